@@ -1,0 +1,139 @@
+/*
+ * thnorm.h -- C ABI of libthnorm.so: LayerNorm / RMSNorm forward and backward for AMD MI355X (gfx950).
+ *
+ * The reference library (TritonHub) has no native boundary: its last host frames before device code are the
+ * Python launch sites in TritonHub/Normalization/layernorm.py and rmsnorm.py.  Each entry point below
+ * replaces one of those launch sites, so a maintainer of the reference can bind it with ctypes in place of
+ * the Triton launch.  The citation on every declaration names the launch site (and device code) replaced.
+ *
+ * Conventions
+ *   - Every pointer is a device pointer owned by the caller.  The library allocates nothing, frees nothing,
+ *     keeps no pointer after the call returns and never synchronises: kernels are enqueued on `stream`
+ *     (a hipStream_t passed as void*; NULL is the default stream) of the CURRENT device.
+ *   - Matrices are row-major (M rows, N columns), unit column stride; row strides are in ELEMENTS.
+ *   - Storage codes: THN_F32 / THN_F16 / THN_BF16 / THN_F64.  Arithmetic is float32 whatever the storage
+ *     (a float64 tensor is narrowed on load and widened on store, as the reference does with
+ *     `.to(tl.float32)`, layernorm.py:31).  Results are rounded to nearest even on store.
+ *   - Return value: THN_OK (0) or a negative THN_E_* code; thn_strerror() names it.  Nothing throws.
+ *   - Thread safe.  The only process state is a per-device cache of the compute-unit count and of kernel
+ *     occupancies, filled on first use.
+ */
+#ifndef THNORM_H_
+#define THNORM_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define THN_ABI_VERSION 1
+
+enum thn_dtype { THN_F32 = 0, THN_F16 = 1, THN_BF16 = 2, THN_F64 = 3 };
+
+enum thn_status {
+    THN_OK = 0,
+    THN_E_DTYPE = -1,         /* unknown storage code */
+    THN_E_FEATURE_DIM = -2,   /* a row is wider than 64 KiB (the reference's RuntimeError, layernorm.py:71-72) */
+    THN_E_NULL = -3,          /* a required pointer is NULL */
+    THN_E_SHAPE = -4,         /* M < 0, N <= 0 or a row stride smaller than N */
+    THN_E_WORKSPACE = -5,     /* workspace smaller than thn_norm_bwd_workspace_bytes() asks for */
+    THN_E_LAUNCH = -6,        /* the HIP runtime refused the launch (hipGetLastError) */
+    THN_E_DEVICE = -7         /* no usable current device */
+};
+
+/* Version of this ABI (THN_ABI_VERSION of the library that was loaded). */
+int thn_abi_version(void);
+
+/* Static description of a status code. */
+const char* thn_strerror(int status);
+
+/*
+ * Forward: y = normalise(x) [* w] [+ b]; writes the float32 row statistics the backward needs.
+ * Replaces `_layernorm_kernel_fwd[(M,)](...)` (layernorm.py:74-86, device code :27-46) when `mean` is not
+ * NULL, and `_rmsnorm_kernel_fwd[(M,)](...)` (rmsnorm.py:60-69, device code :24-38) when `mean` is NULL.
+ *   LayerNorm: mean = sum(x)/N, rstd = 1/sqrt(sum((x-mean)^2)/N + eps), y = (x-mean)*rstd*w + b
+ *   RMSNorm:   rstd = 1/sqrt(sum(x^2)/N + eps),                         y = x*rstd*w        (b must be NULL)
+ * w and b may each be NULL (HAS_WEIGHT / HAS_BIAS false in the reference); both use storage `w_dtype`.
+ * x and y use storage `x_dtype`.  mean, rstd: (M,) float32.  M == 0 is a no-op.
+ */
+int thn_norm_fwd(const void* x, int64_t x_row_stride,
+                 void* y, int64_t y_row_stride,
+                 const void* w, const void* b,
+                 float* mean, float* rstd,
+                 int64_t M, int64_t N, float eps,
+                 int x_dtype, int w_dtype, void* stream);
+
+/*
+ * Bytes of scratch thn_norm_bwd() needs for its per-workgroup partial sums of dW / dB: the counterpart of
+ * the reference's `_dw` / `_db` (sm_count, N) float32 buffers (layernorm.py:183-184, rmsnorm.py:147).
+ * Depends on the current device's compute-unit count.  Returns a negative THN_E_* code on bad arguments,
+ * 0 when neither gradient is requested.
+ */
+int64_t thn_norm_bwd_workspace_bytes(int64_t M, int64_t N, int want_dw, int want_db, int x_dtype);
+
+/*
+ * Backward: dx for every row, and dW / dB summed over rows, from the SAVED statistics.
+ * Replaces `_layernorm_kernel_bwd[(sm_count,)](...)` plus `_dw.sum(0).to(weight.dtype)` /
+ * `_db.sum(0).to(bias.dtype)` (layernorm.py:188-208, device code :113-153) when `mean` is not NULL, and
+ * `_rmsnorm_kernel_bwd[(sm_count,)](...)` plus `_dw.sum(0)` (rmsnorm.py:150-166, device code :92-122) when
+ * `mean` is NULL.
+ *   xhat = (x-mean)*rstd (x*rstd for RMSNorm); wdy = w*dy (dy when w is NULL);
+ *   c1 = sum(xhat*wdy)/N; c2 = sum(wdy)/N (0 for RMSNorm); dx = (wdy - (xhat*c1 + c2))*rstd;
+ *   dW = sum over rows of dy*xhat; dB = sum over rows of dy.
+ * dw / db (storage `w_dtype`, (N,)) may each be NULL when that gradient is not wanted; `workspace` may be
+ * NULL only when both are.  The two-stage sum has a fixed order: results are run-to-run identical.
+ */
+int thn_norm_bwd(const void* x, int64_t x_row_stride,
+                 const void* dy, int64_t dy_row_stride,
+                 void* dx, int64_t dx_row_stride,
+                 const void* w,
+                 const float* mean, const float* rstd,
+                 void* dw, void* db,
+                 void* workspace, int64_t workspace_bytes,
+                 int64_t M, int64_t N,
+                 int x_dtype, int w_dtype, void* stream);
+
+/*
+ * The two stages of thn_norm_bwd() as separate launches, for callers that time or schedule them apart.
+ * Stage 1 replaces the persistent backward kernel alone (layernorm.py:188-206, rmsnorm.py:150-165): it
+ * writes dx and `*num_partials` rows of float32 partial sums into `workspace` (dW partials first, then dB
+ * partials, each (num_partials, N)).  Stage 2 replaces `_dw.sum(0).to(weight.dtype)` / `_db.sum(0)...`
+ * (layernorm.py:207-208, rmsnorm.py:166): it sums the partial rows in a fixed order, in float64, and rounds
+ * once to `w_dtype`.  `want_dw` / `want_db` say which partials stage 1 must produce.
+ */
+int thn_norm_bwd_dx_partials(const void* x, int64_t x_row_stride,
+                             const void* dy, int64_t dy_row_stride,
+                             void* dx, int64_t dx_row_stride,
+                             const void* w,
+                             const float* mean, const float* rstd,
+                             int want_dw, int want_db,
+                             void* workspace, int64_t workspace_bytes, int32_t* num_partials,
+                             int64_t M, int64_t N,
+                             int x_dtype, int w_dtype, void* stream);
+
+int thn_norm_bwd_reduce_partials(const void* workspace, int32_t num_partials,
+                                 void* dw, void* db,
+                                 int64_t N, int w_dtype, void* stream);
+
+/*
+ * Launch-shape control for tuning sweeps (the counterpart of the reference's `triton.autotune` over
+ * num_warps, autotune.py:62-65, which this library replaces by a fixed heuristic on N and the dtype).
+ * `which`: 0 = forward, 1 = backward.  vecs_per_thread / threads_per_row / block_threads select a compiled
+ * kernel shape, blocks_per_cu caps the persistent grid; 0 for any field keeps the heuristic's choice.
+ * Process-wide; meant for benchmarks, not for concurrent production use.  Returns THN_E_SHAPE when no
+ * compiled kernel has that shape.
+ */
+int thn_norm_set_launch_override(int which, int vecs_per_thread, int threads_per_row, int block_threads,
+                                 int blocks_per_cu);
+
+/*
+ * What the heuristic (or the override) would launch for this problem: fills shape[0..4] with
+ * {vecs_per_thread, threads_per_row, block_threads, grid_blocks, vector_path (1) or scalar fallback (0)}.
+ */
+int thn_norm_query_launch(int which, int is_layernorm, int64_t M, int64_t N, int x_dtype, int32_t shape[5]);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* THNORM_H_ */

@@ -1,0 +1,411 @@
+// C ABI of libthnorm.so (declared in include/thnorm.h): argument checks, launch-shape heuristic,
+// persistent-grid sizing and kernel dispatch.  No allocation, no synchronisation, no retained pointers.
+#include "thnorm.h"
+
+#include <atomic>
+#include <mutex>
+#include <unordered_map>
+
+#include "thn_dispatch.h"
+#include "thn_reduce.h"
+
+namespace {
+
+using thn::BwdArgs;
+using thn::FwdArgs;
+using thn::Shape;
+
+constexpr int kMaxDevices = 64;
+constexpr int64_t kMaxRowBytes = 65536;   // the reference's MAX_FUSED_SIZE (layernorm.py:69-72)
+constexpr int kMaxBlocksPerCu = 8;
+
+std::atomic<int> g_cu_count[kMaxDevices];
+
+int current_cu_count() {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+        (void)hipGetLastError();
+        return 0;
+    }
+    int n = g_cu_count[dev].load(std::memory_order_relaxed);
+    if (n == 0) {
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) {
+            (void)hipGetLastError();
+            return 0;
+        }
+        g_cu_count[dev].store(n, std::memory_order_relaxed);
+    }
+    return n;
+}
+
+int elem_bytes(int dtype) {
+    switch (dtype) {
+        case THN_F32: return 4;
+        case THN_F16: return 2;
+        case THN_BF16: return 2;
+        case THN_F64: return 8;
+        default: return 0;
+    }
+}
+
+struct Override {
+    std::atomic<int> k{0}, tpr{0}, block{0}, bpc{0};
+};
+Override g_override[2];
+
+bool shape_compiled(int which, bool aligned, Shape s) {
+#define THN_MATCH(K_, TPR_, BLOCK_) if (s.k == K_ && s.tpr == TPR_ && s.block == BLOCK_) return true;
+    if (!aligned) {
+        THN_SCALAR_SHAPES(THN_MATCH)
+    } else if (which == 0) {
+        THN_FWD_SHAPES(THN_MATCH)
+    } else {
+        THN_BWD_SHAPES(THN_MATCH)
+    }
+#undef THN_MATCH
+    return false;
+}
+
+int launch_fwd(int dtype, bool ln, bool aligned, Shape s, const FwdArgs& a, int grid, hipStream_t st, int* occ) {
+    switch (dtype) {
+        case THN_F32: return thn::launch_fwd_f32(ln, aligned, s, a, grid, st, occ);
+        case THN_F16: return thn::launch_fwd_f16(ln, aligned, s, a, grid, st, occ);
+        case THN_BF16: return thn::launch_fwd_bf16(ln, aligned, s, a, grid, st, occ);
+        default: return thn::launch_fwd_f64(ln, aligned, s, a, grid, st, occ);
+    }
+}
+
+int launch_bwd(int dtype, bool ln, bool aligned, Shape s, const BwdArgs& a, int grid, hipStream_t st, int* occ) {
+    switch (dtype) {
+        case THN_F32: return thn::launch_bwd_f32(ln, aligned, s, a, grid, st, occ);
+        case THN_F16: return thn::launch_bwd_f16(ln, aligned, s, a, grid, st, occ);
+        case THN_BF16: return thn::launch_bwd_bf16(ln, aligned, s, a, grid, st, occ);
+        default: return thn::launch_bwd_f64(ln, aligned, s, a, grid, st, occ);
+    }
+}
+
+// Workgroups of one kernel instance that fit on a compute unit; asked of the runtime once per instance.
+std::mutex g_occ_mutex;
+std::unordered_map<uint64_t, int> g_occ_cache;
+
+int occupancy(int which, int dtype, bool ln, bool aligned, Shape s) {
+    int dev = 0;
+    (void)hipGetDevice(&dev);
+    const uint64_t key = (static_cast<uint64_t>(dev) << 40) | (static_cast<uint64_t>(which) << 36) |
+                         (static_cast<uint64_t>(dtype) << 32) | (static_cast<uint64_t>(ln) << 31) |
+                         (static_cast<uint64_t>(aligned) << 30) | (static_cast<uint64_t>(s.k) << 24) |
+                         (static_cast<uint64_t>(s.tpr) << 12) | static_cast<uint64_t>(s.block);
+    {
+        std::lock_guard<std::mutex> lock(g_occ_mutex);
+        auto it = g_occ_cache.find(key);
+        if (it != g_occ_cache.end()) return it->second;
+    }
+    int occ = 0;
+    int rc;
+    if (which == 0) {
+        FwdArgs dummy{};
+        rc = launch_fwd(dtype, ln, aligned, s, dummy, 0, nullptr, &occ);
+    } else {
+        BwdArgs dummy{};
+        rc = launch_bwd(dtype, ln, aligned, s, dummy, 0, nullptr, &occ);
+    }
+    if (rc != 0 || occ <= 0) occ = 1;
+    if (occ > kMaxBlocksPerCu) occ = kMaxBlocksPerCu;
+    std::lock_guard<std::mutex> lock(g_occ_mutex);
+    g_occ_cache[key] = occ;
+    return occ;
+}
+
+struct Plan {
+    Shape s;
+    int grid;
+    int n_vecs;
+    bool aligned;
+};
+
+constexpr int kTprList[] = {8, 16, 32, 64, 128, 256, 512, 1024};
+
+// The static replacement of the reference's autotune over num_warps (autotune.py:62-65): the fewest
+// threads per row that keep the per-thread register image within budget.
+//   forward : up to 4 vectors per thread;
+//   backward: up to 16 elements per thread (x, dy, w, dW, dB live per element), more only when the row is
+//             too wide for 1024 threads otherwise.
+Shape heuristic_shape(int which, bool ln, bool aligned, int n_vecs, int vec_elems) {
+    (void)ln;
+    int kmax = 4;
+    if (aligned && which == 1) {
+        kmax = 16 / vec_elems;
+        if (kmax < 1) kmax = 1;
+        if (kmax > 4) kmax = 4;
+        while (kmax < 4 && 1024 * kmax < n_vecs) ++kmax;
+    }
+    Shape s{4, 1024, 1024};
+    for (int tpr : kTprList) {
+        if (static_cast<int64_t>(tpr) * kmax >= n_vecs) {
+            s.tpr = tpr;
+            break;
+        }
+    }
+    if (aligned) {
+        s.k = (n_vecs + s.tpr - 1) / s.tpr;
+        if (s.k == 3 && s.tpr < 64) s.k = 4;     // K = 3 is only compiled for TPR >= 64
+        s.block = which == 0 ? (s.tpr > 256 ? s.tpr : 256) : 1024;
+    } else {
+        s.k = 4;
+        s.block = s.tpr > 256 ? s.tpr : 256;
+    }
+    return s;
+}
+
+int plan_launch(int which, bool ln, bool aligned, int64_t M, int64_t N, int dtype, Plan* out) {
+    const int bytes = elem_bytes(dtype);
+    if (bytes == 0) return THN_E_DTYPE;
+    if (M < 0 || N <= 0) return THN_E_SHAPE;
+    if (N * bytes > kMaxRowBytes) return THN_E_FEATURE_DIM;
+    const int vec_elems = 16 / bytes;
+    const int n_vecs = static_cast<int>((N + vec_elems - 1) / vec_elems);
+    const int cus = current_cu_count();
+    if (cus <= 0) return THN_E_DEVICE;
+
+    Shape s = heuristic_shape(which, ln, aligned, n_vecs, vec_elems);
+    const Override& ov = g_override[which];
+    Shape cand = s;
+    if (ov.k.load() > 0) cand.k = ov.k.load();
+    if (ov.tpr.load() > 0) cand.tpr = ov.tpr.load();
+    if (ov.block.load() > 0) cand.block = ov.block.load();
+    else if (cand.block < cand.tpr) cand.block = cand.tpr;
+    if (static_cast<int64_t>(cand.k) * cand.tpr >= n_vecs && cand.block >= cand.tpr &&
+        shape_compiled(which, aligned, cand)) {
+        s = cand;
+    }
+    if (!shape_compiled(which, aligned, s)) return THN_E_SHAPE;
+
+    int bpc = occupancy(which, dtype, ln, aligned, s);
+    const int cap = ov.bpc.load();
+    if (cap > 0 && cap < bpc) bpc = cap;
+    const int rows_per_block = s.block / s.tpr;
+    const int64_t row_blocks = (M + rows_per_block - 1) / rows_per_block;
+    const int64_t grid_max = static_cast<int64_t>(cus) * bpc;
+    int64_t grid = row_blocks;
+    if (grid > grid_max) {
+        const int64_t iters = (row_blocks + grid_max - 1) / grid_max;
+        grid = (row_blocks + iters - 1) / iters;      // every workgroup gets the same number of rows (+-1)
+    }
+    out->s = s;
+    out->grid = static_cast<int>(grid);
+    out->n_vecs = n_vecs;
+    out->aligned = aligned;
+    return THN_OK;
+}
+
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+int64_t partial_pitch(int64_t N) { return (N + 63) / 64 * 64; }
+
+}  // namespace
+
+extern "C" {
+
+int thn_abi_version(void) { return THN_ABI_VERSION; }
+
+const char* thn_strerror(int status) {
+    switch (status) {
+        case THN_OK: return "ok";
+        case THN_E_DTYPE: return "unknown storage type code";
+        case THN_E_FEATURE_DIM: return "This layer norm doesn't support feature dim >= 64KB.";
+        case THN_E_NULL: return "a required pointer is null";
+        case THN_E_SHAPE: return "bad shape, stride or launch shape";
+        case THN_E_WORKSPACE: return "workspace is too small";
+        case THN_E_LAUNCH: return "the HIP runtime refused the kernel launch";
+        case THN_E_DEVICE: return "no usable current HIP device";
+        default: return "unknown status";
+    }
+}
+
+int thn_norm_set_launch_override(int which, int vecs_per_thread, int threads_per_row, int block_threads,
+                                 int blocks_per_cu) {
+    if (which < 0 || which > 1) return THN_E_SHAPE;
+    if (vecs_per_thread < 0 || threads_per_row < 0 || block_threads < 0 || blocks_per_cu < 0) return THN_E_SHAPE;
+    Override& ov = g_override[which];
+    ov.k.store(vecs_per_thread);
+    ov.tpr.store(threads_per_row);
+    ov.block.store(block_threads);
+    ov.bpc.store(blocks_per_cu);
+    return THN_OK;
+}
+
+int thn_norm_query_launch(int which, int is_layernorm, int64_t M, int64_t N, int x_dtype, int32_t shape[5]) {
+    if (which < 0 || which > 1 || shape == nullptr) return THN_E_SHAPE;
+    const int bytes = elem_bytes(x_dtype);
+    if (bytes == 0) return THN_E_DTYPE;
+    Plan p;
+    const bool aligned = N > 0 && (N % (16 / bytes)) == 0;
+    const int rc = plan_launch(which, is_layernorm != 0, aligned, M, N, x_dtype, &p);
+    if (rc != THN_OK) return rc;
+    shape[0] = p.s.k;
+    shape[1] = p.s.tpr;
+    shape[2] = p.s.block;
+    shape[3] = p.grid;
+    shape[4] = p.aligned ? 1 : 0;
+    return THN_OK;
+}
+
+int thn_norm_fwd(const void* x, int64_t x_row_stride, void* y, int64_t y_row_stride, const void* w,
+                 const void* b, float* mean, float* rstd, int64_t M, int64_t N, float eps, int x_dtype,
+                 int w_dtype, void* stream) {
+    const int bytes = elem_bytes(x_dtype);
+    if (bytes == 0 || ((w != nullptr || b != nullptr) && elem_bytes(w_dtype) == 0)) return THN_E_DTYPE;
+    if (M < 0 || N <= 0) return THN_E_SHAPE;
+    if (N * bytes > kMaxRowBytes) return THN_E_FEATURE_DIM;
+    if (M == 0) return THN_OK;
+    if (x == nullptr || y == nullptr || rstd == nullptr) return THN_E_NULL;
+    const bool ln = mean != nullptr;
+    if (!ln && b != nullptr) return THN_E_SHAPE;          // RMSNorm has no bias (rmsnorm.py:13-22)
+    if (x_row_stride < N || y_row_stride < N) return THN_E_SHAPE;
+
+    const int vec_elems = 16 / bytes;
+    const bool aligned = (N % vec_elems) == 0 && aligned16(x) && aligned16(y) && aligned16(w) && aligned16(b) &&
+                         (x_row_stride * bytes) % 16 == 0 && (y_row_stride * bytes) % 16 == 0;
+    Plan p;
+    const int rc = plan_launch(0, ln, aligned, M, N, x_dtype, &p);
+    if (rc != THN_OK) return rc;
+
+    FwdArgs a{};
+    a.x = static_cast<const char*>(x);
+    a.y = static_cast<char*>(y);
+    a.w = w;
+    a.b = b;
+    a.mean = mean;
+    a.rstd = rstd;
+    a.x_stride_bytes = x_row_stride * bytes;
+    a.y_stride_bytes = y_row_stride * bytes;
+    a.M = M;
+    a.n_cols = static_cast<int>(N);
+    a.n_vecs = p.n_vecs;
+    a.w_dtype = w_dtype;
+    a.eps = eps;
+    a.inv_n = 1.0f / static_cast<float>(N);
+    const int lrc = launch_fwd(x_dtype, ln, aligned, p.s, a, p.grid, static_cast<hipStream_t>(stream), nullptr);
+    if (lrc > 0) return THN_E_SHAPE;
+    return lrc == 0 ? THN_OK : THN_E_LAUNCH;
+}
+
+int64_t thn_norm_bwd_workspace_bytes(int64_t M, int64_t N, int want_dw, int want_db, int x_dtype) {
+    const int bytes = elem_bytes(x_dtype);
+    if (bytes == 0) return THN_E_DTYPE;
+    if (M < 0 || N <= 0) return THN_E_SHAPE;
+    if (N * bytes > kMaxRowBytes) return THN_E_FEATURE_DIM;
+    const int n_grads = (want_dw ? 1 : 0) + (want_db ? 1 : 0);
+    if (n_grads == 0 || M == 0) return 0;
+    const int cus = current_cu_count();
+    if (cus <= 0) return THN_E_DEVICE;
+    // Upper bound on the number of partial rows for any launch shape: one per workgroup, at most
+    // kMaxBlocksPerCu workgroups per compute unit, never more than one per row.
+    int64_t parts = static_cast<int64_t>(cus) * kMaxBlocksPerCu;
+    if (parts > M) parts = M;
+    return n_grads * parts * partial_pitch(N) * static_cast<int64_t>(sizeof(float));
+}
+
+int thn_norm_bwd_dx_partials(const void* x, int64_t x_row_stride, const void* dy, int64_t dy_row_stride,
+                             void* dx, int64_t dx_row_stride, const void* w, const float* mean,
+                             const float* rstd, int want_dw, int want_db, void* workspace,
+                             int64_t workspace_bytes, int32_t* num_partials, int64_t M, int64_t N,
+                             int x_dtype, int w_dtype, void* stream) {
+    const int bytes = elem_bytes(x_dtype);
+    if (bytes == 0 || (w != nullptr && elem_bytes(w_dtype) == 0)) return THN_E_DTYPE;
+    if (M < 0 || N <= 0) return THN_E_SHAPE;
+    if (N * bytes > kMaxRowBytes) return THN_E_FEATURE_DIM;
+    if (num_partials != nullptr) *num_partials = 0;
+    if (M == 0) return THN_OK;
+    if (x == nullptr || dy == nullptr || dx == nullptr || rstd == nullptr) return THN_E_NULL;
+    if (x_row_stride < N || dy_row_stride < N || dx_row_stride < N) return THN_E_SHAPE;
+    const bool ln = mean != nullptr;
+    if (!ln) want_db = 0;
+    const int n_grads = (want_dw ? 1 : 0) + (want_db ? 1 : 0);
+    if (n_grads > 0 && (workspace == nullptr || num_partials == nullptr)) return THN_E_NULL;
+    if (n_grads > 0 && !aligned16(workspace)) return THN_E_WORKSPACE;
+
+    const int vec_elems = 16 / bytes;
+    const bool aligned = (N % vec_elems) == 0 && aligned16(x) && aligned16(dy) && aligned16(dx) && aligned16(w) &&
+                         (x_row_stride * bytes) % 16 == 0 && (dy_row_stride * bytes) % 16 == 0 &&
+                         (dx_row_stride * bytes) % 16 == 0;
+    Plan p;
+    const int rc = plan_launch(1, ln, aligned, M, N, x_dtype, &p);
+    if (rc != THN_OK) return rc;
+    const int64_t pitch = partial_pitch(N);
+    const int64_t need = n_grads * static_cast<int64_t>(p.grid) * pitch * static_cast<int64_t>(sizeof(float));
+    if (workspace_bytes < need) return THN_E_WORKSPACE;
+
+    BwdArgs a{};
+    a.x = static_cast<const char*>(x);
+    a.dy = static_cast<const char*>(dy);
+    a.dx = static_cast<char*>(dx);
+    a.w = w;
+    a.mean = mean;
+    a.rstd = rstd;
+    float* ws = static_cast<float*>(workspace);
+    a.dw_part = want_dw ? ws : nullptr;
+    a.db_part = want_db ? ws + (want_dw ? static_cast<int64_t>(p.grid) * pitch : 0) : nullptr;
+    a.x_stride_bytes = x_row_stride * bytes;
+    a.dy_stride_bytes = dy_row_stride * bytes;
+    a.dx_stride_bytes = dx_row_stride * bytes;
+    a.M = M;
+    a.part_pitch = pitch;
+    a.n_cols = static_cast<int>(N);
+    a.n_vecs = p.n_vecs;
+    a.w_dtype = w_dtype;
+    a.inv_n = 1.0f / static_cast<float>(N);
+    const int lrc = launch_bwd(x_dtype, ln, aligned, p.s, a, p.grid, static_cast<hipStream_t>(stream), nullptr);
+    if (lrc > 0) return THN_E_SHAPE;
+    if (lrc < 0) return THN_E_LAUNCH;
+    if (num_partials != nullptr) *num_partials = p.grid;
+    return THN_OK;
+}
+
+// Workspace layout: dW partial rows first (when wanted), dB partial rows after them.  A caller that wants
+// only dB passes dw == NULL and the dB rows start at the beginning.
+int thn_norm_bwd_reduce_partials(const void* workspace, int32_t num_partials, void* dw, void* db, int64_t N,
+                                 int w_dtype, void* stream) {
+    if (elem_bytes(w_dtype) == 0) return THN_E_DTYPE;
+    if (N <= 0 || num_partials < 0) return THN_E_SHAPE;
+    if (dw == nullptr && db == nullptr) return THN_OK;
+    if (workspace == nullptr && num_partials > 0) return THN_E_NULL;
+    const int64_t pitch = partial_pitch(N);
+    const float* ws = static_cast<const float*>(workspace);
+    thn::ReduceArgs r{};
+    int n = 0;
+    if (dw != nullptr) {
+        r.part[n] = ws;
+        r.out[n] = dw;
+        ++n;
+    }
+    if (db != nullptr) {
+        r.part[n] = ws + (dw != nullptr ? static_cast<int64_t>(num_partials) * pitch : 0);
+        r.out[n] = db;
+        ++n;
+    }
+    r.pitch = pitch;
+    r.n_cols = static_cast<int>(N);
+    r.n_parts = num_partials;
+    r.w_dtype = w_dtype;
+    const dim3 grid(static_cast<unsigned>((N + 63) / 64), static_cast<unsigned>(n));
+    hipLaunchKernelGGL(thn::reduce_partials_kernel, grid, dim3(256), 0, static_cast<hipStream_t>(stream), r);
+    return hipGetLastError() == hipSuccess ? THN_OK : THN_E_LAUNCH;
+}
+
+int thn_norm_bwd(const void* x, int64_t x_row_stride, const void* dy, int64_t dy_row_stride, void* dx,
+                 int64_t dx_row_stride, const void* w, const float* mean, const float* rstd, void* dw,
+                 void* db, void* workspace, int64_t workspace_bytes, int64_t M, int64_t N, int x_dtype,
+                 int w_dtype, void* stream) {
+    if ((dw != nullptr || db != nullptr) && elem_bytes(w_dtype) == 0) return THN_E_DTYPE;
+    if (mean == nullptr && db != nullptr) return THN_E_SHAPE;     // RMSNorm has no bias gradient
+    int32_t parts = 0;
+    const int rc = thn_norm_bwd_dx_partials(x, x_row_stride, dy, dy_row_stride, dx, dx_row_stride, w, mean, rstd,
+                                            dw != nullptr, db != nullptr, workspace, workspace_bytes, &parts,
+                                            M, N, x_dtype, w_dtype, stream);
+    if (rc != THN_OK) return rc;
+    // M == 0: no partial rows; the reduction then writes zeros, the sum of an empty set of rows.
+    return thn_norm_bwd_reduce_partials(workspace, parts, dw, db, N, w_dtype, stream);
+}
+
+}  // extern "C"

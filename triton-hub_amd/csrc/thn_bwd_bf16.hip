@@ -1,0 +1,6 @@
+// Backward kernel instances for BF16 storage.
+#include "thn_dispatch.h"
+
+namespace thn {
+THN_DEFINE_BWD_LAUNCHER(bf16, BF16)
+}  // namespace thn

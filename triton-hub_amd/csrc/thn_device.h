@@ -1,0 +1,346 @@
+// Device-side building blocks shared by the forward and backward kernels: 128-bit row I/O for the four
+// storage types, float32 <-> storage conversion, wave64 DPP reductions and the LDS cross-wave reduction.
+// gfx950 (CDNA4) only.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace thn {
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+
+enum : int { kF32 = 0, kF16 = 1, kBF16 = 2, kF64 = 3 };
+
+// Bit casts take their operand BY VALUE in a scalar: applying __builtin_bit_cast directly to an element
+// of an ext_vector (v[i]) reads element 0 whatever i is with this compiler.
+__device__ __forceinline__ float as_f32(uint32_t u) { return __builtin_bit_cast(float, u); }
+__device__ __forceinline__ uint32_t as_u32(float f) { return __builtin_bit_cast(uint32_t, f); }
+
+#ifndef THN_NT_LOAD
+#define THN_NT_LOAD 1
+#endif
+#ifndef THN_NT_STORE
+#define THN_NT_STORE 1
+#endif
+
+__device__ __forceinline__ u32x4 ld128(const void* p) {
+#if THN_NT_LOAD
+    return __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
+#else
+    return *reinterpret_cast<const u32x4*>(p);
+#endif
+}
+__device__ __forceinline__ void st128(void* p, u32x4 v) {
+#if THN_NT_STORE
+    __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(p));
+#else
+    *reinterpret_cast<u32x4*>(p) = v;
+#endif
+}
+
+// s_waitcnt vmcnt(0): every vector-memory operation this wave has issued is complete.  Placed once in front
+// of the row loop so that the loop is entered with nothing outstanding: the compiler derives the loop's own
+// waits from the number of operations in flight on every path into the loop header, and an entry path with
+// the prologue's loads still pending makes it wait for more than the loop body needs on every trip.
+__device__ __forceinline__ void drain_vector_memory() { __builtin_amdgcn_s_waitcnt(0x0F70); }
+
+// ---------------------------------------------------------------------------------------------------
+// Storage traits.  A "vector" is 16 bytes of a row: VEC elements.  unpack() widens a vector to float32,
+// pack() narrows with round-to-nearest-even (v_cvt_pk_bf16_f32 / v_cvt_f16_f32 / v_cvt_f64_f32).
+// ---------------------------------------------------------------------------------------------------
+struct F32 {
+    static constexpr int kCode = kF32, kBytes = 4, VEC = 4;
+    __device__ static __forceinline__ void unpack(u32x4 v, float (&f)[VEC]) {
+        uint32_t a = v[0], b = v[1], c = v[2], d = v[3];
+        f[0] = as_f32(a); f[1] = as_f32(b); f[2] = as_f32(c); f[3] = as_f32(d);
+    }
+    __device__ static __forceinline__ u32x4 pack(const float (&f)[VEC]) {
+        u32x4 v;
+        v[0] = as_u32(f[0]); v[1] = as_u32(f[1]); v[2] = as_u32(f[2]); v[3] = as_u32(f[3]);
+        return v;
+    }
+    __device__ static __forceinline__ float load1(const void* p, int64_t i) {
+        return reinterpret_cast<const float*>(p)[i];
+    }
+    __device__ static __forceinline__ void store1(void* p, int64_t i, float f) {
+        reinterpret_cast<float*>(p)[i] = f;
+    }
+};
+
+struct F16 {
+    static constexpr int kCode = kF16, kBytes = 2, VEC = 8;
+    __device__ static __forceinline__ void unpack_pair(uint32_t u, float& lo, float& hi) {
+        half2_t h = __builtin_bit_cast(half2_t, u);
+        lo = static_cast<float>(h[0]);
+        hi = static_cast<float>(h[1]);
+    }
+    __device__ static __forceinline__ void unpack(u32x4 v, float (&f)[VEC]) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            uint32_t u = v[i];
+            unpack_pair(u, f[2 * i], f[2 * i + 1]);
+        }
+    }
+    __device__ static __forceinline__ u32x4 pack(const float (&f)[VEC]) {
+        u32x4 v;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            half2_t h;
+            h[0] = static_cast<_Float16>(f[2 * i]);
+            h[1] = static_cast<_Float16>(f[2 * i + 1]);
+            v[i] = __builtin_bit_cast(uint32_t, h);
+        }
+        return v;
+    }
+    __device__ static __forceinline__ float load1(const void* p, int64_t i) {
+        return static_cast<float>(reinterpret_cast<const _Float16*>(p)[i]);
+    }
+    __device__ static __forceinline__ void store1(void* p, int64_t i, float f) {
+        reinterpret_cast<_Float16*>(p)[i] = static_cast<_Float16>(f);
+    }
+};
+
+struct BF16 {
+    static constexpr int kCode = kBF16, kBytes = 2, VEC = 8;
+    __device__ static __forceinline__ void unpack_pair(uint32_t u, float& lo, float& hi) {
+        lo = as_f32(u << 16);
+        hi = as_f32(u & 0xffff0000u);
+    }
+    __device__ static __forceinline__ void unpack(u32x4 v, float (&f)[VEC]) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            uint32_t u = v[i];
+            unpack_pair(u, f[2 * i], f[2 * i + 1]);
+        }
+    }
+    __device__ static __forceinline__ u32x4 pack(const float (&f)[VEC]) {
+        u32x4 v;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            bf16x2_t h;
+            h[0] = static_cast<__bf16>(f[2 * i]);
+            h[1] = static_cast<__bf16>(f[2 * i + 1]);
+            v[i] = __builtin_bit_cast(uint32_t, h);
+        }
+        return v;
+    }
+    __device__ static __forceinline__ float load1(const void* p, int64_t i) {
+        return as_f32(static_cast<uint32_t>(reinterpret_cast<const uint16_t*>(p)[i]) << 16);
+    }
+    __device__ static __forceinline__ void store1(void* p, int64_t i, float f) {
+        reinterpret_cast<__bf16*>(p)[i] = static_cast<__bf16>(f);
+    }
+};
+
+struct F64 {
+    static constexpr int kCode = kF64, kBytes = 8, VEC = 2;
+    __device__ static __forceinline__ void unpack(u32x4 v, float (&f)[VEC]) {
+        uint32_t a = v[0], b = v[1], c = v[2], d = v[3];
+        uint64_t lo = (static_cast<uint64_t>(b) << 32) | a;
+        uint64_t hi = (static_cast<uint64_t>(d) << 32) | c;
+        f[0] = static_cast<float>(__builtin_bit_cast(double, lo));
+        f[1] = static_cast<float>(__builtin_bit_cast(double, hi));
+    }
+    __device__ static __forceinline__ u32x4 pack(const float (&f)[VEC]) {
+        uint64_t lo = __builtin_bit_cast(uint64_t, static_cast<double>(f[0]));
+        uint64_t hi = __builtin_bit_cast(uint64_t, static_cast<double>(f[1]));
+        u32x4 v;
+        v[0] = static_cast<uint32_t>(lo); v[1] = static_cast<uint32_t>(lo >> 32);
+        v[2] = static_cast<uint32_t>(hi); v[3] = static_cast<uint32_t>(hi >> 32);
+        return v;
+    }
+    __device__ static __forceinline__ float load1(const void* p, int64_t i) {
+        return static_cast<float>(reinterpret_cast<const double*>(p)[i]);
+    }
+    __device__ static __forceinline__ void store1(void* p, int64_t i, float f) {
+        reinterpret_cast<double*>(p)[i] = static_cast<double>(f);
+    }
+};
+
+// One element of a weight / bias vector whose storage type is only known at run time (cold paths only).
+__device__ __forceinline__ void store_param(void* p, int dtype, int64_t i, float f) {
+    switch (dtype) {
+        case kF32: F32::store1(p, i, f); break;
+        case kF16: F16::store1(p, i, f); break;
+        case kBF16: BF16::store1(p, i, f); break;
+        default: F64::store1(p, i, f); break;
+    }
+}
+
+// VEC consecutive parameter elements of storage type WT starting at column c0, widened to float32, fetched
+// with the widest loads their size allows (the 128-bit path guarantees that the chunk is inside the vector
+// and naturally aligned: the parameter pointer is 16-byte aligned and c0 is a multiple of VEC).
+template <typename WT, int VEC>
+__device__ __forceinline__ void load_param_chunk(const void* p, int c0, float (&out)[VEC]) {
+    constexpr int BYTES = VEC * WT::kBytes;
+    const char* src = static_cast<const char*>(p) + static_cast<int64_t>(c0) * WT::kBytes;
+    if constexpr (BYTES >= 16) {
+        constexpr int PIECES = BYTES / 16;
+        constexpr int EPP = WT::VEC;            // elements per 16-byte piece
+        u32x4 raw[PIECES];
+#pragma unroll
+        for (int i = 0; i < PIECES; ++i) raw[i] = *reinterpret_cast<const u32x4*>(src + 16 * i);
+#pragma unroll
+        for (int i = 0; i < PIECES; ++i) {
+            float f[EPP];
+            WT::unpack(raw[i], f);
+#pragma unroll
+            for (int j = 0; j < EPP; ++j) out[i * EPP + j] = f[j];
+        }
+    } else if constexpr (WT::kBytes == 4) {       // two float32 (VEC == 2)
+        const uint2 raw = *reinterpret_cast<const uint2*>(src);
+        out[0] = as_f32(raw.x);
+        out[1] = as_f32(raw.y);
+    } else {                                      // 16-bit parameters under a wider row type: 4 or 8 bytes
+        static_assert(WT::kBytes == 2 && (VEC == 2 || VEC == 4), "chunk shape");
+        if constexpr (VEC == 4) {
+            const uint2 raw = *reinterpret_cast<const uint2*>(src);
+            WT::unpack_pair(raw.x, out[0], out[1]);
+            WT::unpack_pair(raw.y, out[2], out[3]);
+        } else {
+            const uint32_t raw = *reinterpret_cast<const uint32_t*>(src);
+            WT::unpack_pair(raw, out[0], out[1]);
+        }
+    }
+}
+
+// The K*VEC weight (or bias) elements of a thread's (clamped) vector slots, widened to float32.  The
+// storage type is only known at run time: one uniform branch on it, then independent loads at always valid
+// columns.  voff[k] is the slot's byte offset in a row on the 128-bit path (one wide load per slot), its
+// vector index on the element-wise path (element loads; columns past the row end read as `fill`).
+template <typename WT, int K, int VEC, int ROW_BYTES_PER_ELEM, bool ALIGNED>
+__device__ __forceinline__ void load_params_as(float (&out)[K][VEC], const void* p, const int (&voff)[K],
+                                               int n_cols, float fill) {
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+        if constexpr (ALIGNED) {
+            load_param_chunk<WT, VEC>(p, voff[k] / ROW_BYTES_PER_ELEM, out[k]);
+        } else {
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+                const int c = voff[k] * VEC + e;
+                const float v = WT::load1(p, c < n_cols ? c : n_cols - 1);
+                out[k][e] = c < n_cols ? v : fill;
+            }
+        }
+    }
+}
+
+template <int K, int VEC, bool ALIGNED>
+__device__ __forceinline__ void load_params_clamped(float (&out)[K][VEC], const void* p, int dtype,
+                                                    const int (&voff)[K], int n_cols, float fill) {
+    constexpr int RB = 16 / VEC;    // bytes per row element: byte offset / RB = column
+    if (p == nullptr) {
+#pragma unroll
+        for (int k = 0; k < K; ++k)
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) out[k][e] = fill;
+        return;
+    }
+    switch (dtype) {
+        case kF32: load_params_as<F32, K, VEC, RB, ALIGNED>(out, p, voff, n_cols, fill); break;
+        case kF16: load_params_as<F16, K, VEC, RB, ALIGNED>(out, p, voff, n_cols, fill); break;
+        case kBF16: load_params_as<BF16, K, VEC, RB, ALIGNED>(out, p, voff, n_cols, fill); break;
+        default: load_params_as<F64, K, VEC, RB, ALIGNED>(out, p, voff, n_cols, fill); break;
+    }
+}
+
+// ---------------------------------------------------------------------------------------------------
+// Element-wise row I/O for rows that cannot use 128-bit accesses (N not a multiple of VEC, or a pointer or
+// row stride that is not a multiple of 16 bytes): the same 16-byte register image is assembled from element
+// loads with a per-column bound, so every other part of the kernels is shared with the 128-bit path.
+// ---------------------------------------------------------------------------------------------------
+template <typename T>
+__device__ __forceinline__ u32x4 load_vec_elems(const char* row, int vec, int n_cols) {
+    float f[T::VEC];
+#pragma unroll
+    for (int e = 0; e < T::VEC; ++e) {
+        const int c = vec * T::VEC + e;
+        const float v = T::load1(row, c < n_cols ? c : n_cols - 1);
+        f[e] = c < n_cols ? v : 0.0f;
+    }
+    return T::pack(f);   // exact: every element came from storage type T
+}
+
+template <typename T>
+__device__ __forceinline__ void store_vec_elems(char* row, int vec, int n_cols, const float (&f)[T::VEC]) {
+#pragma unroll
+    for (int e = 0; e < T::VEC; ++e) {
+        const int c = vec * T::VEC + e;
+        if (c < n_cols) T::store1(row, c, f[e]);
+    }
+}
+
+// ---------------------------------------------------------------------------------------------------
+// Wave64 all-reduce (sum) over aligned groups of W lanes, W in {8, 16, 32, 64}.  The first four steps
+// are DPP modifiers fused into v_add_f32 (no LDS traffic); the 16- and 32-lane exchanges use the gfx950
+// v_permlane16_swap / v_permlane32_swap instructions.  Every lane of a group ends with the group's sum,
+// and all lanes of a group add the same values in the same tree, so the result is identical on all of them.
+// ---------------------------------------------------------------------------------------------------
+template <int CTRL>
+__device__ __forceinline__ float dpp_mov(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true));
+}
+
+template <int W>
+__device__ __forceinline__ float group_allreduce(float v) {
+    static_assert(W == 8 || W == 16 || W == 32 || W == 64, "group width");
+    v += dpp_mov<0xB1>(v);    // quad_perm [1,0,3,2]: lane ^ 1
+    v += dpp_mov<0x4E>(v);    // quad_perm [2,3,0,1]: lane ^ 2
+    v += dpp_mov<0x141>(v);   // row_half_mirror: the other quad of each 8 lanes
+    if constexpr (W >= 16) v += dpp_mov<0x140>(v);   // row_mirror: the other half of each 16 lanes
+    if constexpr (W >= 32) {
+        const uint32_t u = as_u32(v);
+        auto r = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+        const uint32_t a = r[0], b = r[1];
+        v = as_f32(a) + as_f32(b);
+    }
+    if constexpr (W >= 64) {
+        const uint32_t u = as_u32(v);
+        auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+        const uint32_t a = r[0], b = r[1];
+        v = as_f32(a) + as_f32(b);
+    }
+    return v;
+}
+
+// Sum NV values over the TPR threads that share a row.  TPR <= 64: pure register exchange.  TPR > 64: each
+// wave publishes its sums in an LDS slot, one workgroup barrier, every thread adds the TPR/64 slots of its
+// row in a fixed order.  The slots are double buffered on `phase`, so one barrier per call is enough: a
+// slot is rewritten two calls later, and no wave can pass the barrier in between before all have read it.
+// All threads of the workgroup must call this together when TPR > 64.
+template <int TPR, int G, int NV>
+__device__ __forceinline__ void row_allreduce(float (&v)[NV], float* red, int& phase, int g, int t) {
+    constexpr int W = TPR < 64 ? TPR : 64;
+#pragma unroll
+    for (int i = 0; i < NV; ++i) v[i] = group_allreduce<W>(v[i]);
+    if constexpr (TPR > 64) {
+        constexpr int WPR = TPR / 64;
+        constexpr int NVP = NV == 3 ? 4 : NV;
+        float* slot = red + (((phase & 1) * G + g) * WPR) * NVP;
+        const int wv = t >> 6;
+        if ((t & 63) == 0) {
+#pragma unroll
+            for (int i = 0; i < NV; ++i) slot[wv * NVP + i] = v[i];
+        }
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < NV; ++i) v[i] = 0.0f;
+#pragma unroll
+        for (int w = 0; w < WPR; ++w) {
+#pragma unroll
+            for (int i = 0; i < NV; ++i) v[i] += slot[w * NVP + i];
+        }
+        ++phase;
+    }
+}
+
+template <int TPR, int G, int NV>
+struct RedSmem {
+    static constexpr int kFloats = TPR > 64 ? 2 * G * (TPR / 64) * (NV == 3 ? 4 : NV) : 1;
+};
+
+}  // namespace thn

@@ -1,0 +1,110 @@
+// Maps a run-time (dtype, flavour, shape) to one compiled kernel instance.  Each storage type has its own
+// pair of translation units (thn_fwd_<dtype>.hip, thn_bwd_<dtype>.hip) that expands these lists, so the types compile in parallel.
+#pragma once
+
+#include "thn_kernels.h"
+
+namespace thn {
+
+struct Shape {
+    int k;       // vectors (16 bytes) per thread
+    int tpr;     // threads per row
+    int block;   // threads per workgroup
+};
+
+// X(K, TPR, BLOCK): shapes of the 128-bit path.
+#define THN_FWD_SHAPES(X)                                                            \
+    X(1, 8, 256) X(2, 8, 256) X(4, 8, 256)                                           \
+    X(1, 16, 256) X(2, 16, 256) X(4, 16, 256)                                        \
+    X(1, 32, 256) X(2, 32, 256) X(4, 32, 256)                                        \
+    X(1, 64, 256) X(2, 64, 256) X(3, 64, 256) X(4, 64, 256)                          \
+    X(1, 128, 256) X(2, 128, 256) X(3, 128, 256) X(4, 128, 256)                      \
+    X(1, 256, 256) X(2, 256, 256) X(3, 256, 256) X(4, 256, 256)                      \
+    X(1, 512, 512) X(2, 512, 512) X(3, 512, 512) X(4, 512, 512)                      \
+    X(1, 1024, 1024) X(2, 1024, 1024) X(3, 1024, 1024) X(4, 1024, 1024)
+
+#define THN_BWD_SHAPES_B(X, B)                                                       \
+    X(1, 8, B) X(2, 8, B) X(4, 8, B)                                                 \
+    X(1, 16, B) X(2, 16, B) X(4, 16, B)                                              \
+    X(1, 32, B) X(2, 32, B) X(4, 32, B)                                              \
+    X(1, 64, B) X(2, 64, B) X(3, 64, B) X(4, 64, B)                                  \
+    X(1, 128, B) X(2, 128, B) X(3, 128, B) X(4, 128, B)                              \
+    X(1, 256, B) X(2, 256, B) X(3, 256, B) X(4, 256, B)
+
+#define THN_BWD_SHAPES(X)                                                            \
+    THN_BWD_SHAPES_B(X, 256) THN_BWD_SHAPES_B(X, 512) THN_BWD_SHAPES_B(X, 1024)      \
+    X(1, 512, 512) X(2, 512, 512) X(3, 512, 512) X(4, 512, 512)                      \
+    X(1, 512, 1024) X(2, 512, 1024) X(3, 512, 1024) X(4, 512, 1024)                  \
+    X(1, 1024, 1024) X(2, 1024, 1024) X(3, 1024, 1024) X(4, 1024, 1024)
+
+// Shapes of the element-wise (unaligned) path: four vectors per thread, any row width.
+#define THN_SCALAR_SHAPES(X)                                                         \
+    X(4, 8, 256) X(4, 16, 256) X(4, 32, 256) X(4, 64, 256) X(4, 128, 256)            \
+    X(4, 256, 256) X(4, 512, 512) X(4, 1024, 1024)
+
+// Return value of the launchers: 0 launched (or occupancy written), 1 no such instance, <0 HIP error.
+// When `occupancy` is not null the kernel is not launched; *occupancy receives the number of workgroups
+// of that instance that fit on one compute unit.
+#define THN_DECLARE_LAUNCHERS(NAME)                                                                        \
+    int launch_fwd_##NAME(bool ln, bool aligned, Shape s, const FwdArgs& a, int grid, hipStream_t st,      \
+                          int* occupancy);                                                                 \
+    int launch_bwd_##NAME(bool ln, bool aligned, Shape s, const BwdArgs& a, int grid, hipStream_t st,      \
+                          int* occupancy);
+
+THN_DECLARE_LAUNCHERS(f32)
+THN_DECLARE_LAUNCHERS(f16)
+THN_DECLARE_LAUNCHERS(bf16)
+THN_DECLARE_LAUNCHERS(f64)
+
+template <typename Args>
+inline int run_kernel(void (*kern)(const Args), const Args& a, int grid, int block, hipStream_t st,
+                      int* occupancy) {
+    if (occupancy != nullptr) {
+        int n = 0;
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, kern, block, 0) != hipSuccess) {
+            (void)hipGetLastError();
+            return -1;
+        }
+        *occupancy = n;
+        return 0;
+    }
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(block), 0, st, a);
+    return hipGetLastError() == hipSuccess ? 0 : -1;
+}
+
+#define THN_CASE(KERNEL, ARGS_T, AL, K_, TPR_, BLOCK_)                                                     \
+    if (s.k == K_ && s.tpr == TPR_ && s.block == BLOCK_) {                                                 \
+        return ln ? run_kernel<ARGS_T>(KERNEL<T, true, K_, TPR_, BLOCK_, AL>, a, grid, BLOCK_, st, occupancy) \
+                  : run_kernel<ARGS_T>(KERNEL<T, false, K_, TPR_, BLOCK_, AL>, a, grid, BLOCK_, st, occupancy); \
+    }
+
+#define THN_DEFINE_FWD_LAUNCHER(NAME, TYPE)                                                                \
+    int launch_fwd_##NAME(bool ln, bool aligned, Shape s, const FwdArgs& a, int grid, hipStream_t st,      \
+                          int* occupancy) {                                                                \
+        using T = TYPE;                                                                                    \
+        if (aligned) {                                                                                     \
+            THN_FWD_SHAPES(THN_FWD_AL)                                                                     \
+        } else {                                                                                           \
+            THN_SCALAR_SHAPES(THN_FWD_SC)                                                                  \
+        }                                                                                                  \
+        return 1;                                                                                          \
+    }
+
+#define THN_DEFINE_BWD_LAUNCHER(NAME, TYPE)                                                                \
+    int launch_bwd_##NAME(bool ln, bool aligned, Shape s, const BwdArgs& a, int grid, hipStream_t st,      \
+                          int* occupancy) {                                                                \
+        using T = TYPE;                                                                                    \
+        if (aligned) {                                                                                     \
+            THN_BWD_SHAPES(THN_BWD_AL)                                                                     \
+        } else {                                                                                           \
+            THN_SCALAR_SHAPES(THN_BWD_SC)                                                                  \
+        }                                                                                                  \
+        return 1;                                                                                          \
+    }
+
+#define THN_FWD_AL(K_, TPR_, BLOCK_) THN_CASE(norm_fwd_kernel, FwdArgs, true, K_, TPR_, BLOCK_)
+#define THN_FWD_SC(K_, TPR_, BLOCK_) THN_CASE(norm_fwd_kernel, FwdArgs, false, K_, TPR_, BLOCK_)
+#define THN_BWD_AL(K_, TPR_, BLOCK_) THN_CASE(norm_bwd_kernel, BwdArgs, true, K_, TPR_, BLOCK_)
+#define THN_BWD_SC(K_, TPR_, BLOCK_) THN_CASE(norm_bwd_kernel, BwdArgs, false, K_, TPR_, BLOCK_)
+
+}  // namespace thn

@@ -1,0 +1,387 @@
+// The forward and backward row kernels.
+//
+// Work decomposition (the same for both): a row of N elements is 16-byte "vectors"; TPR threads share a
+// row and thread t owns vectors t, t+TPR, ..., t+(K-1)*TPR, so a wave touches contiguous 1 KiB segments.
+// A workgroup of BLOCK threads holds G = BLOCK/TPR rows at a time and walks the matrix with a grid stride
+// of gridDim.x*G rows (a persistent grid: the whole chip works on one contiguous window of rows at any
+// moment).  A row lives in registers between its load and its store: x (and dy) are read from HBM exactly
+// once per pass.
+//
+// The row loop is branch free on the 128-bit path.  The vectors of the NEXT row are requested before the
+// current row is reduced, and the hardware returns vector-memory operations in issue order, so the only
+// wait in the loop is "all but the newest loads have landed" (s_waitcnt vmcnt(n)); any branch around a load
+// or store would force the compiler to wait for everything (vmcnt(0)) and serialise the loop on memory
+// latency.  To stay branch free, slots that have no work -- a row past the end in the last grid-stride
+// step, a vector slot past the row end when K*TPR > N/VEC -- are CLAMPED onto the last valid row / vector:
+// they load, compute and store exactly what the owner of that row / vector does (same inputs, same
+// instruction sequence, hence the same bits to the same address), and are only masked out of the row sums
+// and of the dW / dB accumulators.
+#pragma once
+
+#include "thn_device.h"
+
+namespace thn {
+
+struct FwdArgs {
+    const char* x;
+    char* y;
+    const void* w;      // may be null
+    const void* b;      // may be null
+    float* mean;        // null for RMSNorm
+    float* rstd;
+    int64_t x_stride_bytes;
+    int64_t y_stride_bytes;
+    int64_t M;
+    int n_cols;         // N
+    int n_vecs;         // ceil(N / VEC)
+    int w_dtype;
+    float eps;
+    float inv_n;
+};
+
+struct BwdArgs {
+    const char* x;
+    const char* dy;
+    char* dx;
+    const void* w;      // may be null
+    const float* mean;  // null for RMSNorm
+    const float* rstd;
+    float* dw_part;     // (gridDim.x, part_pitch) float32, may be null
+    float* db_part;     // (gridDim.x, part_pitch) float32, may be null
+    int64_t x_stride_bytes;
+    int64_t dy_stride_bytes;
+    int64_t dx_stride_bytes;
+    int64_t M;
+    int64_t part_pitch; // floats between partial rows
+    int n_cols;
+    int n_vecs;
+    int w_dtype;
+    float inv_n;
+};
+
+// Loads the K vectors of one row.  `row` is already clamped to a valid row; voff[k] is the byte offset of
+// the (clamped) vector slot k on the 128-bit path and the vector index on the element-wise path.
+template <typename T, int K, bool ALIGNED>
+__device__ __forceinline__ void load_row(u32x4 (&dst)[K], const char* base, int64_t stride_bytes, int64_t row,
+                                         const int (&voff)[K], int n_cols) {
+    const char* p = base + row * stride_bytes;
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+        if constexpr (ALIGNED) dst[k] = ld128(p + voff[k]);
+        else dst[k] = load_vec_elems<T>(p, voff[k], n_cols);
+    }
+}
+
+template <typename T, bool ALIGNED>
+__device__ __forceinline__ void store_row_vec(char* rowp, int voff, int n_cols, const float (&f)[T::VEC]) {
+    if constexpr (ALIGNED) st128(rowp + voff, T::pack(f));
+    else store_vec_elems<T>(rowp, voff, n_cols, f);
+}
+
+// ---------------------------------------------------------------------------------------------------
+// Forward.  LayerNorm: mean0 = sum(x)/N; d = x - mean0; delta = sum(d)/N; var = sum(d^2)/N - delta^2;
+// rstd = 1/sqrt(var + eps); y = (d - delta)*rstd*w + b; saved mean = mean0 + delta.  The second pass runs
+// on registers; carrying delta (the float32 rounding error of mean0) keeps y accurate when |mean| >> std.
+// RMSNorm: rstd = 1/sqrt(sum(x^2)/N + eps); y = x*rstd*w.
+// ---------------------------------------------------------------------------------------------------
+template <typename T, bool LN, int K, int TPR, int BLOCK, bool ALIGNED>
+__global__ void __launch_bounds__(BLOCK) norm_fwd_kernel(const FwdArgs a) {
+    constexpr int VEC = T::VEC;
+    constexpr int G = BLOCK / TPR;
+    static_assert(BLOCK % TPR == 0 && G >= 1, "a workgroup holds whole rows");
+    __shared__ float red[RedSmem<TPR, G, 2>::kFloats];
+
+    const int tid = threadIdx.x;
+    const int g = tid / TPR;
+    const int t = tid % TPR;
+    int phase = 0;
+
+    // Per-slot masks (1 = this thread owns real columns there) and clamped offsets.
+    int voff[K];
+    bool own[K];
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+        const int v = t + k * TPR;
+        const int vc = v < a.n_vecs ? v : a.n_vecs - 1;
+        voff[k] = ALIGNED ? vc * 16 : vc;
+        own[k] = v < a.n_vecs;
+    }
+
+    const int64_t rows_per_iter = static_cast<int64_t>(gridDim.x) * G;
+    const int64_t last_row = a.M - 1;
+    int64_t row_raw = static_cast<int64_t>(blockIdx.x) * G + g;
+    int64_t row = row_raw < a.M ? row_raw : last_row;
+    u32x4 cur[K];
+    load_row<T, K, ALIGNED>(cur, a.x, a.x_stride_bytes, row, voff, a.n_cols);   // first, so it overlaps the params
+
+    // Parameters of the clamped slot, so that a clamped slot reproduces its owner's output bit for bit.
+    float wr[K][VEC];
+    float br[LN ? K : 1][VEC];
+    load_params_clamped<K, VEC, ALIGNED>(wr, a.w, a.w_dtype, voff, a.n_cols, 1.0f);
+    if constexpr (LN) load_params_clamped<K, VEC, ALIGNED>(br, a.b, a.w_dtype, voff, a.n_cols, 0.0f);
+
+    drain_vector_memory();
+    for (int64_t base = static_cast<int64_t>(blockIdx.x) * G; base < a.M; base += rows_per_iter) {
+        const int64_t nrow_raw = row_raw + rows_per_iter;
+        const int64_t nrow = nrow_raw < a.M ? nrow_raw : last_row;
+        u32x4 nxt[K];
+        load_row<T, K, ALIGNED>(nxt, a.x, a.x_stride_bytes, nrow, voff, a.n_cols);
+
+        float xf[K][VEC];
+#pragma unroll
+        for (int k = 0; k < K; ++k) T::unpack(cur[k], xf[k]);
+
+        float mean = 0.0f, rstd, delta = 0.0f;
+        if constexpr (LN) {
+            float s[1] = {0.0f};
+#pragma unroll
+            for (int k = 0; k < K; ++k) {
+                float sk = 0.0f;
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) sk += xf[k][e];   // element path: absent columns load as 0
+                s[0] += own[k] ? sk : 0.0f;
+            }
+            row_allreduce<TPR, G, 1>(s, red, phase, g, t);
+            const float mean0 = s[0] * a.inv_n;
+            float q[2] = {0.0f, 0.0f};
+#pragma unroll
+            for (int k = 0; k < K; ++k) {
+                float q0 = 0.0f, q1 = 0.0f;
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) {
+                    float d = xf[k][e] - mean0;
+                    if constexpr (!ALIGNED) d = (voff[k] * VEC + e < a.n_cols) ? d : 0.0f;
+                    xf[k][e] = d;
+                    q0 += d;
+                    q1 = fmaf(d, d, q1);
+                }
+                q[0] += own[k] ? q0 : 0.0f;
+                q[1] += own[k] ? q1 : 0.0f;
+            }
+            row_allreduce<TPR, G, 2>(q, red, phase, g, t);
+            delta = q[0] * a.inv_n;
+            const float var = fmaxf(fmaf(-delta, delta, q[1] * a.inv_n), 0.0f);
+            rstd = 1.0f / sqrtf(var + a.eps);
+            mean = mean0 + delta;
+        } else {
+            float q[1] = {0.0f};
+#pragma unroll
+            for (int k = 0; k < K; ++k) {
+                float qk = 0.0f;
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) qk = fmaf(xf[k][e], xf[k][e], qk);
+                q[0] += own[k] ? qk : 0.0f;
+            }
+            row_allreduce<TPR, G, 1>(q, red, phase, g, t);
+            rstd = 1.0f / sqrtf(q[0] * a.inv_n + a.eps);
+        }
+
+        char* yrow = a.y + row * a.y_stride_bytes;
+#pragma unroll
+        for (int k = 0; k < K; ++k) {
+            float yf[VEC];
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+                if constexpr (LN) yf[e] = fmaf((xf[k][e] - delta) * rstd, wr[k][e], br[k][e]);
+                else yf[e] = xf[k][e] * rstd * wr[k][e];
+            }
+            store_row_vec<T, ALIGNED>(yrow, voff[k], a.n_cols, yf);
+        }
+        // Every thread of the row stores the same two words to the same address (one request per wave): a
+        // store under "if (t == 0)" would be a branch, see the note on branches at the top of this file.
+        if constexpr (LN) a.mean[row] = mean;
+        a.rstd[row] = rstd;
+
+#pragma unroll
+        for (int k = 0; k < K; ++k) cur[k] = nxt[k];
+        row_raw = nrow_raw;
+        row = nrow;
+    }
+}
+
+// ---------------------------------------------------------------------------------------------------
+// Backward.  With m, r the saved float32 mean and rstd of the row:
+//   u = (x - m)*r (x*r for RMSNorm); wdy = w*dy; one reduction round of {sum(u*wdy), sum(wdy), sum(u)};
+//   LayerNorm: dlt = sum(u)/N (the part of the mean that float32 m could not hold), xhat = u - dlt,
+//              c2 = sum(wdy)/N, c1 = sum(u*wdy)/N - dlt*c2  (= sum(xhat*wdy)/N);
+//   RMSNorm:   xhat = u, c1 = sum(u*wdy)/N, c2 = 0;
+//   dx = (wdy - (xhat*c1 + c2))*r;  dW += dy*xhat;  dB += dy  (per-thread column accumulators).
+// After the row loop the G row groups of the workgroup are summed through LDS in a fixed binary tree and
+// the workgroup writes ONE float32 partial row of dW (and dB): no atomics, run-to-run deterministic.
+// ---------------------------------------------------------------------------------------------------
+template <int BLOCK, int TPR, int VEC>
+__device__ __forceinline__ void combine_groups(float (&acc)[VEC], float* comb, int g, int t) {
+    constexpr int G = BLOCK / TPR;
+    constexpr int HALF = BLOCK / 2;
+#pragma unroll
+    for (int stride = G / 2; stride >= 1; stride >>= 1) {
+        if (g >= stride && g < 2 * stride) {
+            const int slot = (g - stride) * TPR + t;
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) comb[e * HALF + slot] = acc[e];
+        }
+        __syncthreads();
+        if (g < stride) {
+            const int slot = g * TPR + t;
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) acc[e] += comb[e * HALF + slot];
+        }
+        __syncthreads();
+    }
+}
+
+template <typename T, bool LN, int K, int TPR, int BLOCK, bool ALIGNED>
+__global__ void __launch_bounds__(BLOCK) norm_bwd_kernel(const BwdArgs a) {
+    constexpr int VEC = T::VEC;
+    constexpr int G = BLOCK / TPR;
+    constexpr int NV = LN ? 3 : 1;
+    static_assert(BLOCK % TPR == 0 && G >= 1, "a workgroup holds whole rows");
+    __shared__ float red[RedSmem<TPR, G, NV>::kFloats];
+    __shared__ float comb[G > 1 ? VEC * (BLOCK / 2) : 1];
+
+    const int tid = threadIdx.x;
+    const int g = tid / TPR;
+    const int t = tid % TPR;
+    int phase = 0;
+
+    int voff[K];
+    bool own[K];
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+        const int v = t + k * TPR;
+        const int vc = v < a.n_vecs ? v : a.n_vecs - 1;
+        voff[k] = ALIGNED ? vc * 16 : vc;
+        own[k] = v < a.n_vecs;
+    }
+
+    const int64_t rows_per_iter = static_cast<int64_t>(gridDim.x) * G;
+    const int64_t last_row = a.M - 1;
+    int64_t row_raw = static_cast<int64_t>(blockIdx.x) * G + g;
+    int64_t row = row_raw < a.M ? row_raw : last_row;
+    u32x4 cx[K], cg[K];
+    load_row<T, K, ALIGNED>(cx, a.x, a.x_stride_bytes, row, voff, a.n_cols);    // first, so they overlap the params
+    load_row<T, K, ALIGNED>(cg, a.dy, a.dy_stride_bytes, row, voff, a.n_cols);
+    float c_mean = LN ? a.mean[row] : 0.0f;
+    float c_rstd = a.rstd[row];
+
+    float wr[K][VEC];
+    float dw[K][VEC];
+    float db[LN ? K : 1][VEC];
+    load_params_clamped<K, VEC, ALIGNED>(wr, a.w, a.w_dtype, voff, a.n_cols, 1.0f);
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+            dw[k][e] = 0.0f;
+            if constexpr (LN) db[k][e] = 0.0f;
+        }
+    }
+
+    drain_vector_memory();
+    for (int64_t base = static_cast<int64_t>(blockIdx.x) * G; base < a.M; base += rows_per_iter) {
+        const int64_t nrow_raw = row_raw + rows_per_iter;
+        const int64_t nrow = nrow_raw < a.M ? nrow_raw : last_row;
+        u32x4 nx[K], ng[K];
+        load_row<T, K, ALIGNED>(nx, a.x, a.x_stride_bytes, nrow, voff, a.n_cols);
+        load_row<T, K, ALIGNED>(ng, a.dy, a.dy_stride_bytes, nrow, voff, a.n_cols);
+        const float n_mean = LN ? a.mean[nrow] : 0.0f;
+        const float n_rstd = a.rstd[nrow];
+        const bool live = row_raw < a.M;   // false: this group only mirrors the last row
+
+        float u[K][VEC], gf[K][VEC];
+        float s[NV];
+#pragma unroll
+        for (int i = 0; i < NV; ++i) s[i] = 0.0f;
+#pragma unroll
+        for (int k = 0; k < K; ++k) {
+            T::unpack(cx[k], u[k]);
+            T::unpack(cg[k], gf[k]);
+            float s0 = 0.0f, s1 = 0.0f, s2 = 0.0f;
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+                if constexpr (LN) {
+                    float v = (u[k][e] - c_mean) * c_rstd;
+                    if constexpr (!ALIGNED) v = (voff[k] * VEC + e < a.n_cols) ? v : 0.0f;
+                    u[k][e] = v;
+                } else {
+                    u[k][e] *= c_rstd;
+                }
+                const float wdy = wr[k][e] * gf[k][e];
+                s0 = fmaf(u[k][e], wdy, s0);
+                if constexpr (LN) {
+                    s1 += wdy;
+                    s2 += u[k][e];
+                }
+            }
+            s[0] += own[k] ? s0 : 0.0f;
+            if constexpr (LN) {
+                s[1] += own[k] ? s1 : 0.0f;
+                s[2] += own[k] ? s2 : 0.0f;
+            }
+        }
+        row_allreduce<TPR, G, NV>(s, red, phase, g, t);
+        float c1, c2 = 0.0f, dlt = 0.0f;
+        if constexpr (LN) {
+            dlt = s[2] * a.inv_n;
+            c2 = s[1] * a.inv_n;
+            c1 = fmaf(-dlt, c2, s[0] * a.inv_n);
+        } else {
+            c1 = s[0] * a.inv_n;
+        }
+
+        char* dxrow = a.dx + row * a.dx_stride_bytes;
+#pragma unroll
+        for (int k = 0; k < K; ++k) {
+            float dxf[VEC];
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+                float xhat = u[k][e];
+                if constexpr (LN) {
+                    xhat -= dlt;
+                    if constexpr (!ALIGNED) xhat = (voff[k] * VEC + e < a.n_cols) ? xhat : 0.0f;
+                }
+                const float wdy = wr[k][e] * gf[k][e];
+                dxf[e] = (wdy - fmaf(xhat, c1, c2)) * c_rstd;
+                const float gl = live ? gf[k][e] : 0.0f;         // mirrored rows add nothing to dW / dB
+                dw[k][e] = fmaf(gl, xhat, dw[k][e]);
+                if constexpr (LN) db[k][e] += gl;
+            }
+            store_row_vec<T, ALIGNED>(dxrow, voff[k], a.n_cols, dxf);
+        }
+
+#pragma unroll
+        for (int k = 0; k < K; ++k) { cx[k] = nx[k]; cg[k] = ng[k]; }
+        c_mean = n_mean;
+        c_rstd = n_rstd;
+        row_raw = nrow_raw;
+        row = nrow;
+    }
+
+    // Workgroup partial: tree over the G row groups, then group 0 stores its K vectors of VEC floats.
+    // Clamped vector slots hold a copy of their owner's sums and are simply not written.
+    const bool want_dw = a.dw_part != nullptr;
+    const bool want_db = LN && a.db_part != nullptr;
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+        if constexpr (G > 1) {
+            if (want_dw) combine_groups<BLOCK, TPR, VEC>(dw[k], comb, g, t);
+            if constexpr (LN) {
+                if (want_db) combine_groups<BLOCK, TPR, VEC>(db[k], comb, g, t);
+            }
+        }
+        const int v = t + k * TPR;
+        if (g == 0 && v < a.n_vecs) {
+            // part_pitch is a multiple of 64 floats >= n_vecs*VEC, so whole vectors always fit.
+            const int64_t off = static_cast<int64_t>(blockIdx.x) * a.part_pitch + static_cast<int64_t>(v) * VEC;
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+                if (want_dw) a.dw_part[off + e] = dw[k][e];
+                if constexpr (LN) {
+                    if (want_db) a.db_part[off + e] = db[k][e];
+                }
+            }
+        }
+    }
+}
+
+}  // namespace thn
