@@ -74,36 +74,36 @@ def _check(rc):
         raise RuntimeError(f"norm_oracle.c returned {rc}")
 
 
-def layernorm_fwd(x, weight, bias, eps, out_dtype=None):
+def layernorm_fwd(x, weight, bias, eps, out_dtype=None, want_y=True):
     x, weight, bias = _prep(x), _prep(weight), _prep(bias)
     x2 = x.reshape(-1, x.shape[-1])
     m, n = x2.shape
     wd = _CODES[(weight if weight is not None else bias if bias is not None else x).dtype]
     if weight is not None and bias is not None:
         assert weight.dtype == bias.dtype
-    y, oc = _out(x.shape, out_dtype)
+    y, oc = _out(x.shape if want_y else (0,), out_dtype)
     mean = np.empty(m, dtype=np.float64)
     rstd = np.empty(m, dtype=np.float64)
     _check(lib().thn_oracle_layernorm_fwd(_ptr(x2), _CODES[x.dtype], _ptr(weight), _ptr(bias), wd,
                                           ctypes.c_double(eps), ctypes.c_int64(m), ctypes.c_int64(n),
-                                          _ptr(y), oc, _dp(mean), _dp(rstd)))
-    return _ret(y, out_dtype), mean, rstd
+                                          _ptr(y if want_y else None), oc, _dp(mean), _dp(rstd)))
+    return (_ret(y, out_dtype) if want_y else None), mean, rstd
 
 
-def rmsnorm_fwd(x, weight, eps, out_dtype=None):
+def rmsnorm_fwd(x, weight, eps, out_dtype=None, want_y=True):
     x, weight = _prep(x), _prep(weight)
     x2 = x.reshape(-1, x.shape[-1])
     m, n = x2.shape
     wd = _CODES[(weight if weight is not None else x).dtype]
-    y, oc = _out(x.shape, out_dtype)
+    y, oc = _out(x.shape if want_y else (0,), out_dtype)
     rstd = np.empty(m, dtype=np.float64)
     _check(lib().thn_oracle_rmsnorm_fwd(_ptr(x2), _CODES[x.dtype], _ptr(weight), wd,
                                         ctypes.c_double(eps), ctypes.c_int64(m), ctypes.c_int64(n),
-                                        _ptr(y), oc, _dp(rstd)))
-    return _ret(y, out_dtype), rstd
+                                        _ptr(y if want_y else None), oc, _dp(rstd)))
+    return (_ret(y, out_dtype) if want_y else None), rstd
 
 
-def layernorm_bwd(x, dy, weight, mean, rstd, has_bias=True, out_dtype=None, param_dtype=None):
+def layernorm_bwd(x, dy, weight, mean, rstd, has_bias=True, out_dtype=None, param_dtype=None, want_dx=True):
     x, dy, weight = _prep(x), _prep(dy), _prep(weight)
     assert x.dtype == dy.dtype
     x2 = x.reshape(-1, x.shape[-1])
@@ -111,27 +111,29 @@ def layernorm_bwd(x, dy, weight, mean, rstd, has_bias=True, out_dtype=None, para
     wd = _CODES[(weight if weight is not None else x).dtype]
     mean = np.ascontiguousarray(np.asarray(mean, dtype=np.float64).reshape(-1))
     rstd = np.ascontiguousarray(np.asarray(rstd, dtype=np.float64).reshape(-1))
-    dx, oc = _out(x.shape, out_dtype)
+    dx, oc = _out(x.shape if want_dx else (0,), out_dtype)
     dw, pc = _out((n,), param_dtype)
     db, _ = _out((n,), param_dtype)
     _check(lib().thn_oracle_layernorm_bwd(_ptr(x2), _ptr(dy), _CODES[x.dtype], _ptr(weight), wd,
                                           _dp(mean), _dp(rstd), ctypes.c_int64(m), ctypes.c_int64(n),
-                                          _ptr(dx), oc, _ptr(dw if weight is not None else None),
+                                          _ptr(dx if want_dx else None), oc,
+                                          _ptr(dw if weight is not None else None),
                                           _ptr(db if has_bias else None), pc))
-    return (_ret(dx, out_dtype), _ret(dw, param_dtype) if weight is not None else None,
+    return (_ret(dx, out_dtype) if want_dx else None, _ret(dw, param_dtype) if weight is not None else None,
             _ret(db, param_dtype) if has_bias else None)
 
 
-def rmsnorm_bwd(x, dy, weight, rstd, out_dtype=None, param_dtype=None):
+def rmsnorm_bwd(x, dy, weight, rstd, out_dtype=None, param_dtype=None, want_dx=True):
     x, dy, weight = _prep(x), _prep(dy), _prep(weight)
     assert x.dtype == dy.dtype
     x2 = x.reshape(-1, x.shape[-1])
     m, n = x2.shape
     wd = _CODES[(weight if weight is not None else x).dtype]
     rstd = np.ascontiguousarray(np.asarray(rstd, dtype=np.float64).reshape(-1))
-    dx, oc = _out(x.shape, out_dtype)
+    dx, oc = _out(x.shape if want_dx else (0,), out_dtype)
     dw, pc = _out((n,), param_dtype)
     _check(lib().thn_oracle_rmsnorm_bwd(_ptr(x2), _ptr(dy), _CODES[x.dtype], _ptr(weight), wd,
                                         _dp(rstd), ctypes.c_int64(m), ctypes.c_int64(n),
-                                        _ptr(dx), oc, _ptr(dw if weight is not None else None), pc))
-    return _ret(dx, out_dtype), (_ret(dw, param_dtype) if weight is not None else None)
+                                        _ptr(dx if want_dx else None), oc,
+                                        _ptr(dw if weight is not None else None), pc))
+    return (_ret(dx, out_dtype) if want_dx else None), (_ret(dw, param_dtype) if weight is not None else None)

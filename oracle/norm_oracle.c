@@ -18,7 +18,8 @@
  * Inputs x, dy, w, b are read in their storage type and widened exactly to double.  Outputs y, dx, dw, db
  * are written as float64 when out_dtype == 3 (checking mode: nothing is rounded) or narrowed to
  * out_dtype otherwise (timing mode: double -> float -> half/bfloat16, round to nearest even at each step).
- * mean / rstd are always float64 here.  All matrices are dense row-major (M, N).
+ * mean / rstd are always float64 here.  All matrices are dense row-major (M, N).  y and dx may be NULL
+ * (statistics-only forward, parameter-gradient-only backward).
  */
 #include <math.h>
 #include <stdint.h>
@@ -125,8 +126,9 @@ int thn_oracle_layernorm_fwd(const void* x, int x_dtype, const void* w, const vo
             const double rs = 1.0 / sqrt(q / (double)N + eps);
             mean[r] = mu;
             rstd[r] = rs;
-            for (int64_t j = 0; j < N; ++j)
-                store_elem(y, base + j, out_dtype, (row[j] - mu) * rs * wd[j] + bd[j]);
+            if (y)
+                for (int64_t j = 0; j < N; ++j)
+                    store_elem(y, base + j, out_dtype, (row[j] - mu) * rs * wd[j] + bd[j]);
         }
         free(row);
     }
@@ -148,8 +150,9 @@ int thn_oracle_rmsnorm_fwd(const void* x, int x_dtype, const void* w, int w_dtyp
         for (int64_t j = 0; j < N; ++j) { const double v = load_elem(x, base + j, x_dtype); q += v * v; }
         const double rs = 1.0 / sqrt(q / (double)N + eps);
         rstd[r] = rs;
-        for (int64_t j = 0; j < N; ++j)
-            store_elem(y, base + j, out_dtype, load_elem(x, base + j, x_dtype) * rs * wd[j]);
+        if (y)
+            for (int64_t j = 0; j < N; ++j)
+                store_elem(y, base + j, out_dtype, load_elem(x, base + j, x_dtype) * rs * wd[j]);
     }
     free(wd);
     return 0;
@@ -200,7 +203,7 @@ static int backward(const void* x, const void* dy, int x_dtype, const void* w, i
             const double c2 = mean ? s2 / (double)N : 0.0;
             for (int64_t j = 0; j < N; ++j) {
                 const double wdy = wd[j] * g[j];
-                store_elem(dx, base + j, out_dtype, (wdy - (xh[j] * c1 + c2)) * rs);
+                if (dx) store_elem(dx, base + j, out_dtype, (wdy - (xh[j] * c1 + c2)) * rs);
                 pdw[j] += g[j] * xh[j];
                 pdb[j] += g[j];
             }

@@ -1,0 +1,152 @@
+"""CPU tests of the host side: the C-ABI library loads and exports what include/thnorm.h declares, its
+argument checks answer without a GPU, and the Python modules mirror the reference's operator interface
+(TritonHub/Normalization/layernorm.py:211-252, rmsnorm.py:169-204).  Nothing here launches a kernel."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+from conftest import ROOT
+from TritonHub import Normalization, _native
+from TritonHub.Normalization import LayerNorm, RMSNorm, _launch
+from TritonHub.Normalization.layernorm import layernorm
+from TritonHub.Normalization.rmsnorm import rmsnorm
+
+HEADER = os.path.join(ROOT, "include", "thnorm.h")
+
+
+def declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(thn_[a-z_0-9]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    names = declared_functions()
+    assert len(names) == 9 and "thn_norm_fwd" in names and "thn_norm_bwd" in names
+    handle = ctypes.CDLL(_native.LIB_PATH)
+    for name in names:
+        assert hasattr(handle, name), f"{name} is declared in include/thnorm.h but not exported"
+    assert sorted(_native.SYMBOLS) == names          # the ctypes table binds exactly the declared set
+
+
+def test_abi_version_and_messages():
+    lib = _native.lib()
+    version = int(re.search(r"#define THN_ABI_VERSION (\d+)", open(HEADER).read()).group(1))
+    assert lib.thn_abi_version() == version
+    assert _native.strerror(0) == "ok"
+    # the reference's RuntimeError text (layernorm.py:72, rmsnorm.py:58)
+    assert _native.strerror(_native.E_FEATURE_DIM) == "This layer norm doesn't support feature dim >= 64KB."
+    for code in range(-7, 0):
+        assert _native.strerror(code) not in ("", "unknown status")
+    assert _native.strerror(-99) == "unknown status"
+
+
+def test_argument_checks_answer_without_a_gpu():
+    lib = _native.lib()
+    fwd = lambda m, n, xd, wd=0: lib.thn_norm_fwd(0, n, 0, n, 0, 0, 0, 0, m, n, 1e-5, xd, wd, 0)
+    assert fwd(4, 128, 7) == _native.E_DTYPE
+    assert fwd(4, 0, 0) == _native.E_SHAPE and fwd(-1, 8, 0) == _native.E_SHAPE
+    # 64 KiB row limit per storage type: N <= 16384 (4 bytes), 32768 (2 bytes), 8192 (8 bytes)
+    assert fwd(4, 16385, _native.F32) == _native.E_FEATURE_DIM
+    assert fwd(4, 32769, _native.BF16) == _native.E_FEATURE_DIM
+    assert fwd(4, 8193, _native.F64) == _native.E_FEATURE_DIM
+    assert fwd(0, 128, _native.F16) == _native.OK                     # no rows: nothing to do
+    assert fwd(4, 128, _native.F16) == _native.E_NULL                 # required pointers are null
+    assert lib.thn_norm_bwd_workspace_bytes(4, 128, 1, 1, 9) == _native.E_DTYPE
+    assert lib.thn_norm_bwd_workspace_bytes(4, 40000, 1, 1, _native.F16) == _native.E_FEATURE_DIM
+    assert lib.thn_norm_bwd_workspace_bytes(4, 128, 0, 0, _native.F32) == 0
+    assert lib.thn_norm_bwd_workspace_bytes(0, 128, 1, 1, _native.F32) == 0
+    assert lib.thn_norm_set_launch_override(2, 0, 0, 0, 0) == _native.E_SHAPE
+    assert lib.thn_norm_set_launch_override(0, 0, 0, 0, 0) == _native.OK
+    if not torch.cuda.is_available():
+        assert lib.thn_norm_bwd_workspace_bytes(4, 128, 1, 1, _native.F32) == _native.E_DEVICE
+    with pytest.raises(RuntimeError, match="doesn't support feature dim >= 64KB"):
+        _native.check(_native.E_FEATURE_DIM)
+    with pytest.raises(RuntimeError, match="workspace"):
+        _native.check(_native.E_WORKSPACE)
+
+
+def test_no_cpu_fallback():
+    x = torch.randn(4, 32)
+    for mod in (LayerNorm(32), RMSNorm(32)):
+        with pytest.raises(RuntimeError, match="no CPU fallback"):
+            mod(x)
+
+
+def test_package_surface():
+    assert Normalization.__all__ == ["LayerNorm", "RMSNorm"]
+    assert issubclass(layernorm, torch.autograd.Function) and issubclass(rmsnorm, torch.autograd.Function)
+    import TritonHub
+    assert TritonHub.__version__ == "1.1.1"
+
+
+@pytest.mark.parametrize("affine,bias", [(True, True), (True, False), (False, True), (False, False)])
+def test_layernorm_module_matches_reference_constructor(affine, bias):
+    m = LayerNorm(48, eps=1e-3, elementwise_affine=affine, bias=bias, dtype=torch.bfloat16)
+    assert (m.dim, m.eps, m.elementwise_affine) == (48, 1e-3, affine)
+    assert m.layernorm_fn is not None
+    if affine:
+        assert m.weight.shape == (48,) and m.weight.dtype == torch.bfloat16 and bool((m.weight == 1).all())
+        if bias:
+            assert m.bias.shape == (48,) and bool((m.bias == 0).all())
+        else:
+            assert m.bias is None
+    else:
+        assert m.weight is None and m.bias is None          # bias needs elementwise_affine (layernorm.py:232-240)
+    ref = torch.nn.LayerNorm(48, eps=1e-3, elementwise_affine=affine, bias=bias, dtype=torch.bfloat16)
+    assert list(m.state_dict().keys()) == list(ref.state_dict().keys())
+    assert [n for n, _ in m.named_parameters()] == [n for n, _ in ref.named_parameters()]
+    ref.load_state_dict(m.state_dict())
+    m.load_state_dict(ref.state_dict())
+
+
+@pytest.mark.parametrize("affine", [True, False])
+def test_rmsnorm_module_matches_reference_constructor(affine):
+    m = RMSNorm(64, eps=1e-6, elementwise_affine=affine, dtype=torch.float16)
+    assert (m.dim, m.eps, m.elementwise_affine) == (64, 1e-6, affine)
+    assert m.bias is None and "bias" in m._parameters           # always registered as None (rmsnorm.py:194)
+    assert m.rmsnorm_fn is not None
+    if affine:
+        assert m.weight.shape == (64,) and m.weight.dtype == torch.float16 and bool((m.weight == 1).all())
+    else:
+        assert m.weight is None
+    ref = torch.nn.RMSNorm(64, eps=1e-6, elementwise_affine=affine, dtype=torch.float16)
+    assert list(m.state_dict().keys()) == list(ref.state_dict().keys())
+    m.load_state_dict(ref.state_dict())
+
+
+def test_default_arguments():
+    m = LayerNorm(8)
+    assert m.eps == 1e-5 and m.elementwise_affine and m.bias is not None and m.weight.dtype == torch.float32
+    r = RMSNorm(8)
+    assert r.eps == 1e-5 and r.elementwise_affine
+    m.weight.data.fill_(3.0); m.bias.data.fill_(2.0)
+    m.reset_parameters()
+    assert bool((m.weight == 1).all()) and bool((m.bias == 0).all())
+
+
+def test_host_wrapper_helpers():
+    # flatten to (M, N) with unit column stride, as layernorm.py:49-53 does
+    x = torch.randn(3, 5, 16)
+    assert _launch._rows(x, "input").shape == (15, 16)
+    xt = torch.randn(16, 15).t()                      # last stride != 1 -> made contiguous
+    r = _launch._rows(xt, "input")
+    assert r.stride(-1) == 1 and torch.equal(r, xt)
+    sl = torch.randn(6, 64)[:, :32]                   # row stride 64 is kept, not copied
+    r = _launch._rows(sl, "input")
+    assert r.stride(0) == 64 and r.data_ptr() == sl.data_ptr()
+    ex = torch.randn(1, 16).expand(4, 16)             # broadcast rows are materialised
+    assert _launch._rows(ex, "input").stride(0) == 16
+    with pytest.raises(AssertionError, match=r"expect weight to have shape \(N,\)"):
+        _launch._param(torch.ones(7), 8, "weight")
+    with pytest.raises(AssertionError, match=r"expect bias to have shape \(N,\)"):
+        _launch._param(torch.ones(2, 8), 8, "bias")
+    assert _launch._param(None, 8, "weight") is None
+    with pytest.raises(RuntimeError, match="doesn't support feature dim >= 64KB"):
+        _launch._check_feature_dim(16385, 4)
+    _launch._check_feature_dim(16384, 4)
+    with pytest.raises(TypeError, match="unsupported dtype"):
+        _native.dtype_code(torch.int32)

@@ -1,0 +1,366 @@
+"""GPU parity tests: the HIP path, called through the operator interface and the C ABI, against the CPU
+oracle on the same seeded inputs -- the five BASELINE configurations at full size, the reference's own unit
+test matrix, every constructor variant, ragged / strided / misaligned inputs, the size limits, and
+size-independent properties.  Tolerances are the north-star ones (see conftest.check_*)."""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+from conftest import CONFIGS, make_case, f64
+from parity_util import compare_with_oracle, gpu_forward_backward, run_and_compare
+from TritonHub import _native
+from TritonHub.Normalization import LayerNorm, RMSNorm, _launch
+from TritonHub.Normalization.layernorm import layernorm
+from TritonHub.Normalization.rmsnorm import rmsnorm
+
+pytestmark = pytest.mark.gpu
+
+
+def announce(msg):
+    print(f"\n[case] {msg}", flush=True)
+
+
+# ---- BASELINE configurations, full size ---------------------------------------------------------------------
+@pytest.mark.parametrize("name", list(CONFIGS))
+def test_baseline_config_full_size(name):
+    announce(f"baseline {name} shape={CONFIGS[name][1]}")
+    c = make_case(name)
+    n_elems = c["x"].numel()
+    sample = None if n_elems <= 80_000_000 else 12          # the two 268M-element cases: sampled y / dx chunks
+    worst, out = run_and_compare(c["kind"], c["x"], c["dy"], c["w"], c["b"], c["eps"], name, sample_chunks=sample)
+    print("worst ratios to tolerance:", {k: round(v, 9) for k, v in worst.items()}, flush=True)
+    assert out["y"].dtype == c["dtype"] and out["dx"].dtype == c["dtype"] and out["y"].shape == c["x"].shape
+    assert out["rstd"].dtype == torch.float32 and out["rstd"].shape == (c["x"].numel() // c["x"].shape[-1],)
+
+
+# ---- the reference's own unit-test matrix (UnitTests/Normalization/*_unittest.py:57-67) ------------------------
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32, torch.float64])
+@pytest.mark.parametrize("dim", [32, 64, 128, 256, 512, 1024, 2048])
+@pytest.mark.parametrize("kind", ["ln", "rms"])
+def test_reference_unit_test_matrix(kind, dim, dtype):
+    announce(f"reference matrix {kind} D={dim} {dtype}")
+    torch.manual_seed(42)
+    data = torch.randn(1, 256, 256, dim, device="cuda", dtype=dtype)
+    if kind == "ln":
+        ours = LayerNorm(dimension=dim, eps=1e-5, bias=True, elementwise_affine=True, device="cuda", dtype=dtype)
+        theirs = torch.nn.LayerNorm(dim, eps=1e-5, bias=True, elementwise_affine=True, device="cuda", dtype=dtype)
+    else:
+        ours = RMSNorm(dimension=dim, eps=1e-5, elementwise_affine=True, device="cuda", dtype=dtype)
+        theirs = torch.nn.RMSNorm(dim, eps=1e-5, elementwise_affine=True, device="cuda", dtype=dtype)
+    a = data.clone().requires_grad_(True)
+    r = data.clone().requires_grad_(True)
+    # tolerances of the reference's test (layernorm_unittest.py:30-32)
+    rtol, atol = (3e-4, 1e-3) if dtype == torch.float32 else (5e-3, 1e-2)
+    if dtype == torch.float16:
+        rtol, atol = 1e-2, 5e-2
+    ya, yr = ours(a), theirs(r)
+    assert torch.allclose(ya, yr, atol=atol, rtol=rtol), "Error in forward pass"
+    g = torch.randn_like(ya)
+    ya.backward(g)
+    yr.backward(g)
+    assert torch.allclose(a.grad, r.grad, atol=atol, rtol=rtol), "Error in backward pass"
+    # what the reference's test leaves out: parameter gradients, and the tight tolerance against the oracle
+    assert torch.allclose(ours.weight.grad, theirs.weight.grad, atol=max(atol, 0.3), rtol=rtol)
+    rows = 4096
+    x = data.reshape(-1, dim)[:rows].cpu()
+    gy = g.reshape(-1, dim)[:rows].cpu()
+    w = ours.weight.detach().cpu()
+    b = ours.bias.detach().cpu() if kind == "ln" else None
+    run_and_compare(kind, x, gy, w, b, 1e-5, f"{kind} D={dim} {dtype}")
+
+
+# ---- constructor variants, parameter dtypes, input ranks ---------------------------------------------------------
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("affine,bias", [(True, True), (True, False), (False, False)])
+def test_layernorm_variants(dtype, affine, bias):
+    announce(f"LayerNorm variant affine={affine} bias={bias} {dtype}")
+    g = torch.Generator().manual_seed(7)
+    x = torch.randn(3, 17, 384, generator=g).to(dtype)
+    dy = torch.randn(3, 17, 384, generator=g).to(dtype)
+    mod = LayerNorm(384, eps=1e-5, elementwise_affine=affine, bias=bias, device="cuda", dtype=dtype)
+    if affine:
+        with torch.no_grad():
+            mod.weight.copy_((1 + 0.1 * torch.randn(384, generator=g)).to(dtype))
+            if bias:
+                mod.bias.copy_((0.1 * torch.randn(384, generator=g)).to(dtype))
+    xg = x.cuda().requires_grad_(True)
+    y = mod(xg)
+    assert y.shape == x.shape and y.dtype == dtype
+    saved = y.grad_fn.saved_tensors
+    assert len(saved) == 5 and saved[0] is not None             # (input, weight, bias, mean, rstd), layernorm.py:215
+    assert saved[3].dtype == torch.float32 and saved[3].shape == (51,) and saved[4].shape == (51,)
+    assert (saved[1] is None) == (not affine) and (saved[2] is None) == (not (affine and bias))
+    y.backward(dy.cuda())
+    out = dict(y=y.detach(), dx=xg.grad, dw=mod.weight.grad if affine else None,
+               db=mod.bias.grad if (affine and bias) else None, mean=saved[3], rstd=saved[4])
+    w = mod.weight.detach().cpu() if affine else None
+    b = mod.bias.detach().cpu() if (affine and bias) else None
+    compare_with_oracle("ln", x, dy, w, b, 1e-5, out, "variant")
+    if affine:
+        assert mod.weight.grad.dtype == dtype and mod.weight.grad.shape == (384,)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("affine", [True, False])
+def test_rmsnorm_variants(dtype, affine):
+    announce(f"RMSNorm variant affine={affine} {dtype}")
+    g = torch.Generator().manual_seed(8)
+    x = torch.randn(2, 5, 7, 640, generator=g).to(dtype)
+    dy = torch.randn(2, 5, 7, 640, generator=g).to(dtype)
+    mod = RMSNorm(640, eps=1e-6, elementwise_affine=affine, device="cuda", dtype=dtype)
+    if affine:
+        with torch.no_grad():
+            mod.weight.copy_((1 + 0.1 * torch.randn(640, generator=g)).to(dtype))
+    xg = x.cuda().requires_grad_(True)
+    y = mod(xg)
+    saved = y.grad_fn.saved_tensors
+    assert len(saved) == 3 and saved[2].dtype == torch.float32 and saved[2].shape == (70,)   # (input, weight, rstd)
+    y.backward(dy.cuda())
+    out = dict(y=y.detach(), dx=xg.grad, dw=mod.weight.grad if affine else None, db=None, mean=None, rstd=saved[2])
+    compare_with_oracle("rms", x, dy, mod.weight.detach().cpu() if affine else None, None, 1e-6, out, "variant")
+
+
+def test_mixed_parameter_and_activation_dtypes():
+    # float32 parameters under bfloat16 activations: dW / dB come back in the parameter dtype (layernorm.py:207-208)
+    announce("mixed dtypes")
+    g = torch.Generator().manual_seed(9)
+    x = torch.randn(64, 1024, generator=g).bfloat16(); dy = torch.randn(64, 1024, generator=g).bfloat16()
+    w = 1 + 0.1 * torch.randn(1024, generator=g); b = 0.1 * torch.randn(1024, generator=g)
+    worst, out = run_and_compare("ln", x, dy, w, b, 1e-5, "mixed ln")
+    assert out["dw"].dtype == torch.float32 and out["db"].dtype == torch.float32 and out["y"].dtype == torch.bfloat16
+    worst, out = run_and_compare("rms", x.float(), dy.float(), w.half(), None, 1e-5, "mixed rms")
+    assert out["dw"].dtype == torch.float16 and out["dx"].dtype == torch.float32
+
+
+# ---- ragged, strided and misaligned inputs ---------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16, torch.float64])
+@pytest.mark.parametrize("n", [1, 2, 7, 33, 100, 257, 1000, 4099, 6001])
+@pytest.mark.parametrize("kind", ["ln", "rms"])
+def test_ragged_hidden_sizes(kind, n, dtype):
+    announce(f"ragged {kind} N={n} {dtype}")
+    g = torch.Generator().manual_seed(n)
+    m = 19
+    x = (torch.randn(m, n, generator=g) * 2 + 0.5).to(dtype); dy = torch.randn(m, n, generator=g).to(dtype)
+    w = (1 + 0.1 * torch.randn(n, generator=g)).to(dtype)
+    b = (0.1 * torch.randn(n, generator=g)).to(dtype) if kind == "ln" else None
+    run_and_compare(kind, x, dy, w, b, 1e-5, f"ragged N={n}")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_row_strides_and_misaligned_views(dtype):
+    announce(f"strides {dtype}")
+    g = torch.Generator().manual_seed(13)
+    big = torch.randn(40, 1024, generator=g).to(dtype).cuda()
+    dyb = torch.randn(40, 1024, generator=g).to(dtype).cuda()
+    w = (1 + 0.1 * torch.randn(512, generator=g)).to(dtype)
+    b = (0.1 * torch.randn(512, generator=g)).to(dtype)
+    views = {
+        "row stride 1024, aligned": (big[:, :512], dyb[:, 256:768]),
+        "row stride 1024, base off by one element": (big[:, 1:513], dyb[:, 3:515]),
+        "every other row": (big[::2, 512:], dyb[1::2, :512]),
+    }
+    for label, (xv, dv) in views.items():
+        for kind in ("ln", "rms"):
+            xg = xv.detach().requires_grad_(True)
+            wg = w.cuda().requires_grad_(True)
+            bg = b.cuda().requires_grad_(True) if kind == "ln" else None
+            y = layernorm.apply(xg, wg, bg, 1e-5) if kind == "ln" else rmsnorm.apply(xg, wg, 1e-5)
+            assert y.is_contiguous()
+            saved = y.grad_fn.saved_tensors
+            y.backward(dv)
+            out = dict(y=y.detach(), dx=xg.grad, dw=wg.grad, db=None if bg is None else bg.grad,
+                       mean=saved[3] if kind == "ln" else None, rstd=saved[4] if kind == "ln" else saved[2])
+            compare_with_oracle(kind, xv.cpu().contiguous(), dv.cpu().contiguous(), w, b if kind == "ln" else None,
+                                1e-5, out, f"{label} {kind}")
+    # last stride != 1 is made contiguous by the wrapper (layernorm.py:49-50)
+    xt = torch.randn(96, 24, generator=g).to(dtype).cuda().t()          # shape (24, 96), strides (1, 24)
+    mod = RMSNorm(96, device="cuda", dtype=dtype)
+    y = mod(xt)
+    ref = mod(xt.contiguous())
+    assert torch.equal(y, ref)
+
+
+def test_empty_and_single_row():
+    announce("empty / single row")
+    mod = LayerNorm(64, device="cuda")
+    x = torch.empty(0, 64, device="cuda", requires_grad=True)
+    y = mod(x)
+    assert y.shape == (0, 64)
+    y.backward(torch.empty(0, 64, device="cuda"))
+    assert x.grad.shape == (0, 64)
+    assert torch.equal(mod.weight.grad, torch.zeros(64, device="cuda"))      # the sum over no rows
+    assert torch.equal(mod.bias.grad, torch.zeros(64, device="cuda"))
+    g = torch.Generator().manual_seed(3)
+    x1 = torch.randn(1, 64, generator=g); d1 = torch.randn(1, 64, generator=g)
+    run_and_compare("ln", x1, d1, torch.ones(64), torch.zeros(64), 1e-5, "single row")
+    # N = 1: variance 0, y = bias
+    y = LayerNorm(1, device="cuda")(torch.randn(5, 1, device="cuda"))
+    assert torch.equal(y, torch.zeros(5, 1, device="cuda"))
+
+
+# ---- the 64 KiB row limit (layernorm.py:69-72) -----------------------------------------------------------------
+@pytest.mark.parametrize("dtype,n_max", [(torch.float32, 16384), (torch.bfloat16, 32768), (torch.float16, 32768),
+                                         (torch.float64, 8192)])
+def test_feature_dim_limit(dtype, n_max):
+    announce(f"feature dim limit {dtype} N={n_max}")
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(6, n_max, generator=g).to(dtype); dy = torch.randn(6, n_max, generator=g).to(dtype)
+    w = (1 + 0.1 * torch.randn(n_max, generator=g)).to(dtype); b = (0.1 * torch.randn(n_max, generator=g)).to(dtype)
+    run_and_compare("ln", x, dy, w, b, 1e-5, f"LN N={n_max}")
+    run_and_compare("rms", x, dy, w, None, 1e-5, f"RMS N={n_max}")
+    over = torch.randn(2, n_max + 8, device="cuda").to(dtype)
+    for mod in (LayerNorm(n_max + 8, device="cuda", dtype=dtype), RMSNorm(n_max + 8, device="cuda", dtype=dtype)):
+        with pytest.raises(RuntimeError, match="This layer norm doesn't support feature dim >= 64KB."):
+            mod(over)
+
+
+# ---- size-independent properties at full BASELINE sizes --------------------------------------------------------
+@pytest.mark.parametrize("name", ["c2_rms_bf16_llm", "c5a_ln_f32_hostile", "c4_ln_f32_small_hidden"])
+def test_properties_at_full_size(name):
+    announce(f"properties {name}")
+    rows = 131072 if name.startswith("c4") else None
+    c = make_case(name, rows=rows)
+    kind = c["kind"]
+    a = gpu_forward_backward(kind, c["x"], c["dy"], c["w"], c["b"], c["eps"])
+    # 1. run-to-run determinism, bit for bit (no atomics anywhere on the path)
+    a2 = gpu_forward_backward(kind, c["x"], c["dy"], c["w"], c["b"], c["eps"])
+    for k in ("y", "dx", "dw", "db", "rstd", "mean"):
+        if a[k] is not None:
+            assert torch.equal(a[k], a2[k]), f"{k} differs between two identical runs"
+    # 2. the backward is linear in dy, and scaling by 4 is exact in binary floating point
+    s = gpu_forward_backward(kind, c["x"], c["dy"] * 4, c["w"], c["b"], c["eps"])
+    assert torch.equal(s["dx"], a["dx"] * 4) and torch.equal(s["dw"], a["dw"] * 4)
+    if s["db"] is not None:
+        assert torch.equal(s["db"], a["db"] * 4)
+    # 3. rows are independent: reversing the row order reverses y and dx bit for bit
+    x2 = c["x"].reshape(-1, c["x"].shape[-1]); d2 = c["dy"].reshape(-1, c["x"].shape[-1])
+    r = gpu_forward_backward(kind, x2.flip(0), d2.flip(0), c["w"], c["b"], c["eps"])
+    assert torch.equal(r["y"].flip(0), a["y"].reshape(r["y"].shape))
+    assert torch.equal(r["dx"].flip(0), a["dx"].reshape(r["dx"].shape))
+    assert torch.equal(r["rstd"].flip(0), a["rstd"])
+    # 4. LayerNorm: each dx row sums to ~0 and, without affine parameters, each y row has mean 0 / variance var/(var+eps)
+    if kind == "ln":
+        dxs = a["dx"].double().sum(-1).abs().max().item()
+        bound = 64 * 2.0 ** -24 * a["dx"].double().abs().sum(-1).max().item()
+        assert dxs <= bound, (dxs, bound)
+        plain = gpu_forward_backward("ln", c["x"], c["dy"], None, None, c["eps"])
+        y64 = plain["y"].double()
+        assert y64.mean(-1).abs().max().item() < 1e-5
+        assert (y64.pow(2).mean(-1) - 1).abs().max().item() < 1e-4
+
+
+# ---- the C ABI called directly -------------------------------------------------------------------------------
+def test_c_abi_direct_calls_and_errors():
+    announce("C ABI direct")
+    lib = _native.lib()
+    g = torch.Generator().manual_seed(17)
+    m, n, pitch = 300, 768, 1024
+    st = torch.cuda.current_stream().cuda_stream
+    xb = torch.randn(m, pitch, generator=g).cuda(); db_ = torch.randn(m, pitch, generator=g).cuda()
+    w = (1 + 0.1 * torch.randn(n, generator=g)).cuda(); b = (0.1 * torch.randn(n, generator=g)).cuda()
+    x, dy = xb[:, :n], db_[:, :n]
+    y = torch.full((m, pitch), 7.0, device="cuda"); dx = torch.full((m, pitch), 7.0, device="cuda")
+    mean = torch.empty(m, device="cuda"); rstd = torch.empty(m, device="cuda")
+    rc = lib.thn_norm_fwd(x.data_ptr(), pitch, y.data_ptr(), pitch, w.data_ptr(), b.data_ptr(), mean.data_ptr(),
+                          rstd.data_ptr(), m, n, 1e-5, _native.F32, _native.F32, st)
+    assert rc == 0
+    nbytes = lib.thn_norm_bwd_workspace_bytes(m, n, 1, 1, _native.F32)
+    assert nbytes > 0
+    ws = torch.empty(nbytes // 4, device="cuda")
+    dw = torch.empty(n, device="cuda"); dbias = torch.empty(n, device="cuda")
+    rc = lib.thn_norm_bwd(x.data_ptr(), pitch, dy.data_ptr(), pitch, dx.data_ptr(), pitch, w.data_ptr(),
+                          mean.data_ptr(), rstd.data_ptr(), dw.data_ptr(), dbias.data_ptr(), ws.data_ptr(), nbytes,
+                          m, n, _native.F32, _native.F32, st)
+    assert rc == 0
+    torch.cuda.synchronize()
+    assert bool((y[:, n:] == 7.0).all()) and bool((dx[:, n:] == 7.0).all())      # the padding of strided outputs is untouched
+    out = dict(y=y[:, :n], dx=dx[:, :n], dw=dw, db=dbias, mean=mean, rstd=rstd)
+    compare_with_oracle("ln", x.cpu().contiguous(), dy.cpu().contiguous(), w.cpu(), b.cpu(), 1e-5, out, "C ABI")
+    # the two stages called apart give the same bits as the fused entry point
+    parts = ctypes.c_int32(0)
+    dx2 = torch.empty(m, n, device="cuda"); dw2 = torch.empty(n, device="cuda"); db2 = torch.empty(n, device="cuda")
+    rc = lib.thn_norm_bwd_dx_partials(x.data_ptr(), pitch, dy.data_ptr(), pitch, dx2.data_ptr(), n, w.data_ptr(),
+                                      mean.data_ptr(), rstd.data_ptr(), 1, 1, ws.data_ptr(), nbytes, ctypes.byref(parts),
+                                      m, n, _native.F32, _native.F32, st)
+    assert rc == 0 and parts.value > 0
+    assert lib.thn_norm_bwd_reduce_partials(ws.data_ptr(), parts.value, dw2.data_ptr(), db2.data_ptr(), n,
+                                            _native.F32, st) == 0
+    torch.cuda.synchronize()
+    assert torch.equal(dx2, dx[:, :n]) and torch.equal(dw2, dw) and torch.equal(db2, dbias)
+    # error codes
+    assert lib.thn_norm_bwd(x.data_ptr(), pitch, dy.data_ptr(), pitch, dx.data_ptr(), pitch, w.data_ptr(),
+                            mean.data_ptr(), rstd.data_ptr(), dw.data_ptr(), dbias.data_ptr(), ws.data_ptr(), 64,
+                            m, n, _native.F32, _native.F32, st) == _native.E_WORKSPACE
+    assert lib.thn_norm_bwd(x.data_ptr(), pitch, 0, pitch, dx.data_ptr(), pitch, w.data_ptr(), mean.data_ptr(),
+                            rstd.data_ptr(), dw.data_ptr(), dbias.data_ptr(), ws.data_ptr(), nbytes, m, n,
+                            _native.F32, _native.F32, st) == _native.E_NULL
+    assert lib.thn_norm_fwd(x.data_ptr(), n - 1, y.data_ptr(), pitch, 0, 0, 0, rstd.data_ptr(), m, n, 1e-5,
+                            _native.F32, _native.F32, st) == _native.E_SHAPE         # row stride < N
+    assert lib.thn_norm_fwd(x.data_ptr(), pitch, y.data_ptr(), pitch, 0, b.data_ptr(), 0, rstd.data_ptr(), m, n, 1e-5,
+                            _native.F32, _native.F32, st) == _native.E_SHAPE         # RMSNorm takes no bias
+    # gradients that are not wanted are not computed: dw = db = NULL needs no workspace
+    assert lib.thn_norm_bwd(x.data_ptr(), pitch, dy.data_ptr(), pitch, dx2.data_ptr(), n, w.data_ptr(),
+                            mean.data_ptr(), rstd.data_ptr(), 0, 0, 0, 0, m, n, _native.F32, _native.F32, st) == 0
+    torch.cuda.synchronize()
+    assert torch.equal(dx2, dx[:, :n])
+
+
+# ---- every compiled kernel shape ---------------------------------------------------------------------------------
+def compiled_shapes():
+    import os, re
+    from conftest import ROOT
+    text = open(os.path.join(ROOT, "triton-hub_amd", "csrc", "thn_dispatch.h")).read()
+
+    def expand(macro, block=None):
+        body = re.search(r"#define " + macro + r"\(X(?:, B)?\)(.*?)\n\n", text, re.S).group(1)
+        shapes = []
+        for k, t, b in re.findall(r"X\((\d+), (\d+), (\w+)\)", body):
+            shapes.append((int(k), int(t), block if b == "B" else int(b)))
+        return shapes
+    fwd = expand("THN_FWD_SHAPES")
+    bwd = [s for blk in (256, 512) for s in expand("THN_BWD_SHAPES_B", blk)]
+    tail = re.search(r"#define THN_BWD_SHAPES\(X\)(.*?)\n\n", text, re.S).group(1)
+    bwd += [(int(k), int(t), int(b)) for k, t, b in re.findall(r"X\((\d+), (\d+), (\d+)\)", tail)]
+    return fwd, bwd
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("kind", ["ln", "rms"])
+def test_every_compiled_launch_shape(kind, dtype):
+    """Forces each kernel instance in turn through the launch override and checks it against the oracle, at a
+    row width that fills the shape exactly and at one that leaves vector slots without work."""
+    lib = _native.lib()
+    fwd_shapes, bwd_shapes = compiled_shapes()
+    assert len(fwd_shapes) >= 20 and len(bwd_shapes) >= 40
+    vec = 16 // torch.empty(0, dtype=dtype).element_size()
+    g = torch.Generator().manual_seed(23)
+    pairs = sorted(set((k, t) for k, t, _ in fwd_shapes + bwd_shapes))
+    try:
+        for k, tpr in pairs:
+            for n_vecs in sorted({k * tpr, max((k - 1) * tpr + 1, k * tpr - tpr // 2 - 1)}):
+                n = n_vecs * vec
+                if n * (16 // vec) > 65536:
+                    continue
+                f_blocks = [b for kk, tt, b in fwd_shapes if (kk, tt) == (k, tpr)]
+                b_blocks = [b for kk, tt, b in bwd_shapes if (kk, tt) == (k, tpr)]
+                for fb, bb in zip(f_blocks + [0] * len(b_blocks), b_blocks + [0] * len(f_blocks)):
+                    if fb == 0 and bb == 0:
+                        break
+                    rows_per_block = max(fb, bb, 256) // tpr
+                    m = 2 * rows_per_block + max(1, rows_per_block // 2)
+                    announce(f"shape K={k} TPR={tpr} fwd block={fb} bwd block={bb} N={n} M={m} {kind} {dtype}")
+                    x = torch.randn(m, n, generator=g).to(dtype); dy = torch.randn(m, n, generator=g).to(dtype)
+                    w = (1 + 0.1 * torch.randn(n, generator=g)).to(dtype)
+                    b = (0.1 * torch.randn(n, generator=g)).to(dtype) if kind == "ln" else None
+                    assert lib.thn_norm_set_launch_override(0, k if fb else 0, tpr if fb else 0, fb, 0) == 0
+                    assert lib.thn_norm_set_launch_override(1, k if bb else 0, tpr if bb else 0, bb, 0) == 0
+                    if fb:
+                        assert _launch.query_launch(0, kind == "ln", m, n, dtype)[:3] == (k, tpr, fb)
+                    if bb:
+                        assert _launch.query_launch(1, kind == "ln", m, n, dtype)[:3] == (k, tpr, bb)
+                    run_and_compare(kind, x, dy, w, b, 1e-5, f"K={k} TPR={tpr} blocks=({fb},{bb}) N={n}")
+    finally:
+        lib.thn_norm_set_launch_override(0, 0, 0, 0, 0)
+        lib.thn_norm_set_launch_override(1, 0, 0, 0, 0)

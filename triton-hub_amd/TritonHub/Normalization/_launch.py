@@ -56,6 +56,8 @@ def norm_fwd(x: torch.Tensor, weight, bias, eps: float, layernorm: bool):
     rstd = torch.empty((m,), dtype=torch.float32, device=x.device)
     _check_feature_dim(n, x.element_size())
     x_code = _native.dtype_code(x.dtype)
+    if m == 0:                       # nothing to launch (and empty tensors have no address to pass)
+        return out.reshape(*batch_shape, n), mean, rstd
     params = weight if weight is not None else bias
     if weight is not None and bias is not None and weight.dtype != bias.dtype:
         bias = bias.to(weight.dtype)
@@ -91,6 +93,10 @@ def norm_bwd(x: torch.Tensor, dout: torch.Tensor, weight, bias, mean, rstd, laye
     w_code = _native.dtype_code(grad_dtype)
     dw = torch.empty((n,), dtype=grad_dtype, device=x.device) if weight is not None else None
     db = torch.empty((n,), dtype=grad_dtype, device=x.device) if want_db else None
+    if m == 0:                       # the sum over no rows
+        dw = None if dw is None else dw.zero_()
+        db = None if db is None else db.zero_().to(bias.dtype)
+        return dx.reshape(*batch_shape, n), dw, db
     lib = _native.lib()
     with torch.cuda.device(x.device):
         nbytes = lib.thn_norm_bwd_workspace_bytes(m, n, int(dw is not None), int(db is not None), x_code)

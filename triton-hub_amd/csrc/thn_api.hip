@@ -125,20 +125,24 @@ struct Plan {
 
 constexpr int kTprList[] = {8, 16, 32, 64, 128, 256, 512, 1024};
 
-// The static replacement of the reference's autotune over num_warps (autotune.py:62-65): the fewest
-// threads per row that keep the per-thread register image within budget.
-//   forward : up to 4 vectors per thread;
-//   backward: up to 16 elements per thread (x, dy, w, dW, dB live per element), more only when the row is
-//             too wide for 1024 threads otherwise.
-Shape heuristic_shape(int which, bool ln, bool aligned, int n_vecs, int vec_elems) {
-    (void)ln;
-    int kmax = 4;
-    if (aligned && which == 1) {
-        kmax = 16 / vec_elems;
-        if (kmax < 1) kmax = 1;
-        if (kmax > 4) kmax = 4;
-        while (kmax < 4 && 1024 * kmax < n_vecs) ++kmax;
-    }
+// The static replacement of the reference's autotune over num_warps (autotune.py:62-65), fitted to sweeps
+// over (vectors per thread, threads per row, workgroup size, workgroups per compute unit) on MI355X at row
+// widths from 1 KiB to 64 KiB.  HBM throughput peaks when a compute unit keeps about 1024 (forward) to
+// 2048 (backward: two input streams) 16-byte loads in flight and falls off by up to 15 % beyond that, so:
+// one workgroup per compute unit, and
+//   forward : the fewest threads per row with at most 4 vectors each; LayerNorm rows of 256+ threads x 4
+//             vectors use twice the threads with 2 vectors (its two reduction rounds want 8 waves);
+//   backward: the fewest threads per row with at most 3 vectors each (x, dy, w, dW, dB are live per
+//             element), 4 for rows of at most 2 KiB (they share a wave: the float64 column sums need the
+//             instruction-level parallelism) and for rows that 1024 threads cannot cover otherwise;
+//             512-thread workgroups once a row spans two waves or more, which also halves the number of
+//             partial rows.
+constexpr int kDefaultBlocksPerCu = 1;
+
+int ceil_div(int a, int b) { return (a + b - 1) / b; }
+
+Shape heuristic_shape(int which, bool ln, bool aligned, int n_vecs) {
+    const int kmax = (aligned && which == 1 && n_vecs > 128) ? 3 : 4;
     Shape s{4, 1024, 1024};
     for (int tpr : kTprList) {
         if (static_cast<int64_t>(tpr) * kmax >= n_vecs) {
@@ -146,14 +150,19 @@ Shape heuristic_shape(int which, bool ln, bool aligned, int n_vecs, int vec_elem
             break;
         }
     }
-    if (aligned) {
-        s.k = (n_vecs + s.tpr - 1) / s.tpr;
-        if (s.k == 3 && s.tpr < 64) s.k = 4;     // K = 3 is only compiled for TPR >= 64
-        s.block = which == 0 ? (s.tpr > 256 ? s.tpr : 256) : 1024;
-    } else {
+    if (!aligned) {
         s.k = 4;
         s.block = s.tpr > 256 ? s.tpr : 256;
+        return s;
     }
+    s.k = ceil_div(n_vecs, s.tpr);
+    if (which == 0 && ln && s.k == 4 && s.tpr >= 256 && s.tpr < 1024) {
+        s.tpr *= 2;
+        s.k = ceil_div(n_vecs, s.tpr);
+    }
+    if (s.k == 3 && s.tpr < 64) s.k = 4;     // K = 3 is only compiled for TPR >= 64
+    if (which == 0) s.block = s.tpr > 256 ? s.tpr : 256;
+    else s.block = s.tpr >= 128 ? (s.tpr > 512 ? s.tpr : 512) : 256;
     return s;
 }
 
@@ -167,7 +176,7 @@ int plan_launch(int which, bool ln, bool aligned, int64_t M, int64_t N, int dtyp
     const int cus = current_cu_count();
     if (cus <= 0) return THN_E_DEVICE;
 
-    Shape s = heuristic_shape(which, ln, aligned, n_vecs, vec_elems);
+    Shape s = heuristic_shape(which, ln, aligned, n_vecs);
     const Override& ov = g_override[which];
     Shape cand = s;
     if (ov.k.load() > 0) cand.k = ov.k.load();
@@ -181,8 +190,8 @@ int plan_launch(int which, bool ln, bool aligned, int64_t M, int64_t N, int dtyp
     if (!shape_compiled(which, aligned, s)) return THN_E_SHAPE;
 
     int bpc = occupancy(which, dtype, ln, aligned, s);
-    const int cap = ov.bpc.load();
-    if (cap > 0 && cap < bpc) bpc = cap;
+    const int cap = ov.bpc.load() > 0 ? ov.bpc.load() : kDefaultBlocksPerCu;
+    if (cap < bpc) bpc = cap;
     const int rows_per_block = s.block / s.tpr;
     const int64_t row_blocks = (M + rows_per_block - 1) / rows_per_block;
     const int64_t grid_max = static_cast<int64_t>(cus) * bpc;

@@ -32,9 +32,8 @@ struct Shape {
     X(1, 256, B) X(2, 256, B) X(3, 256, B) X(4, 256, B)
 
 #define THN_BWD_SHAPES(X)                                                            \
-    THN_BWD_SHAPES_B(X, 256) THN_BWD_SHAPES_B(X, 512) THN_BWD_SHAPES_B(X, 1024)      \
+    THN_BWD_SHAPES_B(X, 256) THN_BWD_SHAPES_B(X, 512)                                \
     X(1, 512, 512) X(2, 512, 512) X(3, 512, 512) X(4, 512, 512)                      \
-    X(1, 512, 1024) X(2, 512, 1024) X(3, 512, 1024) X(4, 512, 1024)                  \
     X(1, 1024, 1024) X(2, 1024, 1024) X(3, 1024, 1024) X(4, 1024, 1024)
 
 // Shapes of the element-wise (unaligned) path: four vectors per thread, any row width.

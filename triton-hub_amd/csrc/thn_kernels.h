@@ -206,11 +206,14 @@ __global__ void __launch_bounds__(BLOCK) norm_fwd_kernel(const FwdArgs a) {
 //              c2 = sum(wdy)/N, c1 = sum(u*wdy)/N - dlt*c2  (= sum(xhat*wdy)/N);
 //   RMSNorm:   xhat = u, c1 = sum(u*wdy)/N, c2 = 0;
 //   dx = (wdy - (xhat*c1 + c2))*r;  dW += dy*xhat;  dB += dy  (per-thread column accumulators).
-// After the row loop the G row groups of the workgroup are summed through LDS in a fixed binary tree and
-// the workgroup writes ONE float32 partial row of dW (and dB): no atomics, run-to-run deterministic.
+// After the row loop the G row groups of the workgroup are summed through LDS in a fixed binary tree and the
+// workgroup writes ONE float32 partial row of dW (and dB): no atomics, run-to-run deterministic.
 // ---------------------------------------------------------------------------------------------------
-template <int BLOCK, int TPR, int VEC>
-__device__ __forceinline__ void combine_groups(float (&acc)[VEC], float* comb, int g, int t) {
+template <bool WIDE> struct AccType { using type = double; };
+template <> struct AccType<false> { using type = float; };
+
+template <int BLOCK, int TPR, int VEC, typename Acc>
+__device__ __forceinline__ void combine_groups(Acc (&acc)[VEC], Acc* comb, int g, int t) {
     constexpr int G = BLOCK / TPR;
     constexpr int HALF = BLOCK / 2;
 #pragma unroll
@@ -237,7 +240,14 @@ __global__ void __launch_bounds__(BLOCK) norm_bwd_kernel(const BwdArgs a) {
     constexpr int NV = LN ? 3 : 1;
     static_assert(BLOCK % TPR == 0 && G >= 1, "a workgroup holds whole rows");
     __shared__ float red[RedSmem<TPR, G, NV>::kFloats];
-    __shared__ float comb[G > 1 ? VEC * (BLOCK / 2) : 1];
+    // Column accumulators are float64 where the registers are there: a workgroup adds up to M/gridDim.x rows
+    // per column, and float32 accumulators lose about 10 ulp of the final float32 dW at a million rows; with
+    // float64 the accumulation error vanishes next to the error the float32 xhat terms carry anyway (about
+    // 2^-24 * sqrt(M)).  A 1024-thread workgroup has 128 registers per thread and serves rows of 24 KiB and
+    // more (few rows per workgroup): it accumulates in float32.
+    constexpr bool kWideTotals = BLOCK < 1024;
+    using Acc = typename AccType<kWideTotals>::type;
+    __shared__ Acc comb[G > 1 ? VEC * (BLOCK / 2) : 1];
 
     const int tid = threadIdx.x;
     const int g = tid / TPR;
@@ -265,15 +275,15 @@ __global__ void __launch_bounds__(BLOCK) norm_bwd_kernel(const BwdArgs a) {
     float c_rstd = a.rstd[row];
 
     float wr[K][VEC];
-    float dw[K][VEC];
-    float db[LN ? K : 1][VEC];
+    Acc dw[K][VEC];
+    Acc db[LN ? K : 1][VEC];
     load_params_clamped<K, VEC, ALIGNED>(wr, a.w, a.w_dtype, voff, a.n_cols, 1.0f);
 #pragma unroll
     for (int k = 0; k < K; ++k) {
 #pragma unroll
         for (int e = 0; e < VEC; ++e) {
-            dw[k][e] = 0.0f;
-            if constexpr (LN) db[k][e] = 0.0f;
+            dw[k][e] = Acc(0);
+            if constexpr (LN) db[k][e] = Acc(0);
         }
     }
 
@@ -342,8 +352,8 @@ __global__ void __launch_bounds__(BLOCK) norm_bwd_kernel(const BwdArgs a) {
                 }
                 const float wdy = wr[k][e] * gf[k][e];
                 dxf[e] = (wdy - fmaf(xhat, c1, c2)) * c_rstd;
-                const float gl = live ? gf[k][e] : 0.0f;         // mirrored rows add nothing to dW / dB
-                dw[k][e] = fmaf(gl, xhat, dw[k][e]);
+                const Acc gl = static_cast<Acc>(live ? gf[k][e] : 0.0f);   // mirrored rows add nothing
+                dw[k][e] = fma(gl, static_cast<Acc>(xhat), dw[k][e]);
                 if constexpr (LN) db[k][e] += gl;
             }
             store_row_vec<T, ALIGNED>(dxrow, voff[k], a.n_cols, dxf);
@@ -364,9 +374,9 @@ __global__ void __launch_bounds__(BLOCK) norm_bwd_kernel(const BwdArgs a) {
 #pragma unroll
     for (int k = 0; k < K; ++k) {
         if constexpr (G > 1) {
-            if (want_dw) combine_groups<BLOCK, TPR, VEC>(dw[k], comb, g, t);
+            if (want_dw) combine_groups<BLOCK, TPR, VEC, Acc>(dw[k], comb, g, t);
             if constexpr (LN) {
-                if (want_db) combine_groups<BLOCK, TPR, VEC>(db[k], comb, g, t);
+                if (want_db) combine_groups<BLOCK, TPR, VEC, Acc>(db[k], comb, g, t);
             }
         }
         const int v = t + k * TPR;
@@ -375,9 +385,9 @@ __global__ void __launch_bounds__(BLOCK) norm_bwd_kernel(const BwdArgs a) {
             const int64_t off = static_cast<int64_t>(blockIdx.x) * a.part_pitch + static_cast<int64_t>(v) * VEC;
 #pragma unroll
             for (int e = 0; e < VEC; ++e) {
-                if (want_dw) a.dw_part[off + e] = dw[k][e];
+                if (want_dw) a.dw_part[off + e] = static_cast<float>(dw[k][e]);
                 if constexpr (LN) {
-                    if (want_db) a.db_part[off + e] = db[k][e];
+                    if (want_db) a.db_part[off + e] = static_cast<float>(db[k][e]);
                 }
             }
         }
