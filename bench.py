@@ -1,0 +1,274 @@
+#!/usr/bin/env python3
+"""Benchmark of the LayerNorm / RMSNorm forward + backward path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME]
+
+One step = one forward (`thn_norm_fwd`) plus one backward (`thn_norm_bwd`: the dx / partial-sum kernel and
+the second-stage dW / dB reduction) over one batch of synthetic input that is already resident in HBM,
+called through the C ABI exactly as the Python operator layer calls it.  The default workload is the one the
+headline metric is quoted on: RMSNorm, bfloat16, 16384 rows x 4096, weight = 1 + N(0, 0.1), eps = 1e-6.
+Four independent buffer sets (x, dy, y, dx) are rotated so that no step re-reads what the previous one left
+in the caches.  Prints ONE JSON line.
+
+`value` is algorithmic bytes per step / time per step: 5*M*N*s + 8*M + 3*N*s_w bytes for RMSNorm,
+5*M*N*s + 16*M + 5*N*s_w for LayerNorm (x read by forward and again by backward, dy read, y and dx written,
+float32 row statistics written then read, parameters read, parameter gradients written; the partial-sum
+workspace is overhead and is not counted).
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.join(ROOT, "triton-hub_amd"))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0          # MI355X published peak
+N_BUFFER_SETS = 4
+
+WORKLOADS = {
+    # name: (kind, rows, hidden, dtype name)
+    "rmsnorm_bf16_16384x4096": ("rms", 16384, 4096, "bf16"),
+    "layernorm_bf16_16384x4096": ("ln", 16384, 4096, "bf16"),
+    "layernorm_bf16_32768x8192": ("ln", 32768, 8192, "bf16"),
+    "layernorm_f32_1048576x256": ("ln", 1048576, 256, "f32"),
+    "layernorm_f16_8192x6000_hostile": ("ln", 8192, 6000, "f16"),
+    "layernorm_f32_8192x6000_hostile": ("ln", 8192, 6000, "f32"),
+    "rmsnorm_f16_4096x16384_outliers": ("rms", 4096, 16384, "f16"),
+    "rmsnorm_f32_4096x16384_outliers": ("rms", 4096, 16384, "f32"),
+    "layernorm_f32_200x128_quickstart": ("ln", 200, 128, "f32"),
+}
+
+# HBM bytes per launch of the backward dx / partial-sum kernel, from two rocprofv3 --pmc runs of this script
+# (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch), each scaled by what the same counter reads for a plain
+# copy kernel of known size.  Filled in from the summaries under profiles/; null for workloads not profiled.
+MEASURED_TRAFFIC_BYTES = {
+    # profiles/norm_kernels_rmsnorm_bf16_16384x4096_hbm_counters.txt: 262946 KiB fetched + 135168 KiB written
+    "rmsnorm_bf16_16384x4096": 407669153,
+}
+
+
+def algorithmic_bytes(kind, m, n, s, sw):
+    if kind == "ln":
+        return 2 * m * n * s + 2 * n * sw + 8 * m, 3 * m * n * s + 3 * n * sw + 8 * m
+    return 2 * m * n * s + n * sw + 4 * m, 3 * m * n * s + 2 * n * sw + 4 * m
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--workload", default="rmsnorm_bf16_16384x4096", choices=sorted(WORKLOADS))
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--calibration-copy", action="store_true",
+                    help="append five plain tensor copies of known size (reference points for rocprofv3 counters)")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        sys.exit("bench.py: this path runs on ONE GPU: rows are independent and nothing here uses a second device; "
+                 "run with --gpus 1 (a data-parallel job would only add one all-reduce of dW / dB).")
+
+    import torch
+    from TritonHub import _native
+    from TritonHub.Normalization import _launch
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible; the HIP path has no CPU fallback.")
+    lib = _native.lib()
+    dev = torch.device("cuda", 0)
+    torch.cuda.set_device(dev)
+    kind, m, n, dname = WORKLOADS[args.workload]
+    dtype = {"bf16": torch.bfloat16, "f16": torch.float16, "f32": torch.float32}[dname]
+    s = torch.empty(0, dtype=dtype).element_size()
+    code = _native.dtype_code(dtype)
+    ln = kind == "ln"
+
+    gen = torch.Generator(device=dev).manual_seed(0)
+
+    def rand(*shape):
+        return torch.randn(*shape, device=dev, generator=gen, dtype=torch.float32)
+
+    sets = []
+    for _ in range(N_BUFFER_SETS):
+        x = rand(m, n)
+        if "hostile" in args.workload:
+            x += 1000.0
+        if "outliers" in args.workload:
+            x = torch.where(torch.rand(m, n, device=dev, generator=gen) < 0.001, x * 100.0, x)
+        x = x.to(dtype)
+        dy = rand(m, n).to(dtype)
+        sets.append(dict(x=x, dy=dy, y=torch.empty_like(x), dx=torch.empty_like(x),
+                         mean=torch.empty(m, device=dev) if ln else None, rstd=torch.empty(m, device=dev)))
+    w = (1.0 + 0.1 * rand(n)).to(dtype)
+    b = (0.1 * rand(n)).to(dtype) if ln else None
+    dw = torch.empty_like(w)
+    db = torch.empty_like(w) if ln else None
+    ws_bytes = lib.thn_norm_bwd_workspace_bytes(m, n, 1, int(ln), code)
+    assert ws_bytes >= 0, ws_bytes
+    ws = torch.empty(max(ws_bytes, 16) // 4, device=dev)
+    stream = torch.cuda.current_stream(dev).cuda_stream
+    p = _native.ptr
+    parts = ctypes.c_int32(0)
+
+    def forward(b_):
+        rc = lib.thn_norm_fwd(p(b_["x"]), n, p(b_["y"]), n, p(w), p(b), p(b_["mean"]), p(b_["rstd"]), m, n, 1e-6,
+                              code, code, stream)
+        assert rc == 0, _native.strerror(rc)
+
+    def backward(b_):
+        rc = lib.thn_norm_bwd(p(b_["x"]), n, p(b_["dy"]), n, p(b_["dx"]), n, p(w), p(b_["mean"]), p(b_["rstd"]),
+                              p(dw), p(db), p(ws), ws_bytes, m, n, code, code, stream)
+        assert rc == 0, _native.strerror(rc)
+
+    def backward_stage1(b_):
+        rc = lib.thn_norm_bwd_dx_partials(p(b_["x"]), n, p(b_["dy"]), n, p(b_["dx"]), n, p(w), p(b_["mean"]),
+                                          p(b_["rstd"]), 1, int(ln), p(ws), ws_bytes, ctypes.byref(parts), m, n,
+                                          code, code, stream)
+        assert rc == 0, _native.strerror(rc)
+
+    def backward_stage2():
+        rc = lib.thn_norm_bwd_reduce_partials(p(ws), parts.value, p(dw), p(db), n, code, stream)
+        assert rc == 0, _native.strerror(rc)
+
+    def step(i):
+        b_ = sets[i % N_BUFFER_SETS]
+        forward(b_)
+        backward(b_)
+
+    # ---- the timed region: W warm-up steps, then exactly K steps between two device synchronisations ----
+    for i in range(args.warmup):
+        step(i)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        step(i)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed * 1e3 / args.steps
+    fwd_bytes, bwd_bytes = algorithmic_bytes(kind, m, n, s, s)
+    step_bytes = fwd_bytes + bwd_bytes
+    gbps = step_bytes / (ms_per_step * 1e-3) / 1e9
+
+    # ---- per-kernel durations with HIP events on the stream the kernels are launched on: K back-to-back
+    # launches of one kernel (rotating the buffer sets) between one pair of events, for each kernel in turn.
+    # Bracketing every single launch with its own events would add the event's own few microseconds to it. ----
+    def avg_launch_us(launch):
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        for i in range(min(args.warmup, 5)):
+            launch(sets[i % N_BUFFER_SETS])
+        torch.cuda.synchronize()
+        start.record()
+        for i in range(args.steps):
+            launch(sets[i % N_BUFFER_SETS])
+        stop.record()
+        torch.cuda.synchronize()
+        return start.elapsed_time(stop) * 1e3 / args.steps
+
+    fwd_us = avg_launch_us(forward)
+    bwd1_us = avg_launch_us(backward_stage1)
+    bwd2_us = avg_launch_us(lambda b_: backward_stage2())
+    achieved = bwd_bytes / (bwd1_us * 1e-6) / 1e9
+    if args.calibration_copy:
+        # a plain copy of known size (x -> y: m*n*s bytes read, as many written) for scaling the HBM counters
+        for i in range(5):
+            sets[i % N_BUFFER_SETS]["y"].copy_(sets[i % N_BUFFER_SETS]["x"])
+        torch.cuda.synchronize()
+    fwd_shape = _launch.query_launch(0, ln, m, n, dtype)
+    bwd_shape = _launch.query_launch(1, ln, m, n, dtype)
+
+    out = {
+        "metric": "fwd+bwd HBM GB/s and % of peak, RMSNorm/LayerNorm bf16 16384x4096",
+        "value": round(gbps, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": dname,
+        "data": "synthetic",
+        "config": {"workload": args.workload, "op": "RMSNorm" if kind == "rms" else "LayerNorm", "rows": m,
+                   "hidden": n, "eps": 1e-6, "buffer_sets": N_BUFFER_SETS, "entry_points": "thn_norm_fwd + thn_norm_bwd"},
+        "pct_of_hbm_peak": round(100.0 * gbps / HBM_PEAK_GBPS, 2),
+        "rows_per_s": round(m / (ms_per_step * 1e-3)),
+        "algorithmic_bytes_per_step": step_bytes,
+        "kernels_us": {"forward": round(fwd_us, 2), "backward_dx_partials": round(bwd1_us, 2),
+                       "backward_reduce_partials": round(bwd2_us, 2),
+                       "forward_GBps": round(fwd_bytes / (fwd_us * 1e-6) / 1e9, 1)},
+        "launch": {"forward": {"vecs_per_thread": fwd_shape[0], "threads_per_row": fwd_shape[1],
+                               "block": fwd_shape[2], "grid": fwd_shape[3]},
+                   "backward": {"vecs_per_thread": bwd_shape[0], "threads_per_row": bwd_shape[1],
+                                "block": bwd_shape[2], "grid": bwd_shape[3]}},
+        "roofline": {"bound": "hbm", "kernel": "norm_bwd_kernel (backward dx + dW/dB partials)",
+                     "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBPS, 4),
+                     "algorithmic_bytes_per_launch": bwd_bytes, "avg_launch_us": round(bwd1_us, 2),
+                     "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload)},
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(kind, m, n, dtype, sets[0], w, b, step_bytes)
+    print(json.dumps(out), flush=True)
+
+
+def cpu_baseline(kind, m, n, dtype, buffers, w, b, step_bytes):
+    """The same forward + backward on the host cores: the C restatement of the reference's arithmetic
+    (oracle/norm_oracle.c, OpenMP over rows, storage-dtype outputs), and torch.nn.functional next to it.
+    Bounded sample: the first `rows` rows of the workload, scaled to the whole step by row count."""
+    import torch
+    from oracle import c_oracle as co
+    threads = co.num_threads()
+    rows = min(m, max(256, (1 << 25) // n))            # 32M elements per pass at most
+    x = buffers["x"][:rows].cpu()
+    dy = buffers["dy"][:rows].cpu()
+    wc = w.cpu()
+    bc = None if b is None else b.cpu()
+
+    def oracle_step():
+        if kind == "ln":
+            _, mean, rstd = co.layernorm_fwd(x, wc, bc, 1e-6, out_dtype=dtype)
+            co.layernorm_bwd(x, dy, wc, mean, rstd, has_bias=True, out_dtype=dtype, param_dtype=dtype)
+        else:
+            _, rstd = co.rmsnorm_fwd(x, wc, 1e-6, out_dtype=dtype)
+            co.rmsnorm_bwd(x, dy, wc, rstd, out_dtype=dtype, param_dtype=dtype)
+
+    def torch_step():
+        xr = x.clone().requires_grad_(True)
+        wr = wc.clone().requires_grad_(True)
+        if kind == "ln":
+            br = bc.clone().requires_grad_(True)
+            y = torch.nn.functional.layer_norm(xr, (n,), wr, br, 1e-6)
+        else:
+            y = torch.nn.functional.rms_norm(xr, (n,), wr, 1e-6)
+        y.backward(dy)
+
+    def timed(fn, reps):
+        fn()
+        best = float("inf")
+        for _ in range(reps):
+            t0 = time.perf_counter()
+            fn()
+            best = min(best, time.perf_counter() - t0)
+        return best
+
+    sample_bytes = step_bytes * rows / m
+    t_oracle = timed(oracle_step, 3)
+    t_torch = timed(torch_step, 2)
+    return {
+        "value": round(sample_bytes / t_oracle / 1e9, 2), "unit": "GB/s", "cores": threads, "kind": "port",
+        "sample": f"first {rows} of {m} rows of the same workload, forward + backward, best of 3 passes of "
+                  f"oracle/norm_oracle.c with {threads} OpenMP threads ({t_oracle * 1e3:.1f} ms per pass)",
+        "host_cpu_count": os.cpu_count(),
+        "torch_functional": {"value": round(sample_bytes / t_torch / 1e9, 2), "unit": "GB/s",
+                             "threads": torch.get_num_threads(),
+                             "what": "torch.nn.functional layer_norm / rms_norm forward + autograd backward on the "
+                                     f"host cores, same sample ({t_torch * 1e3:.1f} ms per pass)"},
+    }
+
+
+if __name__ == "__main__":
+    main()
