@@ -42,6 +42,38 @@ def _check_feature_dim(n: int, element_size: int) -> None:
         raise RuntimeError(FEATURE_DIM_MESSAGE)
 
 
+_raw_stream = getattr(torch._C, '_cuda_getCurrentRawStream', None)
+_workspace_bytes_cache = {}
+
+
+def _stream_handle(index: int) -> int:
+    """hipStream_t of torch's current stream on device `index`, as an integer."""
+    if _raw_stream is not None:
+        return _raw_stream(index)
+    return torch.cuda.current_stream(index).cuda_stream
+
+
+class _on_device:
+    """Makes `index` the current HIP device for the duration of a launch; free when it already is
+    (the reference wraps its launches in `with torch.cuda.device(x.device.index)`, layernorm.py:73)."""
+
+    __slots__ = ('index', 'guard')
+
+    def __init__(self, index: int):
+        self.index = index
+        self.guard = None
+
+    def __enter__(self):
+        if torch.cuda.current_device() != self.index:
+            self.guard = torch.cuda.device(self.index)
+            self.guard.__enter__()
+
+    def __exit__(self, *exc):
+        if self.guard is not None:
+            self.guard.__exit__(*exc)
+        return False
+
+
 def norm_fwd(x: torch.Tensor, weight, bias, eps: float, layernorm: bool):
     """Returns (y like x, mean (M,) float32 or None, rstd (M,) float32)."""
     _native.require_gpu(x)
@@ -62,12 +94,14 @@ def norm_fwd(x: torch.Tensor, weight, bias, eps: float, layernorm: bool):
     if weight is not None and bias is not None and weight.dtype != bias.dtype:
         bias = bias.to(weight.dtype)
     w_code = _native.dtype_code(params.dtype) if params is not None else x_code
-    with torch.cuda.device(x.device):
+    index = x.device.index
+    with _on_device(index):
         status = _native.lib().thn_norm_fwd(
             x2.data_ptr(), x2.stride(0) if m > 1 else n, out.data_ptr(), n,
             _native.ptr(weight), _native.ptr(bias), _native.ptr(mean), rstd.data_ptr(),
-            m, n, float(eps), x_code, w_code, _native.current_stream(x.device))
-    _native.check(status)
+            m, n, float(eps), x_code, w_code, _stream_handle(index))
+    if status != 0:
+        _native.check(status)
     return out.reshape(*batch_shape, n), mean, rstd
 
 
@@ -98,17 +132,24 @@ def norm_bwd(x: torch.Tensor, dout: torch.Tensor, weight, bias, mean, rstd, laye
         db = None if db is None else db.zero_().to(bias.dtype)
         return dx.reshape(*batch_shape, n), dw, db
     lib = _native.lib()
-    with torch.cuda.device(x.device):
-        nbytes = lib.thn_norm_bwd_workspace_bytes(m, n, int(dw is not None), int(db is not None), x_code)
-        if nbytes < 0:
-            _native.check(int(nbytes))
-        workspace = torch.empty((max(int(nbytes), 16) // 4,), dtype=torch.float32, device=x.device)
+    index = x.device.index
+    with _on_device(index):
+        key = (index, m, n, dw is not None, db is not None, x_code)
+        nbytes = _workspace_bytes_cache.get(key)
+        if nbytes is None:
+            nbytes = int(lib.thn_norm_bwd_workspace_bytes(m, n, int(dw is not None), int(db is not None), x_code))
+            if nbytes < 0:
+                _native.check(nbytes)
+            _workspace_bytes_cache[key] = nbytes
+        # the counterpart of the reference's per-call _dw / _db buffers (layernorm.py:183-184)
+        workspace = torch.empty((max(nbytes, 16) // 4,), dtype=torch.float32, device=x.device)
         status = lib.thn_norm_bwd(
             x2.data_ptr(), x2.stride(0) if m > 1 else n, d2.data_ptr(), d2.stride(0) if m > 1 else n,
             dx.data_ptr(), n, _native.ptr(weight), _native.ptr(mean), rstd.data_ptr(),
-            _native.ptr(dw), _native.ptr(db), workspace.data_ptr(), int(nbytes), m, n, x_code, w_code,
-            _native.current_stream(x.device))
-    _native.check(status)
+            _native.ptr(dw), _native.ptr(db), workspace.data_ptr(), nbytes, m, n, x_code, w_code,
+            _stream_handle(index))
+    if status != 0:
+        _native.check(status)
     if mixed:
         db = db.to(bias.dtype)
     return dx.reshape(*batch_shape, n), dw, db

@@ -47,6 +47,18 @@ __device__ __forceinline__ void st128(void* p, u32x4 v) {
 // the prologue's loads still pending makes it wait for more than the loop body needs on every trip.
 __device__ __forceinline__ void drain_vector_memory() { __builtin_amdgcn_s_waitcnt(0x0F70); }
 
+// 1/sqrt(v) for v > 0: the hardware estimate (v_rsq_f32, about 1 ulp) refined by one Newton step, which
+// leaves an error of a fraction of an ulp -- well inside the 1e-6 relative bound on the saved rstd -- in 7
+// instructions.  The correctly rounded sqrt followed by a correctly rounded division is about 40, all of them
+// on the serial path between a row's reduction and its stores.
+__device__ __forceinline__ float rsqrt_refined(float v) {
+    const float r = __builtin_amdgcn_rsqf(v);
+    const float h = 0.5f * r;
+    const float e = fmaf(-v * r, r, 1.0f);       // 1 - v*r^2
+    const float refined = fmaf(h, e, r);          // r + r*e/2
+    return v > 0.0f ? refined : r;                // v == 0 (eps == 0, constant row): +inf, as 1/sqrt(0) is
+}
+
 // ---------------------------------------------------------------------------------------------------
 // Storage traits.  A "vector" is 16 bytes of a row: VEC elements.  unpack() widens a vector to float32,
 // pack() narrows with round-to-nearest-even (v_cvt_pk_bf16_f32 / v_cvt_f16_f32 / v_cvt_f64_f32).

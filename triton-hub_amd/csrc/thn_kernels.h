@@ -161,7 +161,7 @@ __global__ void __launch_bounds__(BLOCK) norm_fwd_kernel(const FwdArgs a) {
             row_allreduce<TPR, G, 2>(q, red, phase, g, t);
             delta = q[0] * a.inv_n;
             const float var = fmaxf(fmaf(-delta, delta, q[1] * a.inv_n), 0.0f);
-            rstd = 1.0f / sqrtf(var + a.eps);
+            rstd = rsqrt_refined(var + a.eps);
             mean = mean0 + delta;
         } else {
             float q[1] = {0.0f};
@@ -173,7 +173,7 @@ __global__ void __launch_bounds__(BLOCK) norm_fwd_kernel(const FwdArgs a) {
                 q[0] += own[k] ? qk : 0.0f;
             }
             row_allreduce<TPR, G, 1>(q, red, phase, g, t);
-            rstd = 1.0f / sqrtf(q[0] * a.inv_n + a.eps);
+            rstd = rsqrt_refined(fmaf(q[0], a.inv_n, a.eps));
         }
 
         char* yrow = a.y + row * a.y_stride_bytes;
