@@ -130,8 +130,7 @@ constexpr int kTprList[] = {8, 16, 32, 64, 128, 256, 512, 1024};
 // widths from 1 KiB to 64 KiB.  HBM throughput peaks when a compute unit keeps about 1024 (forward) to
 // 2048 (backward: two input streams) 16-byte loads in flight and falls off by up to 15 % beyond that, so:
 // one workgroup per compute unit, and
-//   forward : the fewest threads per row with at most 4 vectors each; LayerNorm rows of 256+ threads x 4
-//             vectors use twice the threads with 2 vectors (its two reduction rounds want 8 waves);
+//   forward : the fewest threads per row with at most 4 vectors each (256-thread workgroups up to 16 KiB rows);
 //   backward: the fewest threads per row with at most 3 vectors each (x, dy, w, dW, dB are live per
 //             element), 4 for rows of at most 2 KiB (they share a wave: the float64 column sums need the
 //             instruction-level parallelism) and for rows that 1024 threads cannot cover otherwise;
@@ -142,6 +141,7 @@ constexpr int kDefaultBlocksPerCu = 1;
 int ceil_div(int a, int b) { return (a + b - 1) / b; }
 
 Shape heuristic_shape(int which, bool ln, bool aligned, int n_vecs) {
+    (void)ln;
     const int kmax = (aligned && which == 1 && n_vecs > 128) ? 3 : 4;
     Shape s{4, 1024, 1024};
     for (int tpr : kTprList) {
@@ -156,10 +156,6 @@ Shape heuristic_shape(int which, bool ln, bool aligned, int n_vecs) {
         return s;
     }
     s.k = ceil_div(n_vecs, s.tpr);
-    if (which == 0 && ln && s.k == 4 && s.tpr >= 256 && s.tpr < 1024) {
-        s.tpr *= 2;
-        s.k = ceil_div(n_vecs, s.tpr);
-    }
     if (s.k == 3 && s.tpr < 64) s.k = 4;     // K = 3 is only compiled for TPR >= 64
     if (which == 0) s.block = s.tpr > 256 ? s.tpr : 256;
     else s.block = s.tpr >= 128 ? (s.tpr > 512 ? s.tpr : 512) : 256;

@@ -18,6 +18,8 @@
 // and of the dW / dB accumulators.
 #pragma once
 
+#include <type_traits>
+
 #include "thn_device.h"
 
 namespace thn {
@@ -240,12 +242,14 @@ __global__ void __launch_bounds__(BLOCK) norm_bwd_kernel(const BwdArgs a) {
     constexpr int NV = LN ? 3 : 1;
     static_assert(BLOCK % TPR == 0 && G >= 1, "a workgroup holds whole rows");
     __shared__ float red[RedSmem<TPR, G, NV>::kFloats];
-    // Column accumulators are float64 where the registers are there: a workgroup adds up to M/gridDim.x rows
-    // per column, and float32 accumulators lose about 10 ulp of the final float32 dW at a million rows; with
-    // float64 the accumulation error vanishes next to the error the float32 xhat terms carry anyway (about
-    // 2^-24 * sqrt(M)).  A 1024-thread workgroup has 128 registers per thread and serves rows of 24 KiB and
-    // more (few rows per workgroup): it accumulates in float32.
-    constexpr bool kWideTotals = BLOCK < 1024;
+    // Column accumulators: float64 for float32 / float64 rows in workgroups that have the registers (a
+    // workgroup adds up to M/gridDim.x rows per column; float32 accumulators lose about 10 ulp of the final
+    // float32 dW at a million rows, float64 ones leave only the error the float32 xhat terms carry anyway,
+    // about 2^-24 * sqrt(M)).  16-bit rows accumulate in float32: the loop is VALU-latency sensitive (each
+    // instruction per element costs about 1 % of the kernel) and the extra digits would not survive a 16-bit
+    // dW.  A 1024-thread workgroup has 128 registers per thread and serves rows of 24 KiB and more (few rows
+    // per workgroup): float32 too.
+    constexpr bool kWideTotals = BLOCK < 1024 && T::kBytes >= 4;
     using Acc = typename AccType<kWideTotals>::type;
     __shared__ Acc comb[G > 1 ? VEC * (BLOCK / 2) : 1];
 
@@ -287,8 +291,10 @@ __global__ void __launch_bounds__(BLOCK) norm_bwd_kernel(const BwdArgs a) {
         }
     }
 
-    drain_vector_memory();
-    for (int64_t base = static_cast<int64_t>(blockIdx.x) * G; base < a.M; base += rows_per_iter) {
+    // One grid-stride step.  MASKED is only needed for the last step of a workgroup, where some of its row
+    // groups may have run past the end and mirror the last row: they must add nothing to dW / dB.
+    auto step = [&](auto masked_tag) {
+        constexpr bool MASKED = decltype(masked_tag)::value;
         const int64_t nrow_raw = row_raw + rows_per_iter;
         const int64_t nrow = nrow_raw < a.M ? nrow_raw : last_row;
         u32x4 nx[K], ng[K];
@@ -296,9 +302,9 @@ __global__ void __launch_bounds__(BLOCK) norm_bwd_kernel(const BwdArgs a) {
         load_row<T, K, ALIGNED>(ng, a.dy, a.dy_stride_bytes, nrow, voff, a.n_cols);
         const float n_mean = LN ? a.mean[nrow] : 0.0f;
         const float n_rstd = a.rstd[nrow];
-        const bool live = row_raw < a.M;   // false: this group only mirrors the last row
+        const bool live = !MASKED || row_raw < a.M;
 
-        float u[K][VEC], gf[K][VEC];
+        float u[K][VEC], gf[K][VEC], wdy[K][VEC];
         float s[NV];
 #pragma unroll
         for (int i = 0; i < NV; ++i) s[i] = 0.0f;
@@ -316,10 +322,10 @@ __global__ void __launch_bounds__(BLOCK) norm_bwd_kernel(const BwdArgs a) {
                 } else {
                     u[k][e] *= c_rstd;
                 }
-                const float wdy = wr[k][e] * gf[k][e];
-                s0 = fmaf(u[k][e], wdy, s0);
+                wdy[k][e] = wr[k][e] * gf[k][e];
+                s0 = fmaf(u[k][e], wdy[k][e], s0);
                 if constexpr (LN) {
-                    s1 += wdy;
+                    s1 += wdy[k][e];
                     s2 += u[k][e];
                 }
             }
@@ -350,11 +356,12 @@ __global__ void __launch_bounds__(BLOCK) norm_bwd_kernel(const BwdArgs a) {
                     xhat -= dlt;
                     if constexpr (!ALIGNED) xhat = (voff[k] * VEC + e < a.n_cols) ? xhat : 0.0f;
                 }
-                const float wdy = wr[k][e] * gf[k][e];
-                dxf[e] = (wdy - fmaf(xhat, c1, c2)) * c_rstd;
-                const Acc gl = static_cast<Acc>(live ? gf[k][e] : 0.0f);   // mirrored rows add nothing
-                dw[k][e] = fma(gl, static_cast<Acc>(xhat), dw[k][e]);
-                if constexpr (LN) db[k][e] += gl;
+                // subtract first, scale by rstd last: when dx cancels to (almost) nothing -- rstd is huge for a
+                // near-constant row -- the rounding error stays relative to the small difference
+                dxf[e] = (wdy[k][e] - fmaf(xhat, c1, c2)) * c_rstd;
+                const float gl = (MASKED && !live) ? 0.0f : gf[k][e];
+                dw[k][e] = fma(static_cast<Acc>(gl), static_cast<Acc>(xhat), dw[k][e]);
+                if constexpr (LN) db[k][e] += static_cast<Acc>(gl);
             }
             store_row_vec<T, ALIGNED>(dxrow, voff[k], a.n_cols, dxf);
         }
@@ -365,7 +372,12 @@ __global__ void __launch_bounds__(BLOCK) norm_bwd_kernel(const BwdArgs a) {
         c_rstd = n_rstd;
         row_raw = nrow_raw;
         row = nrow;
-    }
+    };
+
+    drain_vector_memory();
+    int64_t base = static_cast<int64_t>(blockIdx.x) * G;
+    for (; base + G <= a.M; base += rows_per_iter) step(std::false_type{});
+    if (base < a.M) step(std::true_type{});
 
     // Workgroup partial: tree over the G row groups, then group 0 stores its K vectors of VEC floats.
     // Clamped vector slots hold a copy of their owner's sums and are simply not written.
