@@ -1,8 +1,10 @@
 /*
- * thnorm.h -- C ABI of libthnorm.so: LayerNorm / RMSNorm forward and backward for AMD MI355X (gfx950).
+ * thnorm.h -- C ABI of libthnorm.so: LayerNorm / RMSNorm, and the Softmax / Softmin / LogSoftmax row
+ * reductions next to them, forward and backward, for AMD MI355X (gfx950).
  *
  * The reference library (TritonHub) has no native boundary: its last host frames before device code are the
- * Python launch sites in TritonHub/Normalization/layernorm.py and rmsnorm.py.  Each entry point below
+ * Python launch sites in TritonHub/Normalization/layernorm.py and rmsnorm.py (and TritonHub/Activations/
+ * softmax.py, softmin.py, logsoftmax.py).  Each entry point below
  * replaces one of those launch sites, so a maintainer of the reference can bind it with ctypes in place of
  * the Triton launch.  The citation on every declaration names the launch site (and device code) replaced.
  *
@@ -11,7 +13,7 @@
  *     keeps no pointer after the call returns and never synchronises: kernels are enqueued on `stream`
  *     (a hipStream_t passed as void*; NULL is the default stream) of the CURRENT device.
  *   - Matrices are row-major (M rows, N columns), unit column stride; row strides are in ELEMENTS.
- *   - Storage codes: THN_F32 / THN_F16 / THN_BF16 / THN_F64.  Arithmetic is float32 whatever the storage
+ *   - Storage codes: THN_F32 / THN_F16 / THN_BF16 / THN_F64.  The norm arithmetic is float32 whatever the storage
  *     (a float64 tensor is narrowed on load and widened on store, as the reference does with
  *     `.to(tl.float32)`, layernorm.py:31).  Results are rounded to nearest even on store.
  *   - Return value: THN_OK (0) or a negative THN_E_* code; thn_strerror() names it.  Nothing throws.
@@ -27,7 +29,7 @@
 extern "C" {
 #endif
 
-#define THN_ABI_VERSION 1
+#define THN_ABI_VERSION 2
 
 enum thn_dtype { THN_F32 = 0, THN_F16 = 1, THN_BF16 = 2, THN_F64 = 3 };
 
@@ -117,10 +119,40 @@ int thn_norm_bwd_reduce_partials(const void* workspace, int32_t num_partials,
                                  int64_t N, int w_dtype, void* stream);
 
 /*
+ * Softmax, Softmin and LogSoftmax over the last dimension (the row-reduction activations next to the norm
+ * path in the reference: TritonHub/Activations/softmax.py, softmin.py, logsoftmax.py).
+ *
+ * thn_softmax_fwd replaces `_softmax_kernel_fwd[grid](...)` (softmax.py:37-40, device code :14-24),
+ * `_softmin_kernel_fwd` (softmin.py:36-39) and `_logsoftmax_kernel_fwd` (logsoftmax.py:39-43, device code
+ * :17-26):  z = x - max(x);  THN_SOFTMAX: y = exp(z)/sum(exp(z));  THN_LOGSOFTMAX: y = z - log(sum(exp(z)));
+ * THN_SOFTMIN: softmax of -x (the reference negates with a separate tensor op, softmin.py:109; here the
+ * sign is applied on load).
+ * thn_softmax_bwd replaces `_softmax_kernel_bwd` (softmax.py:75-79, device code :50-61), `_softmin_kernel_bwd`
+ * (softmin.py:75-79) and `_logsoftmax_kernel_bwd` (logsoftmax.py:88-93, device code :62-78); `y` is the SAVED
+ * OUTPUT of the forward, as in the reference:
+ *   THN_SOFTMAX: dx = y*dy - y*sum(y*dy);  THN_SOFTMIN: the negative of that;  THN_LOGSOFTMAX: dx = dy - exp(y)*sum(dy).
+ * All tensors share one storage code.  Arithmetic is float32, except softmax / softmin on THN_F64 storage,
+ * which run in float64: the reference's softmax kernels compute in the type they load (softmax.py:18-23),
+ * its log-softmax kernels widen to float32 (logsoftmax.py:19, :71).  Rows wider than 64 KiB are refused with
+ * THN_E_FEATURE_DIM (the reference would split such a row into independently normalised chunks).
+ */
+enum thn_softmax_kind { THN_SOFTMAX = 0, THN_SOFTMIN = 1, THN_LOGSOFTMAX = 2 };
+
+int thn_softmax_fwd(const void* x, int64_t x_row_stride,
+                    void* y, int64_t y_row_stride,
+                    int64_t M, int64_t N, int kind, int dtype, void* stream);
+
+int thn_softmax_bwd(const void* y, int64_t y_row_stride,
+                    const void* dy, int64_t dy_row_stride,
+                    void* dx, int64_t dx_row_stride,
+                    int64_t M, int64_t N, int kind, int dtype, void* stream);
+
+/*
  * Launch-shape control for tuning sweeps (the counterpart of the reference's `triton.autotune` over
  * num_warps, autotune.py:62-65, which this library replaces by a fixed heuristic on N and the dtype).
- * `which`: 0 = forward, 1 = backward.  vecs_per_thread / threads_per_row / block_threads select a compiled
- * kernel shape, blocks_per_cu caps the persistent grid; 0 for any field keeps the heuristic's choice.
+ * `which`: 0 = norm forward, 1 = norm backward, 2 = softmax forward, 3 = softmax backward.
+ * vecs_per_thread / threads_per_row / block_threads select a compiled kernel shape, blocks_per_cu caps the
+ * persistent grid; 0 for any field keeps the heuristic's choice.
  * Process-wide; meant for benchmarks, not for concurrent production use.  Returns THN_E_SHAPE when no
  * compiled kernel has that shape.
  */

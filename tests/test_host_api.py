@@ -9,7 +9,7 @@ import pytest
 import torch
 
 from conftest import ROOT
-from TritonHub import Normalization, _native
+from TritonHub import Activations, Normalization, _native
 from TritonHub.Normalization import LayerNorm, RMSNorm, _launch
 from TritonHub.Normalization.layernorm import layernorm
 from TritonHub.Normalization.rmsnorm import rmsnorm
@@ -25,7 +25,7 @@ def declared_functions():
 
 def test_library_exports_every_declared_symbol():
     names = declared_functions()
-    assert len(names) == 9 and "thn_norm_fwd" in names and "thn_norm_bwd" in names
+    assert len(names) == 11 and "thn_norm_fwd" in names and "thn_norm_bwd" in names and "thn_softmax_fwd" in names
     handle = ctypes.CDLL(_native.LIB_PATH)
     for name in names:
         assert hasattr(handle, name), f"{name} is declared in include/thnorm.h but not exported"
@@ -59,7 +59,7 @@ def test_argument_checks_answer_without_a_gpu():
     assert lib.thn_norm_bwd_workspace_bytes(4, 40000, 1, 1, _native.F16) == _native.E_FEATURE_DIM
     assert lib.thn_norm_bwd_workspace_bytes(4, 128, 0, 0, _native.F32) == 0
     assert lib.thn_norm_bwd_workspace_bytes(0, 128, 1, 1, _native.F32) == 0
-    assert lib.thn_norm_set_launch_override(2, 0, 0, 0, 0) == _native.E_SHAPE
+    assert lib.thn_norm_set_launch_override(4, 0, 0, 0, 0) == _native.E_SHAPE
     assert lib.thn_norm_set_launch_override(0, 0, 0, 0, 0) == _native.OK
     if not torch.cuda.is_available():
         assert lib.thn_norm_bwd_workspace_bytes(4, 128, 1, 1, _native.F32) == _native.E_DEVICE
@@ -69,9 +69,25 @@ def test_argument_checks_answer_without_a_gpu():
         _native.check(_native.E_WORKSPACE)
 
 
+def test_softmax_argument_checks_answer_without_a_gpu():
+    lib = _native.lib()
+    fwd = lambda m, n, kind, dt: lib.thn_softmax_fwd(0, n, 0, n, m, n, kind, dt, 0)
+    bwd = lambda m, n, kind, dt: lib.thn_softmax_bwd(0, n, 0, n, 0, n, m, n, kind, dt, 0)
+    for call in (fwd, bwd):
+        assert call(4, 128, 0, 5) == _native.E_DTYPE
+        assert call(4, 128, 3, _native.F32) == _native.E_SHAPE           # unknown kind
+        assert call(4, 0, 0, _native.F32) == _native.E_SHAPE and call(-2, 8, 0, _native.F32) == _native.E_SHAPE
+        assert call(4, 16385, 0, _native.F32) == _native.E_FEATURE_DIM
+        assert call(4, 32769, 2, _native.F16) == _native.E_FEATURE_DIM
+        assert call(4, 8193, 1, _native.F64) == _native.E_FEATURE_DIM
+        assert call(0, 128, 0, _native.BF16) == _native.OK
+        assert call(4, 128, 0, _native.BF16) == _native.E_NULL
+    assert (_native.SOFTMAX, _native.SOFTMIN, _native.LOGSOFTMAX) == (0, 1, 2)   # enum thn_softmax_kind
+
+
 def test_no_cpu_fallback():
     x = torch.randn(4, 32)
-    for mod in (LayerNorm(32), RMSNorm(32)):
+    for mod in (LayerNorm(32), RMSNorm(32), Activations.Softmax(), Activations.Softmin(), Activations.LogSoftmax()):
         with pytest.raises(RuntimeError, match="no CPU fallback"):
             mod(x)
 
@@ -81,6 +97,18 @@ def test_package_surface():
     assert issubclass(layernorm, torch.autograd.Function) and issubclass(rmsnorm, torch.autograd.Function)
     import TritonHub
     assert TritonHub.__version__ == "1.1.1"
+    # the row-reduction activations of TritonHub/Activations/__init__.py (softmax.py:96-100, softmin.py:104-109,
+    # logsoftmax.py:106-110): plain callables holding the Function's apply
+    assert Activations.__all__ == ["Softmax", "Softmin", "LogSoftmax"]
+    from TritonHub.Activations.logsoftmax import logsoftmax
+    from TritonHub.Activations.softmax import softmax
+    from TritonHub.Activations.softmin import softmin
+    for fn in (softmax, softmin, logsoftmax):
+        assert issubclass(fn, torch.autograd.Function)
+    assert Activations.Softmax().softmax_fn is not None and Activations.Softmin().softmin_fn is not None
+    assert Activations.LogSoftmax().logsoftmax_fn is not None
+    with pytest.raises(RuntimeError, match="doesn't support feature dim >= 64KB"):
+        Activations._launch._check_row(16385, 4)
 
 
 @pytest.mark.parametrize("affine,bias", [(True, True), (True, False), (False, True), (False, False)])

@@ -1,0 +1,294 @@
+"""GPU parity tests of Softmax / Softmin / LogSoftmax: the HIP path, called through the operator interface and
+the C ABI, against the float64 CPU oracle on the same seeded inputs.
+
+Tolerances (as for the norm path): float32 storage max(1e-5, 4 float32 ulp); float16 / bfloat16 1 ulp of the
+output type at the oracle's value plus 4 * 2^-24 * (magnitude of the operands that were subtracted to form
+the result); float64 softmax / softmin are computed in float64 (as the reference does) and held to 1e-13,
+float64 log-softmax is float32 arithmetic (logsoftmax.py:19) and held to the float32 bound.
+The backward is a function of the SAVED OUTPUT (softmax.py:99-107): its expected value is the oracle's backward
+evaluated at the very output tensor the GPU saved, so forward rounding does not leak into the comparison.
+"""
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+
+from conftest import ROOT, check_elementwise, f64
+from oracle import softmax_oracle as so
+from TritonHub import _native
+from TritonHub.Activations import LogSoftmax, Softmax, Softmin, _launch
+from TritonHub.Activations.logsoftmax import logsoftmax
+from TritonHub.Activations.softmax import softmax
+from TritonHub.Activations.softmin import softmin
+
+pytestmark = pytest.mark.gpu
+KINDS = ["softmax", "softmin", "logsoftmax"]
+MODULE = {"softmax": Softmax, "softmin": Softmin, "logsoftmax": LogSoftmax}
+CODE = {"softmax": _native.SOFTMAX, "softmin": _native.SOFTMIN, "logsoftmax": _native.LOGSOFTMAX}
+
+
+def announce(msg):
+    print(f"\n[case] {msg}", flush=True)
+
+
+def check(got, ref, scale, dtype, kind, what):
+    if dtype == torch.float64 and kind != "logsoftmax":
+        err = np.abs(f64(got) - ref)
+        bound = 1e-13 * np.maximum(1.0, np.abs(ref))
+        assert (err <= bound).all(), f"{what}: float64 error {err.max():.3e}"
+        return
+    check_elementwise(f64(got), ref, scale, dtype, what)
+
+
+def run_and_compare(kind, x, dy, what, chunk_rows=4096, x_gpu=None, dy_gpu=None):
+    """x, dy: CPU tensors in the storage dtype.  Forward + backward through the callable, compared in row chunks.
+    `x_gpu` / `dy_gpu`: the same values already on the device (to keep a view's strides)."""
+    dtype = x.dtype
+    xg = (x.cuda() if x_gpu is None else x_gpu).requires_grad_(True)
+    y = MODULE[kind]()(xg)
+    y.backward(dy.cuda() if dy_gpu is None else dy_gpu)
+    torch.cuda.synchronize()
+    assert y.dtype == dtype and y.shape == x.shape and xg.grad.dtype == dtype and xg.grad.shape == x.shape
+    n = x.shape[-1]
+    x2, dy2 = x.reshape(-1, n), dy.reshape(-1, n)
+    y2, dx2 = y.detach().reshape(-1, n).cpu(), xg.grad.reshape(-1, n).cpu()
+    for s in range(0, x2.shape[0], chunk_rows):
+        e = min(s + chunk_rows, x2.shape[0])
+        xc, gc = f64(x2[s:e]), f64(dy2[s:e])
+        yo = so.FWD[kind](xc)
+        if kind == "logsoftmax":
+            z = (xc - xc.max(1, keepdims=True))
+            scale = np.abs(z) + np.abs(yo - z)          # y = z - log(sum): the two cancel near the row maximum
+        else:
+            scale = np.abs(yo)
+        check(y2[s:e], yo, scale, dtype, kind, f"{what} y rows {s}:{e}")
+        ys = f64(y2[s:e])                               # the saved output, as stored
+        dxo = so.BWD[kind](ys, gc)
+        if kind == "logsoftmax":
+            scale = np.abs(gc) + np.exp(ys) * np.abs(gc).sum(1, keepdims=True)
+        else:
+            scale = np.abs(ys) * (np.abs(gc) + np.abs(ys * gc).sum(1, keepdims=True))
+        check(dx2[s:e], dxo, scale, dtype, kind, f"{what} dx rows {s}:{e}")
+    return y.detach(), xg.grad
+
+
+def make(shape, dtype, seed, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    x = (torch.randn(shape, generator=g) * scale).to(dtype)
+    dy = torch.randn(shape, generator=g).to(dtype)
+    return x, dy
+
+
+# ---- the reference's unit-test matrix (UnitTests/Activations/softmax_unittest.py:63-68 and twins) ---------------
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32, torch.float64])
+@pytest.mark.parametrize("dim", [32, 64, 128, 256, 512, 1024, 2048])
+@pytest.mark.parametrize("kind", KINDS)
+def test_reference_unit_test_matrix(kind, dim, dtype):
+    announce(f"reference matrix {kind} D={dim} {dtype}")
+    torch.manual_seed(42)
+    data = torch.randn(1, 256, 256, dim, device="cuda", dtype=dtype)
+    theirs = {"softmax": torch.nn.Softmax(dim=-1), "softmin": torch.nn.Softmin(dim=-1),
+              "logsoftmax": torch.nn.LogSoftmax(dim=-1)}[kind]
+    a = data.clone().requires_grad_(True)
+    r = data.clone().requires_grad_(True)
+    rtol, atol = (3e-4, 1e-3) if dtype == torch.float32 else (5e-3, 1e-2)      # softmax_unittest.py:31-33
+    if dtype == torch.float16:
+        rtol, atol = 1e-2, 5e-2
+    ya, yr = MODULE[kind]()(a), theirs(r)
+    assert torch.allclose(ya, yr, atol=atol, rtol=rtol), "Error in forward pass"
+    g = torch.randn_like(ya)
+    ya.backward(g); yr.backward(g)
+    assert torch.allclose(a.grad, r.grad, atol=atol, rtol=rtol), "Error in backward pass"
+    # and the real bar, on a slice of the same data, against the oracle
+    x = data[0, :16].cpu()
+    run_and_compare(kind, x, g[0, :16].cpu(), f"{kind} D={dim} {dtype}")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16, torch.float64])
+@pytest.mark.parametrize("n", [1, 2, 7, 33, 100, 257, 1000, 4099, 6001])
+@pytest.mark.parametrize("kind", KINDS)
+def test_ragged_row_widths(kind, n, dtype):
+    announce(f"ragged {kind} N={n} {dtype}")
+    x, dy = make((37, n), dtype, seed=n, scale=3.0)
+    run_and_compare(kind, x, dy, f"{kind} N={n} {dtype}")
+
+
+@pytest.mark.parametrize("dtype,n_max", [(torch.float32, 16384), (torch.bfloat16, 32768), (torch.float16, 32768),
+                                         (torch.float64, 8192)])
+@pytest.mark.parametrize("kind", KINDS)
+def test_row_width_limit(kind, dtype, n_max):
+    announce(f"row limit {kind} {dtype} N={n_max}")
+    x, dy = make((6, n_max), dtype, seed=5, scale=2.0)
+    run_and_compare(kind, x, dy, f"{kind} N={n_max}")
+    over = torch.randn(2, n_max + 8, device="cuda").to(dtype)
+    with pytest.raises(RuntimeError, match="feature dim >= 64KB"):
+        MODULE[kind]()(over)
+
+
+@pytest.mark.parametrize("kind", KINDS)
+def test_large_logits_and_saturated_rows(kind):
+    """Rows whose entries span hundreds of units (exp underflows for most columns), a row with one dominant entry,
+    a constant row: the maximum is subtracted first, so nothing overflows and the closed forms hold."""
+    announce(f"large logits {kind}")
+    g = torch.Generator().manual_seed(8)
+    x = torch.randn(64, 512, generator=g) * 60.0
+    x[0] = 0.25
+    x[1] = -1000.0; x[1, 17] = 1000.0
+    dy = torch.randn(64, 512, generator=g)
+    y, _ = run_and_compare(kind, x, dy, f"{kind} large logits")
+    assert bool(torch.isfinite(y[2:]).all()) or kind == "logsoftmax"
+    if kind == "logsoftmax":
+        assert torch.allclose(y[0].cpu(), torch.full((512,), -float(np.log(512.0))), atol=2e-6)
+        assert float(y[1, 17]) == 0.0
+    else:
+        assert torch.allclose(y[0].cpu(), torch.full((512,), 1.0 / 512), rtol=1e-6)
+        hot = 17 if kind == "softmax" else None
+        if hot is not None:
+            assert float(y[1, hot]) == 1.0 and float(y[1].sum()) == 1.0
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float64])
+@pytest.mark.parametrize("kind", KINDS)
+def test_strides_views_and_batch_shapes(kind, dtype):
+    announce(f"strides {kind} {dtype}")
+    g = torch.Generator().manual_seed(12)
+    base = (torch.randn(40, 640, generator=g) * 2).to(dtype)
+    gbase = torch.randn(40, 640, generator=g).to(dtype)
+    bg, gg = base.cuda(), gbase.cuda()
+    for i, view in enumerate((lambda t: t[:, :512], lambda t: t[:, 3:515], lambda t: t[::2, 64:576],
+                              lambda t: t.t()[:600, :32], lambda t: t[:, :512].reshape(5, 8, 512),
+                              lambda t: t[0, :512], lambda t: t[:, 5:6], lambda t: t[3:4].expand(6, 640))):
+        xv, gv = view(base), view(gbase)
+        y, dx = run_and_compare(kind, xv.contiguous(), gv.contiguous(), f"{kind} view {i}", x_gpu=view(bg).detach(),
+                                dy_gpu=view(gg))
+        assert y.shape == xv.shape and dx.shape == xv.shape and y.is_contiguous()
+
+
+def test_empty_input_and_single_element_rows():
+    announce("softmax empty / N=1")
+    for kind in KINDS:
+        mod = MODULE[kind]()
+        x = torch.empty(0, 64, device="cuda", requires_grad=True)
+        y = mod(x)
+        y.sum().backward()
+        assert y.shape == (0, 64) and x.grad.shape == (0, 64)
+        one = torch.randn(9, 1, device="cuda", requires_grad=True)
+        y1 = mod(one)
+        y1.backward(torch.randn(9, 1, device="cuda"))
+        expect = 0.0 if kind == "logsoftmax" else 1.0
+        assert bool((y1 == expect).all()) and bool((one.grad == 0).all())
+
+
+def test_softmin_function_and_callable_follow_the_reference():
+    """softmin.apply(z) is softmax(z) (softmin.py:84-96); Softmin()(x) is softmin.apply(-x) (softmin.py:103):
+    values and gradients of the fused callable equal those of the explicit negation bit for bit."""
+    announce("softmin semantics")
+    g = torch.Generator().manual_seed(77)
+    for dtype in (torch.float32, torch.bfloat16, torch.float64):
+        x = (torch.randn(300, 777, generator=g) * 4).to(dtype).cuda()
+        dy = torch.randn(300, 777, generator=g).to(dtype).cuda()
+        a = x.clone().requires_grad_(True)
+        b = x.clone().requires_grad_(True)
+        c = x.clone().requires_grad_(True)
+        ya = Softmin()(a); ya.backward(dy)
+        yb = softmin.apply(-b); yb.backward(dy)
+        yc = softmax.apply(-c); yc.backward(dy)
+        assert torch.equal(ya, yb) and torch.equal(a.grad, b.grad)
+        assert torch.equal(yb, yc) and torch.equal(b.grad, c.grad)
+        assert torch.equal(softmin.apply(x), softmax.apply(x))
+        assert Softmin().softmin_fn is not None
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_properties_at_large_size(dtype):
+    """Size-independent properties on 65536 x 4096: rows sum to one, shift invariance, exp(log-softmax) = softmax,
+    gradients sum to zero over each row, determinism."""
+    announce(f"softmax properties {dtype}")
+    m, n = 65536, 4096
+    g = torch.Generator(device="cuda").manual_seed(3)
+    x = (torch.randn(m, n, device="cuda", generator=g) * 3).to(dtype)
+    dy = torch.randn(m, n, device="cuda", generator=g).to(dtype)
+    p = softmax.apply(x)
+    tol = 2e-6 if dtype == torch.float32 else 4e-3          # half an ulp of bfloat16 is up to 2^-8 relative
+    assert float((p.double().sum(1) - 1).abs().max()) < tol
+    assert torch.equal(softmax.apply(x), p)
+    small = ((x.float().clamp(-7, 7) * 4).round() / 4).to(dtype)      # multiples of 1/4: small + 8 is exact in bfloat16
+    assert torch.equal((small + 8.0).float() - 8.0, small.float())
+    assert torch.equal(softmax.apply(small + 8.0), softmax.apply(small))        # x - max(x) is the same float32 value
+    lp = logsoftmax.apply(x)
+    rel = ((lp.double().exp() - p.double()).abs() / p.double().clamp_min(1e-30)).max()
+    assert float(rel) < (2e-5 if dtype == torch.float32 else 0.09)    # bfloat16: |lp| up to ~25, half an ulp is 0.06
+    dx = _launch.softmax_bwd(p, dy, _native.SOFTMAX)
+    ref_scale = float((p.double() * dy.double().abs()).sum(1).max())
+    assert float(dx.double().sum(1).abs().max()) < (1e-5 if dtype == torch.float32 else 4e-3) * max(1.0, ref_scale) * 4
+    dl = _launch.softmax_bwd(lp, dy, _native.LOGSOFTMAX)
+    assert dl.shape == x.shape and bool(torch.isfinite(dl).all())
+    assert torch.equal(_launch.softmax_bwd(p, dy, _native.SOFTMIN), -dx)
+    # spot rows against the oracle
+    idx = torch.tensor([0, 1, 31337, m - 1], device="cuda")
+    for kind in KINDS:
+        run_and_compare(kind, x[idx].cpu(), dy[idx].cpu(), f"{kind} spot rows")
+
+
+def test_c_abi_direct_calls_and_errors():
+    announce("softmax C ABI direct")
+    lib = _native.lib()
+    st = torch.cuda.current_stream().cuda_stream
+    g = torch.Generator().manual_seed(19)
+    m, n, pitch = 129, 768, 1024
+    xb = (torch.randn(m, pitch, generator=g) * 2).cuda()
+    gb = torch.randn(m, pitch, generator=g).cuda()
+    for kind in KINDS:
+        y = torch.full((m, pitch), 7.0, device="cuda"); dx = torch.full((m, pitch), 7.0, device="cuda")
+        assert lib.thn_softmax_fwd(xb.data_ptr(), pitch, y.data_ptr(), pitch, m, n, CODE[kind], _native.F32, st) == 0
+        assert lib.thn_softmax_bwd(y.data_ptr(), pitch, gb.data_ptr(), pitch, dx.data_ptr(), pitch, m, n, CODE[kind],
+                                   _native.F32, st) == 0
+        torch.cuda.synchronize()
+        assert bool((y[:, n:] == 7.0).all()) and bool((dx[:, n:] == 7.0).all())        # padding untouched
+        yo = so.FWD[kind](f64(xb[:, :n]))
+        check_elementwise(f64(y[:, :n]), yo, np.abs(yo), torch.float32, f"C ABI {kind} y")
+        dxo = so.BWD[kind](f64(y[:, :n]), f64(gb[:, :n]))
+        check_elementwise(f64(dx[:, :n]), dxo, np.abs(dxo), torch.float32, f"C ABI {kind} dx")
+    y = torch.empty(m, n, device="cuda")
+    assert lib.thn_softmax_fwd(xb.data_ptr(), n - 1, y.data_ptr(), n, m, n, 0, _native.F32, st) == _native.E_SHAPE
+    assert lib.thn_softmax_fwd(xb.data_ptr(), pitch, 0, n, m, n, 0, _native.F32, st) == _native.E_NULL
+    assert lib.thn_softmax_fwd(xb.data_ptr(), pitch, y.data_ptr(), n, m, n, 5, _native.F32, st) == _native.E_SHAPE
+    assert lib.thn_softmax_bwd(y.data_ptr(), n, 0, n, y.data_ptr(), n, m, n, 0, _native.F32, st) == _native.E_NULL
+
+
+def compiled_forward_shapes():
+    text = open(os.path.join(ROOT, "triton-hub_amd", "csrc", "thn_dispatch.h")).read()
+    body = re.search(r"#define THN_FWD_SHAPES\(X\)(.*?)\n\n", text, re.S).group(1)
+    return [(int(k), int(t), int(b)) for k, t, b in re.findall(r"X\((\d+), (\d+), (\d+)\)", body)]
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32, torch.float64])
+def test_every_compiled_launch_shape(dtype):
+    """Forces each softmax kernel instance through the launch override (forward: family 2, backward: family 3)."""
+    lib = _native.lib()
+    shapes = compiled_forward_shapes()
+    assert len(shapes) >= 20
+    vec = 16 // torch.empty(0, dtype=dtype).element_size()
+    g = torch.Generator().manual_seed(29)
+    try:
+        for k, tpr, block in shapes:
+            for n_vecs in sorted({k * tpr, max((k - 1) * tpr + 1, k * tpr - tpr // 2 - 1)}):
+                n = n_vecs * vec
+                if n * (16 // vec) > 65536:
+                    continue
+                rows_per_block = block // tpr
+                m = 2 * rows_per_block + max(1, rows_per_block // 2)
+                announce(f"softmax shape K={k} TPR={tpr} block={block} N={n} M={m} {dtype}")
+                assert lib.thn_norm_set_launch_override(2, k, tpr, block, 0) == 0
+                assert lib.thn_norm_set_launch_override(3, k, tpr, block, 0) == 0
+                from TritonHub.Normalization._launch import query_launch
+                assert query_launch(2, False, m, n, dtype)[:3] == (k, tpr, block)
+                assert query_launch(3, False, m, n, dtype)[:3] == (k, tpr, block)
+                x = (torch.randn(m, n, generator=g) * 2).to(dtype); dy = torch.randn(m, n, generator=g).to(dtype)
+                for kind in ("softmax", "logsoftmax"):
+                    run_and_compare(kind, x, dy, f"{kind} K={k} TPR={tpr} block={block} N={n}")
+    finally:
+        lib.thn_norm_set_launch_override(2, 0, 0, 0, 0)
+        lib.thn_norm_set_launch_override(3, 0, 0, 0, 0)

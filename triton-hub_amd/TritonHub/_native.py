@@ -16,6 +16,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, 'libthnorm.so')
 
 F32, F16, BF16, F64 = 0, 1, 2, 3
+SOFTMAX, SOFTMIN, LOGSOFTMAX = 0, 1, 2
 DTYPE_CODES = {torch.float32: F32, torch.float16: F16, torch.bfloat16: BF16, torch.float64: F64}
 
 OK = 0
@@ -33,6 +34,8 @@ SYMBOLS = {
     'thn_norm_bwd_dx_partials': (_i32, [_vp, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _vp, _i32, _i32, _vp, _i64,
                                         ctypes.POINTER(ctypes.c_int32), _i64, _i64, _i32, _i32, _vp]),
     'thn_norm_bwd_reduce_partials': (_i32, [_vp, ctypes.c_int32, _vp, _vp, _i64, _i32, _vp]),
+    'thn_softmax_fwd': (_i32, [_vp, _i64, _vp, _i64, _i64, _i64, _i32, _i32, _vp]),
+    'thn_softmax_bwd': (_i32, [_vp, _i64, _vp, _i64, _vp, _i64, _i64, _i64, _i32, _i32, _vp]),
     'thn_norm_set_launch_override': (_i32, [_i32, _i32, _i32, _i32, _i32]),
     'thn_norm_query_launch': (_i32, [_i32, _i32, _i64, _i64, _i32, ctypes.POINTER(ctypes.c_int32)]),
 }

@@ -8,12 +8,18 @@
 
 #include "thn_dispatch.h"
 #include "thn_reduce.h"
+#include "thn_softmax_dispatch.h"
 
 namespace {
 
 using thn::BwdArgs;
 using thn::FwdArgs;
 using thn::Shape;
+using thn::SoftmaxBwdArgs;
+using thn::SoftmaxFwdArgs;
+
+// `which` throughout this file: the kernel family a launch belongs to.
+enum : int { kNormFwd = 0, kNormBwd = 1, kSoftmaxFwd = 2, kSoftmaxBwd = 3, kFamilies = 4 };
 
 constexpr int kMaxDevices = 64;
 constexpr int64_t kMaxRowBytes = 65536;   // the reference's MAX_FUSED_SIZE (layernorm.py:69-72)
@@ -51,16 +57,16 @@ int elem_bytes(int dtype) {
 struct Override {
     std::atomic<int> k{0}, tpr{0}, block{0}, bpc{0};
 };
-Override g_override[2];
+Override g_override[kFamilies];
 
 bool shape_compiled(int which, bool aligned, Shape s) {
 #define THN_MATCH(K_, TPR_, BLOCK_) if (s.k == K_ && s.tpr == TPR_ && s.block == BLOCK_) return true;
     if (!aligned) {
         THN_SCALAR_SHAPES(THN_MATCH)
-    } else if (which == 0) {
-        THN_FWD_SHAPES(THN_MATCH)
-    } else {
+    } else if (which == kNormBwd) {
         THN_BWD_SHAPES(THN_MATCH)
+    } else {
+        THN_FWD_SHAPES(THN_MATCH)
     }
 #undef THN_MATCH
     return false;
@@ -84,6 +90,26 @@ int launch_bwd(int dtype, bool ln, bool aligned, Shape s, const BwdArgs& a, int 
     }
 }
 
+int launch_softmax_fwd(int dtype, bool is_log, bool aligned, Shape s, const SoftmaxFwdArgs& a, int grid,
+                       hipStream_t st, int* occ) {
+    switch (dtype) {
+        case THN_F32: return thn::launch_softmax_fwd_f32(is_log, aligned, s, a, grid, st, occ);
+        case THN_F16: return thn::launch_softmax_fwd_f16(is_log, aligned, s, a, grid, st, occ);
+        case THN_BF16: return thn::launch_softmax_fwd_bf16(is_log, aligned, s, a, grid, st, occ);
+        default: return thn::launch_softmax_fwd_f64(is_log, aligned, s, a, grid, st, occ);
+    }
+}
+
+int launch_softmax_bwd(int dtype, bool is_log, bool aligned, Shape s, const SoftmaxBwdArgs& a, int grid,
+                       hipStream_t st, int* occ) {
+    switch (dtype) {
+        case THN_F32: return thn::launch_softmax_bwd_f32(is_log, aligned, s, a, grid, st, occ);
+        case THN_F16: return thn::launch_softmax_bwd_f16(is_log, aligned, s, a, grid, st, occ);
+        case THN_BF16: return thn::launch_softmax_bwd_bf16(is_log, aligned, s, a, grid, st, occ);
+        default: return thn::launch_softmax_bwd_f64(is_log, aligned, s, a, grid, st, occ);
+    }
+}
+
 // Workgroups of one kernel instance that fit on a compute unit; asked of the runtime once per instance.
 std::mutex g_occ_mutex;
 std::unordered_map<uint64_t, int> g_occ_cache;
@@ -102,12 +128,18 @@ int occupancy(int which, int dtype, bool ln, bool aligned, Shape s) {
     }
     int occ = 0;
     int rc;
-    if (which == 0) {
+    if (which == kNormFwd) {
         FwdArgs dummy{};
         rc = launch_fwd(dtype, ln, aligned, s, dummy, 0, nullptr, &occ);
-    } else {
+    } else if (which == kNormBwd) {
         BwdArgs dummy{};
         rc = launch_bwd(dtype, ln, aligned, s, dummy, 0, nullptr, &occ);
+    } else if (which == kSoftmaxFwd) {
+        SoftmaxFwdArgs dummy{};
+        rc = launch_softmax_fwd(dtype, ln, aligned, s, dummy, 0, nullptr, &occ);
+    } else {
+        SoftmaxBwdArgs dummy{};
+        rc = launch_softmax_bwd(dtype, ln, aligned, s, dummy, 0, nullptr, &occ);
     }
     if (rc != 0 || occ <= 0) occ = 1;
     if (occ > kMaxBlocksPerCu) occ = kMaxBlocksPerCu;
@@ -142,7 +174,8 @@ int ceil_div(int a, int b) { return (a + b - 1) / b; }
 
 Shape heuristic_shape(int which, bool ln, bool aligned, int n_vecs) {
     (void)ln;
-    const int kmax = (aligned && which == 1 && n_vecs > 128) ? 3 : 4;
+    int kmax = (aligned && which == kNormBwd && n_vecs > 128) ? 3 : 4;
+    if (aligned && which == kSoftmaxBwd && n_vecs <= 2048) kmax = 2;     // two input streams, nothing to hold
     Shape s{4, 1024, 1024};
     for (int tpr : kTprList) {
         if (static_cast<int64_t>(tpr) * kmax >= n_vecs) {
@@ -157,7 +190,7 @@ Shape heuristic_shape(int which, bool ln, bool aligned, int n_vecs) {
     }
     s.k = ceil_div(n_vecs, s.tpr);
     if (s.k == 3 && s.tpr < 64) s.k = 4;     // K = 3 is only compiled for TPR >= 64
-    if (which == 0) s.block = s.tpr > 256 ? s.tpr : 256;
+    if (which != kNormBwd) s.block = s.tpr > 256 ? s.tpr : 256;
     else s.block = s.tpr >= 128 ? (s.tpr > 512 ? s.tpr : 512) : 256;
     return s;
 }
@@ -229,7 +262,7 @@ const char* thn_strerror(int status) {
 
 int thn_norm_set_launch_override(int which, int vecs_per_thread, int threads_per_row, int block_threads,
                                  int blocks_per_cu) {
-    if (which < 0 || which > 1) return THN_E_SHAPE;
+    if (which < 0 || which >= kFamilies) return THN_E_SHAPE;
     if (vecs_per_thread < 0 || threads_per_row < 0 || block_threads < 0 || blocks_per_cu < 0) return THN_E_SHAPE;
     Override& ov = g_override[which];
     ov.k.store(vecs_per_thread);
@@ -240,7 +273,7 @@ int thn_norm_set_launch_override(int which, int vecs_per_thread, int threads_per
 }
 
 int thn_norm_query_launch(int which, int is_layernorm, int64_t M, int64_t N, int x_dtype, int32_t shape[5]) {
-    if (which < 0 || which > 1 || shape == nullptr) return THN_E_SHAPE;
+    if (which < 0 || which >= kFamilies || shape == nullptr) return THN_E_SHAPE;
     const int bytes = elem_bytes(x_dtype);
     if (bytes == 0) return THN_E_DTYPE;
     Plan p;
@@ -272,7 +305,7 @@ int thn_norm_fwd(const void* x, int64_t x_row_stride, void* y, int64_t y_row_str
     const bool aligned = (N % vec_elems) == 0 && aligned16(x) && aligned16(y) && aligned16(w) && aligned16(b) &&
                          (x_row_stride * bytes) % 16 == 0 && (y_row_stride * bytes) % 16 == 0;
     Plan p;
-    const int rc = plan_launch(0, ln, aligned, M, N, x_dtype, &p);
+    const int rc = plan_launch(kNormFwd, ln, aligned, M, N, x_dtype, &p);
     if (rc != THN_OK) return rc;
 
     FwdArgs a{};
@@ -335,7 +368,7 @@ int thn_norm_bwd_dx_partials(const void* x, int64_t x_row_stride, const void* dy
                          (x_row_stride * bytes) % 16 == 0 && (dy_row_stride * bytes) % 16 == 0 &&
                          (dx_row_stride * bytes) % 16 == 0;
     Plan p;
-    const int rc = plan_launch(1, ln, aligned, M, N, x_dtype, &p);
+    const int rc = plan_launch(kNormBwd, ln, aligned, M, N, x_dtype, &p);
     if (rc != THN_OK) return rc;
     const int64_t pitch = partial_pitch(N);
     const int64_t need = n_grads * static_cast<int64_t>(p.grid) * pitch * static_cast<int64_t>(sizeof(float));
@@ -411,6 +444,71 @@ int thn_norm_bwd(const void* x, int64_t x_row_stride, const void* dy, int64_t dy
     if (rc != THN_OK) return rc;
     // M == 0: no partial rows; the reduction then writes zeros, the sum of an empty set of rows.
     return thn_norm_bwd_reduce_partials(workspace, parts, dw, db, N, w_dtype, stream);
+}
+
+// ---- Softmax / Softmin / LogSoftmax -------------------------------------------------------------------------
+
+int thn_softmax_fwd(const void* x, int64_t x_row_stride, void* y, int64_t y_row_stride, int64_t M, int64_t N,
+                    int kind, int dtype, void* stream) {
+    const int bytes = elem_bytes(dtype);
+    if (bytes == 0) return THN_E_DTYPE;
+    if (M < 0 || N <= 0 || kind < THN_SOFTMAX || kind > THN_LOGSOFTMAX) return THN_E_SHAPE;
+    if (N * bytes > kMaxRowBytes) return THN_E_FEATURE_DIM;
+    if (M == 0) return THN_OK;
+    if (x == nullptr || y == nullptr) return THN_E_NULL;
+    if (x_row_stride < N || y_row_stride < N) return THN_E_SHAPE;
+    const int vec_elems = 16 / bytes;
+    const bool aligned = (N % vec_elems) == 0 && aligned16(x) && aligned16(y) && (x_row_stride * bytes) % 16 == 0 &&
+                         (y_row_stride * bytes) % 16 == 0;
+    const bool is_log = kind == THN_LOGSOFTMAX;
+    Plan p;
+    const int rc = plan_launch(kSoftmaxFwd, is_log, aligned, M, N, dtype, &p);
+    if (rc != THN_OK) return rc;
+    SoftmaxFwdArgs a{};
+    a.x = static_cast<const char*>(x);
+    a.y = static_cast<char*>(y);
+    a.x_stride_bytes = x_row_stride * bytes;
+    a.y_stride_bytes = y_row_stride * bytes;
+    a.M = M;
+    a.n_cols = static_cast<int>(N);
+    a.n_vecs = p.n_vecs;
+    a.sign = kind == THN_SOFTMIN ? -1.0f : 1.0f;
+    const int lrc = launch_softmax_fwd(dtype, is_log, aligned, p.s, a, p.grid, static_cast<hipStream_t>(stream), nullptr);
+    if (lrc > 0) return THN_E_SHAPE;
+    return lrc == 0 ? THN_OK : THN_E_LAUNCH;
+}
+
+int thn_softmax_bwd(const void* y, int64_t y_row_stride, const void* dy, int64_t dy_row_stride, void* dx,
+                    int64_t dx_row_stride, int64_t M, int64_t N, int kind, int dtype, void* stream) {
+    const int bytes = elem_bytes(dtype);
+    if (bytes == 0) return THN_E_DTYPE;
+    if (M < 0 || N <= 0 || kind < THN_SOFTMAX || kind > THN_LOGSOFTMAX) return THN_E_SHAPE;
+    if (N * bytes > kMaxRowBytes) return THN_E_FEATURE_DIM;
+    if (M == 0) return THN_OK;
+    if (y == nullptr || dy == nullptr || dx == nullptr) return THN_E_NULL;
+    if (y_row_stride < N || dy_row_stride < N || dx_row_stride < N) return THN_E_SHAPE;
+    const int vec_elems = 16 / bytes;
+    const bool aligned = (N % vec_elems) == 0 && aligned16(y) && aligned16(dy) && aligned16(dx) &&
+                         (y_row_stride * bytes) % 16 == 0 && (dy_row_stride * bytes) % 16 == 0 &&
+                         (dx_row_stride * bytes) % 16 == 0;
+    const bool is_log = kind == THN_LOGSOFTMAX;
+    Plan p;
+    const int rc = plan_launch(kSoftmaxBwd, is_log, aligned, M, N, dtype, &p);
+    if (rc != THN_OK) return rc;
+    SoftmaxBwdArgs a{};
+    a.y = static_cast<const char*>(y);
+    a.dy = static_cast<const char*>(dy);
+    a.dx = static_cast<char*>(dx);
+    a.y_stride_bytes = y_row_stride * bytes;
+    a.dy_stride_bytes = dy_row_stride * bytes;
+    a.dx_stride_bytes = dx_row_stride * bytes;
+    a.M = M;
+    a.n_cols = static_cast<int>(N);
+    a.n_vecs = p.n_vecs;
+    a.sign = kind == THN_SOFTMIN ? -1.0f : 1.0f;
+    const int lrc = launch_softmax_bwd(dtype, is_log, aligned, p.s, a, p.grid, static_cast<hipStream_t>(stream), nullptr);
+    if (lrc > 0) return THN_E_SHAPE;
+    return lrc == 0 ? THN_OK : THN_E_LAUNCH;
 }
 
 }  // extern "C"

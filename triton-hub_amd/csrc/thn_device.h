@@ -287,35 +287,74 @@ __device__ __forceinline__ void store_vec_elems(char* row, int vec, int n_cols, 
 }
 
 // ---------------------------------------------------------------------------------------------------
-// Wave64 all-reduce (sum) over aligned groups of W lanes, W in {8, 16, 32, 64}.  The first four steps
-// are DPP modifiers fused into v_add_f32 (no LDS traffic); the 16- and 32-lane exchanges use the gfx950
+// Wave64 all-reduce (sum, or max with OpMax) over aligned groups of W lanes, W in {8, 16, 32, 64}.  The first four steps
+// are DPP modifiers fused into v_add_f32 / v_max_f32 (no LDS traffic); the 16- and 32-lane exchanges use the gfx950
 // v_permlane16_swap / v_permlane32_swap instructions.  Every lane of a group ends with the group's sum,
 // and all lanes of a group add the same values in the same tree, so the result is identical on all of them.
 // ---------------------------------------------------------------------------------------------------
 template <int CTRL>
-__device__ __forceinline__ float dpp_mov(float v) {
-    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true));
+__device__ __forceinline__ uint32_t dpp_mov_bits(uint32_t v) {
+    return static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v), CTRL, 0xF, 0xF, true));
+}
+template <int CTRL>
+__device__ __forceinline__ float dpp_mov(float v) { return as_f32(dpp_mov_bits<CTRL>(as_u32(v))); }
+// A float64 travels as its two 32-bit halves, each moved with the same lane pattern.
+template <int CTRL>
+__device__ __forceinline__ double dpp_mov(double v) {
+    const uint64_t u = __builtin_bit_cast(uint64_t, v);
+    const uint32_t lo = dpp_mov_bits<CTRL>(static_cast<uint32_t>(u));
+    const uint32_t hi = dpp_mov_bits<CTRL>(static_cast<uint32_t>(u >> 32));
+    return __builtin_bit_cast(double, (static_cast<uint64_t>(hi) << 32) | lo);
 }
 
-template <int W>
-__device__ __forceinline__ float group_allreduce(float v) {
-    static_assert(W == 8 || W == 16 || W == 32 || W == 64, "group width");
-    v += dpp_mov<0xB1>(v);    // quad_perm [1,0,3,2]: lane ^ 1
-    v += dpp_mov<0x4E>(v);    // quad_perm [2,3,0,1]: lane ^ 2
-    v += dpp_mov<0x141>(v);   // row_half_mirror: the other quad of each 8 lanes
-    if constexpr (W >= 16) v += dpp_mov<0x140>(v);   // row_mirror: the other half of each 16 lanes
-    if constexpr (W >= 32) {
-        const uint32_t u = as_u32(v);
-        auto r = __builtin_amdgcn_permlane16_swap(u, u, false, false);
-        const uint32_t a = r[0], b = r[1];
-        v = as_f32(a) + as_f32(b);
-    }
-    if constexpr (W >= 64) {
-        const uint32_t u = as_u32(v);
+struct OpSum {
+    template <typename V> __device__ static __forceinline__ V apply(V a, V b) { return a + b; }
+    template <typename V> __device__ static __forceinline__ V identity() { return V(0); }
+};
+struct OpMax {
+    __device__ static __forceinline__ float apply(float a, float b) { return fmaxf(a, b); }
+    __device__ static __forceinline__ double apply(double a, double b) { return fmax(a, b); }
+    template <typename V> __device__ static __forceinline__ V identity() { return -static_cast<V>(__builtin_inff()); }
+};
+
+// One 32-bit word exchanged with the partner lane 16 (WIDE = false) or 32 (WIDE = true) lanes away: `mine`
+// and `theirs` come back in an order that is the same on both partners' sides of the addition tree.
+template <bool WIDE>
+__device__ __forceinline__ void swap_lanes(uint32_t u, uint32_t& first, uint32_t& second) {
+    if constexpr (WIDE) {
         auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
-        const uint32_t a = r[0], b = r[1];
-        v = as_f32(a) + as_f32(b);
+        first = r[0]; second = r[1];
+    } else {
+        auto r = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+        first = r[0]; second = r[1];
     }
+}
+template <bool WIDE, typename Op>
+__device__ __forceinline__ float swap_combine(float v) {
+    uint32_t a, b;
+    swap_lanes<WIDE>(as_u32(v), a, b);
+    return Op::apply(as_f32(a), as_f32(b));
+}
+template <bool WIDE, typename Op>
+__device__ __forceinline__ double swap_combine(double v) {
+    const uint64_t u = __builtin_bit_cast(uint64_t, v);
+    uint32_t al, bl, ah, bh;
+    swap_lanes<WIDE>(static_cast<uint32_t>(u), al, bl);
+    swap_lanes<WIDE>(static_cast<uint32_t>(u >> 32), ah, bh);
+    const double a = __builtin_bit_cast(double, (static_cast<uint64_t>(ah) << 32) | al);
+    const double b = __builtin_bit_cast(double, (static_cast<uint64_t>(bh) << 32) | bl);
+    return Op::apply(a, b);
+}
+
+template <int W, typename Op = OpSum, typename V = float>
+__device__ __forceinline__ V group_allreduce(V v) {
+    static_assert(W == 8 || W == 16 || W == 32 || W == 64, "group width");
+    v = Op::apply(v, dpp_mov<0xB1>(v));    // quad_perm [1,0,3,2]: lane ^ 1
+    v = Op::apply(v, dpp_mov<0x4E>(v));    // quad_perm [2,3,0,1]: lane ^ 2
+    v = Op::apply(v, dpp_mov<0x141>(v));   // row_half_mirror: the other quad of each 8 lanes
+    if constexpr (W >= 16) v = Op::apply(v, dpp_mov<0x140>(v));   // row_mirror: the other half of each 16 lanes
+    if constexpr (W >= 32) v = swap_combine<false, Op>(v);
+    if constexpr (W >= 64) v = swap_combine<true, Op>(v);
     return v;
 }
 
@@ -324,15 +363,15 @@ __device__ __forceinline__ float group_allreduce(float v) {
 // row in a fixed order.  The slots are double buffered on `phase`, so one barrier per call is enough: a
 // slot is rewritten two calls later, and no wave can pass the barrier in between before all have read it.
 // All threads of the workgroup must call this together when TPR > 64.
-template <int TPR, int G, int NV>
-__device__ __forceinline__ void row_allreduce(float (&v)[NV], float* red, int& phase, int g, int t) {
+template <int TPR, int G, int NV, typename Op = OpSum, typename V = float>
+__device__ __forceinline__ void row_allreduce(V (&v)[NV], V* red, int& phase, int g, int t) {
     constexpr int W = TPR < 64 ? TPR : 64;
 #pragma unroll
-    for (int i = 0; i < NV; ++i) v[i] = group_allreduce<W>(v[i]);
+    for (int i = 0; i < NV; ++i) v[i] = group_allreduce<W, Op, V>(v[i]);
     if constexpr (TPR > 64) {
         constexpr int WPR = TPR / 64;
         constexpr int NVP = NV == 3 ? 4 : NV;
-        float* slot = red + (((phase & 1) * G + g) * WPR) * NVP;
+        V* slot = red + (((phase & 1) * G + g) * WPR) * NVP;
         const int wv = t >> 6;
         if ((t & 63) == 0) {
 #pragma unroll
@@ -340,11 +379,11 @@ __device__ __forceinline__ void row_allreduce(float (&v)[NV], float* red, int& p
         }
         __syncthreads();
 #pragma unroll
-        for (int i = 0; i < NV; ++i) v[i] = 0.0f;
+        for (int i = 0; i < NV; ++i) v[i] = Op::template identity<V>();
 #pragma unroll
         for (int w = 0; w < WPR; ++w) {
 #pragma unroll
-            for (int i = 0; i < NV; ++i) v[i] += slot[w * NVP + i];
+            for (int i = 0; i < NV; ++i) v[i] = Op::apply(v[i], slot[w * NVP + i]);
         }
         ++phase;
     }

@@ -1,0 +1,274 @@
+// Softmax / Softmin / LogSoftmax over the last dimension, forward and backward: the reference's
+// TritonHub/Activations/softmax.py, softmin.py and logsoftmax.py on the row engine of the norm kernels
+// (same decomposition, same branch-free prefetching loop; see thn_kernels.h).
+#pragma once
+
+#include <type_traits>
+
+#include "thn_kernels.h"
+
+namespace thn {
+
+struct SoftmaxFwdArgs {
+    const char* x;
+    char* y;
+    int64_t x_stride_bytes;
+    int64_t y_stride_bytes;
+    int64_t M;
+    int n_cols;
+    int n_vecs;
+    float sign;      // -1: the input is negated on load (Softmin of x = Softmax of -x)
+};
+
+struct SoftmaxBwdArgs {
+    const char* y;   // the SAVED OUTPUT of the forward (softmax.py:99-107, logsoftmax.py:119-127)
+    const char* dy;
+    char* dx;
+    int64_t y_stride_bytes;
+    int64_t dy_stride_bytes;
+    int64_t dx_stride_bytes;
+    int64_t M;
+    int n_cols;
+    int n_vecs;
+    float sign;      // -1: the gradient is negated on store (fused Softmin)
+};
+
+// Arithmetic type.  Float32 for 16- and 32-bit storage and for every log-softmax (logsoftmax.py:19, :71 widen
+// to float32 explicitly).  The reference's softmax / softmin kernels compute in the type they load
+// (softmax.py:18-23), so float64 rows are computed in float64.
+template <typename T, bool LOG> struct SoftmaxCompute { using type = float; };
+template <> struct SoftmaxCompute<F64, false> { using type = double; };
+
+template <typename T>
+__device__ __forceinline__ void unpack_as(u32x4 v, float (&f)[T::VEC]) { T::unpack(v, f); }
+template <typename T>
+__device__ __forceinline__ void unpack_as(u32x4 v, double (&f)[T::VEC]) {
+    static_assert(T::kBytes == 8, "float64 arithmetic is for float64 storage only");
+    const uint32_t a = v[0], b = v[1], c = v[2], d = v[3];
+    f[0] = __builtin_bit_cast(double, (static_cast<uint64_t>(b) << 32) | a);
+    f[1] = __builtin_bit_cast(double, (static_cast<uint64_t>(d) << 32) | c);
+}
+
+__device__ __forceinline__ u32x4 pack_f64(const double (&f)[2]) {
+    const uint64_t lo = __builtin_bit_cast(uint64_t, f[0]), hi = __builtin_bit_cast(uint64_t, f[1]);
+    u32x4 v;
+    v[0] = static_cast<uint32_t>(lo); v[1] = static_cast<uint32_t>(lo >> 32);
+    v[2] = static_cast<uint32_t>(hi); v[3] = static_cast<uint32_t>(hi >> 32);
+    return v;
+}
+
+// load_row for arithmetic type C: the element path of the float32 engine narrows float64 storage on load,
+// which the float64 path must not do.
+template <typename T, typename C, int K, bool ALIGNED>
+__device__ __forceinline__ void load_row_as(u32x4 (&dst)[K], const char* base, int64_t stride_bytes, int64_t row,
+                                            const int (&voff)[K], int n_cols) {
+    if constexpr (ALIGNED || std::is_same<C, float>::value) {
+        load_row<T, K, ALIGNED>(dst, base, stride_bytes, row, voff, n_cols);
+    } else {
+        const double* p = reinterpret_cast<const double*>(base + row * stride_bytes);
+#pragma unroll
+        for (int k = 0; k < K; ++k) {
+            double f[2];
+#pragma unroll
+            for (int e = 0; e < 2; ++e) {
+                const int c = voff[k] * 2 + e;
+                const double v = p[c < n_cols ? c : n_cols - 1];
+                f[e] = c < n_cols ? v : 0.0;
+            }
+            dst[k] = pack_f64(f);
+        }
+    }
+}
+
+template <typename T, bool ALIGNED>
+__device__ __forceinline__ void store_row_as(char* rowp, int voff, int n_cols, const float (&f)[T::VEC]) {
+    store_row_vec<T, ALIGNED>(rowp, voff, n_cols, f);
+}
+template <typename T, bool ALIGNED>
+__device__ __forceinline__ void store_row_as(char* rowp, int voff, int n_cols, const double (&f)[T::VEC]) {
+    static_assert(T::kBytes == 8, "float64 arithmetic is for float64 storage only");
+    if constexpr (ALIGNED) {
+        st128(rowp + voff, pack_f64(f));
+    } else {
+#pragma unroll
+        for (int e = 0; e < 2; ++e) {
+            const int c = voff * 2 + e;
+            if (c < n_cols) reinterpret_cast<double*>(rowp)[c] = f[e];
+        }
+    }
+}
+
+__device__ __forceinline__ float exp_c(float z) { return __expf(z); }
+__device__ __forceinline__ double exp_c(double z) { return exp(z); }
+
+// Forward (softmax.py:17-23, logsoftmax.py:19-24): z = x - max(x); softmax: exp(z) / sum(exp(z));
+// log-softmax: z - log(sum(exp(z))).  One rounding on store.
+template <typename T, bool LOG, int K, int TPR, int BLOCK, bool ALIGNED>
+__global__ void __launch_bounds__(BLOCK) softmax_fwd_kernel(const SoftmaxFwdArgs a) {
+    constexpr int VEC = T::VEC;
+    constexpr int G = BLOCK / TPR;
+    static_assert(BLOCK % TPR == 0 && G >= 1, "a workgroup holds whole rows");
+    using C = typename SoftmaxCompute<T, LOG>::type;
+    __shared__ C red[RedSmem<TPR, G, 1>::kFloats];
+
+    const int tid = threadIdx.x;
+    const int g = tid / TPR;
+    const int t = tid % TPR;
+    int phase = 0;
+
+    int voff[K];
+    bool own[K];
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+        const int v = t + k * TPR;
+        const int vc = v < a.n_vecs ? v : a.n_vecs - 1;
+        voff[k] = ALIGNED ? vc * 16 : vc;
+        own[k] = v < a.n_vecs;
+    }
+    const C sign = static_cast<C>(a.sign);
+    const C neg_inf = OpMax::identity<C>();
+
+    const int64_t rows_per_iter = static_cast<int64_t>(gridDim.x) * G;
+    const int64_t last_row = a.M - 1;
+    int64_t row_raw = static_cast<int64_t>(blockIdx.x) * G + g;
+    int64_t row = row_raw < a.M ? row_raw : last_row;
+    u32x4 cur[K];
+    load_row_as<T, C, K, ALIGNED>(cur, a.x, a.x_stride_bytes, row, voff, a.n_cols);
+
+    drain_vector_memory();
+    for (int64_t base = static_cast<int64_t>(blockIdx.x) * G; base < a.M; base += rows_per_iter) {
+        const int64_t nrow_raw = row_raw + rows_per_iter;
+        const int64_t nrow = nrow_raw < a.M ? nrow_raw : last_row;
+        u32x4 nxt[K];
+        load_row_as<T, C, K, ALIGNED>(nxt, a.x, a.x_stride_bytes, nrow, voff, a.n_cols);
+
+        C xf[K][VEC];
+        C m[1] = {neg_inf};
+#pragma unroll
+        for (int k = 0; k < K; ++k) {
+            unpack_as<T>(cur[k], xf[k]);
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+                C v = xf[k][e] * sign;
+                if constexpr (!ALIGNED) v = (voff[k] * VEC + e < a.n_cols) ? v : neg_inf;
+                xf[k][e] = v;
+                m[0] = OpMax::apply(m[0], v);      // clamped slots repeat real columns: harmless for a maximum
+            }
+        }
+        row_allreduce<TPR, G, 1, OpMax, C>(m, red, phase, g, t);
+
+        C s[1] = {C(0)};
+#pragma unroll
+        for (int k = 0; k < K; ++k) {
+            C sk = C(0);
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+                const C z = xf[k][e] - m[0];
+                const C ez = exp_c(z);              // columns past the row end: exp(-inf) = 0
+                xf[k][e] = LOG ? z : ez;
+                sk += ez;
+            }
+            s[0] += own[k] ? sk : C(0);
+        }
+        row_allreduce<TPR, G, 1, OpSum, C>(s, red, phase, g, t);
+        C scale;
+        if constexpr (LOG) scale = logf(s[0]);
+        else scale = C(1) / s[0];
+
+        char* yrow = a.y + row * a.y_stride_bytes;
+#pragma unroll
+        for (int k = 0; k < K; ++k) {
+            C yf[VEC];
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) yf[e] = LOG ? xf[k][e] - scale : xf[k][e] * scale;
+            store_row_as<T, ALIGNED>(yrow, voff[k], a.n_cols, yf);
+        }
+
+#pragma unroll
+        for (int k = 0; k < K; ++k) cur[k] = nxt[k];
+        row_raw = nrow_raw;
+        row = nrow;
+    }
+}
+
+// Backward from the saved output y and the upstream gradient g:
+//   softmax (softmax.py:57-60):       dx = y*g - y*sum(y*g)
+//   log-softmax (logsoftmax.py:73-76): dx = g - exp(y)*sum(g)
+template <typename T, bool LOG, int K, int TPR, int BLOCK, bool ALIGNED>
+__global__ void __launch_bounds__(BLOCK) softmax_bwd_kernel(const SoftmaxBwdArgs a) {
+    constexpr int VEC = T::VEC;
+    constexpr int G = BLOCK / TPR;
+    static_assert(BLOCK % TPR == 0 && G >= 1, "a workgroup holds whole rows");
+    using C = typename SoftmaxCompute<T, LOG>::type;
+    __shared__ C red[RedSmem<TPR, G, 1>::kFloats];
+
+    const int tid = threadIdx.x;
+    const int g = tid / TPR;
+    const int t = tid % TPR;
+    int phase = 0;
+
+    int voff[K];
+    bool own[K];
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+        const int v = t + k * TPR;
+        const int vc = v < a.n_vecs ? v : a.n_vecs - 1;
+        voff[k] = ALIGNED ? vc * 16 : vc;
+        own[k] = v < a.n_vecs;
+    }
+
+    const int64_t rows_per_iter = static_cast<int64_t>(gridDim.x) * G;
+    const int64_t last_row = a.M - 1;
+    int64_t row_raw = static_cast<int64_t>(blockIdx.x) * G + g;
+    int64_t row = row_raw < a.M ? row_raw : last_row;
+    const C sign = static_cast<C>(a.sign);
+    u32x4 cy[K], cg[K];
+    load_row_as<T, C, K, ALIGNED>(cy, a.y, a.y_stride_bytes, row, voff, a.n_cols);
+    load_row_as<T, C, K, ALIGNED>(cg, a.dy, a.dy_stride_bytes, row, voff, a.n_cols);
+
+    drain_vector_memory();
+    for (int64_t base = static_cast<int64_t>(blockIdx.x) * G; base < a.M; base += rows_per_iter) {
+        const int64_t nrow_raw = row_raw + rows_per_iter;
+        const int64_t nrow = nrow_raw < a.M ? nrow_raw : last_row;
+        u32x4 ny[K], ng[K];
+        load_row_as<T, C, K, ALIGNED>(ny, a.y, a.y_stride_bytes, nrow, voff, a.n_cols);
+        load_row_as<T, C, K, ALIGNED>(ng, a.dy, a.dy_stride_bytes, nrow, voff, a.n_cols);
+
+        C yf[K][VEC], gf[K][VEC];
+        C s[1] = {C(0)};
+#pragma unroll
+        for (int k = 0; k < K; ++k) {
+            unpack_as<T>(cy[k], yf[k]);
+            unpack_as<T>(cg[k], gf[k]);      // element path: columns past the row end load as 0
+            C sk = C(0);
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+                if constexpr (LOG) sk += gf[k][e];
+                else sk = fma(yf[k][e], gf[k][e], sk);
+            }
+            s[0] += own[k] ? sk : C(0);
+        }
+        row_allreduce<TPR, G, 1, OpSum, C>(s, red, phase, g, t);
+
+        char* dxrow = a.dx + row * a.dx_stride_bytes;
+#pragma unroll
+        for (int k = 0; k < K; ++k) {
+            C dxf[VEC];
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+                C d;
+                if constexpr (LOG) d = fma(-exp_c(yf[k][e]), s[0], gf[k][e]);
+                else d = yf[k][e] * (gf[k][e] - s[0]);
+                dxf[e] = d * sign;
+            }
+            store_row_as<T, ALIGNED>(dxrow, voff[k], a.n_cols, dxf);
+        }
+
+#pragma unroll
+        for (int k = 0; k < K; ++k) { cy[k] = ny[k]; cg[k] = ng[k]; }
+        row_raw = nrow_raw;
+        row = nrow;
+    }
+}
+
+}  // namespace thn

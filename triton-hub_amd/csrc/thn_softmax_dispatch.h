@@ -1,0 +1,53 @@
+// Run-time (dtype, flavour, shape) -> compiled softmax kernel instance; one translation unit per storage type.
+#pragma once
+
+#include "thn_dispatch.h"
+#include "thn_softmax.h"
+
+namespace thn {
+
+#define THN_DECLARE_SOFTMAX_LAUNCHERS(NAME)                                                                     \
+    int launch_softmax_fwd_##NAME(bool is_log, bool aligned, Shape s, const SoftmaxFwdArgs& a, int grid,        \
+                                  hipStream_t st, int* occupancy);                                              \
+    int launch_softmax_bwd_##NAME(bool is_log, bool aligned, Shape s, const SoftmaxBwdArgs& a, int grid,        \
+                                  hipStream_t st, int* occupancy);
+
+THN_DECLARE_SOFTMAX_LAUNCHERS(f32)
+THN_DECLARE_SOFTMAX_LAUNCHERS(f16)
+THN_DECLARE_SOFTMAX_LAUNCHERS(bf16)
+THN_DECLARE_SOFTMAX_LAUNCHERS(f64)
+
+#define THN_SM_CASE(KERNEL, ARGS_T, AL, K_, TPR_, BLOCK_)                                                      \
+    if (s.k == K_ && s.tpr == TPR_ && s.block == BLOCK_) {                                                     \
+        return is_log ? run_kernel<ARGS_T>(KERNEL<T, true, K_, TPR_, BLOCK_, AL>, a, grid, BLOCK_, st, occupancy) \
+                      : run_kernel<ARGS_T>(KERNEL<T, false, K_, TPR_, BLOCK_, AL>, a, grid, BLOCK_, st, occupancy); \
+    }
+#define THN_SMF_AL(K_, TPR_, BLOCK_) THN_SM_CASE(softmax_fwd_kernel, SoftmaxFwdArgs, true, K_, TPR_, BLOCK_)
+#define THN_SMF_SC(K_, TPR_, BLOCK_) THN_SM_CASE(softmax_fwd_kernel, SoftmaxFwdArgs, false, K_, TPR_, BLOCK_)
+#define THN_SMB_AL(K_, TPR_, BLOCK_) THN_SM_CASE(softmax_bwd_kernel, SoftmaxBwdArgs, true, K_, TPR_, BLOCK_)
+#define THN_SMB_SC(K_, TPR_, BLOCK_) THN_SM_CASE(softmax_bwd_kernel, SoftmaxBwdArgs, false, K_, TPR_, BLOCK_)
+
+// Both directions use the forward shape list of the norm kernels (no per-column accumulators to hold).
+#define THN_DEFINE_SOFTMAX_LAUNCHERS(NAME, TYPE)                                                                \
+    int launch_softmax_fwd_##NAME(bool is_log, bool aligned, Shape s, const SoftmaxFwdArgs& a, int grid,        \
+                                  hipStream_t st, int* occupancy) {                                             \
+        using T = TYPE;                                                                                         \
+        if (aligned) {                                                                                          \
+            THN_FWD_SHAPES(THN_SMF_AL)                                                                          \
+        } else {                                                                                                \
+            THN_SCALAR_SHAPES(THN_SMF_SC)                                                                       \
+        }                                                                                                       \
+        return 1;                                                                                               \
+    }                                                                                                           \
+    int launch_softmax_bwd_##NAME(bool is_log, bool aligned, Shape s, const SoftmaxBwdArgs& a, int grid,        \
+                                  hipStream_t st, int* occupancy) {                                             \
+        using T = TYPE;                                                                                         \
+        if (aligned) {                                                                                          \
+            THN_FWD_SHAPES(THN_SMB_AL)                                                                          \
+        } else {                                                                                                \
+            THN_SCALAR_SHAPES(THN_SMB_SC)                                                                       \
+        }                                                                                                       \
+        return 1;                                                                                               \
+    }
+
+}  // namespace thn
