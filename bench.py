@@ -1,5 +1,5 @@
 #!/usr/bin/env python3
-"""Benchmark of the LayerNorm / RMSNorm forward + backward path on one MI355X.
+"""Benchmark of the LayerNorm / RMSNorm (and Softmax-family) forward + backward path on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME]
 
@@ -40,7 +40,15 @@ WORKLOADS = {
     "rmsnorm_f16_4096x16384_outliers": ("rms", 4096, 16384, "f16"),
     "rmsnorm_f32_4096x16384_outliers": ("rms", 4096, 16384, "f32"),
     "layernorm_f32_200x128_quickstart": ("ln", 200, 128, "f32"),
+    # the row-reduction activations next to the norm path (thn_softmax_fwd + thn_softmax_bwd per step)
+    "softmax_bf16_16384x4096": ("softmax", 16384, 4096, "bf16"),
+    "softmax_f32_16384x4096": ("softmax", 16384, 4096, "f32"),
+    "softmax_f16_65536x1024": ("softmax", 65536, 1024, "f16"),
+    "softmin_bf16_16384x4096": ("softmin", 16384, 4096, "bf16"),
+    "logsoftmax_bf16_8192x32768": ("logsoftmax", 8192, 32768, "bf16"),
+    "logsoftmax_f32_16384x4096": ("logsoftmax", 16384, 4096, "f32"),
 }
+SOFTMAX_KINDS = ("softmax", "softmin", "logsoftmax")
 
 # HBM bytes per launch of the backward dx / partial-sum kernel, from two rocprofv3 --pmc runs of this script
 # (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch), each scaled by what the same counter reads for a plain
@@ -52,6 +60,8 @@ MEASURED_TRAFFIC_BYTES = {
 
 
 def algorithmic_bytes(kind, m, n, s, sw):
+    if kind in SOFTMAX_KINDS:                 # forward: x read, y written; backward: y and dy read, dx written
+        return 2 * m * n * s, 3 * m * n * s
     if kind == "ln":
         return 2 * m * n * s + 2 * n * sw + 8 * m, 3 * m * n * s + 3 * n * sw + 8 * m
     return 2 * m * n * s + n * sw + 4 * m, 3 * m * n * s + 2 * n * sw + 4 * m
@@ -82,6 +92,8 @@ def main():
     torch.cuda.set_device(dev)
     kind, m, n, dname = WORKLOADS[args.workload]
     dtype = {"bf16": torch.bfloat16, "f16": torch.float16, "f32": torch.float32}[dname]
+    if kind in SOFTMAX_KINDS:
+        return softmax_main(args, lib, dev, kind, m, n, dname, dtype)
     s = torch.empty(0, dtype=dtype).element_size()
     code = _native.dtype_code(dtype)
     ln = kind == "ln"
@@ -213,6 +225,133 @@ def main():
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(kind, m, n, dtype, sets[0], w, b, step_bytes)
     print(json.dumps(out), flush=True)
+
+
+def softmax_main(args, lib, dev, kind, m, n, dname, dtype):
+    """One step = thn_softmax_fwd + thn_softmax_bwd (the backward reads the output the forward just wrote,
+    as the autograd Function does) over one of four rotating buffer sets."""
+    import torch
+    from TritonHub import _native
+    from TritonHub.Normalization import _launch
+    s = torch.empty(0, dtype=dtype).element_size()
+    code = _native.dtype_code(dtype)
+    kcode = {"softmax": _native.SOFTMAX, "softmin": _native.SOFTMIN, "logsoftmax": _native.LOGSOFTMAX}[kind]
+    gen = torch.Generator(device=dev).manual_seed(0)
+    sets = []
+    for _ in range(N_BUFFER_SETS):
+        x = (3.0 * torch.randn(m, n, device=dev, generator=gen)).to(dtype)
+        dy = torch.randn(m, n, device=dev, generator=gen).to(dtype)
+        sets.append(dict(x=x, dy=dy, y=torch.empty_like(x), dx=torch.empty_like(x)))
+    stream = torch.cuda.current_stream(dev).cuda_stream
+    p = _native.ptr
+
+    def forward(b_):
+        rc = lib.thn_softmax_fwd(p(b_["x"]), n, p(b_["y"]), n, m, n, kcode, code, stream)
+        assert rc == 0, _native.strerror(rc)
+
+    def backward(b_):
+        rc = lib.thn_softmax_bwd(p(b_["y"]), n, p(b_["dy"]), n, p(b_["dx"]), n, m, n, kcode, code, stream)
+        assert rc == 0, _native.strerror(rc)
+
+    def step(i):
+        forward(sets[i % N_BUFFER_SETS])
+        backward(sets[i % N_BUFFER_SETS])
+
+    for i in range(args.warmup):
+        step(i)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        step(i)
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    fwd_bytes, bwd_bytes = algorithmic_bytes(kind, m, n, s, s)
+    step_bytes = fwd_bytes + bwd_bytes
+    gbps = step_bytes / (ms_per_step * 1e-3) / 1e9
+
+    def avg_launch_us(launch):
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        for i in range(min(args.warmup, 5)):
+            launch(sets[i % N_BUFFER_SETS])
+        torch.cuda.synchronize()
+        start.record()
+        for i in range(args.steps):
+            launch(sets[i % N_BUFFER_SETS])
+        stop.record()
+        torch.cuda.synchronize()
+        return start.elapsed_time(stop) * 1e3 / args.steps
+
+    fwd_us = avg_launch_us(forward)
+    bwd_us = avg_launch_us(backward)
+    if args.calibration_copy:
+        for i in range(5):
+            sets[i % N_BUFFER_SETS]["dx"].copy_(sets[i % N_BUFFER_SETS]["x"])
+        torch.cuda.synchronize()
+    achieved = bwd_bytes / (bwd_us * 1e-6) / 1e9
+    fs = _launch.query_launch(2, kind == "logsoftmax", m, n, dtype)
+    bs = _launch.query_launch(3, kind == "logsoftmax", m, n, dtype)
+    out = {
+        "metric": f"fwd+bwd HBM GB/s and % of peak, {kind} {dname} {m}x{n}",
+        "value": round(gbps, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": dname, "data": "synthetic",
+        "config": {"workload": args.workload, "op": kind, "rows": m, "row_width": n, "buffer_sets": N_BUFFER_SETS,
+                   "entry_points": "thn_softmax_fwd + thn_softmax_bwd"},
+        "pct_of_hbm_peak": round(100.0 * gbps / HBM_PEAK_GBPS, 2),
+        "rows_per_s": round(m / (ms_per_step * 1e-3)),
+        "algorithmic_bytes_per_step": step_bytes,
+        "kernels_us": {"forward": round(fwd_us, 2), "backward": round(bwd_us, 2),
+                       "forward_GBps": round(fwd_bytes / (fwd_us * 1e-6) / 1e9, 1)},
+        "launch": {"forward": dict(zip(("vecs_per_thread", "threads_per_row", "block", "grid"), fs[:4])),
+                   "backward": dict(zip(("vecs_per_thread", "threads_per_row", "block", "grid"), bs[:4]))},
+        "roofline": {"bound": "hbm", "kernel": "softmax_bwd_kernel", "achieved": round(achieved, 1),
+                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
+                     "algorithmic_bytes_per_launch": bwd_bytes, "avg_launch_us": round(bwd_us, 2),
+                     "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload)},
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = softmax_cpu_baseline(kind, m, n, dtype, sets[0], step_bytes)
+    print(json.dumps(out), flush=True)
+
+
+def softmax_cpu_baseline(kind, m, n, dtype, buffers, step_bytes):
+    """The numpy restatement of the reference's kernels (oracle/softmax_oracle.py, one thread, float64) on a
+    bounded sample of the same rows, and torch.nn.functional on the host cores next to it."""
+    import torch
+    from oracle import softmax_oracle as so
+    rows = min(m, max(64, (1 << 23) // n))             # 8M elements per pass at most
+    x = buffers["x"][:rows].cpu()
+    dy = buffers["dy"][:rows].cpu()
+    x64, dy64 = x.double().numpy(), dy.double().numpy()
+
+    def oracle_step():
+        so.BWD[kind](so.FWD[kind](x64), dy64)
+
+    fn = {"softmax": torch.softmax, "softmin": lambda t, d: torch.softmax(-t, d), "logsoftmax": torch.log_softmax}[kind]
+
+    def torch_step():
+        xr = x.clone().requires_grad_(True)
+        fn(xr, -1).backward(dy)
+
+    def timed(f, reps):
+        f()
+        best = float("inf")
+        for _ in range(reps):
+            t0 = time.perf_counter()
+            f()
+            best = min(best, time.perf_counter() - t0)
+        return best
+
+    sample_bytes = step_bytes * rows / m
+    t_oracle, t_torch = timed(oracle_step, 3), timed(torch_step, 3)
+    return {"value": round(sample_bytes / t_oracle / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
+            "sample": f"first {rows} of {m} rows of the same workload, forward + backward, best of 3 passes of "
+                      f"oracle/softmax_oracle.py (numpy float64, one thread; {t_oracle * 1e3:.1f} ms per pass)",
+            "host_cpu_count": os.cpu_count(),
+            "torch_functional": {"value": round(sample_bytes / t_torch / 1e9, 2), "unit": "GB/s",
+                                 "threads": torch.get_num_threads(),
+                                 "what": f"torch {kind} forward + autograd backward on the host cores, same sample "
+                                         f"({t_torch * 1e3:.1f} ms per pass)"}}
 
 
 def cpu_baseline(kind, m, n, dtype, buffers, w, b, step_bytes):

@@ -122,18 +122,18 @@ int thn_norm_bwd_reduce_partials(const void* workspace, int32_t num_partials,
  * Softmax, Softmin and LogSoftmax over the last dimension (the row-reduction activations next to the norm
  * path in the reference: TritonHub/Activations/softmax.py, softmin.py, logsoftmax.py).
  *
- * thn_softmax_fwd replaces `_softmax_kernel_fwd[grid](...)` (softmax.py:37-40, device code :14-24),
- * `_softmin_kernel_fwd` (softmin.py:36-39) and `_logsoftmax_kernel_fwd` (logsoftmax.py:39-43, device code
- * :17-26):  z = x - max(x);  THN_SOFTMAX: y = exp(z)/sum(exp(z));  THN_LOGSOFTMAX: y = z - log(sum(exp(z)));
- * THN_SOFTMIN: softmax of -x (the reference negates with a separate tensor op, softmin.py:109; here the
+ * thn_softmax_fwd replaces `_softmax_kernel_fwd[grid](...)` (softmax.py:37-40, device code :11-24),
+ * `_softmin_kernel_fwd` (softmin.py:37-40) and `_logsoftmax_kernel_fwd` (logsoftmax.py:39-43, device code
+ * :11-24):  z = x - max(x);  THN_SOFTMAX: y = exp(z)/sum(exp(z));  THN_LOGSOFTMAX: y = z - log(sum(exp(z)));
+ * THN_SOFTMIN: softmax of -x (the reference negates with a separate tensor op, softmin.py:103; here the
  * sign is applied on load).
- * thn_softmax_bwd replaces `_softmax_kernel_bwd` (softmax.py:75-79, device code :50-61), `_softmin_kernel_bwd`
- * (softmin.py:75-79) and `_logsoftmax_kernel_bwd` (logsoftmax.py:88-93, device code :62-78); `y` is the SAVED
+ * thn_softmax_bwd replaces `_softmax_kernel_bwd` (softmax.py:79-83, device code :48-62), `_softmin_kernel_bwd`
+ * (softmin.py:79-83) and `_logsoftmax_kernel_bwd` (logsoftmax.py:85-90, device code :51-67); `y` is the SAVED
  * OUTPUT of the forward, as in the reference:
  *   THN_SOFTMAX: dx = y*dy - y*sum(y*dy);  THN_SOFTMIN: the negative of that;  THN_LOGSOFTMAX: dx = dy - exp(y)*sum(dy).
  * All tensors share one storage code.  Arithmetic is float32, except softmax / softmin on THN_F64 storage,
  * which run in float64: the reference's softmax kernels compute in the type they load (softmax.py:18-23),
- * its log-softmax kernels widen to float32 (logsoftmax.py:19, :71).  Rows wider than 64 KiB are refused with
+ * its log-softmax kernels widen to float32 (logsoftmax.py:19, :61-62).  Rows wider than 64 KiB are refused with
  * THN_E_FEATURE_DIM (the reference would split such a row into independently normalised chunks).
  */
 enum thn_softmax_kind { THN_SOFTMAX = 0, THN_SOFTMIN = 1, THN_LOGSOFTMAX = 2 };

@@ -3,11 +3,11 @@
 Float64 numpy restatement of the reference's row-reduction activation kernels; imported by ``tests/`` only.
 
 * ``softmax_fwd``     follows ``TritonHub/Activations/softmax.py:17-23``   (z = x - max; exp(z)/sum(exp(z)))
-* ``softmax_bwd``     follows ``TritonHub/Activations/softmax.py:56-60``   (from the SAVED OUTPUT y: y*dy - y*sum(y*dy))
-* ``softmin_fwd/bwd`` follow  ``TritonHub/Activations/softmin.py:109`` + ``:17-23`` / ``:57-61``: the callable
+* ``softmax_bwd``     follows ``TritonHub/Activations/softmax.py:57-61``   (from the SAVED OUTPUT y: y*dy - y*sum(y*dy))
+* ``softmin_fwd/bwd`` follow  ``TritonHub/Activations/softmin.py:103`` + ``:17-23`` / ``:57-61``: the callable
   negates its input and applies the softmax kernels; the gradient w.r.t. the callable's input carries the sign.
 * ``logsoftmax_fwd``  follows ``TritonHub/Activations/logsoftmax.py:19-24`` (z - log(sum(exp(z))))
-* ``logsoftmax_bwd``  follows ``TritonHub/Activations/logsoftmax.py:71-76`` (from the saved output y: dy - exp(y)*sum(dy))
+* ``logsoftmax_bwd``  follows ``TritonHub/Activations/logsoftmax.py:61-67`` (from the saved output y: dy - exp(y)*sum(dy))
 
 For rows within the reference's 64 KiB block the kernels see the whole row; wider rows are split by the
 reference into independently normalised chunks (softmax.py:34-36), which this oracle -- and the product --

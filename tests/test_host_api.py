@@ -97,7 +97,7 @@ def test_package_surface():
     assert issubclass(layernorm, torch.autograd.Function) and issubclass(rmsnorm, torch.autograd.Function)
     import TritonHub
     assert TritonHub.__version__ == "1.1.1"
-    # the row-reduction activations of TritonHub/Activations/__init__.py (softmax.py:96-100, softmin.py:104-109,
+    # the row-reduction activations of TritonHub/Activations/__init__.py (softmax.py:99-103, softmin.py:99-103,
     # logsoftmax.py:106-110): plain callables holding the Function's apply
     assert Activations.__all__ == ["Softmax", "Softmin", "LogSoftmax"]
     from TritonHub.Activations.logsoftmax import logsoftmax

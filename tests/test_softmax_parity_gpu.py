@@ -5,7 +5,7 @@ Tolerances (as for the norm path): float32 storage max(1e-5, 4 float32 ulp); flo
 output type at the oracle's value plus 4 * 2^-24 * (magnitude of the operands that were subtracted to form
 the result); float64 softmax / softmin are computed in float64 (as the reference does) and held to 1e-13,
 float64 log-softmax is float32 arithmetic (logsoftmax.py:19) and held to the float32 bound.
-The backward is a function of the SAVED OUTPUT (softmax.py:99-107): its expected value is the oracle's backward
+The backward is a function of the SAVED OUTPUT (softmax.py:86-97): its expected value is the oracle's backward
 evaluated at the very output tensor the GPU saved, so forward rounding does not leak into the comparison.
 """
 import os
@@ -81,7 +81,7 @@ def make(shape, dtype, seed, scale=1.0):
     return x, dy
 
 
-# ---- the reference's unit-test matrix (UnitTests/Activations/softmax_unittest.py:63-68 and twins) ---------------
+# ---- the reference's unit-test matrix (UnitTests/Activations/softmax_unittest.py:57-65 and twins) ---------------
 @pytest.mark.parametrize("dtype", [torch.float16, torch.float32, torch.float64])
 @pytest.mark.parametrize("dim", [32, 64, 128, 256, 512, 1024, 2048])
 @pytest.mark.parametrize("kind", KINDS)
@@ -93,7 +93,7 @@ def test_reference_unit_test_matrix(kind, dim, dtype):
               "logsoftmax": torch.nn.LogSoftmax(dim=-1)}[kind]
     a = data.clone().requires_grad_(True)
     r = data.clone().requires_grad_(True)
-    rtol, atol = (3e-4, 1e-3) if dtype == torch.float32 else (5e-3, 1e-2)      # softmax_unittest.py:31-33
+    rtol, atol = (3e-4, 1e-3) if dtype == torch.float32 else (5e-3, 1e-2)      # softmax_unittest.py:30-32
     if dtype == torch.float16:
         rtol, atol = 1e-2, 5e-2
     ya, yr = MODULE[kind]()(a), theirs(r)
@@ -182,7 +182,7 @@ def test_empty_input_and_single_element_rows():
 
 
 def test_softmin_function_and_callable_follow_the_reference():
-    """softmin.apply(z) is softmax(z) (softmin.py:84-96); Softmin()(x) is softmin.apply(-x) (softmin.py:103):
+    """softmin.apply(z) is softmax(z) (softmin.py:86-97); Softmin()(x) is softmin.apply(-x) (softmin.py:103):
     values and gradients of the fused callable equal those of the explicit negation bit for bit."""
     announce("softmin semantics")
     g = torch.Generator().manual_seed(77)

@@ -1,6 +1,6 @@
 """Host launch wrappers of the softmax family.
 
-They do what the reference's ``_softmax_fwd`` / ``_softmax_bwd`` (softmax.py:25-41, :63-80) and their softmin /
+They do what the reference's ``_softmax_fwd`` / ``_softmax_bwd`` (softmax.py:25-41, :64-84) and their softmin /
 logsoftmax twins do on the host -- make the last dimension contiguous, flatten to (M, N), allocate the output
 with the same assertion messages -- and then call the C ABI of libthnorm.so on the current stream.
 """
@@ -47,7 +47,7 @@ def softmax_fwd(x: torch.Tensor, kind: int) -> torch.Tensor:
 
 
 def softmax_bwd(y: torch.Tensor, dout: torch.Tensor, kind: int) -> torch.Tensor:
-    """`y` is the saved OUTPUT of the forward (softmax.py:99-107)."""
+    """`y` is the saved OUTPUT of the forward (softmax.py:86-97)."""
     _native.require_gpu(y)
     batch_shape = y.shape[:-1]
     y2 = _rows(y)

@@ -1,5 +1,5 @@
 """LogSoftmax over the last dimension: drop-in for ``TritonHub/Activations/logsoftmax.py`` of the reference
-(the ``logsoftmax`` autograd Function, logsoftmax.py:112-124, and the ``LogSoftmax`` callable, :126-130)."""
+(the ``logsoftmax`` autograd Function, logsoftmax.py:93-110, and the ``LogSoftmax`` callable, :126-130)."""
 import torch
 
 from .. import _native

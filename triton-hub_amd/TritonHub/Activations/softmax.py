@@ -1,5 +1,5 @@
 """Softmax over the last dimension: drop-in for ``TritonHub/Activations/softmax.py`` of the reference
-(the ``softmax`` autograd Function, softmax.py:82-94, and the ``Softmax`` callable, :96-100)."""
+(the ``softmax`` autograd Function, softmax.py:86-97, and the ``Softmax`` callable, :99-103)."""
 import torch
 
 from .. import _native

@@ -1,7 +1,7 @@
 """Softmin over the last dimension: drop-in for ``TritonHub/Activations/softmin.py`` of the reference.
 
-In the reference the ``softmin`` autograd Function is a softmax of ITS input (softmin.py:11-24, :84-96) and the
-``Softmin`` callable negates first: ``self.softmin_fn(-x)`` (softmin.py:109).  Both are kept: ``softmin.apply(z)``
+In the reference the ``softmin`` autograd Function is a softmax of ITS input (softmin.py:11-24, :86-97) and the
+``Softmin`` callable negates first: ``self.softmin_fn(-x)`` (softmin.py:103).  Both are kept: ``softmin.apply(z)``
 is softmax(z), ``Softmin()(x)`` is softmax(-x).  The callable does not spend a pass of its own on the
 negation: it calls a second Function whose kernels negate on load (forward) and on store (backward), which
 gives the same values and gradients as negating with a tensor op.

@@ -21,7 +21,7 @@ struct SoftmaxFwdArgs {
 };
 
 struct SoftmaxBwdArgs {
-    const char* y;   // the SAVED OUTPUT of the forward (softmax.py:99-107, logsoftmax.py:119-127)
+    const char* y;   // the SAVED OUTPUT of the forward (softmax.py:86-97, logsoftmax.py:93-104)
     const char* dy;
     char* dx;
     int64_t y_stride_bytes;
@@ -33,7 +33,7 @@ struct SoftmaxBwdArgs {
     float sign;      // -1: the gradient is negated on store (fused Softmin)
 };
 
-// Arithmetic type.  Float32 for 16- and 32-bit storage and for every log-softmax (logsoftmax.py:19, :71 widen
+// Arithmetic type.  Float32 for 16- and 32-bit storage and for every log-softmax (logsoftmax.py:19, :61-62 widen
 // to float32 explicitly).  The reference's softmax / softmin kernels compute in the type they load
 // (softmax.py:18-23), so float64 rows are computed in float64.
 template <typename T, bool LOG> struct SoftmaxCompute { using type = float; };
@@ -192,8 +192,8 @@ __global__ void __launch_bounds__(BLOCK) softmax_fwd_kernel(const SoftmaxFwdArgs
 }
 
 // Backward from the saved output y and the upstream gradient g:
-//   softmax (softmax.py:57-60):       dx = y*g - y*sum(y*g)
-//   log-softmax (logsoftmax.py:73-76): dx = g - exp(y)*sum(g)
+//   softmax (softmax.py:57-61):       dx = y*g - y*sum(y*g)
+//   log-softmax (logsoftmax.py:61-67): dx = g - exp(y)*sum(g)
 template <typename T, bool LOG, int K, int TPR, int BLOCK, bool ALIGNED>
 __global__ void __launch_bounds__(BLOCK) softmax_bwd_kernel(const SoftmaxBwdArgs a) {
     constexpr int VEC = T::VEC;
