@@ -56,6 +56,8 @@ SOFTMAX_KINDS = ("softmax", "softmin", "logsoftmax")
 MEASURED_TRAFFIC_BYTES = {
     # profiles/norm_kernels_rmsnorm_bf16_16384x4096_hbm_counters.txt: 262946 KiB fetched + 135168 KiB written
     "rmsnorm_bf16_16384x4096": 407669153,
+    # profiles/softmax_kernels_softmax_bf16_16384x4096_stats_and_hbm_counters.txt (softmax_bwd_kernel)
+    "softmax_bf16_16384x4096": 402815465,
 }
 
 

@@ -175,7 +175,9 @@ int ceil_div(int a, int b) { return (a + b - 1) / b; }
 Shape heuristic_shape(int which, bool ln, bool aligned, int n_vecs) {
     (void)ln;
     int kmax = (aligned && which == kNormBwd && n_vecs > 128) ? 3 : 4;
-    if (aligned && which == kSoftmaxBwd && n_vecs <= 2048) kmax = 2;     // two input streams, nothing to hold
+    // Softmax backward: two input streams and nothing to hold; 2 vectors per thread per stream measured best,
+    // except for 2 KiB rows, where one full wave per row (2 x 64) is 8 % slower than half a wave (4 x 32).
+    if (aligned && which == kSoftmaxBwd && n_vecs <= 2048 && !(n_vecs > 64 && n_vecs <= 128)) kmax = 2;
     Shape s{4, 1024, 1024};
     for (int tpr : kTprList) {
         if (static_cast<int64_t>(tpr) * kmax >= n_vecs) {
