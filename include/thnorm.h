@@ -1,10 +1,10 @@
 /*
- * thnorm.h -- C ABI of libthnorm.so: LayerNorm / RMSNorm, and the Softmax / Softmin / LogSoftmax row
- * reductions next to them, forward and backward, for AMD MI355X (gfx950).
+ * thnorm.h -- C ABI of libthnorm.so: LayerNorm / RMSNorm, and the row reductions next to them (Softmax /
+ * Softmin / LogSoftmax, row p-norm / normalize), forward and backward, for AMD MI355X (gfx950).
  *
  * The reference library (TritonHub) has no native boundary: its last host frames before device code are the
  * Python launch sites in TritonHub/Normalization/layernorm.py and rmsnorm.py (and TritonHub/Activations/
- * softmax.py, softmin.py, logsoftmax.py).  Each entry point below
+ * softmax.py, softmin.py, logsoftmax.py, TritonHub/Ops/norm.py, normalize.py).  Each entry point below
  * replaces one of those launch sites, so a maintainer of the reference can bind it with ctypes in place of
  * the Triton launch.  The citation on every declaration names the launch site (and device code) replaced.
  *
@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define THN_ABI_VERSION 2
+#define THN_ABI_VERSION 3
 
 enum thn_dtype { THN_F32 = 0, THN_F16 = 1, THN_BF16 = 2, THN_F64 = 3 };
 
@@ -148,9 +148,54 @@ int thn_softmax_bwd(const void* y, int64_t y_row_stride,
                     int64_t M, int64_t N, int kind, int dtype, void* stream);
 
 /*
+ * Row p-norm and p-normalisation over the last dimension of a (B, M, K) tensor (the reference's
+ * TritonHub/Ops/norm.py and normalize.py).  x, y, dy, dx: element-contiguous rows, batch and row strides in
+ * ELEMENTS; norms, dnorms: contiguous (B*M,) vectors.  All tensors share one storage code; arithmetic is
+ * float32 (the reference's `dtype` is float32 unless the tensor is float16 / bfloat16, norm.py:53).
+ * p is any real number in [1, 6] and eps >= 0 (the reference's constructor assertions, norm.py:148-149), else
+ * THN_E_SHAPE.  There is no row-width limit: rows of more than 64 KiB, and p that is not an integer, take a
+ * slower looping kernel.
+ *
+ * thn_pnorm_fwd replaces `_norm_fwd_kernel[grid](...)` (norm.py:56-59, device code :11-45):
+ *   norms = max((sum |x|^p)^(1/p), eps), rounded to the storage type.
+ * thn_normalize_fwd replaces the two launches of `_normalize_fwd` (normalize.py:47-54: `_norm_fwd_kernel`, then
+ *   `_normalize_fwd_kernel`, device code :11-33) by one pass over x: norms as above, y = x / norms with norms
+ *   ALREADY ROUNDED to the storage type (the reference reads them back from the tensor the first kernel wrote).
+ * thn_pnorm_bwd replaces `_norm_bwd_kernel[grid](...)` (norm.py:120-125, device code :66-102); `norms` is the
+ *   saved output of the forward (not read when p == 1, may then be NULL), `dnorms` its upstream gradient:
+ *   p=1: dx = g*sign(x);  p=2: dx = g*x/n;  else dx = g*sign(x)*|x|^(p-1) / n^(p-1).
+ * thn_normalize_bwd replaces `_normalize_bwd_kernel[grid](...)` (normalize.py:136-141, device code :61-117); y
+ *   and norms are the saved outputs of the forward:  proj = sum(y*dy) (p=1: sum(x*dy));
+ *   p=1: dx = dy/n - sign(x)*(proj/(n*n));  p=2: dx = (dy - y*proj)/n;
+ *   else dx = dy/n - sign(x)*|x|^(p-1)*(proj/(n^(p-1)*n)).   x is not read when p == 2, y not when p == 1
+ *   (each may then be NULL).
+ */
+int thn_pnorm_fwd(const void* x, int64_t x_batch_stride, int64_t x_row_stride,
+                  void* norms,
+                  int64_t B, int64_t M, int64_t K, float p, float eps, int dtype, void* stream);
+
+int thn_normalize_fwd(const void* x, int64_t x_batch_stride, int64_t x_row_stride,
+                      void* y, int64_t y_batch_stride, int64_t y_row_stride,
+                      void* norms,
+                      int64_t B, int64_t M, int64_t K, float p, float eps, int dtype, void* stream);
+
+int thn_pnorm_bwd(const void* x, int64_t x_batch_stride, int64_t x_row_stride,
+                  const void* norms, const void* dnorms,
+                  void* dx, int64_t dx_batch_stride, int64_t dx_row_stride,
+                  int64_t B, int64_t M, int64_t K, float p, int dtype, void* stream);
+
+int thn_normalize_bwd(const void* x, int64_t x_batch_stride, int64_t x_row_stride,
+                      const void* y, int64_t y_batch_stride, int64_t y_row_stride,
+                      const void* norms,
+                      const void* dy, int64_t dy_batch_stride, int64_t dy_row_stride,
+                      void* dx, int64_t dx_batch_stride, int64_t dx_row_stride,
+                      int64_t B, int64_t M, int64_t K, float p, int dtype, void* stream);
+
+/*
  * Launch-shape control for tuning sweeps (the counterpart of the reference's `triton.autotune` over
  * num_warps, autotune.py:62-65, which this library replaces by a fixed heuristic on N and the dtype).
- * `which`: 0 = norm forward, 1 = norm backward, 2 = softmax forward, 3 = softmax backward.
+ * `which`: 0 = norm forward, 1 = norm backward, 2 = softmax forward, 3 = softmax backward, 4 = p-norm /
+ * normalize forward, 5 = p-norm backward, 6 = normalize backward.
  * vecs_per_thread / threads_per_row / block_threads select a compiled kernel shape, blocks_per_cu caps the
  * persistent grid; 0 for any field keeps the heuristic's choice.
  * Process-wide; meant for benchmarks, not for concurrent production use.  Returns THN_E_SHAPE when no

@@ -25,7 +25,7 @@ def declared_functions():
 
 def test_library_exports_every_declared_symbol():
     names = declared_functions()
-    assert len(names) == 11 and "thn_norm_fwd" in names and "thn_norm_bwd" in names and "thn_softmax_fwd" in names
+    assert len(names) == 15 and "thn_pnorm_fwd" in names and "thn_normalize_bwd" in names and "thn_norm_fwd" in names and "thn_norm_bwd" in names and "thn_softmax_fwd" in names
     handle = ctypes.CDLL(_native.LIB_PATH)
     for name in names:
         assert hasattr(handle, name), f"{name} is declared in include/thnorm.h but not exported"
@@ -59,7 +59,7 @@ def test_argument_checks_answer_without_a_gpu():
     assert lib.thn_norm_bwd_workspace_bytes(4, 40000, 1, 1, _native.F16) == _native.E_FEATURE_DIM
     assert lib.thn_norm_bwd_workspace_bytes(4, 128, 0, 0, _native.F32) == 0
     assert lib.thn_norm_bwd_workspace_bytes(0, 128, 1, 1, _native.F32) == 0
-    assert lib.thn_norm_set_launch_override(4, 0, 0, 0, 0) == _native.E_SHAPE
+    assert lib.thn_norm_set_launch_override(7, 0, 0, 0, 0) == _native.E_SHAPE
     assert lib.thn_norm_set_launch_override(0, 0, 0, 0, 0) == _native.OK
     if not torch.cuda.is_available():
         assert lib.thn_norm_bwd_workspace_bytes(4, 128, 1, 1, _native.F32) == _native.E_DEVICE
@@ -83,6 +83,54 @@ def test_softmax_argument_checks_answer_without_a_gpu():
         assert call(0, 128, 0, _native.BF16) == _native.OK
         assert call(4, 128, 0, _native.BF16) == _native.E_NULL
     assert (_native.SOFTMAX, _native.SOFTMIN, _native.LOGSOFTMAX) == (0, 1, 2)   # enum thn_softmax_kind
+
+
+def test_pnorm_argument_checks_answer_without_a_gpu():
+    lib = _native.lib()
+    fwd = lambda b, m, k, p, eps, dt: lib.thn_pnorm_fwd(0, m * k, k, 0, b, m, k, p, eps, dt, 0)
+    nfwd = lambda b, m, k, p, eps, dt: lib.thn_normalize_fwd(0, m * k, k, 0, m * k, k, 0, b, m, k, p, eps, dt, 0)
+    bwd = lambda b, m, k, p, dt: lib.thn_pnorm_bwd(0, m * k, k, 0, 0, 0, m * k, k, b, m, k, p, dt, 0)
+    nbwd = lambda b, m, k, p, dt: lib.thn_normalize_bwd(0, m * k, k, 0, m * k, k, 0, 0, m * k, k, 0, m * k, k, b, m, k,
+                                                       p, dt, 0)
+    for call in (fwd, nfwd):
+        assert call(2, 3, 8, 2.0, 1e-6, 9) == _native.E_DTYPE
+        assert call(2, 3, 0, 2.0, 1e-6, _native.F32) == _native.E_SHAPE and call(-1, 3, 8, 2.0, 1e-6, 0) == _native.E_SHAPE
+        assert call(2, 3, 8, 0.5, 1e-6, _native.F32) == _native.E_SHAPE        # p must be in [1, 6] (Ops/norm.py:148)
+        assert call(2, 3, 8, 6.5, 1e-6, _native.F32) == _native.E_SHAPE
+        assert call(2, 3, 8, float("nan"), 1e-6, _native.F32) == _native.E_SHAPE
+        assert call(2, 3, 8, 2.0, -1.0, _native.F32) == _native.E_SHAPE        # eps must be non-negative (:149)
+        assert call(0, 3, 8, 2.0, 1e-6, _native.F16) == _native.OK and call(2, 0, 8, 2.0, 1e-6, _native.F16) == _native.OK
+        assert call(2, 3, 8, 2.0, 1e-6, _native.BF16) == _native.E_NULL
+        assert call(2, 3, 100000, 2.5, 1e-6, _native.F32) == _native.E_NULL    # no row-width limit, any real p
+    for call in (bwd, nbwd):
+        assert call(2, 3, 8, 2.0, 7) == _native.E_DTYPE
+        assert call(2, 3, 8, 7.0, _native.F32) == _native.E_SHAPE
+        assert call(2, 0, 8, 2.0, _native.F32) == _native.OK
+        assert call(2, 3, 8, 3.0, _native.F32) == _native.E_NULL
+
+
+def test_ops_surface_matches_the_reference():
+    from TritonHub import Ops
+    from TritonHub.Ops.norm import Norm
+    from TritonHub.Ops.normalize import Normalize
+    assert Ops.__all__ == ["normalize", "norm"]                     # Ops/__init__.py:2-5 without bmm
+    assert issubclass(Norm, torch.autograd.Function) and issubclass(Normalize, torch.autograd.Function)
+    n = Ops.norm()
+    assert (n.p, n.eps) == (2, 1e-6) and n.norm is not None           # Ops/norm.py:147-152
+    z = Ops.normalize(p=3, eps=0.0)
+    assert (z.p, z.eps) == (3, 0.0) and z.normalize is not None       # Ops/normalize.py:163-168
+    for cls in (Ops.norm, Ops.normalize):
+        with pytest.raises(AssertionError, match=r"p must be in \[1, 6\] for numerical stability"):
+            cls(p=0.5)
+        with pytest.raises(AssertionError, match=r"p must be in \[1, 6\]"):
+            cls(p=7)
+        with pytest.raises(AssertionError, match="eps must be non-negative"):
+            cls(eps=-1e-3)
+    for op in (n, z):
+        with pytest.raises(AssertionError, match="Expected Tensor to be 3D"):
+            op(torch.randn(4, 8))
+        with pytest.raises(RuntimeError, match="no CPU fallback"):
+            op(torch.randn(2, 4, 8))
 
 
 def test_no_cpu_fallback():

@@ -36,6 +36,11 @@ SYMBOLS = {
     'thn_norm_bwd_reduce_partials': (_i32, [_vp, ctypes.c_int32, _vp, _vp, _i64, _i32, _vp]),
     'thn_softmax_fwd': (_i32, [_vp, _i64, _vp, _i64, _i64, _i64, _i32, _i32, _vp]),
     'thn_softmax_bwd': (_i32, [_vp, _i64, _vp, _i64, _vp, _i64, _i64, _i64, _i32, _i32, _vp]),
+    'thn_pnorm_fwd': (_i32, [_vp, _i64, _i64, _vp, _i64, _i64, _i64, _f32, _f32, _i32, _vp]),
+    'thn_normalize_fwd': (_i32, [_vp, _i64, _i64, _vp, _i64, _i64, _vp, _i64, _i64, _i64, _f32, _f32, _i32, _vp]),
+    'thn_pnorm_bwd': (_i32, [_vp, _i64, _i64, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _f32, _i32, _vp]),
+    'thn_normalize_bwd': (_i32, [_vp, _i64, _i64, _vp, _i64, _i64, _vp, _vp, _i64, _i64, _vp, _i64, _i64,
+                                 _i64, _i64, _i64, _f32, _i32, _vp]),
     'thn_norm_set_launch_override': (_i32, [_i32, _i32, _i32, _i32, _i32]),
     'thn_norm_query_launch': (_i32, [_i32, _i32, _i64, _i64, _i32, ctypes.POINTER(ctypes.c_int32)]),
 }

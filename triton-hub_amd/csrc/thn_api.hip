@@ -8,18 +8,26 @@
 
 #include "thn_dispatch.h"
 #include "thn_reduce.h"
+#include "thn_pnorm_dispatch.h"
 #include "thn_softmax_dispatch.h"
 
 namespace {
 
 using thn::BwdArgs;
 using thn::FwdArgs;
+using thn::NormalizeBwdArgs;
+using thn::PnormBwdArgs;
+using thn::PnormFwdArgs;
+using thn::RowMap;
 using thn::Shape;
 using thn::SoftmaxBwdArgs;
 using thn::SoftmaxFwdArgs;
 
 // `which` throughout this file: the kernel family a launch belongs to.
-enum : int { kNormFwd = 0, kNormBwd = 1, kSoftmaxFwd = 2, kSoftmaxBwd = 3, kFamilies = 4 };
+enum : int {
+    kNormFwd = 0, kNormBwd = 1, kSoftmaxFwd = 2, kSoftmaxBwd = 3, kPnormFwd = 4, kPnormBwd = 5, kNormalizeBwd = 6,
+    kFamilies = 7
+};
 
 constexpr int kMaxDevices = 64;
 constexpr int64_t kMaxRowBytes = 65536;   // the reference's MAX_FUSED_SIZE (layernorm.py:69-72)
@@ -65,6 +73,8 @@ bool shape_compiled(int which, bool aligned, Shape s) {
         THN_SCALAR_SHAPES(THN_MATCH)
     } else if (which == kNormBwd) {
         THN_BWD_SHAPES(THN_MATCH)
+    } else if (which >= kPnormFwd) {
+        THN_ROW_SHAPES(THN_MATCH)
     } else {
         THN_FWD_SHAPES(THN_MATCH)
     }
@@ -110,15 +120,49 @@ int launch_softmax_bwd(int dtype, bool is_log, bool aligned, Shape s, const Soft
     }
 }
 
+// `variant` of the p-norm families: the p mode (thn::kP1 / kP2 / kPInt), plus 4 when the forward also normalises.
+int launch_pnorm_fwd(int dtype, int variant, bool aligned, Shape s, const PnormFwdArgs& a, int grid, hipStream_t st,
+                     int* occ) {
+    const int mode = variant & 3;
+    const bool nz = (variant & 4) != 0;
+    switch (dtype) {
+        case THN_F32: return thn::launch_pnorm_fwd_f32(mode, nz, aligned, s, a, grid, st, occ);
+        case THN_F16: return thn::launch_pnorm_fwd_f16(mode, nz, aligned, s, a, grid, st, occ);
+        case THN_BF16: return thn::launch_pnorm_fwd_bf16(mode, nz, aligned, s, a, grid, st, occ);
+        default: return thn::launch_pnorm_fwd_f64(mode, nz, aligned, s, a, grid, st, occ);
+    }
+}
+
+int launch_pnorm_bwd(int dtype, int mode, bool aligned, Shape s, const PnormBwdArgs& a, int grid, hipStream_t st,
+                     int* occ) {
+    switch (dtype) {
+        case THN_F32: return thn::launch_pnorm_bwd_f32(mode, aligned, s, a, grid, st, occ);
+        case THN_F16: return thn::launch_pnorm_bwd_f16(mode, aligned, s, a, grid, st, occ);
+        case THN_BF16: return thn::launch_pnorm_bwd_bf16(mode, aligned, s, a, grid, st, occ);
+        default: return thn::launch_pnorm_bwd_f64(mode, aligned, s, a, grid, st, occ);
+    }
+}
+
+int launch_normalize_bwd(int dtype, int mode, bool aligned, Shape s, const NormalizeBwdArgs& a, int grid,
+                         hipStream_t st, int* occ) {
+    switch (dtype) {
+        case THN_F32: return thn::launch_normalize_bwd_f32(mode, aligned, s, a, grid, st, occ);
+        case THN_F16: return thn::launch_normalize_bwd_f16(mode, aligned, s, a, grid, st, occ);
+        case THN_BF16: return thn::launch_normalize_bwd_bf16(mode, aligned, s, a, grid, st, occ);
+        default: return thn::launch_normalize_bwd_f64(mode, aligned, s, a, grid, st, occ);
+    }
+}
+
 // Workgroups of one kernel instance that fit on a compute unit; asked of the runtime once per instance.
 std::mutex g_occ_mutex;
 std::unordered_map<uint64_t, int> g_occ_cache;
 
-int occupancy(int which, int dtype, bool ln, bool aligned, Shape s) {
+// `ln`: the kernel flavour within the family (LayerNorm / log-softmax: 1; p-norm families: the variant above).
+int occupancy(int which, int dtype, int ln, bool aligned, Shape s) {
     int dev = 0;
     (void)hipGetDevice(&dev);
-    const uint64_t key = (static_cast<uint64_t>(dev) << 40) | (static_cast<uint64_t>(which) << 36) |
-                         (static_cast<uint64_t>(dtype) << 32) | (static_cast<uint64_t>(ln) << 31) |
+    const uint64_t key = (static_cast<uint64_t>(dev) << 44) | (static_cast<uint64_t>(which) << 40) |
+                         (static_cast<uint64_t>(dtype) << 36) | (static_cast<uint64_t>(ln) << 32) |
                          (static_cast<uint64_t>(aligned) << 30) | (static_cast<uint64_t>(s.k) << 24) |
                          (static_cast<uint64_t>(s.tpr) << 12) | static_cast<uint64_t>(s.block);
     {
@@ -137,9 +181,18 @@ int occupancy(int which, int dtype, bool ln, bool aligned, Shape s) {
     } else if (which == kSoftmaxFwd) {
         SoftmaxFwdArgs dummy{};
         rc = launch_softmax_fwd(dtype, ln, aligned, s, dummy, 0, nullptr, &occ);
-    } else {
+    } else if (which == kSoftmaxBwd) {
         SoftmaxBwdArgs dummy{};
         rc = launch_softmax_bwd(dtype, ln, aligned, s, dummy, 0, nullptr, &occ);
+    } else if (which == kPnormFwd) {
+        PnormFwdArgs dummy{};
+        rc = launch_pnorm_fwd(dtype, ln, aligned, s, dummy, 0, nullptr, &occ);
+    } else if (which == kPnormBwd) {
+        PnormBwdArgs dummy{};
+        rc = launch_pnorm_bwd(dtype, ln, aligned, s, dummy, 0, nullptr, &occ);
+    } else {
+        NormalizeBwdArgs dummy{};
+        rc = launch_normalize_bwd(dtype, ln, aligned, s, dummy, 0, nullptr, &occ);
     }
     if (rc != 0 || occ <= 0) occ = 1;
     if (occ > kMaxBlocksPerCu) occ = kMaxBlocksPerCu;
@@ -172,12 +225,13 @@ constexpr int kDefaultBlocksPerCu = 1;
 
 int ceil_div(int a, int b) { return (a + b - 1) / b; }
 
-Shape heuristic_shape(int which, bool ln, bool aligned, int n_vecs) {
+Shape heuristic_shape(int which, int ln, bool aligned, int n_vecs) {
     (void)ln;
     int kmax = (aligned && which == kNormBwd && n_vecs > 128) ? 3 : 4;
     // Softmax backward: two input streams and nothing to hold; 2 vectors per thread per stream measured best,
     // except for 2 KiB rows, where one full wave per row (2 x 64) is 8 % slower than half a wave (4 x 32).
     if (aligned && which == kSoftmaxBwd && n_vecs <= 2048 && !(n_vecs > 64 && n_vecs <= 128)) kmax = 2;
+    if (aligned && which == kNormalizeBwd && n_vecs <= 2048) kmax = 2;    // two or three input streams
     Shape s{4, 1024, 1024};
     for (int tpr : kTprList) {
         if (static_cast<int64_t>(tpr) * kmax >= n_vecs) {
@@ -197,7 +251,7 @@ Shape heuristic_shape(int which, bool ln, bool aligned, int n_vecs) {
     return s;
 }
 
-int plan_launch(int which, bool ln, bool aligned, int64_t M, int64_t N, int dtype, Plan* out) {
+int plan_launch(int which, int ln, bool aligned, int64_t M, int64_t N, int dtype, Plan* out) {
     const int bytes = elem_bytes(dtype);
     if (bytes == 0) return THN_E_DTYPE;
     if (M < 0 || N <= 0) return THN_E_SHAPE;
@@ -242,6 +296,110 @@ bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) ==
 
 int64_t partial_pitch(int64_t N) { return (N + 63) / 64 * 64; }
 
+
+// ---- row p-norm / normalize ---------------------------------------------------------------------------------
+struct RowProblem {
+    int bytes;
+    int64_t rows;
+    int p_int;          // p when it is an integer in [1, 6], else 0
+    bool engine;        // rows fit the row engine (at most 64 KiB, integer p); otherwise the looping kernels
+    bool aligned;
+};
+
+// Common argument checks of the four p-norm entry points.  Returns THN_OK with *done = true when there is
+// nothing to launch.
+int check_row_problem(int64_t B, int64_t M, int64_t K, float p, int dtype, RowProblem* out, bool* done) {
+    *done = false;
+    out->bytes = elem_bytes(dtype);
+    if (out->bytes == 0) return THN_E_DTYPE;
+    if (B < 0 || M < 0 || K <= 0) return THN_E_SHAPE;
+    if (!(p >= 1.0f && p <= 6.0f)) return THN_E_SHAPE;          // "p must be in [1, 6]" (Ops/norm.py:148)
+    out->rows = B * M;
+    if (out->rows == 0) {
+        *done = true;
+        return THN_OK;
+    }
+    const int pi = static_cast<int>(p);
+    out->p_int = static_cast<float>(pi) == p ? pi : 0;
+    out->engine = out->p_int != 0 && K * out->bytes <= kMaxRowBytes;
+    out->aligned = (K % (16 / out->bytes)) == 0;
+    return THN_OK;
+}
+
+// One (B, M, K) operand: fills its row map and folds its alignment into *aligned.  Returns false when the
+// strides cannot be addressed.
+bool map_rows(const void* base, int64_t batch_stride, int64_t row_stride, int64_t B, int64_t M, int64_t K,
+              int bytes, RowMap* map, bool* aligned) {
+    if (batch_stride < 0 || row_stride < 0 || (M > 1 && row_stride < K)) return false;
+    map->batch_stride_bytes = 0;
+    map->rows_per_batch = 0;
+    if (M == 1) {
+        map->row_stride_bytes = batch_stride * bytes;                  // one row per batch: the rows are the batches
+    } else if (B == 1 || batch_stride == M * row_stride) {
+        map->row_stride_bytes = row_stride * bytes;
+    } else {
+        if (B * M >= (int64_t{1} << 31)) return false;
+        map->row_stride_bytes = row_stride * bytes;
+        map->batch_stride_bytes = batch_stride * bytes;
+        map->rows_per_batch = static_cast<uint32_t>(M);
+    }
+    *aligned = *aligned && aligned16(base) && (map->row_stride_bytes % 16) == 0 && (map->batch_stride_bytes % 16) == 0;
+    return true;
+}
+
+int mode_of(int p_int) { return p_int == 1 ? thn::kP1 : (p_int == 2 ? thn::kP2 : thn::kPInt); }
+
+int loop_grid(int64_t rows) {
+    const int64_t cap = static_cast<int64_t>(current_cu_count()) * 8;
+    return static_cast<int>(rows < cap ? rows : cap);
+}
+
+int pnorm_forward(const void* x, int64_t x_batch_stride, int64_t x_row_stride, void* y, int64_t y_batch_stride,
+                  int64_t y_row_stride, void* norms, int64_t B, int64_t M, int64_t K, float p, float eps, int dtype,
+                  bool normalize, void* stream) {
+    RowProblem rp;
+    bool done;
+    const int crc = check_row_problem(B, M, K, p, dtype, &rp, &done);
+    if (crc != THN_OK) return crc;
+    if (!(eps >= 0.0f)) return THN_E_SHAPE;                      // "eps must be non-negative" (Ops/norm.py:149)
+    if (done) return THN_OK;
+    if (x == nullptr || norms == nullptr || (normalize && y == nullptr)) return THN_E_NULL;
+    if (current_cu_count() <= 0) return THN_E_DEVICE;
+    PnormFwdArgs a{};
+    bool aligned = rp.aligned;
+    if (!map_rows(x, x_batch_stride, x_row_stride, B, M, K, rp.bytes, &a.xmap, &aligned)) return THN_E_SHAPE;
+    if (normalize && !map_rows(y, y_batch_stride, y_row_stride, B, M, K, rp.bytes, &a.ymap, &aligned)) return THN_E_SHAPE;
+    a.x = static_cast<const char*>(x);
+    a.y = static_cast<char*>(y);
+    a.norms = norms;
+    a.rows = rp.rows;
+    a.n_cols64 = K;
+    a.n_cols = static_cast<int>(K < INT32_MAX ? K : INT32_MAX);
+    a.p_int = rp.p_int;
+    a.p = p;
+    a.eps = eps;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    int lrc;
+    if (rp.engine) {
+        const int variant = mode_of(rp.p_int) | (normalize ? 4 : 0);
+        Plan plan;
+        const int rc = plan_launch(kPnormFwd, variant, aligned, rp.rows, K, dtype, &plan);
+        if (rc != THN_OK) return rc;
+        a.n_vecs = plan.n_vecs;
+        lrc = launch_pnorm_fwd(dtype, variant, aligned, plan.s, a, plan.grid, st, nullptr);
+    } else {
+        const int grid = loop_grid(rp.rows);
+        switch (dtype) {
+            case THN_F32: lrc = thn::launch_pnorm_fwd_loop_f32(normalize, a, grid, st); break;
+            case THN_F16: lrc = thn::launch_pnorm_fwd_loop_f16(normalize, a, grid, st); break;
+            case THN_BF16: lrc = thn::launch_pnorm_fwd_loop_bf16(normalize, a, grid, st); break;
+            default: lrc = thn::launch_pnorm_fwd_loop_f64(normalize, a, grid, st); break;
+        }
+    }
+    if (lrc > 0) return THN_E_SHAPE;
+    return lrc == 0 ? THN_OK : THN_E_LAUNCH;
+}
+
 }  // namespace
 
 extern "C" {
@@ -280,7 +438,8 @@ int thn_norm_query_launch(int which, int is_layernorm, int64_t M, int64_t N, int
     if (bytes == 0) return THN_E_DTYPE;
     Plan p;
     const bool aligned = N > 0 && (N % (16 / bytes)) == 0;
-    const int rc = plan_launch(which, is_layernorm != 0, aligned, M, N, x_dtype, &p);
+    const int flavour = which >= kPnormFwd ? static_cast<int>(thn::kP2) : (is_layernorm != 0 ? 1 : 0);
+    const int rc = plan_launch(which, flavour, aligned, M, N, x_dtype, &p);
     if (rc != THN_OK) return rc;
     shape[0] = p.s.k;
     shape[1] = p.s.tpr;
@@ -509,6 +668,117 @@ int thn_softmax_bwd(const void* y, int64_t y_row_stride, const void* dy, int64_t
     a.n_vecs = p.n_vecs;
     a.sign = kind == THN_SOFTMIN ? -1.0f : 1.0f;
     const int lrc = launch_softmax_bwd(dtype, is_log, aligned, p.s, a, p.grid, static_cast<hipStream_t>(stream), nullptr);
+    if (lrc > 0) return THN_E_SHAPE;
+    return lrc == 0 ? THN_OK : THN_E_LAUNCH;
+}
+
+int thn_pnorm_fwd(const void* x, int64_t x_batch_stride, int64_t x_row_stride, void* norms, int64_t B, int64_t M,
+                  int64_t K, float p, float eps, int dtype, void* stream) {
+    return pnorm_forward(x, x_batch_stride, x_row_stride, nullptr, 0, 0, norms, B, M, K, p, eps, dtype, false, stream);
+}
+
+int thn_normalize_fwd(const void* x, int64_t x_batch_stride, int64_t x_row_stride, void* y, int64_t y_batch_stride,
+                      int64_t y_row_stride, void* norms, int64_t B, int64_t M, int64_t K, float p, float eps,
+                      int dtype, void* stream) {
+    return pnorm_forward(x, x_batch_stride, x_row_stride, y, y_batch_stride, y_row_stride, norms, B, M, K, p, eps,
+                         dtype, true, stream);
+}
+
+int thn_pnorm_bwd(const void* x, int64_t x_batch_stride, int64_t x_row_stride, const void* norms, const void* dnorms,
+                  void* dx, int64_t dx_batch_stride, int64_t dx_row_stride, int64_t B, int64_t M, int64_t K, float p,
+                  int dtype, void* stream) {
+    RowProblem rp;
+    bool done;
+    const int crc = check_row_problem(B, M, K, p, dtype, &rp, &done);
+    if (crc != THN_OK) return crc;
+    if (done) return THN_OK;
+    if (x == nullptr || dnorms == nullptr || dx == nullptr || (norms == nullptr && p != 1.0f)) return THN_E_NULL;
+    if (current_cu_count() <= 0) return THN_E_DEVICE;
+    PnormBwdArgs a{};
+    bool aligned = rp.aligned;
+    if (!map_rows(x, x_batch_stride, x_row_stride, B, M, K, rp.bytes, &a.xmap, &aligned)) return THN_E_SHAPE;
+    if (!map_rows(dx, dx_batch_stride, dx_row_stride, B, M, K, rp.bytes, &a.dxmap, &aligned)) return THN_E_SHAPE;
+    a.x = static_cast<const char*>(x);
+    a.norms = norms;
+    a.g = dnorms;
+    a.dx = static_cast<char*>(dx);
+    a.rows = rp.rows;
+    a.n_cols64 = K;
+    a.n_cols = static_cast<int>(K < INT32_MAX ? K : INT32_MAX);
+    a.p_int = rp.p_int;
+    a.p = p;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    int lrc;
+    if (rp.engine) {
+        const int mode = mode_of(rp.p_int);
+        Plan plan;
+        const int rc = plan_launch(kPnormBwd, mode, aligned, rp.rows, K, dtype, &plan);
+        if (rc != THN_OK) return rc;
+        a.n_vecs = plan.n_vecs;
+        lrc = launch_pnorm_bwd(dtype, mode, aligned, plan.s, a, plan.grid, st, nullptr);
+    } else {
+        const int grid = loop_grid(rp.rows);
+        switch (dtype) {
+            case THN_F32: lrc = thn::launch_pnorm_bwd_loop_f32(a, grid, st); break;
+            case THN_F16: lrc = thn::launch_pnorm_bwd_loop_f16(a, grid, st); break;
+            case THN_BF16: lrc = thn::launch_pnorm_bwd_loop_bf16(a, grid, st); break;
+            default: lrc = thn::launch_pnorm_bwd_loop_f64(a, grid, st); break;
+        }
+    }
+    if (lrc > 0) return THN_E_SHAPE;
+    return lrc == 0 ? THN_OK : THN_E_LAUNCH;
+}
+
+int thn_normalize_bwd(const void* x, int64_t x_batch_stride, int64_t x_row_stride, const void* y,
+                      int64_t y_batch_stride, int64_t y_row_stride, const void* norms, const void* dy,
+                      int64_t dy_batch_stride, int64_t dy_row_stride, void* dx, int64_t dx_batch_stride,
+                      int64_t dx_row_stride, int64_t B, int64_t M, int64_t K, float p, int dtype, void* stream) {
+    RowProblem rp;
+    bool done;
+    const int crc = check_row_problem(B, M, K, p, dtype, &rp, &done);
+    if (crc != THN_OK) return crc;
+    if (done) return THN_OK;
+    const bool need_x = p != 2.0f, need_y = p != 1.0f;
+    if (norms == nullptr || dy == nullptr || dx == nullptr || (need_x && x == nullptr) || (need_y && y == nullptr)) {
+        return THN_E_NULL;
+    }
+    if (current_cu_count() <= 0) return THN_E_DEVICE;
+    NormalizeBwdArgs a{};
+    bool aligned = rp.aligned;
+    if (need_x && !map_rows(x, x_batch_stride, x_row_stride, B, M, K, rp.bytes, &a.xmap, &aligned)) return THN_E_SHAPE;
+    if (need_y && !map_rows(y, y_batch_stride, y_row_stride, B, M, K, rp.bytes, &a.ymap, &aligned)) return THN_E_SHAPE;
+    if (!map_rows(dy, dy_batch_stride, dy_row_stride, B, M, K, rp.bytes, &a.gmap, &aligned)) return THN_E_SHAPE;
+    if (!map_rows(dx, dx_batch_stride, dx_row_stride, B, M, K, rp.bytes, &a.dxmap, &aligned)) return THN_E_SHAPE;
+    a.x = static_cast<const char*>(need_x ? x : dy);         // never dereferenced when not needed
+    a.y = static_cast<const char*>(need_y ? y : dy);
+    if (!need_x) a.xmap = a.gmap;
+    if (!need_y) a.ymap = a.gmap;
+    a.norms = norms;
+    a.g = static_cast<const char*>(dy);
+    a.dx = static_cast<char*>(dx);
+    a.rows = rp.rows;
+    a.n_cols64 = K;
+    a.n_cols = static_cast<int>(K < INT32_MAX ? K : INT32_MAX);
+    a.p_int = rp.p_int;
+    a.p = p;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    int lrc;
+    if (rp.engine) {
+        const int mode = mode_of(rp.p_int);
+        Plan plan;
+        const int rc = plan_launch(kNormalizeBwd, mode, aligned, rp.rows, K, dtype, &plan);
+        if (rc != THN_OK) return rc;
+        a.n_vecs = plan.n_vecs;
+        lrc = launch_normalize_bwd(dtype, mode, aligned, plan.s, a, plan.grid, st, nullptr);
+    } else {
+        const int grid = loop_grid(rp.rows);
+        switch (dtype) {
+            case THN_F32: lrc = thn::launch_normalize_bwd_loop_f32(a, grid, st); break;
+            case THN_F16: lrc = thn::launch_normalize_bwd_loop_f16(a, grid, st); break;
+            case THN_BF16: lrc = thn::launch_normalize_bwd_loop_bf16(a, grid, st); break;
+            default: lrc = thn::launch_normalize_bwd_loop_f64(a, grid, st); break;
+        }
+    }
     if (lrc > 0) return THN_E_SHAPE;
     return lrc == 0 ? THN_OK : THN_E_LAUNCH;
 }

@@ -1,0 +1,482 @@
+// Row p-norm and p-normalisation over the last dimension of a (B, M, K) tensor, forward and backward: the
+// reference's TritonHub/Ops/norm.py and normalize.py.  Rows of at most 64 KiB run on the row engine of the norm
+// kernels (see thn_kernels.h: 16-byte vectors, TPR threads per row, next row prefetched, branch-free clamped
+// slots).  Everything else -- wider rows, a p that is not an integer -- runs on the looping kernels at the end
+// of this file.
+//
+//   norm forward       (norm.py:24-45):        n = max((sum |x|^p)^(1/p), eps), stored in the storage type
+//   normalize forward  (normalize.py:27-33):   y = x / n, with n ALREADY ROUNDED to the storage type (the
+//                                              reference reads it back from the tensor the norm kernel wrote);
+//                                              here one pass does both: x is read once
+//   norm backward      (norm.py:83-102):       p=1: g*sign(x);  p=2: g*x/n;  else g*sign(x)*|x|^(p-1) / n^(p-1)
+//   normalize backward (normalize.py:81-117):  proj = sum(y*g)  (p=1: sum(x*g));
+//                                              p=1: g/n - sign(x)*(proj/(n*n));  p=2: (g - y*proj)/n;
+//                                              else g/n - sign(x)*|x|^(p-1) * (proj/(n^(p-1)*n))
+// Arithmetic is float32 whatever the storage type (the reference's `dtype` is float32 for anything that is not
+// float16 / bfloat16, norm.py:53).
+#pragma once
+
+#include <type_traits>
+
+#include "thn_kernels.h"
+
+namespace thn {
+
+// Address of row r of a (B, M, K) tensor with element-contiguous rows.  rows_per_batch == 0: the batch and row
+// strides collapse into one (batch_stride == M * row_stride), the common case.
+struct RowMap {
+    int64_t batch_stride_bytes;
+    int64_t row_stride_bytes;
+    uint32_t rows_per_batch;
+};
+
+__device__ __forceinline__ int64_t row_offset(const RowMap& m, int64_t r) {
+    if (m.rows_per_batch == 0) return r * m.row_stride_bytes;
+    const uint32_t r32 = static_cast<uint32_t>(r);          // the host refuses B*M >= 2^31 for such layouts
+    const uint32_t b = r32 / m.rows_per_batch;
+    return b * m.batch_stride_bytes + (r32 - b * m.rows_per_batch) * m.row_stride_bytes;
+}
+
+enum : int { kP1 = 1, kP2 = 2, kPInt = 3 };   // MODE of the row-engine kernels; kPInt: p in {3, 4, 5, 6}
+
+struct PnormFwdArgs {
+    const char* x;
+    char* y;            // normalize only
+    void* norms;        // (rows,) storage type
+    RowMap xmap, ymap;
+    int64_t rows;
+    int64_t n_cols64;   // looping kernels
+    int n_cols;
+    int n_vecs;
+    int p_int;          // p when it is an integer in [1, 6], else 0
+    float p;
+    float eps;
+};
+
+struct PnormBwdArgs {
+    const char* x;
+    const void* norms;  // (rows,) storage type: the saved output of the forward
+    const void* g;      // (rows,) storage type: upstream gradient of the norms
+    char* dx;
+    RowMap xmap, dxmap;
+    int64_t rows;
+    int64_t n_cols64;
+    int n_cols;
+    int n_vecs;
+    int p_int;
+    float p;
+};
+
+struct NormalizeBwdArgs {
+    const char* x;      // read unless p == 2
+    const char* y;      // the saved normalised output; read unless p == 1
+    const void* norms;
+    const char* g;      // upstream gradient of y, (B, M, K)
+    char* dx;
+    RowMap xmap, ymap, gmap, dxmap;
+    int64_t rows;
+    int64_t n_cols64;
+    int n_cols;
+    int n_vecs;
+    int p_int;
+    float p;
+};
+
+// a^e for a >= 0 and a launch-uniform integer e in [2, 6], without a branch.
+__device__ __forceinline__ float pow_small(float a, int e) {
+    const float a2 = a * a, a3 = a2 * a, a4 = a2 * a2;
+    float r = a2;
+    r = e == 3 ? a3 : r;
+    r = e == 4 ? a4 : r;
+    r = e == 5 ? a4 * a : r;
+    r = e == 6 ? a3 * a3 : r;
+    return r;
+}
+
+__device__ __forceinline__ float sign_of(float x) { return x > 0.0f ? 1.0f : (x < 0.0f ? -1.0f : 0.0f); }
+
+// num / den with the row's correctly rounded reciprocal `rden` = 1/den: one multiplication and one residual
+// correction (q + (num - q*den)*rden), which is the correctly rounded quotient except for isolated
+// significand patterns, at 3 instructions per element instead of the ~10 of a full division.  |num/den| must
+// be representable (true here: every quotient is bounded by the row's norm) and den must not be subnormal
+// (then rden is infinite and the quotient is infinite or NaN where exact division would give a huge finite
+// number; the norms are clamped from below by eps, so this needs eps = 0 and a row of subnormals).
+__device__ __forceinline__ float div_by_row(float num, float den, float rden) {
+    const float q = num * rden;
+    return __builtin_fmaf(__builtin_fmaf(-q, den, num), rden, q);
+}
+
+// x rounded to storage type T and widened again.
+template <typename T>
+__device__ __forceinline__ float round_to_storage(float f) {
+    if constexpr (T::kBytes >= 4) {
+        return f;
+    } else {
+        float tmp[T::VEC];
+#pragma unroll
+        for (int e = 0; e < T::VEC; ++e) tmp[e] = f;
+        const u32x4 v = T::pack(tmp);
+        T::unpack(v, tmp);
+        return tmp[0];
+    }
+}
+
+template <int MODE>
+__device__ __forceinline__ float norm_term(float x, int p_int) {
+    if constexpr (MODE == kP1) return __builtin_fabsf(x);
+    else if constexpr (MODE == kP2) return x * x;
+    else return pow_small(__builtin_fabsf(x), p_int);
+}
+
+template <int MODE>
+__device__ __forceinline__ float norm_root(float acc, float p) {
+    if constexpr (MODE == kP1) return acc;
+    else if constexpr (MODE == kP2) return sqrtf(acc);
+    else return powf(acc, 1.0f / p);
+}
+
+// ---------------------------------------------------------------------------------------------------
+// Forward on the row engine.  NORMALIZE = false: norms only (x read once: K*s bytes per row).
+// NORMALIZE = true: norms and y = x / norms from the registers (x read once, y written once: 2*K*s bytes).
+// ---------------------------------------------------------------------------------------------------
+template <typename T, int MODE, bool NORMALIZE, int K, int TPR, int BLOCK, bool ALIGNED>
+__global__ void __launch_bounds__(BLOCK) pnorm_fwd_kernel(const PnormFwdArgs a) {
+    constexpr int VEC = T::VEC;
+    constexpr int G = BLOCK / TPR;
+    static_assert(BLOCK % TPR == 0 && G >= 1, "a workgroup holds whole rows");
+    __shared__ float red[RedSmem<TPR, G, 1>::kFloats];
+
+    const int tid = threadIdx.x;
+    const int g = tid / TPR;
+    const int t = tid % TPR;
+    int phase = 0;
+
+    int voff[K];
+    bool own[K];
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+        const int v = t + k * TPR;
+        const int vc = v < a.n_vecs ? v : a.n_vecs - 1;
+        voff[k] = ALIGNED ? vc * 16 : vc;
+        own[k] = v < a.n_vecs;
+    }
+
+    const int64_t rows_per_iter = static_cast<int64_t>(gridDim.x) * G;
+    const int64_t last_row = a.rows - 1;
+    int64_t row_raw = static_cast<int64_t>(blockIdx.x) * G + g;
+    int64_t row = row_raw < a.rows ? row_raw : last_row;
+    u32x4 cur[K];
+    load_row<T, K, ALIGNED>(cur, a.x + row_offset(a.xmap, row), 0, 0, voff, a.n_cols);
+
+    drain_vector_memory();
+    for (int64_t base = static_cast<int64_t>(blockIdx.x) * G; base < a.rows; base += rows_per_iter) {
+        const int64_t nrow_raw = row_raw + rows_per_iter;
+        const int64_t nrow = nrow_raw < a.rows ? nrow_raw : last_row;
+        u32x4 nxt[K];
+        load_row<T, K, ALIGNED>(nxt, a.x + row_offset(a.xmap, nrow), 0, 0, voff, a.n_cols);
+
+        float xf[K][VEC];
+        float s[1] = {0.0f};
+#pragma unroll
+        for (int k = 0; k < K; ++k) {
+            T::unpack(cur[k], xf[k]);
+            float sk = 0.0f;
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) sk += norm_term<MODE>(xf[k][e], a.p_int);   // absent columns load as 0
+            s[0] += own[k] ? sk : 0.0f;
+        }
+        row_allreduce<TPR, G, 1>(s, red, phase, g, t);
+        const float n = fmaxf(norm_root<MODE>(s[0], a.p), a.eps);
+        // Every thread of the row stores the same value to the same address (one request per wave).
+        T::store1(a.norms, row, n);
+
+        if constexpr (NORMALIZE) {
+            const float nr = round_to_storage<T>(n);
+            const float rn = 1.0f / nr;
+            char* yrow = a.y + row_offset(a.ymap, row);
+#pragma unroll
+            for (int k = 0; k < K; ++k) {
+                float yf[VEC];
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) yf[e] = div_by_row(xf[k][e], nr, rn);
+                store_row_vec<T, ALIGNED>(yrow, voff[k], a.n_cols, yf);
+            }
+        }
+
+#pragma unroll
+        for (int k = 0; k < K; ++k) cur[k] = nxt[k];
+        row_raw = nrow_raw;
+        row = nrow;
+    }
+}
+
+// ---------------------------------------------------------------------------------------------------
+// Norm backward: element-wise with two per-row scalars; x read once, dx written once (2*K*s bytes per row).
+// ---------------------------------------------------------------------------------------------------
+template <typename T, int MODE, int K, int TPR, int BLOCK, bool ALIGNED>
+__global__ void __launch_bounds__(BLOCK) pnorm_bwd_kernel(const PnormBwdArgs a) {
+    constexpr int VEC = T::VEC;
+    constexpr int G = BLOCK / TPR;
+    static_assert(BLOCK % TPR == 0 && G >= 1, "a workgroup holds whole rows");
+
+    const int tid = threadIdx.x;
+    const int g = tid / TPR;
+    const int t = tid % TPR;
+
+    int voff[K];
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+        const int v = t + k * TPR;
+        const int vc = v < a.n_vecs ? v : a.n_vecs - 1;
+        voff[k] = ALIGNED ? vc * 16 : vc;
+    }
+
+    const int64_t rows_per_iter = static_cast<int64_t>(gridDim.x) * G;
+    const int64_t last_row = a.rows - 1;
+    int64_t row_raw = static_cast<int64_t>(blockIdx.x) * G + g;
+    int64_t row = row_raw < a.rows ? row_raw : last_row;
+    u32x4 cur[K];
+    load_row<T, K, ALIGNED>(cur, a.x + row_offset(a.xmap, row), 0, 0, voff, a.n_cols);
+    float c_n = MODE == kP1 ? 1.0f : T::load1(a.norms, row);
+    float c_g = T::load1(a.g, row);
+
+    drain_vector_memory();
+    for (int64_t base = static_cast<int64_t>(blockIdx.x) * G; base < a.rows; base += rows_per_iter) {
+        const int64_t nrow_raw = row_raw + rows_per_iter;
+        const int64_t nrow = nrow_raw < a.rows ? nrow_raw : last_row;
+        u32x4 nxt[K];
+        load_row<T, K, ALIGNED>(nxt, a.x + row_offset(a.xmap, nrow), 0, 0, voff, a.n_cols);
+        const float n_n = MODE == kP1 ? 1.0f : T::load1(a.norms, nrow);
+        const float n_g = T::load1(a.g, nrow);
+
+        float den = c_n;
+        if constexpr (MODE == kPInt) den = pow_small(c_n, a.p_int - 1);     // norms^(p-1), norm.py:86-87
+        const float rden = 1.0f / den;
+        char* dxrow = a.dx + row_offset(a.dxmap, row);
+#pragma unroll
+        for (int k = 0; k < K; ++k) {
+            float xf[VEC], df[VEC];
+            T::unpack(cur[k], xf);
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+                const float x = xf[e];
+                if constexpr (MODE == kP1) df[e] = c_g * sign_of(x);
+                else if constexpr (MODE == kP2) df[e] = div_by_row(c_g * x, den, rden);
+                else df[e] = div_by_row(c_g * sign_of(x) * pow_small(__builtin_fabsf(x), a.p_int - 1), den, rden);
+            }
+            store_row_vec<T, ALIGNED>(dxrow, voff[k], a.n_cols, df);
+        }
+
+#pragma unroll
+        for (int k = 0; k < K; ++k) cur[k] = nxt[k];
+        c_n = n_n;
+        c_g = n_g;
+        row_raw = nrow_raw;
+        row = nrow;
+    }
+}
+
+// ---------------------------------------------------------------------------------------------------
+// Normalize backward.  p = 2 reads y and g (3*K*s bytes per row with the dx store), p = 1 reads x and g
+// (3*K*s), other p read x, y and g (4*K*s).  One reduction round per row.
+// ---------------------------------------------------------------------------------------------------
+template <typename T, int MODE, int K, int TPR, int BLOCK, bool ALIGNED>
+__global__ void __launch_bounds__(BLOCK) normalize_bwd_kernel(const NormalizeBwdArgs a) {
+    constexpr int VEC = T::VEC;
+    constexpr int G = BLOCK / TPR;
+    constexpr bool NEED_X = MODE != kP2;
+    constexpr bool NEED_Y = MODE != kP1;
+    static_assert(BLOCK % TPR == 0 && G >= 1, "a workgroup holds whole rows");
+    __shared__ float red[RedSmem<TPR, G, 1>::kFloats];
+
+    const int tid = threadIdx.x;
+    const int g = tid / TPR;
+    const int t = tid % TPR;
+    int phase = 0;
+
+    int voff[K];
+    bool own[K];
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+        const int v = t + k * TPR;
+        const int vc = v < a.n_vecs ? v : a.n_vecs - 1;
+        voff[k] = ALIGNED ? vc * 16 : vc;
+        own[k] = v < a.n_vecs;
+    }
+
+    const int64_t rows_per_iter = static_cast<int64_t>(gridDim.x) * G;
+    const int64_t last_row = a.rows - 1;
+    int64_t row_raw = static_cast<int64_t>(blockIdx.x) * G + g;
+    int64_t row = row_raw < a.rows ? row_raw : last_row;
+    u32x4 cx[NEED_X ? K : 1], cy[NEED_Y ? K : 1], cg[K];
+    if constexpr (NEED_X) load_row<T, K, ALIGNED>(cx, a.x + row_offset(a.xmap, row), 0, 0, voff, a.n_cols);
+    if constexpr (NEED_Y) load_row<T, K, ALIGNED>(cy, a.y + row_offset(a.ymap, row), 0, 0, voff, a.n_cols);
+    load_row<T, K, ALIGNED>(cg, a.g + row_offset(a.gmap, row), 0, 0, voff, a.n_cols);
+    float c_n = T::load1(a.norms, row);
+
+    drain_vector_memory();
+    for (int64_t base = static_cast<int64_t>(blockIdx.x) * G; base < a.rows; base += rows_per_iter) {
+        const int64_t nrow_raw = row_raw + rows_per_iter;
+        const int64_t nrow = nrow_raw < a.rows ? nrow_raw : last_row;
+        u32x4 nx[NEED_X ? K : 1], ny[NEED_Y ? K : 1], ng[K];
+        if constexpr (NEED_X) load_row<T, K, ALIGNED>(nx, a.x + row_offset(a.xmap, nrow), 0, 0, voff, a.n_cols);
+        if constexpr (NEED_Y) load_row<T, K, ALIGNED>(ny, a.y + row_offset(a.ymap, nrow), 0, 0, voff, a.n_cols);
+        load_row<T, K, ALIGNED>(ng, a.g + row_offset(a.gmap, nrow), 0, 0, voff, a.n_cols);
+        const float n_n = T::load1(a.norms, nrow);
+
+        float xf[NEED_X ? K : 1][VEC], yf[NEED_Y ? K : 1][VEC], gf[K][VEC];
+        float s[1] = {0.0f};
+#pragma unroll
+        for (int k = 0; k < K; ++k) {
+            if constexpr (NEED_X) T::unpack(cx[k], xf[k]);
+            if constexpr (NEED_Y) T::unpack(cy[k], yf[k]);
+            T::unpack(cg[k], gf[k]);
+            float sk = 0.0f;
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+                if constexpr (MODE == kP1) sk = __builtin_fmaf(xf[k][e], gf[k][e], sk);       // normalize.py:92
+                else sk = __builtin_fmaf(yf[k][e], gf[k][e], sk);                             // normalize.py:96
+            }
+            s[0] += own[k] ? sk : 0.0f;
+        }
+        row_allreduce<TPR, G, 1>(s, red, phase, g, t);
+        const float proj = s[0];
+        const float n = c_n;
+        const float rn = 1.0f / n;
+        float coef = 0.0f;                                                                    // per-row factor of sign(x)*...
+        if constexpr (MODE == kP1) coef = proj / (n * n);                                     // normalize.py:106
+        if constexpr (MODE == kPInt) coef = proj / (pow_small(n, a.p_int - 1) * n);           // normalize.py:115
+
+        char* dxrow = a.dx + row_offset(a.dxmap, row);
+#pragma unroll
+        for (int k = 0; k < K; ++k) {
+            float df[VEC];
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+                const float gg = gf[k][e];
+                if constexpr (MODE == kP2) {
+                    df[e] = div_by_row(gg - yf[k][e] * proj, n, rn);                          // normalize.py:110
+                } else if constexpr (MODE == kP1) {
+                    df[e] = div_by_row(gg, n, rn) - sign_of(xf[k][e]) * coef;
+                } else {
+                    const float x = xf[k][e];
+                    df[e] = div_by_row(gg, n, rn) - sign_of(x) * pow_small(__builtin_fabsf(x), a.p_int - 1) * coef;
+                }
+            }
+            store_row_vec<T, ALIGNED>(dxrow, voff[k], a.n_cols, df);
+        }
+
+#pragma unroll
+        for (int k = 0; k < K; ++k) {
+            if constexpr (NEED_X) cx[k] = nx[k];
+            if constexpr (NEED_Y) cy[k] = ny[k];
+            cg[k] = ng[k];
+        }
+        c_n = n_n;
+        row_raw = nrow_raw;
+        row = nrow;
+    }
+}
+
+// ---------------------------------------------------------------------------------------------------
+// Looping kernels: one 256-thread workgroup per row (grid-stride over rows), the row walked in strides of
+// 256 elements as often as the formula needs it (the second walk of a row comes from the L2).  Any row
+// width, any real p in [1, 6] (accurate powf), any alignment.  This is the path of rows wider than 64 KiB
+// and of non-integer p; it is not tuned.
+// ---------------------------------------------------------------------------------------------------
+constexpr int kLoopBlock = 256;
+
+// ax^e for ax >= 0; e_int is e when e is an integer in [0, 6], else -1.
+__device__ __forceinline__ float pow_abs_any(float ax, float e, int e_int) {
+    if (e_int == 0) return 1.0f;
+    if (e_int == 1) return ax;
+    if (e_int >= 2 && e_int <= 6) return pow_small(ax, e_int);
+    return powf(ax, e);
+}
+
+template <typename T, bool NORMALIZE>
+__global__ void __launch_bounds__(kLoopBlock) pnorm_fwd_loop_kernel(const PnormFwdArgs a) {
+    __shared__ float red[RedSmem<kLoopBlock, 1, 1>::kFloats];
+    int phase = 0;
+    const int t = threadIdx.x;
+    for (int64_t row = blockIdx.x; row < a.rows; row += gridDim.x) {
+        const char* xrow = a.x + row_offset(a.xmap, row);
+        float s[1] = {0.0f};
+        for (int64_t c = t; c < a.n_cols64; c += kLoopBlock) {
+            const float x = T::load1(xrow, c);
+            s[0] += a.p_int == 2 ? x * x : pow_abs_any(__builtin_fabsf(x), a.p, a.p_int > 0 ? a.p_int : -1);
+        }
+        row_allreduce<kLoopBlock, 1, 1>(s, red, phase, 0, t);
+        float n = s[0];
+        if (a.p_int == 2) n = sqrtf(n);
+        else if (a.p_int != 1) n = powf(n, 1.0f / a.p);
+        n = fmaxf(n, a.eps);
+        if (t == 0) T::store1(a.norms, row, n);
+        if constexpr (NORMALIZE) {
+            const float nr = round_to_storage<T>(n);
+            char* yrow = a.y + row_offset(a.ymap, row);
+            for (int64_t c = t; c < a.n_cols64; c += kLoopBlock) T::store1(yrow, c, T::load1(xrow, c) / nr);
+        }
+    }
+}
+
+template <typename T>
+__global__ void __launch_bounds__(kLoopBlock) pnorm_bwd_loop_kernel(const PnormBwdArgs a) {
+    const int t = threadIdx.x;
+    for (int64_t row = blockIdx.x; row < a.rows; row += gridDim.x) {
+        const char* xrow = a.x + row_offset(a.xmap, row);
+        char* dxrow = a.dx + row_offset(a.dxmap, row);
+        const float g = T::load1(a.g, row);
+        float den = 1.0f;
+        if (a.p_int != 1) {
+            const float n = T::load1(a.norms, row);
+            den = a.p_int == 2 ? n : pow_abs_any(n, a.p - 1.0f, a.p_int > 0 ? a.p_int - 1 : -1);
+        }
+        for (int64_t c = t; c < a.n_cols64; c += kLoopBlock) {
+            const float x = T::load1(xrow, c);
+            float d;
+            if (a.p_int == 1) d = g * sign_of(x);
+            else if (a.p_int == 2) d = (g * x) / den;
+            else d = (g * sign_of(x) * pow_abs_any(__builtin_fabsf(x), a.p - 1.0f, a.p_int > 0 ? a.p_int - 1 : -1)) / den;
+            T::store1(dxrow, c, d);
+        }
+    }
+}
+
+template <typename T>
+__global__ void __launch_bounds__(kLoopBlock) normalize_bwd_loop_kernel(const NormalizeBwdArgs a) {
+    __shared__ float red[RedSmem<kLoopBlock, 1, 1>::kFloats];
+    int phase = 0;
+    const int t = threadIdx.x;
+    const int e_int = a.p_int > 0 ? a.p_int - 1 : -1;
+    for (int64_t row = blockIdx.x; row < a.rows; row += gridDim.x) {
+        const char* xrow = a.x + row_offset(a.xmap, row);
+        const char* yrow = a.y + row_offset(a.ymap, row);
+        const char* grow = a.g + row_offset(a.gmap, row);
+        char* dxrow = a.dx + row_offset(a.dxmap, row);
+        const float n = T::load1(a.norms, row);
+        float s[1] = {0.0f};
+        for (int64_t c = t; c < a.n_cols64; c += kLoopBlock) {
+            const float other = a.p_int == 1 ? T::load1(xrow, c) : T::load1(yrow, c);
+            s[0] = __builtin_fmaf(other, T::load1(grow, c), s[0]);
+        }
+        row_allreduce<kLoopBlock, 1, 1>(s, red, phase, 0, t);
+        const float proj = s[0];
+        float coef = 0.0f;
+        if (a.p_int == 1) coef = proj / (n * n);
+        else if (a.p_int != 2) coef = proj / (pow_abs_any(n, a.p - 1.0f, e_int) * n);
+        for (int64_t c = t; c < a.n_cols64; c += kLoopBlock) {
+            const float gg = T::load1(grow, c);
+            float d;
+            if (a.p_int == 2) {
+                d = (gg - T::load1(yrow, c) * proj) / n;
+            } else {
+                const float x = T::load1(xrow, c);
+                d = gg / n - sign_of(x) * pow_abs_any(__builtin_fabsf(x), a.p - 1.0f, e_int) * coef;
+            }
+            T::store1(dxrow, c, d);
+        }
+    }
+}
+
+}  // namespace thn
