@@ -47,6 +47,14 @@ WORKLOADS = {
     "softmin_bf16_16384x4096": ("softmin", 16384, 4096, "bf16"),
     "logsoftmax_bf16_8192x32768": ("logsoftmax", 8192, 32768, "bf16"),
     "logsoftmax_f32_16384x4096": ("logsoftmax", 16384, 4096, "f32"),
+    # row p-norm / normalize of a (1, rows, K) tensor (thn_normalize_fwd + thn_normalize_bwd, or thn_pnorm_*)
+    "normalize_p2_bf16_16384x4096": ("normalize_p2", 16384, 4096, "bf16"),
+    "normalize_p2_f32_16384x4096": ("normalize_p2", 16384, 4096, "f32"),
+    "normalize_p2_f16_65536x1024": ("normalize_p2", 65536, 1024, "f16"),
+    "normalize_p1_bf16_16384x4096": ("normalize_p1", 16384, 4096, "bf16"),
+    "normalize_p3_bf16_16384x4096": ("normalize_p3", 16384, 4096, "bf16"),
+    "pnorm_p2_bf16_16384x4096": ("pnorm_p2", 16384, 4096, "bf16"),
+    "pnorm_p3_f32_16384x4096": ("pnorm_p3", 16384, 4096, "f32"),
 }
 SOFTMAX_KINDS = ("softmax", "softmin", "logsoftmax")
 
@@ -62,6 +70,11 @@ MEASURED_TRAFFIC_BYTES = {
 
 
 def algorithmic_bytes(kind, m, n, s, sw):
+    if kind.startswith("normalize"):          # forward: x read, y + norms written; backward: y (x for p=1; x and y for
+        extra = 0 if kind[-1] in "12" else 1  # other p), dy and norms read, dx written
+        return 2 * m * n * s + m * s, (3 + extra) * m * n * s + m * s
+    if kind.startswith("pnorm"):              # forward: x read, norms written; backward: x, norms, dnorms read, dx written
+        return m * n * s + m * s, 2 * m * n * s + 2 * m * s
     if kind in SOFTMAX_KINDS:                 # forward: x read, y written; backward: y and dy read, dx written
         return 2 * m * n * s, 3 * m * n * s
     if kind == "ln":
@@ -94,7 +107,7 @@ def main():
     torch.cuda.set_device(dev)
     kind, m, n, dname = WORKLOADS[args.workload]
     dtype = {"bf16": torch.bfloat16, "f16": torch.float16, "f32": torch.float32}[dname]
-    if kind in SOFTMAX_KINDS:
+    if kind in SOFTMAX_KINDS or kind.startswith(("normalize", "pnorm")):
         return softmax_main(args, lib, dev, kind, m, n, dname, dtype)
     s = torch.empty(0, dtype=dtype).element_size()
     code = _native.dtype_code(dtype)
@@ -237,22 +250,40 @@ def softmax_main(args, lib, dev, kind, m, n, dname, dtype):
     from TritonHub.Normalization import _launch
     s = torch.empty(0, dtype=dtype).element_size()
     code = _native.dtype_code(dtype)
-    kcode = {"softmax": _native.SOFTMAX, "softmin": _native.SOFTMIN, "logsoftmax": _native.LOGSOFTMAX}[kind]
+    kcode = {"softmax": _native.SOFTMAX, "softmin": _native.SOFTMIN, "logsoftmax": _native.LOGSOFTMAX}.get(kind)
+    row_op = None if kcode is not None else kind.split("_")[0]          # "normalize" or "pnorm"
+    pval = float(kind[-1]) if row_op else 0.0
     gen = torch.Generator(device=dev).manual_seed(0)
     sets = []
     for _ in range(N_BUFFER_SETS):
         x = (3.0 * torch.randn(m, n, device=dev, generator=gen)).to(dtype)
         dy = torch.randn(m, n, device=dev, generator=gen).to(dtype)
-        sets.append(dict(x=x, dy=dy, y=torch.empty_like(x), dx=torch.empty_like(x)))
+        sets.append(dict(x=x, dy=dy, y=torch.empty_like(x), dx=torch.empty_like(x),
+                         norms=torch.empty(m, device=dev, dtype=dtype),
+                         dnorms=torch.rand(m, device=dev, generator=gen).to(dtype)))
     stream = torch.cuda.current_stream(dev).cuda_stream
     p = _native.ptr
+    mn = m * n
 
     def forward(b_):
-        rc = lib.thn_softmax_fwd(p(b_["x"]), n, p(b_["y"]), n, m, n, kcode, code, stream)
+        if row_op == "normalize":
+            rc = lib.thn_normalize_fwd(p(b_["x"]), mn, n, p(b_["y"]), mn, n, p(b_["norms"]), 1, m, n, pval, 1e-12, code,
+                                       stream)
+        elif row_op == "pnorm":
+            rc = lib.thn_pnorm_fwd(p(b_["x"]), mn, n, p(b_["norms"]), 1, m, n, pval, 1e-12, code, stream)
+        else:
+            rc = lib.thn_softmax_fwd(p(b_["x"]), n, p(b_["y"]), n, m, n, kcode, code, stream)
         assert rc == 0, _native.strerror(rc)
 
     def backward(b_):
-        rc = lib.thn_softmax_bwd(p(b_["y"]), n, p(b_["dy"]), n, p(b_["dx"]), n, m, n, kcode, code, stream)
+        if row_op == "normalize":
+            rc = lib.thn_normalize_bwd(p(b_["x"]), mn, n, p(b_["y"]), mn, n, p(b_["norms"]), p(b_["dy"]), mn, n,
+                                       p(b_["dx"]), mn, n, 1, m, n, pval, code, stream)
+        elif row_op == "pnorm":
+            rc = lib.thn_pnorm_bwd(p(b_["x"]), mn, n, p(b_["norms"]), p(b_["dnorms"]), p(b_["dx"]), mn, n, 1, m, n,
+                                   pval, code, stream)
+        else:
+            rc = lib.thn_softmax_bwd(p(b_["y"]), n, p(b_["dy"]), n, p(b_["dx"]), n, m, n, kcode, code, stream)
         assert rc == 0, _native.strerror(rc)
 
     def step(i):
@@ -290,15 +321,19 @@ def softmax_main(args, lib, dev, kind, m, n, dname, dtype):
             sets[i % N_BUFFER_SETS]["dx"].copy_(sets[i % N_BUFFER_SETS]["x"])
         torch.cuda.synchronize()
     achieved = bwd_bytes / (bwd_us * 1e-6) / 1e9
-    fs = _launch.query_launch(2, kind == "logsoftmax", m, n, dtype)
-    bs = _launch.query_launch(3, kind == "logsoftmax", m, n, dtype)
+    fam = {None: (2, 3), "normalize": (4, 6), "pnorm": (4, 5)}[row_op]
+    fs = _launch.query_launch(fam[0], kind == "logsoftmax", m, n, dtype)
+    bs = _launch.query_launch(fam[1], kind == "logsoftmax", m, n, dtype)
+    bwd_kernel = {None: "softmax_bwd_kernel", "normalize": "normalize_bwd_kernel", "pnorm": "pnorm_bwd_kernel"}[row_op]
+    entry = {None: "thn_softmax_fwd + thn_softmax_bwd", "normalize": "thn_normalize_fwd + thn_normalize_bwd",
+             "pnorm": "thn_pnorm_fwd + thn_pnorm_bwd"}[row_op]
     out = {
         "metric": f"fwd+bwd HBM GB/s and % of peak, {kind} {dname} {m}x{n}",
         "value": round(gbps, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": dname, "data": "synthetic",
         "config": {"workload": args.workload, "op": kind, "rows": m, "row_width": n, "buffer_sets": N_BUFFER_SETS,
-                   "entry_points": "thn_softmax_fwd + thn_softmax_bwd"},
+                   "entry_points": entry},
         "pct_of_hbm_peak": round(100.0 * gbps / HBM_PEAK_GBPS, 2),
         "rows_per_s": round(m / (ms_per_step * 1e-3)),
         "algorithmic_bytes_per_step": step_bytes,
@@ -306,14 +341,61 @@ def softmax_main(args, lib, dev, kind, m, n, dname, dtype):
                        "forward_GBps": round(fwd_bytes / (fwd_us * 1e-6) / 1e9, 1)},
         "launch": {"forward": dict(zip(("vecs_per_thread", "threads_per_row", "block", "grid"), fs[:4])),
                    "backward": dict(zip(("vecs_per_thread", "threads_per_row", "block", "grid"), bs[:4]))},
-        "roofline": {"bound": "hbm", "kernel": "softmax_bwd_kernel", "achieved": round(achieved, 1),
+        "roofline": {"bound": "hbm", "kernel": bwd_kernel, "achieved": round(achieved, 1),
                      "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
                      "algorithmic_bytes_per_launch": bwd_bytes, "avg_launch_us": round(bwd_us, 2),
                      "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload)},
     }
     if not args.no_cpu_baseline:
-        out["cpu_baseline"] = softmax_cpu_baseline(kind, m, n, dtype, sets[0], step_bytes)
+        out["cpu_baseline"] = (row_op_cpu_baseline if row_op else softmax_cpu_baseline)(kind, m, n, dtype, sets[0], step_bytes)
     print(json.dumps(out), flush=True)
+
+
+def row_op_cpu_baseline(kind, m, n, dtype, buffers, step_bytes):
+    """oracle/pnorm_oracle.py (numpy float64, one thread) on a bounded sample of the same rows, and torch on the
+    host cores next to it."""
+    import torch
+    from oracle import pnorm_oracle as po
+    op, pval = kind.split("_")[0], int(kind[-1])
+    rows = min(m, max(64, (1 << 23) // n))
+    x = buffers["x"][:rows].cpu()
+    dy = buffers["dy"][:rows].cpu()
+    gn = buffers["dnorms"][:rows].cpu()
+    x64, dy64, gn64 = x.double().numpy(), dy.double().numpy(), gn.double().numpy()
+
+    def oracle_step():
+        nrm = po.norm_fwd(x64, pval, 1e-12)
+        if op == "normalize":
+            po.normalize_bwd(x64, po.normalize_fwd(x64, nrm), nrm, dy64, pval)
+        else:
+            po.norm_bwd(x64, nrm, gn64, pval)
+
+    def torch_step():
+        xr = x.clone().requires_grad_(True)
+        if op == "normalize":
+            torch.nn.functional.normalize(xr, p=pval, dim=-1, eps=1e-12).backward(dy)
+        else:
+            torch.norm(xr, p=pval, dim=-1).backward(gn)
+
+    def timed(f, reps):
+        f()
+        best = float("inf")
+        for _ in range(reps):
+            t0 = time.perf_counter()
+            f()
+            best = min(best, time.perf_counter() - t0)
+        return best
+
+    sample_bytes = step_bytes * rows / m
+    t_oracle, t_torch = timed(oracle_step, 3), timed(torch_step, 3)
+    return {"value": round(sample_bytes / t_oracle / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
+            "sample": f"first {rows} of {m} rows of the same workload, forward + backward, best of 3 passes of "
+                      f"oracle/pnorm_oracle.py (numpy float64, one thread; {t_oracle * 1e3:.1f} ms per pass)",
+            "host_cpu_count": os.cpu_count(),
+            "torch_functional": {"value": round(sample_bytes / t_torch / 1e9, 2), "unit": "GB/s",
+                                 "threads": torch.get_num_threads(),
+                                 "what": f"torch {op} forward + autograd backward on the host cores, same sample "
+                                         f"({t_torch * 1e3:.1f} ms per pass)"}}
 
 
 def softmax_cpu_baseline(kind, m, n, dtype, buffers, step_bytes):

@@ -275,7 +275,10 @@ int plan_launch(int which, int ln, bool aligned, int64_t M, int64_t N, int dtype
     if (!shape_compiled(which, aligned, s)) return THN_E_SHAPE;
 
     int bpc = occupancy(which, dtype, ln, aligned, s);
-    const int cap = ov.bpc.load() > 0 ? ov.bpc.load() : kDefaultBlocksPerCu;
+    // The p-norm families in 256-thread workgroups (rows up to 16 KiB) measured 5-25 % faster with two workgroups
+    // per compute unit; everything else with one.
+    const int family_bpc = (which >= kPnormFwd && s.block <= 256) ? 2 : kDefaultBlocksPerCu;
+    const int cap = ov.bpc.load() > 0 ? ov.bpc.load() : family_bpc;
     if (cap < bpc) bpc = cap;
     const int rows_per_block = s.block / s.tpr;
     const int64_t row_blocks = (M + rows_per_block - 1) / rows_per_block;
@@ -326,25 +329,27 @@ int check_row_problem(int64_t B, int64_t M, int64_t K, float p, int dtype, RowPr
     return THN_OK;
 }
 
-// One (B, M, K) operand: fills its row map and folds its alignment into *aligned.  Returns false when the
-// strides cannot be addressed.
+// One (B, M, K) operand: fills its row map, folds its alignment into *aligned and clears *uniform when its batch
+// stride is not M row strides.  Returns false when the strides cannot be addressed.
 bool map_rows(const void* base, int64_t batch_stride, int64_t row_stride, int64_t B, int64_t M, int64_t K,
-              int bytes, RowMap* map, bool* aligned) {
+              int bytes, RowMap* map, bool* aligned, bool* uniform) {
     if (batch_stride < 0 || row_stride < 0 || (M > 1 && row_stride < K)) return false;
-    map->batch_stride_bytes = 0;
-    map->rows_per_batch = 0;
-    if (M == 1) {
-        map->row_stride_bytes = batch_stride * bytes;                  // one row per batch: the rows are the batches
-    } else if (B == 1 || batch_stride == M * row_stride) {
-        map->row_stride_bytes = row_stride * bytes;
-    } else {
-        if (B * M >= (int64_t{1} << 31)) return false;
-        map->row_stride_bytes = row_stride * bytes;
-        map->batch_stride_bytes = batch_stride * bytes;
-        map->rows_per_batch = static_cast<uint32_t>(M);
-    }
-    *aligned = *aligned && aligned16(base) && (map->row_stride_bytes % 16) == 0 && (map->batch_stride_bytes % 16) == 0;
+    if (M == 1) row_stride = batch_stride;            // one row per batch: the rows are the batches
+    else if (B > 1 && batch_stride != M * row_stride) *uniform = false;
+    map->batch_stride_bytes = batch_stride * bytes;
+    map->row_stride_bytes = row_stride * bytes;
+    *aligned = *aligned && aligned16(base) && (map->row_stride_bytes % 16) == 0 &&
+               (B == 1 || (map->batch_stride_bytes % 16) == 0);
     return true;
+}
+
+// The (batch, row) walk of a launch whose row groups advance by rows_per_iter rows per step.
+thn::RowWalk make_walk(bool uniform, int64_t M, int64_t rows, int64_t rows_per_iter) {
+    thn::RowWalk w;
+    w.rows_per_batch = uniform ? rows : M;
+    w.step_batch = rows_per_iter / w.rows_per_batch;
+    w.step_row = rows_per_iter % w.rows_per_batch;
+    return w;
 }
 
 int mode_of(int p_int) { return p_int == 1 ? thn::kP1 : (p_int == 2 ? thn::kP2 : thn::kPInt); }
@@ -366,9 +371,11 @@ int pnorm_forward(const void* x, int64_t x_batch_stride, int64_t x_row_stride, v
     if (x == nullptr || norms == nullptr || (normalize && y == nullptr)) return THN_E_NULL;
     if (current_cu_count() <= 0) return THN_E_DEVICE;
     PnormFwdArgs a{};
-    bool aligned = rp.aligned;
-    if (!map_rows(x, x_batch_stride, x_row_stride, B, M, K, rp.bytes, &a.xmap, &aligned)) return THN_E_SHAPE;
-    if (normalize && !map_rows(y, y_batch_stride, y_row_stride, B, M, K, rp.bytes, &a.ymap, &aligned)) return THN_E_SHAPE;
+    bool aligned = rp.aligned, uniform = true;
+    if (!map_rows(x, x_batch_stride, x_row_stride, B, M, K, rp.bytes, &a.xmap, &aligned, &uniform)) return THN_E_SHAPE;
+    if (normalize && !map_rows(y, y_batch_stride, y_row_stride, B, M, K, rp.bytes, &a.ymap, &aligned, &uniform)) {
+        return THN_E_SHAPE;
+    }
     a.x = static_cast<const char*>(x);
     a.y = static_cast<char*>(y);
     a.norms = norms;
@@ -386,9 +393,11 @@ int pnorm_forward(const void* x, int64_t x_batch_stride, int64_t x_row_stride, v
         const int rc = plan_launch(kPnormFwd, variant, aligned, rp.rows, K, dtype, &plan);
         if (rc != THN_OK) return rc;
         a.n_vecs = plan.n_vecs;
+        a.walk = make_walk(uniform, M, rp.rows, static_cast<int64_t>(plan.grid) * (plan.s.block / plan.s.tpr));
         lrc = launch_pnorm_fwd(dtype, variant, aligned, plan.s, a, plan.grid, st, nullptr);
     } else {
         const int grid = loop_grid(rp.rows);
+        a.walk = make_walk(uniform, M, rp.rows, grid);
         switch (dtype) {
             case THN_F32: lrc = thn::launch_pnorm_fwd_loop_f32(normalize, a, grid, st); break;
             case THN_F16: lrc = thn::launch_pnorm_fwd_loop_f16(normalize, a, grid, st); break;
@@ -695,9 +704,9 @@ int thn_pnorm_bwd(const void* x, int64_t x_batch_stride, int64_t x_row_stride, c
     if (x == nullptr || dnorms == nullptr || dx == nullptr || (norms == nullptr && p != 1.0f)) return THN_E_NULL;
     if (current_cu_count() <= 0) return THN_E_DEVICE;
     PnormBwdArgs a{};
-    bool aligned = rp.aligned;
-    if (!map_rows(x, x_batch_stride, x_row_stride, B, M, K, rp.bytes, &a.xmap, &aligned)) return THN_E_SHAPE;
-    if (!map_rows(dx, dx_batch_stride, dx_row_stride, B, M, K, rp.bytes, &a.dxmap, &aligned)) return THN_E_SHAPE;
+    bool aligned = rp.aligned, uniform = true;
+    if (!map_rows(x, x_batch_stride, x_row_stride, B, M, K, rp.bytes, &a.xmap, &aligned, &uniform)) return THN_E_SHAPE;
+    if (!map_rows(dx, dx_batch_stride, dx_row_stride, B, M, K, rp.bytes, &a.dxmap, &aligned, &uniform)) return THN_E_SHAPE;
     a.x = static_cast<const char*>(x);
     a.norms = norms;
     a.g = dnorms;
@@ -715,9 +724,11 @@ int thn_pnorm_bwd(const void* x, int64_t x_batch_stride, int64_t x_row_stride, c
         const int rc = plan_launch(kPnormBwd, mode, aligned, rp.rows, K, dtype, &plan);
         if (rc != THN_OK) return rc;
         a.n_vecs = plan.n_vecs;
+        a.walk = make_walk(uniform, M, rp.rows, static_cast<int64_t>(plan.grid) * (plan.s.block / plan.s.tpr));
         lrc = launch_pnorm_bwd(dtype, mode, aligned, plan.s, a, plan.grid, st, nullptr);
     } else {
         const int grid = loop_grid(rp.rows);
+        a.walk = make_walk(uniform, M, rp.rows, grid);
         switch (dtype) {
             case THN_F32: lrc = thn::launch_pnorm_bwd_loop_f32(a, grid, st); break;
             case THN_F16: lrc = thn::launch_pnorm_bwd_loop_f16(a, grid, st); break;
@@ -744,11 +755,11 @@ int thn_normalize_bwd(const void* x, int64_t x_batch_stride, int64_t x_row_strid
     }
     if (current_cu_count() <= 0) return THN_E_DEVICE;
     NormalizeBwdArgs a{};
-    bool aligned = rp.aligned;
-    if (need_x && !map_rows(x, x_batch_stride, x_row_stride, B, M, K, rp.bytes, &a.xmap, &aligned)) return THN_E_SHAPE;
-    if (need_y && !map_rows(y, y_batch_stride, y_row_stride, B, M, K, rp.bytes, &a.ymap, &aligned)) return THN_E_SHAPE;
-    if (!map_rows(dy, dy_batch_stride, dy_row_stride, B, M, K, rp.bytes, &a.gmap, &aligned)) return THN_E_SHAPE;
-    if (!map_rows(dx, dx_batch_stride, dx_row_stride, B, M, K, rp.bytes, &a.dxmap, &aligned)) return THN_E_SHAPE;
+    bool aligned = rp.aligned, uniform = true;
+    if (need_x && !map_rows(x, x_batch_stride, x_row_stride, B, M, K, rp.bytes, &a.xmap, &aligned, &uniform)) return THN_E_SHAPE;
+    if (need_y && !map_rows(y, y_batch_stride, y_row_stride, B, M, K, rp.bytes, &a.ymap, &aligned, &uniform)) return THN_E_SHAPE;
+    if (!map_rows(dy, dy_batch_stride, dy_row_stride, B, M, K, rp.bytes, &a.gmap, &aligned, &uniform)) return THN_E_SHAPE;
+    if (!map_rows(dx, dx_batch_stride, dx_row_stride, B, M, K, rp.bytes, &a.dxmap, &aligned, &uniform)) return THN_E_SHAPE;
     a.x = static_cast<const char*>(need_x ? x : dy);         // never dereferenced when not needed
     a.y = static_cast<const char*>(need_y ? y : dy);
     if (!need_x) a.xmap = a.gmap;
@@ -769,9 +780,11 @@ int thn_normalize_bwd(const void* x, int64_t x_batch_stride, int64_t x_row_strid
         const int rc = plan_launch(kNormalizeBwd, mode, aligned, rp.rows, K, dtype, &plan);
         if (rc != THN_OK) return rc;
         a.n_vecs = plan.n_vecs;
+        a.walk = make_walk(uniform, M, rp.rows, static_cast<int64_t>(plan.grid) * (plan.s.block / plan.s.tpr));
         lrc = launch_normalize_bwd(dtype, mode, aligned, plan.s, a, plan.grid, st, nullptr);
     } else {
         const int grid = loop_grid(rp.rows);
+        a.walk = make_walk(uniform, M, rp.rows, grid);
         switch (dtype) {
             case THN_F32: lrc = thn::launch_normalize_bwd_loop_f32(a, grid, st); break;
             case THN_F16: lrc = thn::launch_normalize_bwd_loop_f16(a, grid, st); break;

@@ -22,19 +22,57 @@
 
 namespace thn {
 
-// Address of row r of a (B, M, K) tensor with element-contiguous rows.  rows_per_batch == 0: the batch and row
-// strides collapse into one (batch_stride == M * row_stride), the common case.
+// Addressing of the rows of a (B, M, K) tensor with element-contiguous rows.  Row r is (batch r / rows_per_batch,
+// row r % rows_per_batch) and sits at batch*batch_stride + row*row_stride.  When every operand of a launch has
+// batch_stride == M*row_stride the host folds the batches away (rows_per_batch = B*M, one "batch").
+// The row kernels never divide inside their loop: each row group keeps a (batch, row) cursor and advances it by
+// the launch-uniform grid stride, split by the host into (step_batch, step_row) -- a division, or a branch
+// around one, inside the loop would cost the loop its precise memory waits (see thn_kernels.h).
 struct RowMap {
     int64_t batch_stride_bytes;
     int64_t row_stride_bytes;
-    uint32_t rows_per_batch;
 };
 
-__device__ __forceinline__ int64_t row_offset(const RowMap& m, int64_t r) {
-    if (m.rows_per_batch == 0) return r * m.row_stride_bytes;
-    const uint32_t r32 = static_cast<uint32_t>(r);          // the host refuses B*M >= 2^31 for such layouts
-    const uint32_t b = r32 / m.rows_per_batch;
-    return b * m.batch_stride_bytes + (r32 - b * m.rows_per_batch) * m.row_stride_bytes;
+struct RowWalk {
+    int64_t rows_per_batch;
+    int64_t step_batch;     // (gridDim.x * G) / rows_per_batch
+    int64_t step_row;       // (gridDim.x * G) % rows_per_batch
+};
+
+struct RowCursor {
+    int64_t b, m;
+    __device__ __forceinline__ void init(const RowWalk& w, int64_t row) {
+        b = row / w.rows_per_batch;
+        m = row - b * w.rows_per_batch;
+    }
+    __device__ __forceinline__ void advance(const RowWalk& w) {
+        m += w.step_row;
+        b += w.step_batch;
+        const bool carry = m >= w.rows_per_batch;
+        m -= carry ? w.rows_per_batch : 0;
+        b += carry ? 1 : 0;
+    }
+};
+
+__device__ __forceinline__ int64_t row_offset(const RowMap& map, const RowCursor& c) {
+    return c.b * map.batch_stride_bytes + c.m * map.row_stride_bytes;
+}
+
+// The cursor of the next row, or of the tensor's last row when the row group has run past the end (slots without
+// work mirror the last row).  A select on the two small integers, not on the offsets: selecting between a computed
+// offset and a constant makes the compiler branch around the multiplications.
+__device__ __forceinline__ RowCursor clamp_cursor(const RowCursor& c, const RowCursor& last, bool in_range) {
+    RowCursor r;
+    r.b = in_range ? c.b : last.b;
+    r.m = in_range ? c.m : last.m;
+    return r;
+}
+
+// For the looping kernels, which may divide.
+__device__ __forceinline__ int64_t row_offset(const RowMap& map, const RowWalk& w, int64_t r) {
+    RowCursor c;
+    c.init(w, r);
+    return row_offset(map, c);
 }
 
 enum : int { kP1 = 1, kP2 = 2, kPInt = 3 };   // MODE of the row-engine kernels; kPInt: p in {3, 4, 5, 6}
@@ -44,6 +82,7 @@ struct PnormFwdArgs {
     char* y;            // normalize only
     void* norms;        // (rows,) storage type
     RowMap xmap, ymap;
+    RowWalk walk;
     int64_t rows;
     int64_t n_cols64;   // looping kernels
     int n_cols;
@@ -59,6 +98,7 @@ struct PnormBwdArgs {
     const void* g;      // (rows,) storage type: upstream gradient of the norms
     char* dx;
     RowMap xmap, dxmap;
+    RowWalk walk;
     int64_t rows;
     int64_t n_cols64;
     int n_cols;
@@ -74,6 +114,7 @@ struct NormalizeBwdArgs {
     const char* g;      // upstream gradient of y, (B, M, K)
     char* dx;
     RowMap xmap, ymap, gmap, dxmap;
+    RowWalk walk;
     int64_t rows;
     int64_t n_cols64;
     int n_cols;
@@ -128,11 +169,21 @@ __device__ __forceinline__ float norm_term(float x, int p_int) {
     else return pow_small(__builtin_fabsf(x), p_int);
 }
 
+// acc^(1/p) for integer p in [3, 6]: the hardware log2 / exp2 give the root to a few float32 ulp, one Newton step
+// on r^p = acc (r^p by multiplication) brings it to about 1 ulp, at a tenth of the instructions of powf -- every
+// thread of a row evaluates this once per row.
+__device__ __forceinline__ float root_small(float acc, int p_int, float p) {
+    const float r = __builtin_amdgcn_exp2f(__builtin_amdgcn_logf(acc) / p);
+    const float rp1 = pow_small(r, p_int - 1);                     // r^(p-1)
+    const float better = r - (rp1 * r - acc) / (p * rp1);
+    return acc > 0.0f && acc < 3.0e38f && rp1 > 0.0f ? better : (acc > 0.0f ? powf(acc, 1.0f / p) : 0.0f);
+}
+
 template <int MODE>
-__device__ __forceinline__ float norm_root(float acc, float p) {
+__device__ __forceinline__ float norm_root(float acc, int p_int, float p) {
     if constexpr (MODE == kP1) return acc;
     else if constexpr (MODE == kP2) return sqrtf(acc);
-    else return powf(acc, 1.0f / p);
+    else return root_small(acc, p_int, p);
 }
 
 // ---------------------------------------------------------------------------------------------------
@@ -165,15 +216,23 @@ __global__ void __launch_bounds__(BLOCK) pnorm_fwd_kernel(const PnormFwdArgs a) 
     const int64_t last_row = a.rows - 1;
     int64_t row_raw = static_cast<int64_t>(blockIdx.x) * G + g;
     int64_t row = row_raw < a.rows ? row_raw : last_row;
+    RowCursor cursor;
+    cursor.init(a.walk, row);
+    RowCursor last;
+    last.init(a.walk, last_row);
+    int64_t y_off = NORMALIZE ? row_offset(a.ymap, cursor) : 0;
     u32x4 cur[K];
-    load_row<T, K, ALIGNED>(cur, a.x + row_offset(a.xmap, row), 0, 0, voff, a.n_cols);
+    load_row<T, K, ALIGNED>(cur, a.x + row_offset(a.xmap, cursor), 0, 0, voff, a.n_cols);
 
     drain_vector_memory();
     for (int64_t base = static_cast<int64_t>(blockIdx.x) * G; base < a.rows; base += rows_per_iter) {
         const int64_t nrow_raw = row_raw + rows_per_iter;
-        const int64_t nrow = nrow_raw < a.rows ? nrow_raw : last_row;
+        const bool more = nrow_raw < a.rows;
+        const int64_t nrow = more ? nrow_raw : last_row;
+        cursor.advance(a.walk);
+        const RowCursor ncur = clamp_cursor(cursor, last, more);
         u32x4 nxt[K];
-        load_row<T, K, ALIGNED>(nxt, a.x + row_offset(a.xmap, nrow), 0, 0, voff, a.n_cols);
+        load_row<T, K, ALIGNED>(nxt, a.x + row_offset(a.xmap, ncur), 0, 0, voff, a.n_cols);
 
         float xf[K][VEC];
         float s[1] = {0.0f};
@@ -186,14 +245,14 @@ __global__ void __launch_bounds__(BLOCK) pnorm_fwd_kernel(const PnormFwdArgs a) 
             s[0] += own[k] ? sk : 0.0f;
         }
         row_allreduce<TPR, G, 1>(s, red, phase, g, t);
-        const float n = fmaxf(norm_root<MODE>(s[0], a.p), a.eps);
+        const float n = fmaxf(norm_root<MODE>(s[0], a.p_int, a.p), a.eps);
         // Every thread of the row stores the same value to the same address (one request per wave).
         T::store1(a.norms, row, n);
 
         if constexpr (NORMALIZE) {
             const float nr = round_to_storage<T>(n);
             const float rn = 1.0f / nr;
-            char* yrow = a.y + row_offset(a.ymap, row);
+            char* yrow = a.y + y_off;
 #pragma unroll
             for (int k = 0; k < K; ++k) {
                 float yf[VEC];
@@ -201,6 +260,7 @@ __global__ void __launch_bounds__(BLOCK) pnorm_fwd_kernel(const PnormFwdArgs a) 
                 for (int e = 0; e < VEC; ++e) yf[e] = div_by_row(xf[k][e], nr, rn);
                 store_row_vec<T, ALIGNED>(yrow, voff[k], a.n_cols, yf);
             }
+            y_off = row_offset(a.ymap, ncur);
         }
 
 #pragma unroll
@@ -235,24 +295,33 @@ __global__ void __launch_bounds__(BLOCK) pnorm_bwd_kernel(const PnormBwdArgs a) 
     const int64_t last_row = a.rows - 1;
     int64_t row_raw = static_cast<int64_t>(blockIdx.x) * G + g;
     int64_t row = row_raw < a.rows ? row_raw : last_row;
+    RowCursor cursor;
+    cursor.init(a.walk, row);
+    RowCursor last;
+    last.init(a.walk, last_row);
+    int64_t dx_off = row_offset(a.dxmap, cursor);
     u32x4 cur[K];
-    load_row<T, K, ALIGNED>(cur, a.x + row_offset(a.xmap, row), 0, 0, voff, a.n_cols);
+    load_row<T, K, ALIGNED>(cur, a.x + row_offset(a.xmap, cursor), 0, 0, voff, a.n_cols);
     float c_n = MODE == kP1 ? 1.0f : T::load1(a.norms, row);
     float c_g = T::load1(a.g, row);
 
     drain_vector_memory();
     for (int64_t base = static_cast<int64_t>(blockIdx.x) * G; base < a.rows; base += rows_per_iter) {
         const int64_t nrow_raw = row_raw + rows_per_iter;
-        const int64_t nrow = nrow_raw < a.rows ? nrow_raw : last_row;
+        const bool more = nrow_raw < a.rows;
+        const int64_t nrow = more ? nrow_raw : last_row;
+        cursor.advance(a.walk);
+        const RowCursor ncur = clamp_cursor(cursor, last, more);
         u32x4 nxt[K];
-        load_row<T, K, ALIGNED>(nxt, a.x + row_offset(a.xmap, nrow), 0, 0, voff, a.n_cols);
+        load_row<T, K, ALIGNED>(nxt, a.x + row_offset(a.xmap, ncur), 0, 0, voff, a.n_cols);
         const float n_n = MODE == kP1 ? 1.0f : T::load1(a.norms, nrow);
         const float n_g = T::load1(a.g, nrow);
 
         float den = c_n;
         if constexpr (MODE == kPInt) den = pow_small(c_n, a.p_int - 1);     // norms^(p-1), norm.py:86-87
         const float rden = 1.0f / den;
-        char* dxrow = a.dx + row_offset(a.dxmap, row);
+        char* dxrow = a.dx + dx_off;
+        dx_off = row_offset(a.dxmap, ncur);
 #pragma unroll
         for (int k = 0; k < K; ++k) {
             float xf[VEC], df[VEC];
@@ -308,20 +377,28 @@ __global__ void __launch_bounds__(BLOCK) normalize_bwd_kernel(const NormalizeBwd
     const int64_t last_row = a.rows - 1;
     int64_t row_raw = static_cast<int64_t>(blockIdx.x) * G + g;
     int64_t row = row_raw < a.rows ? row_raw : last_row;
+    RowCursor cursor;
+    cursor.init(a.walk, row);
+    RowCursor last;
+    last.init(a.walk, last_row);
+    int64_t dx_off = row_offset(a.dxmap, cursor);
     u32x4 cx[NEED_X ? K : 1], cy[NEED_Y ? K : 1], cg[K];
-    if constexpr (NEED_X) load_row<T, K, ALIGNED>(cx, a.x + row_offset(a.xmap, row), 0, 0, voff, a.n_cols);
-    if constexpr (NEED_Y) load_row<T, K, ALIGNED>(cy, a.y + row_offset(a.ymap, row), 0, 0, voff, a.n_cols);
-    load_row<T, K, ALIGNED>(cg, a.g + row_offset(a.gmap, row), 0, 0, voff, a.n_cols);
+    if constexpr (NEED_X) load_row<T, K, ALIGNED>(cx, a.x + row_offset(a.xmap, cursor), 0, 0, voff, a.n_cols);
+    if constexpr (NEED_Y) load_row<T, K, ALIGNED>(cy, a.y + row_offset(a.ymap, cursor), 0, 0, voff, a.n_cols);
+    load_row<T, K, ALIGNED>(cg, a.g + row_offset(a.gmap, cursor), 0, 0, voff, a.n_cols);
     float c_n = T::load1(a.norms, row);
 
     drain_vector_memory();
     for (int64_t base = static_cast<int64_t>(blockIdx.x) * G; base < a.rows; base += rows_per_iter) {
         const int64_t nrow_raw = row_raw + rows_per_iter;
-        const int64_t nrow = nrow_raw < a.rows ? nrow_raw : last_row;
+        const bool more = nrow_raw < a.rows;
+        const int64_t nrow = more ? nrow_raw : last_row;
+        cursor.advance(a.walk);
+        const RowCursor ncur = clamp_cursor(cursor, last, more);
         u32x4 nx[NEED_X ? K : 1], ny[NEED_Y ? K : 1], ng[K];
-        if constexpr (NEED_X) load_row<T, K, ALIGNED>(nx, a.x + row_offset(a.xmap, nrow), 0, 0, voff, a.n_cols);
-        if constexpr (NEED_Y) load_row<T, K, ALIGNED>(ny, a.y + row_offset(a.ymap, nrow), 0, 0, voff, a.n_cols);
-        load_row<T, K, ALIGNED>(ng, a.g + row_offset(a.gmap, nrow), 0, 0, voff, a.n_cols);
+        if constexpr (NEED_X) load_row<T, K, ALIGNED>(nx, a.x + row_offset(a.xmap, ncur), 0, 0, voff, a.n_cols);
+        if constexpr (NEED_Y) load_row<T, K, ALIGNED>(ny, a.y + row_offset(a.ymap, ncur), 0, 0, voff, a.n_cols);
+        load_row<T, K, ALIGNED>(ng, a.g + row_offset(a.gmap, ncur), 0, 0, voff, a.n_cols);
         const float n_n = T::load1(a.norms, nrow);
 
         float xf[NEED_X ? K : 1][VEC], yf[NEED_Y ? K : 1][VEC], gf[K][VEC];
@@ -347,7 +424,8 @@ __global__ void __launch_bounds__(BLOCK) normalize_bwd_kernel(const NormalizeBwd
         if constexpr (MODE == kP1) coef = proj / (n * n);                                     // normalize.py:106
         if constexpr (MODE == kPInt) coef = proj / (pow_small(n, a.p_int - 1) * n);           // normalize.py:115
 
-        char* dxrow = a.dx + row_offset(a.dxmap, row);
+        char* dxrow = a.dx + dx_off;
+        dx_off = row_offset(a.dxmap, ncur);
 #pragma unroll
         for (int k = 0; k < K; ++k) {
             float df[VEC];
@@ -400,7 +478,7 @@ __global__ void __launch_bounds__(kLoopBlock) pnorm_fwd_loop_kernel(const PnormF
     int phase = 0;
     const int t = threadIdx.x;
     for (int64_t row = blockIdx.x; row < a.rows; row += gridDim.x) {
-        const char* xrow = a.x + row_offset(a.xmap, row);
+        const char* xrow = a.x + row_offset(a.xmap, a.walk, row);
         float s[1] = {0.0f};
         for (int64_t c = t; c < a.n_cols64; c += kLoopBlock) {
             const float x = T::load1(xrow, c);
@@ -414,7 +492,7 @@ __global__ void __launch_bounds__(kLoopBlock) pnorm_fwd_loop_kernel(const PnormF
         if (t == 0) T::store1(a.norms, row, n);
         if constexpr (NORMALIZE) {
             const float nr = round_to_storage<T>(n);
-            char* yrow = a.y + row_offset(a.ymap, row);
+            char* yrow = a.y + row_offset(a.ymap, a.walk, row);
             for (int64_t c = t; c < a.n_cols64; c += kLoopBlock) T::store1(yrow, c, T::load1(xrow, c) / nr);
         }
     }
@@ -424,8 +502,8 @@ template <typename T>
 __global__ void __launch_bounds__(kLoopBlock) pnorm_bwd_loop_kernel(const PnormBwdArgs a) {
     const int t = threadIdx.x;
     for (int64_t row = blockIdx.x; row < a.rows; row += gridDim.x) {
-        const char* xrow = a.x + row_offset(a.xmap, row);
-        char* dxrow = a.dx + row_offset(a.dxmap, row);
+        const char* xrow = a.x + row_offset(a.xmap, a.walk, row);
+        char* dxrow = a.dx + row_offset(a.dxmap, a.walk, row);
         const float g = T::load1(a.g, row);
         float den = 1.0f;
         if (a.p_int != 1) {
@@ -450,10 +528,10 @@ __global__ void __launch_bounds__(kLoopBlock) normalize_bwd_loop_kernel(const No
     const int t = threadIdx.x;
     const int e_int = a.p_int > 0 ? a.p_int - 1 : -1;
     for (int64_t row = blockIdx.x; row < a.rows; row += gridDim.x) {
-        const char* xrow = a.x + row_offset(a.xmap, row);
-        const char* yrow = a.y + row_offset(a.ymap, row);
-        const char* grow = a.g + row_offset(a.gmap, row);
-        char* dxrow = a.dx + row_offset(a.dxmap, row);
+        const char* xrow = a.x + row_offset(a.xmap, a.walk, row);
+        const char* yrow = a.y + row_offset(a.ymap, a.walk, row);
+        const char* grow = a.g + row_offset(a.gmap, a.walk, row);
+        char* dxrow = a.dx + row_offset(a.dxmap, a.walk, row);
         const float n = T::load1(a.norms, row);
         float s[1] = {0.0f};
         for (int64_t c = t; c < a.n_cols64; c += kLoopBlock) {
