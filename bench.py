@@ -66,6 +66,8 @@ MEASURED_TRAFFIC_BYTES = {
     "rmsnorm_bf16_16384x4096": 407669153,
     # profiles/softmax_kernels_softmax_bf16_16384x4096_stats_and_hbm_counters.txt (softmax_bwd_kernel)
     "softmax_bf16_16384x4096": 402815465,
+    # profiles/pnorm_kernels_normalize_p2_bf16_16384x4096_stats_and_hbm_counters.txt (normalize_bwd_kernel)
+    "normalize_p2_bf16_16384x4096": 403121728,
 }
 
 
