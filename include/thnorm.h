@@ -1,6 +1,7 @@
 /*
- * thnorm.h -- C ABI of libthnorm.so: LayerNorm / RMSNorm, and the row reductions next to them (Softmax /
- * Softmin / LogSoftmax, row p-norm / normalize), forward and backward, for AMD MI355X (gfx950).
+ * thnorm.h -- C ABI of libthnorm.so: LayerNorm / RMSNorm, the row reductions next to them (Softmax / Softmin /
+ * LogSoftmax, row p-norm / normalize) and the element-wise activations, forward and backward, for AMD MI355X
+ * (gfx950).
  *
  * The reference library (TritonHub) has no native boundary: its last host frames before device code are the
  * Python launch sites in TritonHub/Normalization/layernorm.py and rmsnorm.py (and TritonHub/Activations/
@@ -29,7 +30,7 @@
 extern "C" {
 #endif
 
-#define THN_ABI_VERSION 3
+#define THN_ABI_VERSION 4
 
 enum thn_dtype { THN_F32 = 0, THN_F16 = 1, THN_BF16 = 2, THN_F64 = 3 };
 
@@ -192,10 +193,54 @@ int thn_normalize_bwd(const void* x, int64_t x_batch_stride, int64_t x_row_strid
                       int64_t B, int64_t M, int64_t K, float p, int dtype, void* stream);
 
 /*
+ * Element-wise activations (the reference's TritonHub/Activations/gelu.py, silu.py, relu.py, leaky_relu.py,
+ * relu6.py, sigmoid.py, tanh.py, mish.py, softplus.py, threshold.py).  (M, N) row-major, unit column stride, row
+ * strides in ELEMENTS; one storage code for all tensors; no row-width limit.  `out` must not alias an input.
+ *
+ * thn_act_fwd replaces the `_<name>_kernel_fwd[grid](...)` launches (gelu.py:45, silu.py:35, relu.py:35,
+ * leaky_relu.py:36, relu6.py:36, sigmoid.py:35, tanh.py:37, mish.py:39, softplus.py:37, threshold.py:36);
+ * thn_act_bwd the `_<name>_kernel_bwd[grid](...)` launches (gelu.py:100, silu.py:76, relu.py:75,
+ * leaky_relu.py:78, relu6.py:77, sigmoid.py:75, tanh.py:77, mish.py:85, softplus.py:81, threshold.py:78).
+ *   THN_ACT_GELU        y = 0.5*x*(1 + erf(x/sqrt 2));                    dx = dy*(cdf + x*pdf)
+ *   THN_ACT_GELU_TANH   y = 0.5*x*(1 + tanh(sqrt(2/pi)*(x + 0.044715 x^3))); dx as gelu.py:71-75
+ *   THN_ACT_SILU        y = x*sigmoid(x);                                 dx = dy*(s*(1 + x*(1 - s)))
+ *   THN_ACT_RELU        y = x > 0 ? x : 0;                                dx = x > 0 ? dy : 0
+ *   THN_ACT_LEAKY_RELU  y = x > 0 ? x : param0*x;                         dx = x > 0 ? dy : param0*dy
+ *   THN_ACT_RELU6       y = min(max(x, 0), 6);                            dx = 0 < x < 6 ? dy : 0
+ *   THN_ACT_SIGMOID     y = 1/(1 + exp(-x));                              dx = dy*y*(1 - y)      (saved: OUTPUT)
+ *   THN_ACT_TANH        y = tanh(x);                                      dx = dy*(1 - y*y)      (saved: OUTPUT)
+ *   THN_ACT_MISH        y = x*tanh(softplus(x));                          dx as mish.py:60-66
+ *   THN_ACT_SOFTPLUS    y = x*param0 > param1 ? x : log(1 + exp(param0*x))/param0   (param0 = beta, param1 = threshold)
+ *                       dx = x*param0 > param1 ? dy : dy/(1 + exp(-param0*x))
+ *   THN_ACT_THRESHOLD   y = x > param0 ? x : param1;                      dx = x > param0 ? dy : 0
+ * `saved` of thn_act_bwd is what the reference's Function saves: the forward's input, or its OUTPUT for
+ * THN_ACT_SIGMOID and THN_ACT_TANH (sigmoid.py:81-92, tanh.py:83-94).
+ * Arithmetic is float32, except RELU / LEAKY_RELU / RELU6 / SOFTPLUS / THRESHOLD on THN_F64 storage, which the
+ * reference computes in the loaded type (no `.to(tl.float32)`, relu.py:18): float64 there.  Where the
+ * reference's tanh-as-exponentials overflows to NaN for large |x| (tanh.py:19-21, mish.py:20-22, gelu.py:24-25)
+ * the same function is evaluated in a form that cannot overflow.
+ */
+enum thn_act {
+    THN_ACT_GELU = 0, THN_ACT_GELU_TANH = 1, THN_ACT_SILU = 2, THN_ACT_RELU = 3, THN_ACT_LEAKY_RELU = 4,
+    THN_ACT_RELU6 = 5, THN_ACT_SIGMOID = 6, THN_ACT_TANH = 7, THN_ACT_MISH = 8, THN_ACT_SOFTPLUS = 9,
+    THN_ACT_THRESHOLD = 10
+};
+
+int thn_act_fwd(const void* x, int64_t x_row_stride,
+                void* y, int64_t y_row_stride,
+                int64_t M, int64_t N, int act, float param0, float param1, int dtype, void* stream);
+
+int thn_act_bwd(const void* saved, int64_t saved_row_stride,
+                const void* dy, int64_t dy_row_stride,
+                void* dx, int64_t dx_row_stride,
+                int64_t M, int64_t N, int act, float param0, float param1, int dtype, void* stream);
+
+/*
  * Launch-shape control for tuning sweeps (the counterpart of the reference's `triton.autotune` over
  * num_warps, autotune.py:62-65, which this library replaces by a fixed heuristic on N and the dtype).
  * `which`: 0 = norm forward, 1 = norm backward, 2 = softmax forward, 3 = softmax backward, 4 = p-norm /
- * normalize forward, 5 = p-norm backward, 6 = normalize backward.
+ * normalize forward, 5 = p-norm backward, 6 = normalize backward, 7 / 8 = element-wise activation forward /
+ * backward (only blocks_per_cu applies to them; thn_norm_query_launch does not cover them).
  * vecs_per_thread / threads_per_row / block_threads select a compiled kernel shape, blocks_per_cu caps the
  * persistent grid; 0 for any field keeps the heuristic's choice.
  * Process-wide; meant for benchmarks, not for concurrent production use.  Returns THN_E_SHAPE when no

@@ -25,7 +25,7 @@ def declared_functions():
 
 def test_library_exports_every_declared_symbol():
     names = declared_functions()
-    assert len(names) == 15 and "thn_pnorm_fwd" in names and "thn_normalize_bwd" in names and "thn_norm_fwd" in names and "thn_norm_bwd" in names and "thn_softmax_fwd" in names
+    assert len(names) == 17 and "thn_act_fwd" in names and "thn_pnorm_fwd" in names and "thn_normalize_bwd" in names and "thn_norm_fwd" in names and "thn_norm_bwd" in names and "thn_softmax_fwd" in names
     handle = ctypes.CDLL(_native.LIB_PATH)
     for name in names:
         assert hasattr(handle, name), f"{name} is declared in include/thnorm.h but not exported"
@@ -59,7 +59,7 @@ def test_argument_checks_answer_without_a_gpu():
     assert lib.thn_norm_bwd_workspace_bytes(4, 40000, 1, 1, _native.F16) == _native.E_FEATURE_DIM
     assert lib.thn_norm_bwd_workspace_bytes(4, 128, 0, 0, _native.F32) == 0
     assert lib.thn_norm_bwd_workspace_bytes(0, 128, 1, 1, _native.F32) == 0
-    assert lib.thn_norm_set_launch_override(7, 0, 0, 0, 0) == _native.E_SHAPE
+    assert lib.thn_norm_set_launch_override(9, 0, 0, 0, 0) == _native.E_SHAPE
     assert lib.thn_norm_set_launch_override(0, 0, 0, 0, 0) == _native.OK
     if not torch.cuda.is_available():
         assert lib.thn_norm_bwd_workspace_bytes(4, 128, 1, 1, _native.F32) == _native.E_DEVICE
@@ -109,6 +109,47 @@ def test_pnorm_argument_checks_answer_without_a_gpu():
         assert call(2, 3, 8, 3.0, _native.F32) == _native.E_NULL
 
 
+def test_act_argument_checks_answer_without_a_gpu():
+    lib = _native.lib()
+    fwd = lambda m, n, act, dt: lib.thn_act_fwd(0, n, 0, n, m, n, act, 0.0, 0.0, dt, 0)
+    bwd = lambda m, n, act, dt: lib.thn_act_bwd(0, n, 0, n, 0, n, m, n, act, 0.0, 0.0, dt, 0)
+    for call in (fwd, bwd):
+        assert call(4, 128, 0, 6) == _native.E_DTYPE
+        assert call(4, 128, 11, _native.F32) == _native.E_SHAPE and call(4, 128, -1, _native.F32) == _native.E_SHAPE
+        assert call(4, 0, 0, _native.F32) == _native.E_SHAPE and call(-1, 8, 0, _native.F32) == _native.E_SHAPE
+        assert call(0, 128, 3, _native.F16) == _native.OK
+        assert call(4, 1 << 20, 3, _native.F32) == _native.E_NULL        # no row-width limit
+    assert [_native.ACT_GELU, _native.ACT_GELU_TANH, _native.ACT_SILU, _native.ACT_RELU, _native.ACT_LEAKY_RELU,
+            _native.ACT_RELU6, _native.ACT_SIGMOID, _native.ACT_TANH, _native.ACT_MISH, _native.ACT_SOFTPLUS,
+            _native.ACT_THRESHOLD] == list(range(11))                   # enum thn_act
+    header = open(HEADER).read()
+    for i, name in enumerate(["GELU", "GELU_TANH", "SILU", "RELU", "LEAKY_RELU", "RELU6", "SIGMOID", "TANH", "MISH",
+                              "SOFTPLUS", "THRESHOLD"]):
+        assert re.search(rf"THN_ACT_{name} = {i}\b", header)
+
+
+def test_activation_callables_match_the_reference_constructors():
+    A = Activations
+    assert A.GeLU().approximate == "none" and A.GeLU("tanh").gelu_fn is not None        # gelu.py:122-127
+    with pytest.raises(AssertionError, match="GeLU approximate must be either none or tanh"):
+        A.GeLU("fast")
+    assert A.LeakyReLU().negative_slope == 0.01 and A.LeakyReLU(0.2).leakyrelu_fn is not None     # leaky_relu.py:100-102
+    sp = A.Softplus()
+    assert (sp.beta, sp.threshold) == (1.0, 20) and sp.softplus_fn is not None         # softplus.py:105-108
+    th = A.Threshold(0.5, -1.0)
+    assert (th.threshold, th.value) == (0.5, -1.0) and th.threshold_fn is not None     # threshold.py:103-106
+    with pytest.raises(TypeError):
+        A.Threshold()                                                                  # both arguments are required
+    for cls, attr in ((A.SiLU, "silu_fn"), (A.ReLU, "relu_fn"), (A.ReLU6, "relu6_fn"), (A.Sigmoid, "sigmoid_fn"),
+                      (A.Tanh, "tanh_fn"), (A.Mish, "mish_fn")):
+        assert getattr(cls(), attr) is not None
+    x = torch.randn(3, 16)
+    for mod in (A.GeLU(), A.GeLU("tanh"), A.SiLU(), A.ReLU(), A.LeakyReLU(), A.ReLU6(), A.Sigmoid(), A.Tanh(), A.Mish(),
+                A.Softplus(), A.Threshold(0.1, 0.0)):
+        with pytest.raises(RuntimeError, match="no CPU fallback"):
+            mod(x)
+
+
 def test_ops_surface_matches_the_reference():
     from TritonHub import Ops
     from TritonHub.Ops.norm import Norm
@@ -147,7 +188,8 @@ def test_package_surface():
     assert TritonHub.__version__ == "1.1.1"
     # the row-reduction activations of TritonHub/Activations/__init__.py (softmax.py:99-103, softmin.py:99-103,
     # logsoftmax.py:106-110): plain callables holding the Function's apply
-    assert Activations.__all__ == ["Softmax", "Softmin", "LogSoftmax"]
+    assert Activations.__all__ == ['GeLU', 'SiLU', 'ReLU', 'LeakyReLU', 'Softmax', 'Softplus', 'Tanh', 'Softmin', 'Sigmoid',
+                                   'Mish', 'ReLU6', 'Threshold', 'LogSoftmax']      # Activations/__init__.py:15
     from TritonHub.Activations.logsoftmax import logsoftmax
     from TritonHub.Activations.softmax import softmax
     from TritonHub.Activations.softmin import softmin

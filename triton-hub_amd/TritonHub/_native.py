@@ -17,6 +17,8 @@ LIB_PATH = os.path.join(_HERE, 'libthnorm.so')
 
 F32, F16, BF16, F64 = 0, 1, 2, 3
 SOFTMAX, SOFTMIN, LOGSOFTMAX = 0, 1, 2
+(ACT_GELU, ACT_GELU_TANH, ACT_SILU, ACT_RELU, ACT_LEAKY_RELU, ACT_RELU6, ACT_SIGMOID, ACT_TANH, ACT_MISH, ACT_SOFTPLUS,
+ ACT_THRESHOLD) = range(11)
 DTYPE_CODES = {torch.float32: F32, torch.float16: F16, torch.bfloat16: BF16, torch.float64: F64}
 
 OK = 0
@@ -41,6 +43,8 @@ SYMBOLS = {
     'thn_pnorm_bwd': (_i32, [_vp, _i64, _i64, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _f32, _i32, _vp]),
     'thn_normalize_bwd': (_i32, [_vp, _i64, _i64, _vp, _i64, _i64, _vp, _vp, _i64, _i64, _vp, _i64, _i64,
                                  _i64, _i64, _i64, _f32, _i32, _vp]),
+    'thn_act_fwd': (_i32, [_vp, _i64, _vp, _i64, _i64, _i64, _i32, _f32, _f32, _i32, _vp]),
+    'thn_act_bwd': (_i32, [_vp, _i64, _vp, _i64, _vp, _i64, _i64, _i64, _i32, _f32, _f32, _i32, _vp]),
     'thn_norm_set_launch_override': (_i32, [_i32, _i32, _i32, _i32, _i32]),
     'thn_norm_query_launch': (_i32, [_i32, _i32, _i64, _i64, _i32, ctypes.POINTER(ctypes.c_int32)]),
 }

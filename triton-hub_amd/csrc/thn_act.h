@@ -1,0 +1,240 @@
+// Element-wise activations, forward and backward: GeLU (exact / tanh), SiLU, ReLU, LeakyReLU, ReLU6, Sigmoid,
+// Tanh, Mish, Softplus, Threshold -- the reference's TritonHub/Activations/{gelu,silu,relu,leaky_relu,relu6,
+// sigmoid,tanh,mish,softplus,threshold}.py.  Pure streaming: the forward reads x and writes y (2*s bytes per
+// element), the backward reads the saved tensor and dy and writes dx (3*s bytes per element).
+//
+// Arithmetic type, as in the reference: float32 for the kernels that widen on load (gelu.py:20, silu.py:18,
+// sigmoid.py:18, tanh.py:18, mish.py:18); the loaded type for the others (relu.py:18, leaky_relu.py:19,
+// relu6.py:18, softplus.py:20, threshold.py:19), which for 16-bit storage still means float32 arithmetic with
+// one rounding on store (their float32 scalar arguments promote the expression) and for float64 storage means
+// float64 -- a ReLU of a float64 tensor returns its input bits.
+//
+// Where the reference's formula overflows to NaN for large |x| although the function is finite -- tanh as
+// (e^x - e^-x)/(e^x + e^-x) (tanh.py:19-21, mish.py:20-22), GeLU's tanh as (e^2u - 1)/(e^2u + 1) (gelu.py:24-25)
+// -- the same function is evaluated in a form that cannot overflow; the values agree wherever the reference's
+// are finite.
+#pragma once
+
+#include <type_traits>
+
+#include "thn_kernels.h"
+
+namespace thn {
+
+enum : int {
+    kGelu = 0, kGeluTanh = 1, kSilu = 2, kRelu = 3, kLeakyRelu = 4, kRelu6 = 5, kSigmoid = 6, kTanh = 7, kMish = 8,
+    kSoftplus = 9, kThreshold = 10, kNumActs = 11
+};
+
+constexpr bool act_uses_loaded_type(int act) {
+    return act == kRelu || act == kLeakyRelu || act == kRelu6 || act == kSoftplus || act == kThreshold;
+}
+// Sigmoid and Tanh save their OUTPUT for the backward (sigmoid.py:81-92, tanh.py:83-94); the others their input.
+
+template <typename T, int ACT>
+struct ActCompute {
+    using type = typename std::conditional<T::kBytes == 8 && act_uses_loaded_type(ACT), double, float>::type;
+};
+
+struct ActArgs {
+    const char* x;        // forward: input.  backward: the saved tensor (input, or output for Sigmoid / Tanh)
+    const char* g;        // backward: upstream gradient
+    char* out;            // y, or dx
+    int64_t total_vecs;   // flat kernels: whole 16-byte vectors
+    int64_t total_elems;  // flat kernels
+    int64_t x_stride_bytes, g_stride_bytes, out_stride_bytes;   // row kernels
+    int64_t M, N;         // row kernels
+    float p0, p1;         // negative_slope | beta, threshold | threshold, value
+};
+
+__device__ __forceinline__ float log_c(float z) { return __logf(z); }
+__device__ __forceinline__ double log_c(double z) { return log(z); }
+
+// tanh(u) = sign(u) * (1 - t)/(1 + t) with t = exp(-2|u|): no overflow for any u.
+__device__ __forceinline__ float tanh_safe(float u) {
+    const float t = __expf(-2.0f * __builtin_fabsf(u));
+    const float r = (1.0f - t) / (1.0f + t);
+    return u < 0.0f ? -r : r;
+}
+
+__device__ __forceinline__ float sigmoid_f(float x) { return 1.0f / (1.0f + __expf(-x)); }
+
+// softplus of mish.py:19: x > 20 ? x : log(1 + exp(x))
+__device__ __forceinline__ float mish_softplus(float x) { return x > 20.0f ? x : __logf(1.0f + __expf(x)); }
+
+template <int ACT, typename C>
+__device__ __forceinline__ C act_fwd(C x, C p0, C p1) {
+    if constexpr (ACT == kGelu) {
+        return 0.5f * x * (1.0f + erff(x * 0.70710678118654752440f));                      // gelu.py:28
+    } else if constexpr (ACT == kGeluTanh) {
+        const float u = 0.79788456080286535588f * (x + 0.044715f * x * x * x);            // gelu.py:23
+        return 0.5f * x * (1.0f + tanh_safe(u));                                           // gelu.py:26
+    } else if constexpr (ACT == kSilu) {
+        return x * sigmoid_f(x);                                                           // silu.py:19
+    } else if constexpr (ACT == kRelu) {
+        return x > C(0) ? x : C(0);                                                        // relu.py:19
+    } else if constexpr (ACT == kLeakyRelu) {
+        return x > C(0) ? x : p0 * x;                                                      // leaky_relu.py:20
+    } else if constexpr (ACT == kRelu6) {
+        const C r = x > C(0) ? x : C(0);                                                   // relu6.py:19-20
+        return r < C(6) ? r : C(6);
+    } else if constexpr (ACT == kSigmoid) {
+        return sigmoid_f(x);                                                               // sigmoid.py:19
+    } else if constexpr (ACT == kTanh) {
+        return tanh_safe(x);                                                               // tanh.py:19-21
+    } else if constexpr (ACT == kMish) {
+        return x * tanh_safe(mish_softplus(x));                                            // mish.py:19-23
+    } else if constexpr (ACT == kSoftplus) {
+        return x * p0 > p1 ? x : log_c(C(1) + exp_c(p0 * x)) / p0;                         // softplus.py:21
+    } else {
+        return x > p0 ? x : p1;                                                            // threshold.py:20
+    }
+}
+
+// `s` is the saved tensor: the forward's input, or its output for Sigmoid and Tanh.
+template <int ACT, typename C>
+__device__ __forceinline__ C act_bwd(C s, C g, C p0, C p1) {
+    if constexpr (ACT == kGelu) {
+        const float cdf = 0.5f * (1.0f + erff(s * 0.70710678118654752440f));               // gelu.py:77-80
+        const float pdf = __expf(-0.5f * s * s) * 0.39894228040143267794f;
+        return g * (cdf + s * pdf);
+    } else if constexpr (ACT == kGeluTanh) {
+        const float k = 0.79788456080286535588f;                                           // gelu.py:71-75
+        const float t = tanh_safe(k * (s + 0.044715f * s * s * s));
+        const float gp = k * (1.0f + 3.0f * 0.044715f * s * s);
+        const float sech2 = 1.0f - t * t;                          // exactly 0 once |s| > ~6: keeps 0 * inf out for huge |s|
+        const float tail = sech2 == 0.0f ? 0.0f : s * sech2 * gp;
+        return g * (0.5f * (1.0f + t + tail));
+    } else if constexpr (ACT == kSilu) {
+        const float sg = sigmoid_f(s);                                                     // silu.py:56-57
+        return g * (sg * (1.0f + s * (1.0f - sg)));
+    } else if constexpr (ACT == kRelu) {
+        return s > C(0) ? g : C(0);                                                        // relu.py:56
+    } else if constexpr (ACT == kLeakyRelu) {
+        return s > C(0) ? g : p0 * g;                                                      // leaky_relu.py:59
+    } else if constexpr (ACT == kRelu6) {
+        const C r = s > C(0) ? g : C(0);                                                   // relu6.py:57-58
+        return s < C(6) ? r : C(0);
+    } else if constexpr (ACT == kSigmoid) {
+        return g * (s * (1.0f - s));                                                       // sigmoid.py:56
+    } else if constexpr (ACT == kTanh) {
+        return g * (1.0f - s * s);                                                         // tanh.py:58
+    } else if constexpr (ACT == kMish) {
+        const float t = tanh_safe(mish_softplus(s));                                       // mish.py:60-66
+        return g * (t + s * (1.0f - t * t) * sigmoid_f(s));
+    } else if constexpr (ACT == kSoftplus) {
+        return s * p0 > p1 ? g : g / (C(1) + exp_c(-p0 * s));                              // softplus.py:62
+    } else {
+        return s > p0 ? g : C(0);                                                          // threshold.py:59
+    }
+}
+
+template <typename T, typename C>
+__device__ __forceinline__ u32x4 pack_as(const C (&f)[T::VEC]) {
+    if constexpr (std::is_same<C, double>::value) return pack_f64(f);
+    else return T::pack(f);
+}
+
+template <typename T, typename C>
+__device__ __forceinline__ C load_elem(const void* p, int64_t i) {
+    if constexpr (std::is_same<C, double>::value) return reinterpret_cast<const double*>(p)[i];
+    else return T::load1(p, i);
+}
+
+template <typename T, typename C>
+__device__ __forceinline__ void store_elem(void* p, int64_t i, C v) {
+    if constexpr (std::is_same<C, double>::value) reinterpret_cast<double*>(p)[i] = v;
+    else T::store1(p, i, v);
+}
+
+// ---------------------------------------------------------------------------------------------------
+// Contiguous tensors: one flat stream of 16-byte vectors.  A persistent grid; every thread owns U vectors per
+// grid step (vector v0 + u*BLOCK, so a wave touches contiguous 1 KiB segments), requests the next step's
+// vectors before it computes the current ones, and clamps vector slots past the end onto the last vector (they
+// recompute and re-store its values), which keeps the loop free of branches around memory operations.
+// The last total_elems % VEC elements are handled one by one after the loop.
+// ---------------------------------------------------------------------------------------------------
+constexpr int kActBlock = 256;
+
+template <typename T, int ACT, bool BWD, int U>
+__global__ void __launch_bounds__(kActBlock) act_flat_kernel(const ActArgs a) {
+    using C = typename ActCompute<T, ACT>::type;
+    constexpr int VEC = T::VEC;
+    const C p0 = static_cast<C>(a.p0), p1 = static_cast<C>(a.p1);
+
+    if (a.total_vecs > 0) {
+        const int64_t step = static_cast<int64_t>(gridDim.x) * kActBlock * U;
+        const int64_t last = a.total_vecs - 1;
+        int64_t v0 = static_cast<int64_t>(blockIdx.x) * kActBlock * U + threadIdx.x;
+        u32x4 cx[U], cg[BWD ? U : 1];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int64_t v = v0 + u * kActBlock;
+            const int64_t vc = (v < last ? v : last) * 16;
+            cx[u] = ld128(a.x + vc);
+            if constexpr (BWD) cg[u] = ld128(a.g + vc);
+        }
+        drain_vector_memory();
+        for (int64_t base = static_cast<int64_t>(blockIdx.x) * kActBlock * U; base < a.total_vecs; base += step) {
+            const int64_t n0 = v0 + step;
+            u32x4 nx[U], ng[BWD ? U : 1];
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int64_t v = n0 + u * kActBlock;
+                const int64_t vc = (v < last ? v : last) * 16;
+                nx[u] = ld128(a.x + vc);
+                if constexpr (BWD) ng[u] = ld128(a.g + vc);
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                C xf[VEC], gf[VEC], of[VEC];
+                unpack_as<T>(cx[u], xf);
+                if constexpr (BWD) unpack_as<T>(cg[u], gf);
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) {
+                    if constexpr (BWD) of[e] = act_bwd<ACT, C>(xf[e], gf[e], p0, p1);
+                    else of[e] = act_fwd<ACT, C>(xf[e], p0, p1);
+                }
+                const int64_t v = v0 + u * kActBlock;
+                st128(a.out + (v < last ? v : last) * 16, pack_as<T, C>(of));
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                cx[u] = nx[u];
+                if constexpr (BWD) cg[u] = ng[u];
+            }
+            v0 = n0;
+        }
+    }
+    // the tail that does not fill a vector
+    const int64_t tail0 = a.total_vecs * VEC;
+    const int64_t i = tail0 + threadIdx.x;
+    if (blockIdx.x == 0 && i < a.total_elems) {
+        const C x = load_elem<T, C>(a.x, i);
+        if constexpr (BWD) store_elem<T, C>(a.out, i, act_bwd<ACT, C>(x, load_elem<T, C>(a.g, i), p0, p1));
+        else store_elem<T, C>(a.out, i, act_fwd<ACT, C>(x, p0, p1));
+    }
+}
+
+// ---------------------------------------------------------------------------------------------------
+// Strided rows, or pointers that are not 16-byte aligned: one element per thread and step.  Correct for any
+// layout the reference accepts (unit column stride, arbitrary row strides); not tuned.
+// ---------------------------------------------------------------------------------------------------
+template <typename T, int ACT, bool BWD>
+__global__ void __launch_bounds__(kActBlock) act_rows_kernel(const ActArgs a) {
+    using C = typename ActCompute<T, ACT>::type;
+    const C p0 = static_cast<C>(a.p0), p1 = static_cast<C>(a.p1);
+    for (int64_t row = blockIdx.y; row < a.M; row += gridDim.y) {
+        const char* xr = a.x + row * a.x_stride_bytes;
+        const char* gr = BWD ? a.g + row * a.g_stride_bytes : nullptr;
+        char* outr = a.out + row * a.out_stride_bytes;
+        for (int64_t c = static_cast<int64_t>(blockIdx.x) * kActBlock + threadIdx.x; c < a.N;
+             c += static_cast<int64_t>(gridDim.x) * kActBlock) {
+            const C x = load_elem<T, C>(xr, c);
+            if constexpr (BWD) store_elem<T, C>(outr, c, act_bwd<ACT, C>(x, load_elem<T, C>(gr, c), p0, p1));
+            else store_elem<T, C>(outr, c, act_fwd<ACT, C>(x, p0, p1));
+        }
+    }
+}
+
+}  // namespace thn

@@ -8,11 +8,13 @@
 
 #include "thn_dispatch.h"
 #include "thn_reduce.h"
+#include "thn_act_dispatch.h"
 #include "thn_pnorm_dispatch.h"
 #include "thn_softmax_dispatch.h"
 
 namespace {
 
+using thn::ActArgs;
 using thn::BwdArgs;
 using thn::FwdArgs;
 using thn::NormalizeBwdArgs;
@@ -26,7 +28,7 @@ using thn::SoftmaxFwdArgs;
 // `which` throughout this file: the kernel family a launch belongs to.
 enum : int {
     kNormFwd = 0, kNormBwd = 1, kSoftmaxFwd = 2, kSoftmaxBwd = 3, kPnormFwd = 4, kPnormBwd = 5, kNormalizeBwd = 6,
-    kFamilies = 7
+    kActFwd = 7, kActBwd = 8, kFamilies = 9
 };
 
 constexpr int kMaxDevices = 64;
@@ -409,6 +411,65 @@ int pnorm_forward(const void* x, int64_t x_batch_stride, int64_t x_row_stride, v
     return lrc == 0 ? THN_OK : THN_E_LAUNCH;
 }
 
+// ---- element-wise activations --------------------------------------------------------------------------------
+int act_launch(const void* x, int64_t x_row_stride, const void* g, int64_t g_row_stride, void* out,
+               int64_t out_row_stride, int64_t M, int64_t N, int act, float p0, float p1, int dtype, bool bwd,
+               void* stream) {
+    const int bytes = elem_bytes(dtype);
+    if (bytes == 0) return THN_E_DTYPE;
+    if (M < 0 || N <= 0 || act < 0 || act >= thn::kNumActs) return THN_E_SHAPE;
+    if (M == 0) return THN_OK;
+    if (x == nullptr || out == nullptr || (bwd && g == nullptr)) return THN_E_NULL;
+    if (M > 1 && (x_row_stride < N || out_row_stride < N || (bwd && g_row_stride < N))) return THN_E_SHAPE;
+    const int cus = current_cu_count();
+    if (cus <= 0) return THN_E_DEVICE;
+    const int which = bwd ? kActBwd : kActFwd;
+    const int bpc_override = g_override[which].bpc.load();
+    ActArgs a{};
+    a.x = static_cast<const char*>(x);
+    a.g = static_cast<const char*>(g);
+    a.out = static_cast<char*>(out);
+    a.p0 = p0;
+    a.p1 = p1;
+    const bool contiguous = M == 1 || (x_row_stride == N && out_row_stride == N && (!bwd || g_row_stride == N));
+    const bool flat = contiguous && aligned16(x) && aligned16(out) && (!bwd || aligned16(g));
+    dim3 grid;
+    if (flat) {
+        const int vec_elems = 16 / bytes;
+        a.total_elems = M * N;
+        a.total_vecs = a.total_elems / vec_elems;
+        const int per_block = thn::kActBlock * (bwd ? thn::kActBwdVecs : thn::kActFwdVecs);
+        const int64_t blocks = (a.total_vecs + per_block - 1) / per_block;
+        // two 256-thread workgroups per compute unit: the same in-flight budget as the row kernels
+        const int64_t cap = static_cast<int64_t>(cus) * (bpc_override > 0 ? bpc_override : 2);
+        int64_t n = blocks < cap ? blocks : cap;
+        if (n > 1 && n == cap) {
+            const int64_t iters = (blocks + cap - 1) / cap;
+            n = (blocks + iters - 1) / iters;           // every workgroup takes the same number of steps
+        }
+        grid = dim3(static_cast<unsigned>(n < 1 ? 1 : n));
+    } else {
+        a.M = M;
+        a.N = N;
+        a.x_stride_bytes = x_row_stride * bytes;
+        a.g_stride_bytes = g_row_stride * bytes;
+        a.out_stride_bytes = out_row_stride * bytes;
+        const int64_t col_blocks = (N + thn::kActBlock - 1) / thn::kActBlock;
+        grid = dim3(static_cast<unsigned>(col_blocks < 1024 ? col_blocks : 1024),
+                    static_cast<unsigned>(M < 65535 ? M : 65535));
+    }
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    int lrc;
+    switch (dtype) {
+        case THN_F32: lrc = thn::launch_act_f32(act, bwd, flat, a, grid, st); break;
+        case THN_F16: lrc = thn::launch_act_f16(act, bwd, flat, a, grid, st); break;
+        case THN_BF16: lrc = thn::launch_act_bf16(act, bwd, flat, a, grid, st); break;
+        default: lrc = thn::launch_act_f64(act, bwd, flat, a, grid, st); break;
+    }
+    if (lrc > 0) return THN_E_SHAPE;
+    return lrc == 0 ? THN_OK : THN_E_LAUNCH;
+}
+
 }  // namespace
 
 extern "C" {
@@ -442,7 +503,7 @@ int thn_norm_set_launch_override(int which, int vecs_per_thread, int threads_per
 }
 
 int thn_norm_query_launch(int which, int is_layernorm, int64_t M, int64_t N, int x_dtype, int32_t shape[5]) {
-    if (which < 0 || which >= kFamilies || shape == nullptr) return THN_E_SHAPE;
+    if (which < 0 || which >= kActFwd || shape == nullptr) return THN_E_SHAPE;    // element-wise kernels have no row shape
     const int bytes = elem_bytes(x_dtype);
     if (bytes == 0) return THN_E_DTYPE;
     Plan p;
@@ -794,6 +855,18 @@ int thn_normalize_bwd(const void* x, int64_t x_batch_stride, int64_t x_row_strid
     }
     if (lrc > 0) return THN_E_SHAPE;
     return lrc == 0 ? THN_OK : THN_E_LAUNCH;
+}
+
+int thn_act_fwd(const void* x, int64_t x_row_stride, void* y, int64_t y_row_stride, int64_t M, int64_t N, int act,
+                float param0, float param1, int dtype, void* stream) {
+    return act_launch(x, x_row_stride, nullptr, 0, y, y_row_stride, M, N, act, param0, param1, dtype, false, stream);
+}
+
+int thn_act_bwd(const void* saved, int64_t saved_row_stride, const void* dy, int64_t dy_row_stride, void* dx,
+                int64_t dx_row_stride, int64_t M, int64_t N, int act, float param0, float param1, int dtype,
+                void* stream) {
+    return act_launch(saved, saved_row_stride, dy, dy_row_stride, dx, dx_row_stride, M, N, act, param0, param1, dtype,
+                      true, stream);
 }
 
 }  // extern "C"

@@ -286,6 +286,30 @@ __device__ __forceinline__ void store_vec_elems(char* row, int vec, int n_cols, 
     }
 }
 
+// Unpacking / packing for kernels whose arithmetic type C is float64 on float64 storage (the float32 traits
+// narrow on load).
+template <typename T>
+__device__ __forceinline__ void unpack_as(u32x4 v, float (&f)[T::VEC]) { T::unpack(v, f); }
+template <typename T>
+__device__ __forceinline__ void unpack_as(u32x4 v, double (&f)[T::VEC]) {
+    static_assert(T::kBytes == 8, "float64 arithmetic is for float64 storage only");
+    const uint32_t a = v[0], b = v[1], c = v[2], d = v[3];
+    f[0] = __builtin_bit_cast(double, (static_cast<uint64_t>(b) << 32) | a);
+    f[1] = __builtin_bit_cast(double, (static_cast<uint64_t>(d) << 32) | c);
+}
+
+__device__ __forceinline__ u32x4 pack_f64(const double (&f)[2]) {
+    const uint64_t lo = __builtin_bit_cast(uint64_t, f[0]), hi = __builtin_bit_cast(uint64_t, f[1]);
+    u32x4 v;
+    v[0] = static_cast<uint32_t>(lo); v[1] = static_cast<uint32_t>(lo >> 32);
+    v[2] = static_cast<uint32_t>(hi); v[3] = static_cast<uint32_t>(hi >> 32);
+    return v;
+}
+
+__device__ __forceinline__ float exp_c(float z) { return __expf(z); }
+__device__ __forceinline__ double exp_c(double z) { return exp(z); }
+
+
 // ---------------------------------------------------------------------------------------------------
 // Wave64 all-reduce (sum, or max with OpMax) over aligned groups of W lanes, W in {8, 16, 32, 64}.  The first four steps
 // are DPP modifiers fused into v_add_f32 / v_max_f32 (no LDS traffic); the 16- and 32-lane exchanges use the gfx950

@@ -39,24 +39,6 @@ struct SoftmaxBwdArgs {
 template <typename T, bool LOG> struct SoftmaxCompute { using type = float; };
 template <> struct SoftmaxCompute<F64, false> { using type = double; };
 
-template <typename T>
-__device__ __forceinline__ void unpack_as(u32x4 v, float (&f)[T::VEC]) { T::unpack(v, f); }
-template <typename T>
-__device__ __forceinline__ void unpack_as(u32x4 v, double (&f)[T::VEC]) {
-    static_assert(T::kBytes == 8, "float64 arithmetic is for float64 storage only");
-    const uint32_t a = v[0], b = v[1], c = v[2], d = v[3];
-    f[0] = __builtin_bit_cast(double, (static_cast<uint64_t>(b) << 32) | a);
-    f[1] = __builtin_bit_cast(double, (static_cast<uint64_t>(d) << 32) | c);
-}
-
-__device__ __forceinline__ u32x4 pack_f64(const double (&f)[2]) {
-    const uint64_t lo = __builtin_bit_cast(uint64_t, f[0]), hi = __builtin_bit_cast(uint64_t, f[1]);
-    u32x4 v;
-    v[0] = static_cast<uint32_t>(lo); v[1] = static_cast<uint32_t>(lo >> 32);
-    v[2] = static_cast<uint32_t>(hi); v[3] = static_cast<uint32_t>(hi >> 32);
-    return v;
-}
-
 // load_row for arithmetic type C: the element path of the float32 engine narrows float64 storage on load,
 // which the float64 path must not do.
 template <typename T, typename C, int K, bool ALIGNED>
@@ -97,9 +79,6 @@ __device__ __forceinline__ void store_row_as(char* rowp, int voff, int n_cols, c
         }
     }
 }
-
-__device__ __forceinline__ float exp_c(float z) { return __expf(z); }
-__device__ __forceinline__ double exp_c(double z) { return exp(z); }
 
 // Forward (softmax.py:17-23, logsoftmax.py:19-24): z = x - max(x); softmax: exp(z) / sum(exp(z));
 // log-softmax: z - log(sum(exp(z))).  One rounding on store.
