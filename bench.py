@@ -55,7 +55,18 @@ WORKLOADS = {
     "normalize_p3_bf16_16384x4096": ("normalize_p3", 16384, 4096, "bf16"),
     "pnorm_p2_bf16_16384x4096": ("pnorm_p2", 16384, 4096, "bf16"),
     "pnorm_p3_f32_16384x4096": ("pnorm_p3", 16384, 4096, "f32"),
+    # element-wise activations (thn_act_fwd + thn_act_bwd per step)
+    "act_gelu_bf16_16384x4096": ("act_gelu", 16384, 4096, "bf16"),
+    "act_gelu_tanh_bf16_16384x4096": ("act_gelu_tanh", 16384, 4096, "bf16"),
+    "act_gelu_f32_16384x4096": ("act_gelu", 16384, 4096, "f32"),
+    "act_silu_bf16_16384x4096": ("act_silu", 16384, 4096, "bf16"),
+    "act_relu_bf16_16384x4096": ("act_relu", 16384, 4096, "bf16"),
+    "act_mish_bf16_16384x4096": ("act_mish", 16384, 4096, "bf16"),
+    "act_softplus_f16_16384x4096": ("act_softplus", 16384, 4096, "f16"),
+    "act_sigmoid_f32_16384x4096": ("act_sigmoid", 16384, 4096, "f32"),
 }
+ACT_NAMES = ["gelu", "gelu_tanh", "silu", "relu", "leaky_relu", "relu6", "sigmoid", "tanh", "mish", "softplus", "threshold"]
+ACT_PARAMS = {"leaky_relu": (0.01, 0.0), "softplus": (1.0, 20.0), "threshold": (0.1, 20.0)}
 SOFTMAX_KINDS = ("softmax", "softmin", "logsoftmax")
 
 # HBM bytes per launch of the backward dx / partial-sum kernel, from two rocprofv3 --pmc runs of this script
@@ -77,7 +88,7 @@ def algorithmic_bytes(kind, m, n, s, sw):
         return 2 * m * n * s + m * s, (3 + extra) * m * n * s + m * s
     if kind.startswith("pnorm"):              # forward: x read, norms written; backward: x, norms, dnorms read, dx written
         return m * n * s + m * s, 2 * m * n * s + 2 * m * s
-    if kind in SOFTMAX_KINDS:                 # forward: x read, y written; backward: y and dy read, dx written
+    if kind in SOFTMAX_KINDS or kind.startswith("act_"):   # forward: x read, y written; backward: saved and dy read, dx written
         return 2 * m * n * s, 3 * m * n * s
     if kind == "ln":
         return 2 * m * n * s + 2 * n * sw + 8 * m, 3 * m * n * s + 3 * n * sw + 8 * m
@@ -109,7 +120,7 @@ def main():
     torch.cuda.set_device(dev)
     kind, m, n, dname = WORKLOADS[args.workload]
     dtype = {"bf16": torch.bfloat16, "f16": torch.float16, "f32": torch.float32}[dname]
-    if kind in SOFTMAX_KINDS or kind.startswith(("normalize", "pnorm")):
+    if kind in SOFTMAX_KINDS or kind.startswith(("normalize", "pnorm", "act_")):
         return softmax_main(args, lib, dev, kind, m, n, dname, dtype)
     s = torch.empty(0, dtype=dtype).element_size()
     code = _native.dtype_code(dtype)
@@ -253,8 +264,12 @@ def softmax_main(args, lib, dev, kind, m, n, dname, dtype):
     s = torch.empty(0, dtype=dtype).element_size()
     code = _native.dtype_code(dtype)
     kcode = {"softmax": _native.SOFTMAX, "softmin": _native.SOFTMIN, "logsoftmax": _native.LOGSOFTMAX}.get(kind)
-    row_op = None if kcode is not None else kind.split("_")[0]          # "normalize" or "pnorm"
-    pval = float(kind[-1]) if row_op else 0.0
+    row_op = None if kcode is not None else kind.split("_")[0]          # "normalize", "pnorm" or "act"
+    pval = float(kind[-1]) if row_op in ("normalize", "pnorm") else 0.0
+    act_name = kind[4:] if row_op == "act" else None
+    act_code = ACT_NAMES.index(act_name) if act_name else -1
+    ap0, ap1 = ACT_PARAMS.get(act_name, (0.0, 0.0))
+    saves_output = act_name in ("sigmoid", "tanh")
     gen = torch.Generator(device=dev).manual_seed(0)
     sets = []
     for _ in range(N_BUFFER_SETS):
@@ -273,6 +288,8 @@ def softmax_main(args, lib, dev, kind, m, n, dname, dtype):
                                        stream)
         elif row_op == "pnorm":
             rc = lib.thn_pnorm_fwd(p(b_["x"]), mn, n, p(b_["norms"]), 1, m, n, pval, 1e-12, code, stream)
+        elif row_op == "act":
+            rc = lib.thn_act_fwd(p(b_["x"]), n, p(b_["y"]), n, m, n, act_code, ap0, ap1, code, stream)
         else:
             rc = lib.thn_softmax_fwd(p(b_["x"]), n, p(b_["y"]), n, m, n, kcode, code, stream)
         assert rc == 0, _native.strerror(rc)
@@ -284,6 +301,9 @@ def softmax_main(args, lib, dev, kind, m, n, dname, dtype):
         elif row_op == "pnorm":
             rc = lib.thn_pnorm_bwd(p(b_["x"]), mn, n, p(b_["norms"]), p(b_["dnorms"]), p(b_["dx"]), mn, n, 1, m, n,
                                    pval, code, stream)
+        elif row_op == "act":
+            rc = lib.thn_act_bwd(p(b_["y"] if saves_output else b_["x"]), n, p(b_["dy"]), n, p(b_["dx"]), n, m, n,
+                                 act_code, ap0, ap1, code, stream)
         else:
             rc = lib.thn_softmax_bwd(p(b_["y"]), n, p(b_["dy"]), n, p(b_["dx"]), n, m, n, kcode, code, stream)
         assert rc == 0, _native.strerror(rc)
@@ -323,12 +343,16 @@ def softmax_main(args, lib, dev, kind, m, n, dname, dtype):
             sets[i % N_BUFFER_SETS]["dx"].copy_(sets[i % N_BUFFER_SETS]["x"])
         torch.cuda.synchronize()
     achieved = bwd_bytes / (bwd_us * 1e-6) / 1e9
-    fam = {None: (2, 3), "normalize": (4, 6), "pnorm": (4, 5)}[row_op]
-    fs = _launch.query_launch(fam[0], kind == "logsoftmax", m, n, dtype)
-    bs = _launch.query_launch(fam[1], kind == "logsoftmax", m, n, dtype)
-    bwd_kernel = {None: "softmax_bwd_kernel", "normalize": "normalize_bwd_kernel", "pnorm": "pnorm_bwd_kernel"}[row_op]
+    fam = {None: (2, 3), "normalize": (4, 6), "pnorm": (4, 5), "act": None}[row_op]
+    if fam is not None:
+        fs = _launch.query_launch(fam[0], kind == "logsoftmax", m, n, dtype)
+        bs = _launch.query_launch(fam[1], kind == "logsoftmax", m, n, dtype)
+    else:                                   # flat element-wise kernels: 4 / 2 vectors per thread, no rows
+        fs, bs = (4, 0, 256, 0), (2, 0, 256, 0)
+    bwd_kernel = {None: "softmax_bwd_kernel", "normalize": "normalize_bwd_kernel", "pnorm": "pnorm_bwd_kernel",
+                  "act": "act_flat_kernel (backward)"}[row_op]
     entry = {None: "thn_softmax_fwd + thn_softmax_bwd", "normalize": "thn_normalize_fwd + thn_normalize_bwd",
-             "pnorm": "thn_pnorm_fwd + thn_pnorm_bwd"}[row_op]
+             "pnorm": "thn_pnorm_fwd + thn_pnorm_bwd", "act": "thn_act_fwd + thn_act_bwd"}[row_op]
     out = {
         "metric": f"fwd+bwd HBM GB/s and % of peak, {kind} {dname} {m}x{n}",
         "value": round(gbps, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -349,8 +373,55 @@ def softmax_main(args, lib, dev, kind, m, n, dname, dtype):
                      "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload)},
     }
     if not args.no_cpu_baseline:
-        out["cpu_baseline"] = (row_op_cpu_baseline if row_op else softmax_cpu_baseline)(kind, m, n, dtype, sets[0], step_bytes)
+        baseline = {None: softmax_cpu_baseline, "act": act_cpu_baseline}.get(row_op, row_op_cpu_baseline)
+        out["cpu_baseline"] = baseline(kind, m, n, dtype, sets[0], step_bytes)
     print(json.dumps(out), flush=True)
+
+
+def act_cpu_baseline(kind, m, n, dtype, buffers, step_bytes):
+    """oracle/act_oracle.py (numpy float64, one thread) on a bounded sample of the same rows, and torch on the host
+    cores next to it."""
+    import torch
+    import torch.nn.functional as F
+    from oracle import act_oracle as ao
+    name = kind[4:]
+    p0, p1 = ACT_PARAMS.get(name, (0.0, 0.0))
+    rows = min(m, max(64, (1 << 23) // n))
+    x = buffers["x"][:rows].cpu()
+    dy = buffers["dy"][:rows].cpu()
+    x64, dy64 = x.double().numpy(), dy.double().numpy()
+
+    def oracle_step():
+        y = ao.fwd(name, x64, p0, p1)
+        ao.bwd(name, y if name in ao.SAVES_OUTPUT else x64, dy64, p0, p1)
+
+    fn = {"gelu": F.gelu, "gelu_tanh": lambda t: F.gelu(t, approximate="tanh"), "silu": F.silu, "relu": F.relu,
+          "leaky_relu": lambda t: F.leaky_relu(t, p0), "relu6": F.relu6, "sigmoid": torch.sigmoid, "tanh": torch.tanh,
+          "mish": F.mish, "softplus": lambda t: F.softplus(t, p0, p1), "threshold": lambda t: F.threshold(t, p0, p1)}[name]
+
+    def torch_step():
+        xr = x.clone().requires_grad_(True)
+        fn(xr).backward(dy)
+
+    def timed(f, reps):
+        f()
+        best = float("inf")
+        for _ in range(reps):
+            t0 = time.perf_counter()
+            f()
+            best = min(best, time.perf_counter() - t0)
+        return best
+
+    sample_bytes = step_bytes * rows / m
+    t_oracle, t_torch = timed(oracle_step, 3), timed(torch_step, 3)
+    return {"value": round(sample_bytes / t_oracle / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
+            "sample": f"first {rows} of {m} rows of the same workload, forward + backward, best of 3 passes of "
+                      f"oracle/act_oracle.py (numpy float64, one thread; {t_oracle * 1e3:.1f} ms per pass)",
+            "host_cpu_count": os.cpu_count(),
+            "torch_functional": {"value": round(sample_bytes / t_torch / 1e9, 2), "unit": "GB/s",
+                                 "threads": torch.get_num_threads(),
+                                 "what": f"torch {name} forward + autograd backward on the host cores, same sample "
+                                         f"({t_torch * 1e3:.1f} ms per pass)"}}
 
 
 def row_op_cpu_baseline(kind, m, n, dtype, buffers, step_bytes):

@@ -412,6 +412,18 @@ int pnorm_forward(const void* x, int64_t x_batch_stride, int64_t x_row_stride, v
 }
 
 // ---- element-wise activations --------------------------------------------------------------------------------
+// Workgroups per compute unit of the flat kernels, from sweeps on MI355X: the selections and the backward passes
+// that need one or two instructions per element stream best with one workgroup (2.5 % over two); everything with
+// an exponential in it wants two to overlap arithmetic and memory; the exact GeLU on 16-bit storage is bound by
+// arithmetic (about 30 instruction slots per element) and takes four.
+int act_blocks_per_cu(int act, bool bwd, int bytes) {
+    const bool gelu = act == thn::kGelu;
+    if (gelu && bytes == 2) return 4;
+    const bool heavy_bwd = gelu || act == thn::kGeluTanh || act == thn::kMish || (act == thn::kSilu && bytes == 2);
+    if (bwd) return heavy_bwd ? 2 : 1;
+    return 2;
+}
+
 int act_launch(const void* x, int64_t x_row_stride, const void* g, int64_t g_row_stride, void* out,
                int64_t out_row_stride, int64_t M, int64_t N, int act, float p0, float p1, int dtype, bool bwd,
                void* stream) {
@@ -440,8 +452,7 @@ int act_launch(const void* x, int64_t x_row_stride, const void* g, int64_t g_row
         a.total_vecs = a.total_elems / vec_elems;
         const int per_block = thn::kActBlock * (bwd ? thn::kActBwdVecs : thn::kActFwdVecs);
         const int64_t blocks = (a.total_vecs + per_block - 1) / per_block;
-        // two 256-thread workgroups per compute unit: the same in-flight budget as the row kernels
-        const int64_t cap = static_cast<int64_t>(cus) * (bpc_override > 0 ? bpc_override : 2);
+        const int64_t cap = static_cast<int64_t>(cus) * (bpc_override > 0 ? bpc_override : act_blocks_per_cu(act, bwd, bytes));
         int64_t n = blocks < cap ? blocks : cap;
         if (n > 1 && n == cap) {
             const int64_t iters = (blocks + cap - 1) / cap;
