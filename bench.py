@@ -79,6 +79,8 @@ MEASURED_TRAFFIC_BYTES = {
     "softmax_bf16_16384x4096": 402815465,
     # profiles/pnorm_kernels_normalize_p2_bf16_16384x4096_stats_and_hbm_counters.txt (normalize_bwd_kernel)
     "normalize_p2_bf16_16384x4096": 403121728,
+    # profiles/act_kernels_gelu_tanh_bf16_16384x4096_stats_and_hbm_counters.txt (act_flat_kernel backward)
+    "act_gelu_tanh_bf16_16384x4096": 402681390,
 }
 
 
