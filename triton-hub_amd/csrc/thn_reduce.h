@@ -7,8 +7,10 @@ namespace thn {
 
 // ---------------------------------------------------------------------------------------------------
 // Second stage: out[c] = sum over the P partial rows of part[p][c], added in a fixed order in float64 and
-// rounded once to the parameter's storage type.  A workgroup owns 64 columns (16 lanes x float4); its 16
-// row slices each add every 16th partial row, then slice sums are added in slice order through LDS.
+// rounded once to the parameter's storage type.  The stage is pure latency (a few MiB, one dependent launch),
+// so it is cut for parallelism: a workgroup owns 16 columns (4 lanes x float4) and has 64 row slices, each
+// adding every 64th partial row (4 independent loads for 256 partial rows); the slice sums are then added in
+// slice order through LDS.  N / 16 workgroups: every compute unit takes part from N = 4096 on.
 // blockIdx.y selects dW (0) or dB (1).
 // ---------------------------------------------------------------------------------------------------
 struct ReduceArgs {
@@ -20,17 +22,24 @@ struct ReduceArgs {
     int w_dtype;
 };
 
+#ifndef THN_REDUCE_COLS
+#define THN_REDUCE_COLS 16
+#endif
+constexpr int kReduceCols = THN_REDUCE_COLS;        // columns per workgroup
+constexpr int kReduceSlices = 1024 / kReduceCols;   // row slices per workgroup (256 threads x float4)
+
 __global__ void __launch_bounds__(256) reduce_partials_kernel(const ReduceArgs a) {
-    __shared__ double acc[16][64];
+    __shared__ double acc[kReduceSlices][kReduceCols];
     const int which = blockIdx.y;
     const float* part = a.part[which];
     void* out = a.out[which];
-    const int lane = threadIdx.x & 15;
-    const int slice = threadIdx.x >> 4;
-    const int col = blockIdx.x * 64 + lane * 4;
+    constexpr int kLanes = kReduceCols / 4;
+    const int lane = threadIdx.x % kLanes;
+    const int slice = threadIdx.x / kLanes;
+    const int col = blockIdx.x * kReduceCols + lane * 4;
     double s0 = 0.0, s1 = 0.0, s2 = 0.0, s3 = 0.0;
     if (col < a.n_cols) {     // the pitch is a multiple of 64 floats: the whole float4 is inside the row
-        for (int p = slice; p < a.n_parts; p += 16) {
+        for (int p = slice; p < a.n_parts; p += kReduceSlices) {
             const float4 v = *reinterpret_cast<const float4*>(part + static_cast<int64_t>(p) * a.pitch + col);
             s0 += v.x; s1 += v.y; s2 += v.z; s3 += v.w;
         }
@@ -40,12 +49,12 @@ __global__ void __launch_bounds__(256) reduce_partials_kernel(const ReduceArgs a
     acc[slice][lane * 4 + 2] = s2;
     acc[slice][lane * 4 + 3] = s3;
     __syncthreads();
-    if (threadIdx.x < 64) {
-        const int c = blockIdx.x * 64 + threadIdx.x;
+    if (threadIdx.x < kReduceCols) {
+        const int c = blockIdx.x * kReduceCols + threadIdx.x;
         if (c < a.n_cols) {
             double s = 0.0;
 #pragma unroll
-            for (int i = 0; i < 16; ++i) s += acc[i][threadIdx.x];
+            for (int i = 0; i < kReduceSlices; ++i) s += acc[i][threadIdx.x];
             if (a.w_dtype == kF64) reinterpret_cast<double*>(out)[c] = s;
             else store_param(out, a.w_dtype, c, static_cast<float>(s));
         }
