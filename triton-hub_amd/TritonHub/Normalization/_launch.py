@@ -31,7 +31,8 @@ def _rows(t: torch.Tensor, what: str) -> torch.Tensor:
 def _param(p, n: int, name: str):
     if p is None:
         return None
-    p = p.contiguous()
+    if not p.is_contiguous():
+        p = p.contiguous()
     assert p.shape == (n,), f'expect {name} to have shape (N,)'
     assert p.stride(-1) == 1, f'expect {name} to be row-major'
     return p
@@ -43,7 +44,10 @@ def _check_feature_dim(n: int, element_size: int) -> None:
 
 
 _raw_stream = getattr(torch._C, '_cuda_getCurrentRawStream', None)
+_get_device = getattr(torch._C, '_cuda_getDevice', None)
 _workspace_bytes_cache = {}
+_workspace_cache = {}           # (device index, stream handle) -> uint8 tensor, grown on demand
+_F32 = torch.float32
 
 
 def _stream_handle(index: int) -> int:
@@ -51,6 +55,10 @@ def _stream_handle(index: int) -> int:
     if _raw_stream is not None:
         return _raw_stream(index)
     return torch.cuda.current_stream(index).cuda_stream
+
+
+def _current_device() -> int:
+    return _get_device() if _get_device is not None else torch.cuda.current_device()
 
 
 class _on_device:
@@ -64,7 +72,7 @@ class _on_device:
         self.guard = None
 
     def __enter__(self):
-        if torch.cuda.current_device() != self.index:
+        if _current_device() != self.index:
             self.guard = torch.cuda.device(self.index)
             self.guard.__enter__()
 
@@ -74,66 +82,110 @@ class _on_device:
         return False
 
 
+def _flatten(t: torch.Tensor, what: str):
+    """(tensor to pass, M, N, row stride in elements, needs un-flattening).  A contiguous tensor is passed as it
+    is -- its rows are already N apart -- which skips two reshapes per call on the common path."""
+    n = t.shape[-1]
+    if t.is_contiguous() and t.dim() >= 1 and n > 0:
+        return t, t.numel() // n, n, n, False
+    t2 = _rows(t, what)
+    m = t2.shape[0]
+    return t2, m, n, (t2.stride(0) if m > 1 else n), True
+
+
+def _workspace(index: int, stream: int, nbytes: int, device) -> torch.Tensor:
+    """The counterpart of the reference's per-call `_dw` / `_db` partial buffers (layernorm.py:183-184).  One buffer
+    per (device, stream) is kept and grown on demand: both stages of a backward are enqueued on that stream, so a
+    later call on the same stream can only reuse the buffer after they have run."""
+    key = (index, stream)
+    ws = _workspace_cache.get(key)
+    if ws is None or ws.numel() < nbytes:
+        ws = torch.empty((max(nbytes, 16),), dtype=torch.uint8, device=device)
+        _workspace_cache[key] = ws
+    return ws
+
+
 def norm_fwd(x: torch.Tensor, weight, bias, eps: float, layernorm: bool):
     """Returns (y like x, mean (M,) float32 or None, rstd (M,) float32)."""
-    _native.require_gpu(x)
-    batch_shape = x.shape[:-1]
-    x2 = _rows(x, 'input')
-    m, n = x2.shape
-    weight = _param(weight, n, 'weight')
-    bias = _param(bias, n, 'bias')
-    out = torch.empty((m, n), dtype=x.dtype, device=x.device)
+    if not x.is_cuda:
+        _native.require_gpu(x)
+    x2, m, n, x_stride, reshaped = _flatten(x, 'input')
+    if weight is not None:
+        weight = _param(weight, n, 'weight')
+    if bias is not None:
+        bias = _param(bias, n, 'bias')
+    device = x.device
+    out = torch.empty((m, n), dtype=x.dtype, device=device) if reshaped else torch.empty_like(x)
     assert out.stride(-1) == 1, 'expect output to be row-major'
-    mean = torch.empty((m,), dtype=torch.float32, device=x.device) if layernorm else None
-    rstd = torch.empty((m,), dtype=torch.float32, device=x.device)
-    _check_feature_dim(n, x.element_size())
+    mean = torch.empty((m,), dtype=_F32, device=device) if layernorm else None
+    rstd = torch.empty((m,), dtype=_F32, device=device)
+    if n * x.element_size() > 65536:
+        raise RuntimeError(FEATURE_DIM_MESSAGE)
     x_code = _native.dtype_code(x.dtype)
     if m == 0:                       # nothing to launch (and empty tensors have no address to pass)
-        return out.reshape(*batch_shape, n), mean, rstd
-    params = weight if weight is not None else bias
-    if weight is not None and bias is not None and weight.dtype != bias.dtype:
-        bias = bias.to(weight.dtype)
-    w_code = _native.dtype_code(params.dtype) if params is not None else x_code
-    index = x.device.index
-    with _on_device(index):
+        return (out.reshape(*x.shape[:-1], n) if reshaped else out), mean, rstd
+    w_code = x_code
+    if weight is not None:
+        w_code = _native.dtype_code(weight.dtype)
+        if bias is not None and weight.dtype != bias.dtype:
+            bias = bias.to(weight.dtype)
+    elif bias is not None:
+        w_code = _native.dtype_code(bias.dtype)
+    index = device.index
+    other_device = _current_device() != index
+    if other_device:
+        guard = torch.cuda.device(index)
+        guard.__enter__()
+    try:
         status = _native.lib().thn_norm_fwd(
-            x2.data_ptr(), x2.stride(0) if m > 1 else n, out.data_ptr(), n,
-            _native.ptr(weight), _native.ptr(bias), _native.ptr(mean), rstd.data_ptr(),
+            x2.data_ptr(), x_stride, out.data_ptr(), n,
+            0 if weight is None else weight.data_ptr(), 0 if bias is None else bias.data_ptr(),
+            0 if mean is None else mean.data_ptr(), rstd.data_ptr(),
             m, n, float(eps), x_code, w_code, _stream_handle(index))
+    finally:
+        if other_device:
+            guard.__exit__(None, None, None)
     if status != 0:
         _native.check(status)
-    return out.reshape(*batch_shape, n), mean, rstd
+    return (out.reshape(*x.shape[:-1], n) if reshaped else out), mean, rstd
 
 
 def norm_bwd(x: torch.Tensor, dout: torch.Tensor, weight, bias, mean, rstd, layernorm: bool):
     """Returns (dx like x, dw or None, db or None); dw/db take the dtype of weight/bias (layernorm.py:207-208)."""
-    _native.require_gpu(x)
-    batch_shape = x.shape[:-1]
-    x2 = _rows(x, 'input')
-    m, n = x2.shape
-    d2 = _rows(dout, 'output')
-    assert d2.shape == (m, n), 'expect input and output shape to be the same'
+    if not x.is_cuda:
+        _native.require_gpu(x)
+    x2, m, n, x_stride, reshaped = _flatten(x, 'input')
+    d2, dm, dn, d_stride, _ = _flatten(dout, 'output')
+    assert dm == m and dn == n, 'expect input and output shape to be the same'
     if d2.dtype != x2.dtype:
         d2 = d2.to(x2.dtype)
-    weight = _param(weight, n, 'weight')
-    bias = _param(bias, n, 'bias')
-    dx = torch.empty((m, n), dtype=x.dtype, device=x.device)
+    if weight is not None:
+        weight = _param(weight, n, 'weight')
+    if bias is not None:
+        bias = _param(bias, n, 'bias')
+    device = x.device
+    dx = torch.empty((m, n), dtype=x.dtype, device=device) if reshaped else torch.empty_like(x)
     assert dx.stride(-1) == 1, 'expect derivative to be row-major'
-    _check_feature_dim(n, x.element_size())
+    if n * x.element_size() > 65536:
+        raise RuntimeError(FEATURE_DIM_MESSAGE)
     x_code = _native.dtype_code(x.dtype)
     want_db = layernorm and bias is not None
     mixed = weight is not None and want_db and weight.dtype != bias.dtype
     grad_dtype = weight.dtype if weight is not None else (bias.dtype if want_db else x.dtype)
     w_code = _native.dtype_code(grad_dtype)
-    dw = torch.empty((n,), dtype=grad_dtype, device=x.device) if weight is not None else None
-    db = torch.empty((n,), dtype=grad_dtype, device=x.device) if want_db else None
+    dw = torch.empty((n,), dtype=grad_dtype, device=device) if weight is not None else None
+    db = torch.empty((n,), dtype=grad_dtype, device=device) if want_db else None
     if m == 0:                       # the sum over no rows
         dw = None if dw is None else dw.zero_()
         db = None if db is None else db.zero_().to(bias.dtype)
-        return dx.reshape(*batch_shape, n), dw, db
+        return (dx.reshape(*x.shape[:-1], n) if reshaped else dx), dw, db
     lib = _native.lib()
-    index = x.device.index
-    with _on_device(index):
+    index = device.index
+    other_device = _current_device() != index
+    if other_device:
+        guard = torch.cuda.device(index)
+        guard.__enter__()
+    try:
         key = (index, m, n, dw is not None, db is not None, x_code)
         nbytes = _workspace_bytes_cache.get(key)
         if nbytes is None:
@@ -141,18 +193,21 @@ def norm_bwd(x: torch.Tensor, dout: torch.Tensor, weight, bias, mean, rstd, laye
             if nbytes < 0:
                 _native.check(nbytes)
             _workspace_bytes_cache[key] = nbytes
-        # the counterpart of the reference's per-call _dw / _db buffers (layernorm.py:183-184)
-        workspace = torch.empty((max(nbytes, 16) // 4,), dtype=torch.float32, device=x.device)
+        stream = _stream_handle(index)
+        workspace = _workspace(index, stream, nbytes, device) if nbytes > 0 else None
         status = lib.thn_norm_bwd(
-            x2.data_ptr(), x2.stride(0) if m > 1 else n, d2.data_ptr(), d2.stride(0) if m > 1 else n,
-            dx.data_ptr(), n, _native.ptr(weight), _native.ptr(mean), rstd.data_ptr(),
-            _native.ptr(dw), _native.ptr(db), workspace.data_ptr(), nbytes, m, n, x_code, w_code,
-            _stream_handle(index))
+            x2.data_ptr(), x_stride, d2.data_ptr(), d_stride, dx.data_ptr(), n,
+            0 if weight is None else weight.data_ptr(), 0 if mean is None else mean.data_ptr(), rstd.data_ptr(),
+            0 if dw is None else dw.data_ptr(), 0 if db is None else db.data_ptr(),
+            0 if workspace is None else workspace.data_ptr(), nbytes, m, n, x_code, w_code, stream)
+    finally:
+        if other_device:
+            guard.__exit__(None, None, None)
     if status != 0:
         _native.check(status)
     if mixed:
         db = db.to(bias.dtype)
-    return dx.reshape(*batch_shape, n), dw, db
+    return (dx.reshape(*x.shape[:-1], n) if reshaped else dx), dw, db
 
 
 def query_launch(which: int, layernorm: bool, m: int, n: int, dtype: torch.dtype):

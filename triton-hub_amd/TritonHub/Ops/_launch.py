@@ -8,7 +8,7 @@ on the current stream.  The (B, M) tensors cross the boundary as contiguous vect
 import torch
 
 from .. import _native
-from ..Normalization._launch import _on_device, _stream_handle
+from ..Activations._launch import _call
 
 
 def _rows3d(t: torch.Tensor) -> torch.Tensor:
@@ -18,13 +18,6 @@ def _rows3d(t: torch.Tensor) -> torch.Tensor:
     return t
 
 
-def _launch(fn_name, device_index, *args):
-    with _on_device(device_index):
-        status = getattr(_native.lib(), fn_name)(*args, _stream_handle(device_index))
-    if status != 0:
-        _native.check(status)
-
-
 def norm_fwd(x, p=2, eps=1e-6):
     _native.require_gpu(x)
     x = _rows3d(x)
@@ -32,7 +25,7 @@ def norm_fwd(x, p=2, eps=1e-6):
     norms_x = torch.empty((B, M), memory_format=torch.contiguous_format, device=x.device, dtype=x.dtype)
     assert x.stride(-1) == 1, "Output tensors must be contiguous"
     if B * M > 0:
-        _launch('thn_pnorm_fwd', x.device.index, x.data_ptr(), x.stride(0), x.stride(1), norms_x.data_ptr(),
+        _call(x.device, 'thn_pnorm_fwd', x.data_ptr(), x.stride(0), x.stride(1), norms_x.data_ptr(),
                 B, M, K, float(p), float(eps), _native.dtype_code(x.dtype))
     return norms_x
 
@@ -51,7 +44,7 @@ def norm_bwd(x, norms_x, dout, p=2):
     dx = torch.empty((B, M, K), memory_format=torch.contiguous_format, device=norms_x.device, dtype=norms_x.dtype)
     assert dx.stride(-1) == 1, "Output tensors must be contiguous"
     if B * M > 0:
-        _launch('thn_pnorm_bwd', x.device.index, x.data_ptr(), x.stride(0), x.stride(1), norms_x.data_ptr(),
+        _call(x.device, 'thn_pnorm_bwd', x.data_ptr(), x.stride(0), x.stride(1), norms_x.data_ptr(),
                 dout.data_ptr(), dx.data_ptr(), M * K, K, B, M, K, float(p), _native.dtype_code(x.dtype))
     return dx
 
@@ -64,7 +57,7 @@ def normalize_fwd(x, p=2, eps=1e-6):
     norms_x = torch.empty((B, M), memory_format=torch.contiguous_format, device=x.device, dtype=x.dtype)
     assert x.stride(-1) == 1, "Output tensors must be contiguous"
     if B * M > 0:
-        _launch('thn_normalize_fwd', x.device.index, x.data_ptr(), x.stride(0), x.stride(1), x_norm.data_ptr(),
+        _call(x.device, 'thn_normalize_fwd', x.data_ptr(), x.stride(0), x.stride(1), x_norm.data_ptr(),
                 M * K, K, norms_x.data_ptr(), B, M, K, float(p), float(eps), _native.dtype_code(x.dtype))
     return x_norm, norms_x
 
@@ -81,7 +74,7 @@ def normalize_bwd(x, x_norm, norms_x, dout, p=2):
     dx = torch.empty((B, M, K), memory_format=torch.contiguous_format, device=x_norm.device, dtype=x_norm.dtype)
     assert dx.stride(-1) == 1, "Output tensors must be contiguous"
     if B * M > 0:
-        _launch('thn_normalize_bwd', x_norm.device.index, x.data_ptr(), x.stride(0), x.stride(1), x_norm.data_ptr(),
+        _call(x_norm.device, 'thn_normalize_bwd', x.data_ptr(), x.stride(0), x.stride(1), x_norm.data_ptr(),
                 x_norm.stride(0), x_norm.stride(1), norms_x.data_ptr(), dout.data_ptr(), dout.stride(0),
                 dout.stride(1), dx.data_ptr(), M * K, K, B, M, K, float(p), _native.dtype_code(x_norm.dtype))
     return dx
