@@ -1,0 +1,102 @@
+"""GPU tests of the stream contract of the C ABI: every kernel is enqueued on the stream it is given, nothing
+synchronises, allocates or touches another stream -- so the calls can run on a side stream and can be captured
+into a HIP graph and replayed."""
+import ctypes
+
+import pytest
+import torch
+
+from TritonHub import _native
+from TritonHub.Activations import GeLU, Softmax
+from TritonHub.Normalization import LayerNorm, RMSNorm
+from TritonHub.Ops import normalize
+
+pytestmark = pytest.mark.gpu
+
+
+def announce(msg):
+    print(f"\n[case] {msg}", flush=True)
+
+
+def test_operators_on_a_side_stream():
+    """The operator layer launches on torch's CURRENT stream: results computed on a side stream equal those of the
+    default stream, and the side stream's work is ordered after the producer it waited on."""
+    announce("side stream")
+    torch.manual_seed(0)
+    x = torch.randn(512, 1024, device="cuda")
+    dy = torch.randn(512, 1024, device="cuda")
+    mods = [LayerNorm(1024, device="cuda"), RMSNorm(1024, device="cuda"), Softmax(), GeLU("tanh")]
+    expected = []
+    for mod in mods:
+        a = x.clone().requires_grad_(True)
+        y = mod(a); y.backward(dy)
+        expected.append((y.detach().clone(), a.grad.clone()))
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    got = []
+    with torch.cuda.stream(side):
+        big = torch.randn(4096, 8192, device="cuda")
+        for _ in range(3):
+            big = big * 1.0001                      # keeps the side stream busy: the launches below must queue behind it
+        for mod in mods:
+            a = x.clone().requires_grad_(True)
+            y = mod(a); y.backward(dy)
+            got.append((y.detach(), a.grad))
+    side.synchronize()
+    for (ye, ge), (yg, gg) in zip(expected, got):
+        assert torch.equal(ye, yg) and torch.equal(ge, gg)
+    x3 = x.reshape(4, 128, 1024).clone().requires_grad_(True)
+    with torch.cuda.stream(side):
+        side.wait_stream(torch.cuda.current_stream())
+        y = normalize()(x3); y.backward(dy.reshape(4, 128, 1024))
+    side.synchronize()
+    ref = torch.nn.functional.normalize(x.reshape(4, 128, 1024), dim=-1, eps=1e-6)
+    assert torch.allclose(y, ref, atol=1e-6)
+
+
+def test_c_abi_calls_replay_from_a_hip_graph():
+    """Forward + backward of RMSNorm, softmax and an activation captured into one graph through the C ABI (no
+    allocation, no synchronisation inside the library), replayed three times on changing inputs with eager work
+    and synchronisations in between; every replay must equal the eager result bit for bit."""
+    announce("graph capture")
+    lib = _native.lib()
+    m, n = 2048, 1024
+    code = _native.BF16
+    dt = torch.bfloat16
+    g = torch.Generator(device="cuda").manual_seed(1)
+    x = torch.randn(m, n, device="cuda", generator=g).to(dt); dy = torch.randn(m, n, device="cuda", generator=g).to(dt)
+    w = (1 + 0.1 * torch.randn(n, device="cuda", generator=g)).to(dt)
+    y = torch.empty_like(x); dx = torch.empty_like(x); dw = torch.empty_like(w); rstd = torch.empty(m, device="cuda")
+    sm = torch.empty_like(x); dsm = torch.empty_like(x); act = torch.empty_like(x); dact = torch.empty_like(x)
+    nbytes = lib.thn_norm_bwd_workspace_bytes(m, n, 1, 0, code)
+    ws = torch.empty(nbytes, dtype=torch.uint8, device="cuda")
+    p = _native.ptr
+
+    def enqueue(st):
+        assert lib.thn_norm_fwd(p(x), n, p(y), n, p(w), 0, 0, p(rstd), m, n, 1e-6, code, code, st) == 0
+        assert lib.thn_norm_bwd(p(x), n, p(dy), n, p(dx), n, p(w), 0, p(rstd), p(dw), 0, p(ws), nbytes, m, n, code, code, st) == 0
+        assert lib.thn_softmax_fwd(p(y), n, p(sm), n, m, n, _native.SOFTMAX, code, st) == 0
+        assert lib.thn_softmax_bwd(p(sm), n, p(dy), n, p(dsm), n, m, n, _native.SOFTMAX, code, st) == 0
+        assert lib.thn_act_fwd(p(y), n, p(act), n, m, n, _native.ACT_SILU, 0.0, 0.0, code, st) == 0
+        assert lib.thn_act_bwd(p(y), n, p(dy), n, p(dact), n, m, n, _native.ACT_SILU, 0.0, 0.0, code, st) == 0
+
+    outputs = (y, dx, dw, rstd, sm, dsm, act, dact)
+    enqueue(torch.cuda.current_stream().cuda_stream)          # eager warm-up (fills the library's occupancy cache)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        enqueue(torch.cuda.current_stream().cuda_stream)       # the capture stream
+    for trial in range(3):
+        x.copy_(torch.randn(m, n, device="cuda", generator=g).to(dt))
+        dy.copy_(torch.randn(m, n, device="cuda", generator=g).to(dt))
+        enqueue(torch.cuda.current_stream().cuda_stream)
+        torch.cuda.synchronize()
+        eager = [t.clone() for t in outputs]
+        for t in outputs:
+            t.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for name, e, t in zip("y dx dw rstd sm dsm act dact".split(), eager, outputs):
+            assert torch.equal(e, t), f"replay {trial}: {name} differs from the eager result"
