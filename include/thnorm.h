@@ -30,7 +30,7 @@
 extern "C" {
 #endif
 
-#define THN_ABI_VERSION 4
+#define THN_ABI_VERSION 5
 
 enum thn_dtype { THN_F32 = 0, THN_F16 = 1, THN_BF16 = 2, THN_F64 = 3 };
 
@@ -236,11 +236,44 @@ int thn_act_bwd(const void* saved, int64_t saved_row_stride,
                 int64_t M, int64_t N, int act, float param0, float param1, int dtype, void* stream);
 
 /*
+ * LayerNorm / RMSNorm with an activation epilogue: y = act(normalise(x)*w + b) in ONE pass over the tensor.
+ * The reference has no such operator; its quick start chains the two (README.md:47-48: `x = layernorm(x)`,
+ * then `x = gelu(x)`), i.e. `_layernorm_kernel_fwd` (layernorm.py:74-86) followed by `_gelu_kernel_fwd`
+ * (gelu.py:45), and in the backward `_gelu_kernel_bwd` (gelu.py:100) followed by `_layernorm_kernel_bwd` plus the
+ * partial sums (layernorm.py:188-208).  These two entry points replace each pair by one launch (plus the
+ * second-stage reduction): the activation is applied to the float32 value before the single rounding on store,
+ * and the backward recomputes the pre-activation z = xhat*w + b from the saved statistics (nothing extra is
+ * saved), replaces dy by dy*act'(z) and continues as thn_norm_bwd.  Five passes over the tensor instead of ten.
+ * `act`: THN_ACT_GELU, THN_ACT_GELU_TANH, THN_ACT_SILU or THN_ACT_RELU (the parameter-free activations whose
+ * backward needs only their input); anything else is THN_E_SHAPE.  All other arguments, the workspace
+ * (thn_norm_bwd_workspace_bytes) and the NULL conventions are those of thn_norm_fwd / thn_norm_bwd; `b` is the
+ * forward's bias (NULL when there is none).  Because the intermediate is never rounded to the storage type, the
+ * result is closer to exact arithmetic than the chained operators', not bit-identical to them.
+ */
+int thn_norm_act_fwd(const void* x, int64_t x_row_stride,
+                     void* y, int64_t y_row_stride,
+                     const void* w, const void* b,
+                     float* mean, float* rstd,
+                     int64_t M, int64_t N, float eps, int act,
+                     int x_dtype, int w_dtype, void* stream);
+
+int thn_norm_act_bwd(const void* x, int64_t x_row_stride,
+                     const void* dy, int64_t dy_row_stride,
+                     void* dx, int64_t dx_row_stride,
+                     const void* w, const void* b,
+                     const float* mean, const float* rstd,
+                     void* dw, void* db,
+                     void* workspace, int64_t workspace_bytes,
+                     int64_t M, int64_t N, int act,
+                     int x_dtype, int w_dtype, void* stream);
+
+/*
  * Launch-shape control for tuning sweeps (the counterpart of the reference's `triton.autotune` over
  * num_warps, autotune.py:62-65, which this library replaces by a fixed heuristic on N and the dtype).
  * `which`: 0 = norm forward, 1 = norm backward, 2 = softmax forward, 3 = softmax backward, 4 = p-norm /
  * normalize forward, 5 = p-norm backward, 6 = normalize backward, 7 / 8 = element-wise activation forward /
- * backward (only blocks_per_cu applies to them; thn_norm_query_launch does not cover them).
+ * backward (only blocks_per_cu applies to them; thn_norm_query_launch does not cover them), 9 / 10 = norm with
+ * activation epilogue forward / backward.
  * vecs_per_thread / threads_per_row / block_threads select a compiled kernel shape, blocks_per_cu caps the
  * persistent grid; 0 for any field keeps the heuristic's choice.
  * Process-wide; meant for benchmarks, not for concurrent production use.  Returns THN_E_SHAPE when no

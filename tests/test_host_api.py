@@ -25,7 +25,7 @@ def declared_functions():
 
 def test_library_exports_every_declared_symbol():
     names = declared_functions()
-    assert len(names) == 17 and "thn_act_fwd" in names and "thn_pnorm_fwd" in names and "thn_normalize_bwd" in names and "thn_norm_fwd" in names and "thn_norm_bwd" in names and "thn_softmax_fwd" in names
+    assert len(names) == 19 and "thn_norm_act_fwd" in names and "thn_norm_act_bwd" in names and "thn_act_fwd" in names and "thn_pnorm_fwd" in names and "thn_normalize_bwd" in names and "thn_norm_fwd" in names and "thn_norm_bwd" in names and "thn_softmax_fwd" in names
     handle = ctypes.CDLL(_native.LIB_PATH)
     for name in names:
         assert hasattr(handle, name), f"{name} is declared in include/thnorm.h but not exported"
@@ -59,7 +59,7 @@ def test_argument_checks_answer_without_a_gpu():
     assert lib.thn_norm_bwd_workspace_bytes(4, 40000, 1, 1, _native.F16) == _native.E_FEATURE_DIM
     assert lib.thn_norm_bwd_workspace_bytes(4, 128, 0, 0, _native.F32) == 0
     assert lib.thn_norm_bwd_workspace_bytes(0, 128, 1, 1, _native.F32) == 0
-    assert lib.thn_norm_set_launch_override(9, 0, 0, 0, 0) == _native.E_SHAPE
+    assert lib.thn_norm_set_launch_override(11, 0, 0, 0, 0) == _native.E_SHAPE
     assert lib.thn_norm_set_launch_override(0, 0, 0, 0, 0) == _native.OK
     if not torch.cuda.is_available():
         assert lib.thn_norm_bwd_workspace_bytes(4, 128, 1, 1, _native.F32) == _native.E_DEVICE
@@ -148,6 +148,33 @@ def test_activation_callables_match_the_reference_constructors():
                 A.Softplus(), A.Threshold(0.1, 0.0)):
         with pytest.raises(RuntimeError, match="no CPU fallback"):
             mod(x)
+
+
+def test_fused_norm_activation_surface_and_argument_checks():
+    from TritonHub.Normalization.fused import ACTIVATIONS, LayerNormActivation, RMSNormActivation
+    lib = _native.lib()
+    fwd = lambda m, n, act, xd: lib.thn_norm_act_fwd(0, n, 0, n, 0, 0, 0, 0, m, n, 1e-5, act, xd, 0, 0)
+    bwd = lambda m, n, act, xd: lib.thn_norm_act_bwd(0, n, 0, n, 0, n, 0, 0, 0, 0, 0, 0, 0, 0, m, n, act, xd, 0, 0)
+    for call in (fwd, bwd):
+        for act in (-1, _native.ACT_LEAKY_RELU, _native.ACT_SIGMOID, _native.ACT_THRESHOLD, 11):
+            assert call(4, 128, act, _native.F32) == _native.E_SHAPE        # only gelu, gelu_tanh, silu, relu ride along
+        assert call(4, 128, _native.ACT_GELU, 9) == _native.E_DTYPE
+        assert call(4, 32769, _native.ACT_SILU, _native.BF16) == _native.E_FEATURE_DIM
+        assert call(0, 128, _native.ACT_RELU, _native.F16) == _native.OK
+        assert call(4, 128, _native.ACT_GELU_TANH, _native.F16) == _native.E_NULL
+    assert ACTIVATIONS == {"gelu": 0, "gelu_tanh": 1, "silu": 2, "relu": 3}
+    m = LayerNormActivation(48, "gelu_tanh", eps=1e-3, bias=False, dtype=torch.bfloat16)
+    assert isinstance(m, LayerNorm) and (m.dim, m.eps, m.activation, m.act) == (48, 1e-3, "gelu_tanh", 1)
+    assert m.bias is None and m.weight.dtype == torch.bfloat16
+    assert list(m.state_dict()) == list(LayerNorm(48, bias=False).state_dict())
+    r = RMSNormActivation(64)
+    assert isinstance(r, RMSNorm) and (r.activation, r.act, r.eps) == ("silu", 2, 1e-5) and r.bias is None
+    with pytest.raises(AssertionError, match="activation must be one of"):
+        LayerNormActivation(8, "mish")
+    for mod in (m, r):
+        with pytest.raises(RuntimeError, match="no CPU fallback"):
+            mod(torch.randn(2, mod.dim, dtype=mod.weight.dtype))
+    assert Normalization.__all__ == ["LayerNorm", "RMSNorm"]          # the reference's surface is unchanged
 
 
 def test_ops_surface_matches_the_reference():

@@ -105,8 +105,9 @@ def _workspace(index: int, stream: int, nbytes: int, device) -> torch.Tensor:
     return ws
 
 
-def norm_fwd(x: torch.Tensor, weight, bias, eps: float, layernorm: bool):
-    """Returns (y like x, mean (M,) float32 or None, rstd (M,) float32)."""
+def norm_fwd(x: torch.Tensor, weight, bias, eps: float, layernorm: bool, act: int = -1):
+    """Returns (y like x, mean (M,) float32 or None, rstd (M,) float32).  `act` >= 0: the activation with that
+    code is applied in the same pass (thn_norm_act_fwd)."""
     if not x.is_cuda:
         _native.require_gpu(x)
     x2, m, n, x_stride, reshaped = _flatten(x, 'input')
@@ -137,11 +138,18 @@ def norm_fwd(x: torch.Tensor, weight, bias, eps: float, layernorm: bool):
         guard = torch.cuda.device(index)
         guard.__enter__()
     try:
-        status = _native.lib().thn_norm_fwd(
-            x2.data_ptr(), x_stride, out.data_ptr(), n,
-            0 if weight is None else weight.data_ptr(), 0 if bias is None else bias.data_ptr(),
-            0 if mean is None else mean.data_ptr(), rstd.data_ptr(),
-            m, n, float(eps), x_code, w_code, _stream_handle(index))
+        if act < 0:
+            status = _native.lib().thn_norm_fwd(
+                x2.data_ptr(), x_stride, out.data_ptr(), n,
+                0 if weight is None else weight.data_ptr(), 0 if bias is None else bias.data_ptr(),
+                0 if mean is None else mean.data_ptr(), rstd.data_ptr(),
+                m, n, float(eps), x_code, w_code, _stream_handle(index))
+        else:
+            status = _native.lib().thn_norm_act_fwd(
+                x2.data_ptr(), x_stride, out.data_ptr(), n,
+                0 if weight is None else weight.data_ptr(), 0 if bias is None else bias.data_ptr(),
+                0 if mean is None else mean.data_ptr(), rstd.data_ptr(),
+                m, n, float(eps), act, x_code, w_code, _stream_handle(index))
     finally:
         if other_device:
             guard.__exit__(None, None, None)
@@ -150,8 +158,9 @@ def norm_fwd(x: torch.Tensor, weight, bias, eps: float, layernorm: bool):
     return (out.reshape(*x.shape[:-1], n) if reshaped else out), mean, rstd
 
 
-def norm_bwd(x: torch.Tensor, dout: torch.Tensor, weight, bias, mean, rstd, layernorm: bool):
-    """Returns (dx like x, dw or None, db or None); dw/db take the dtype of weight/bias (layernorm.py:207-208)."""
+def norm_bwd(x: torch.Tensor, dout: torch.Tensor, weight, bias, mean, rstd, layernorm: bool, act: int = -1):
+    """Returns (dx like x, dw or None, db or None); dw/db take the dtype of weight/bias (layernorm.py:207-208).
+    `act` >= 0: the backward of norm_fwd(..., act) (thn_norm_act_bwd)."""
     if not x.is_cuda:
         _native.require_gpu(x)
     x2, m, n, x_stride, reshaped = _flatten(x, 'input')
@@ -195,11 +204,22 @@ def norm_bwd(x: torch.Tensor, dout: torch.Tensor, weight, bias, mean, rstd, laye
             _workspace_bytes_cache[key] = nbytes
         stream = _stream_handle(index)
         workspace = _workspace(index, stream, nbytes, device) if nbytes > 0 else None
-        status = lib.thn_norm_bwd(
-            x2.data_ptr(), x_stride, d2.data_ptr(), d_stride, dx.data_ptr(), n,
-            0 if weight is None else weight.data_ptr(), 0 if mean is None else mean.data_ptr(), rstd.data_ptr(),
-            0 if dw is None else dw.data_ptr(), 0 if db is None else db.data_ptr(),
-            0 if workspace is None else workspace.data_ptr(), nbytes, m, n, x_code, w_code, stream)
+        if act < 0:
+            status = lib.thn_norm_bwd(
+                x2.data_ptr(), x_stride, d2.data_ptr(), d_stride, dx.data_ptr(), n,
+                0 if weight is None else weight.data_ptr(), 0 if mean is None else mean.data_ptr(), rstd.data_ptr(),
+                0 if dw is None else dw.data_ptr(), 0 if db is None else db.data_ptr(),
+                0 if workspace is None else workspace.data_ptr(), nbytes, m, n, x_code, w_code, stream)
+        else:
+            fwd_bias = bias if layernorm else None
+            if fwd_bias is not None and weight is not None and fwd_bias.dtype != weight.dtype:
+                fwd_bias = fwd_bias.to(weight.dtype)
+            status = lib.thn_norm_act_bwd(
+                x2.data_ptr(), x_stride, d2.data_ptr(), d_stride, dx.data_ptr(), n,
+                0 if weight is None else weight.data_ptr(), 0 if fwd_bias is None else fwd_bias.data_ptr(),
+                0 if mean is None else mean.data_ptr(), rstd.data_ptr(),
+                0 if dw is None else dw.data_ptr(), 0 if db is None else db.data_ptr(),
+                0 if workspace is None else workspace.data_ptr(), nbytes, m, n, act, x_code, w_code, stream)
     finally:
         if other_device:
             guard.__exit__(None, None, None)

@@ -45,6 +45,9 @@ SYMBOLS = {
                                  _i64, _i64, _i64, _f32, _i32, _vp]),
     'thn_act_fwd': (_i32, [_vp, _i64, _vp, _i64, _i64, _i64, _i32, _f32, _f32, _i32, _vp]),
     'thn_act_bwd': (_i32, [_vp, _i64, _vp, _i64, _vp, _i64, _i64, _i64, _i32, _f32, _f32, _i32, _vp]),
+    'thn_norm_act_fwd': (_i32, [_vp, _i64, _vp, _i64, _vp, _vp, _vp, _vp, _i64, _i64, _f32, _i32, _i32, _i32, _vp]),
+    'thn_norm_act_bwd': (_i32, [_vp, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64,
+                                _i32, _i32, _i32, _vp]),
     'thn_norm_set_launch_override': (_i32, [_i32, _i32, _i32, _i32, _i32]),
     'thn_norm_query_launch': (_i32, [_i32, _i32, _i64, _i64, _i32, ctypes.POINTER(ctypes.c_int32)]),
 }

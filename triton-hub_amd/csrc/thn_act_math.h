@@ -1,0 +1,148 @@
+// Element-wise activation formulas, forward and derivative, shared by the streaming activation kernels (thn_act.h)
+// and by the activation epilogue of the norm kernels (thn_kernels.h).  Each formula cites the line of the
+// reference it restates (TritonHub/Activations/*.py).
+#pragma once
+
+#include <type_traits>
+
+#include "thn_device.h"
+
+namespace thn {
+
+enum : int {
+    kGelu = 0, kGeluTanh = 1, kSilu = 2, kRelu = 3, kLeakyRelu = 4, kRelu6 = 5, kSigmoid = 6, kTanh = 7, kMish = 8,
+    kSoftplus = 9, kThreshold = 10, kNumActs = 11
+};
+
+__device__ __forceinline__ float log_c(float z) { return __logf(z); }
+__device__ __forceinline__ double log_c(double z) { return log(z); }
+
+// The float32 formulas below are written for the instruction budget of a streaming kernel: at 16-bit storage a
+// compute unit must finish an element in about 25 instruction slots to keep up with HBM, and the quarter-rate
+// v_exp_f32 / v_log_f32 / v_rcp_f32 cost four slots each.  Quotients use the hardware reciprocal (1 ulp) and a
+// multiplication instead of an IEEE division (10 slots); every result stays within a few float32 ulp of the exact
+// function, far inside the test tolerances.
+__device__ __forceinline__ float rcp_fast(float x) { return __builtin_amdgcn_rcpf(x); }
+
+// tanh(u) = sign(u) * (1 - t)/(1 + t) with t = exp(-2|u|): no overflow for any u.
+__device__ __forceinline__ float tanh_safe(float u) {
+    const float t = __expf(-2.0f * __builtin_fabsf(u));
+    const float r = (1.0f - t) * rcp_fast(1.0f + t);
+    return u < 0.0f ? -r : r;
+}
+
+__device__ __forceinline__ float sigmoid_f(float x) { return rcp_fast(1.0f + __expf(-x)); }
+
+// Phi(x) = 0.5*(1 + erf(x/sqrt 2)), the normal distribution function of GeLU, from the complementary error
+// function erfc(z) = t*exp(-z^2 + P(t)), t = 1/(1 + z/2), z >= 0 (Chebyshev fit, relative error below 1.2e-7 for
+// every z, Numerical Recipes 6.2): branch free, a third of the instructions of the library erff, and accurate in
+// the negative tail, where 1 + erf(..) cancels.
+__device__ __forceinline__ float normal_cdf(float x) {
+    const float z = __builtin_fabsf(x) * 0.70710678118654752440f;
+    const float t = rcp_fast(__builtin_fmaf(0.5f, z, 1.0f));
+    float p = 0.17087277f;
+    p = __builtin_fmaf(p, t, -0.82215223f);
+    p = __builtin_fmaf(p, t, 1.48851587f);
+    p = __builtin_fmaf(p, t, -1.13520398f);
+    p = __builtin_fmaf(p, t, 0.27886807f);
+    p = __builtin_fmaf(p, t, -0.18628806f);
+    p = __builtin_fmaf(p, t, 0.09678418f);
+    p = __builtin_fmaf(p, t, 0.37409196f);
+    p = __builtin_fmaf(p, t, 1.00002368f);
+    p = __builtin_fmaf(p, t, -1.26551223f);
+    const float half_erfc = 0.5f * t * __expf(__builtin_fmaf(-z, z, p));
+    return x < 0.0f ? half_erfc : 1.0f - half_erfc;
+}
+
+// Mish needs t = tanh(softplus(x)) with softplus(x) = x > 20 ? x : log(1 + e^x) (mish.py:19-22).  With w = e^x and
+// n = w*(w + 2):  tanh(log(1 + w)) = n/(n + 2)  and  1 - t^2 = 4*(n + 1)/(n + 2)^2 : one exponential, one
+// reciprocal, no cancellation for very negative x (where log(1 + e^x) rounds to 0 in float32).  Above 20 the
+// reference's branch gives tanh(x), which is 1 in float32.
+struct MishParts { float t, one_minus_t2, sig; };
+__device__ __forceinline__ MishParts mish_parts(float x) {
+    const float w = __expf(x < 20.0f ? x : 20.0f);
+    const float n = w * (w + 2.0f);
+    const float r = rcp_fast(n + 2.0f);
+    MishParts m;
+    const bool big = x > 20.0f;
+    m.t = big ? 1.0f : n * r;
+    m.one_minus_t2 = big ? 0.0f : 4.0f * (n + 1.0f) * r * r;
+    m.sig = big ? 1.0f : w * rcp_fast(1.0f + w);          // sigmoid(x) = w/(1 + w); 1 in float32 above 20
+    return m;
+}
+
+template <int ACT, typename C>
+__device__ __forceinline__ C act_fwd(C x, C p0, C p1) {
+    if constexpr (ACT == kGelu) {
+        return x * normal_cdf(x);                                                          // gelu.py:28
+    } else if constexpr (ACT == kGeluTanh) {
+        const float u = 0.79788456080286535588f * (x + 0.044715f * x * x * x);            // gelu.py:23
+        return 0.5f * x * (1.0f + tanh_safe(u));                                           // gelu.py:26
+    } else if constexpr (ACT == kSilu) {
+        return x * sigmoid_f(x);                                                           // silu.py:19
+    } else if constexpr (ACT == kRelu) {
+        return x > C(0) ? x : C(0);                                                        // relu.py:19
+    } else if constexpr (ACT == kLeakyRelu) {
+        return x > C(0) ? x : p0 * x;                                                      // leaky_relu.py:20
+    } else if constexpr (ACT == kRelu6) {
+        const C r = x > C(0) ? x : C(0);                                                   // relu6.py:19-20
+        return r < C(6) ? r : C(6);
+    } else if constexpr (ACT == kSigmoid) {
+        return sigmoid_f(x);                                                               // sigmoid.py:19
+    } else if constexpr (ACT == kTanh) {
+        return tanh_safe(x);                                                               // tanh.py:19-21
+    } else if constexpr (ACT == kMish) {
+        return x * mish_parts(x).t;                                                        // mish.py:19-23
+    } else if constexpr (ACT == kSoftplus) {
+        if constexpr (std::is_same<C, float>::value) {                                     // softplus.py:21
+            return x * p0 > p1 ? x : __logf(1.0f + __expf(p0 * x)) * rcp_fast(p0);
+        } else {
+            return x * p0 > p1 ? x : log_c(C(1) + exp_c(p0 * x)) / p0;
+        }
+    } else {
+        return x > p0 ? x : p1;                                                            // threshold.py:20
+    }
+}
+
+// `s` is the saved tensor: the forward's input, or its output for Sigmoid and Tanh.
+template <int ACT, typename C>
+__device__ __forceinline__ C act_bwd(C s, C g, C p0, C p1) {
+    if constexpr (ACT == kGelu) {
+        const float pdf = __expf(-0.5f * s * s) * 0.39894228040143267794f;                 // gelu.py:77-80
+        return g * __builtin_fmaf(s, pdf, normal_cdf(s));
+    } else if constexpr (ACT == kGeluTanh) {
+        const float k = 0.79788456080286535588f;                                           // gelu.py:71-75
+        const float t = tanh_safe(k * (s + 0.044715f * s * s * s));
+        const float gp = k * (1.0f + 3.0f * 0.044715f * s * s);
+        const float sech2 = 1.0f - t * t;                          // exactly 0 once |s| > ~6: keeps 0 * inf out for huge |s|
+        const float tail = sech2 == 0.0f ? 0.0f : s * sech2 * gp;
+        return g * (0.5f * (1.0f + t + tail));
+    } else if constexpr (ACT == kSilu) {
+        const float sg = sigmoid_f(s);                                                     // silu.py:56-57
+        return g * (sg * (1.0f + s * (1.0f - sg)));
+    } else if constexpr (ACT == kRelu) {
+        return s > C(0) ? g : C(0);                                                        // relu.py:56
+    } else if constexpr (ACT == kLeakyRelu) {
+        return s > C(0) ? g : p0 * g;                                                      // leaky_relu.py:59
+    } else if constexpr (ACT == kRelu6) {
+        const C r = s > C(0) ? g : C(0);                                                   // relu6.py:57-58
+        return s < C(6) ? r : C(0);
+    } else if constexpr (ACT == kSigmoid) {
+        return g * (s * (1.0f - s));                                                       // sigmoid.py:56
+    } else if constexpr (ACT == kTanh) {
+        return g * (1.0f - s * s);                                                         // tanh.py:58
+    } else if constexpr (ACT == kMish) {
+        const MishParts m = mish_parts(s);                                                 // mish.py:60-66
+        return g * (m.t + s * m.one_minus_t2 * m.sig);
+    } else if constexpr (ACT == kSoftplus) {
+        if constexpr (std::is_same<C, float>::value) {                                     // softplus.py:62
+            return s * p0 > p1 ? g : g * rcp_fast(1.0f + __expf(-p0 * s));
+        } else {
+            return s * p0 > p1 ? g : g / (C(1) + exp_c(-p0 * s));
+        }
+    } else {
+        return s > p0 ? g : C(0);                                                          // threshold.py:59
+    }
+}
+
+}  // namespace thn

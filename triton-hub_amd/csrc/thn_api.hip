@@ -7,6 +7,7 @@
 #include <unordered_map>
 
 #include "thn_dispatch.h"
+#include "thn_fused_dispatch.h"
 #include "thn_reduce.h"
 #include "thn_act_dispatch.h"
 #include "thn_pnorm_dispatch.h"
@@ -28,7 +29,7 @@ using thn::SoftmaxFwdArgs;
 // `which` throughout this file: the kernel family a launch belongs to.
 enum : int {
     kNormFwd = 0, kNormBwd = 1, kSoftmaxFwd = 2, kSoftmaxBwd = 3, kPnormFwd = 4, kPnormBwd = 5, kNormalizeBwd = 6,
-    kActFwd = 7, kActBwd = 8, kFamilies = 9
+    kActFwd = 7, kActBwd = 8, kFusedFwd = 9, kFusedBwd = 10, kFamilies = 11
 };
 
 constexpr int kMaxDevices = 64;
@@ -75,6 +76,10 @@ bool shape_compiled(int which, bool aligned, Shape s) {
         THN_SCALAR_SHAPES(THN_MATCH)
     } else if (which == kNormBwd) {
         THN_BWD_SHAPES(THN_MATCH)
+    } else if (which == kFusedFwd) {
+        THN_FUSED_FWD_SHAPES(THN_MATCH)
+    } else if (which == kFusedBwd) {
+        THN_FUSED_BWD_SHAPES(THN_MATCH)
     } else if (which >= kPnormFwd) {
         THN_ROW_SHAPES(THN_MATCH)
     } else {
@@ -119,6 +124,29 @@ int launch_softmax_bwd(int dtype, bool is_log, bool aligned, Shape s, const Soft
         case THN_F16: return thn::launch_softmax_bwd_f16(is_log, aligned, s, a, grid, st, occ);
         case THN_BF16: return thn::launch_softmax_bwd_bf16(is_log, aligned, s, a, grid, st, occ);
         default: return thn::launch_softmax_bwd_f64(is_log, aligned, s, a, grid, st, occ);
+    }
+}
+
+// `variant` of the fused families: bit 0 = LayerNorm, bits 1.. = the activation code.
+int launch_fused_fwd(int dtype, int variant, bool aligned, Shape s, const FwdArgs& a, int grid, hipStream_t st, int* occ) {
+    const bool ln = (variant & 1) != 0;
+    const int act = variant >> 1;
+    switch (dtype) {
+        case THN_F32: return thn::launch_fused_fwd_f32(ln, act, aligned, s, a, grid, st, occ);
+        case THN_F16: return thn::launch_fused_fwd_f16(ln, act, aligned, s, a, grid, st, occ);
+        case THN_BF16: return thn::launch_fused_fwd_bf16(ln, act, aligned, s, a, grid, st, occ);
+        default: return thn::launch_fused_fwd_f64(ln, act, aligned, s, a, grid, st, occ);
+    }
+}
+
+int launch_fused_bwd(int dtype, int variant, bool aligned, Shape s, const BwdArgs& a, int grid, hipStream_t st, int* occ) {
+    const bool ln = (variant & 1) != 0;
+    const int act = variant >> 1;
+    switch (dtype) {
+        case THN_F32: return thn::launch_fused_bwd_f32(ln, act, aligned, s, a, grid, st, occ);
+        case THN_F16: return thn::launch_fused_bwd_f16(ln, act, aligned, s, a, grid, st, occ);
+        case THN_BF16: return thn::launch_fused_bwd_bf16(ln, act, aligned, s, a, grid, st, occ);
+        default: return thn::launch_fused_bwd_f64(ln, act, aligned, s, a, grid, st, occ);
     }
 }
 
@@ -186,6 +214,12 @@ int occupancy(int which, int dtype, int ln, bool aligned, Shape s) {
     } else if (which == kSoftmaxBwd) {
         SoftmaxBwdArgs dummy{};
         rc = launch_softmax_bwd(dtype, ln, aligned, s, dummy, 0, nullptr, &occ);
+    } else if (which == kFusedFwd) {
+        FwdArgs dummy{};
+        rc = launch_fused_fwd(dtype, ln, aligned, s, dummy, 0, nullptr, &occ);
+    } else if (which == kFusedBwd) {
+        BwdArgs dummy{};
+        rc = launch_fused_bwd(dtype, ln, aligned, s, dummy, 0, nullptr, &occ);
     } else if (which == kPnormFwd) {
         PnormFwdArgs dummy{};
         rc = launch_pnorm_fwd(dtype, ln, aligned, s, dummy, 0, nullptr, &occ);
@@ -234,6 +268,7 @@ Shape heuristic_shape(int which, int ln, bool aligned, int n_vecs) {
     // except for 2 KiB rows, where one full wave per row (2 x 64) is 8 % slower than half a wave (4 x 32).
     if (aligned && which == kSoftmaxBwd && n_vecs <= 2048 && !(n_vecs > 64 && n_vecs <= 128)) kmax = 2;
     if (aligned && which == kNormalizeBwd && n_vecs <= 2048) kmax = 2;    // two or three input streams
+    if (aligned && which == kFusedBwd && n_vecs <= 2048) kmax = 2;        // bias and pre-activation are live too
     Shape s{4, 1024, 1024};
     for (int tpr : kTprList) {
         if (static_cast<int64_t>(tpr) * kmax >= n_vecs) {
@@ -248,7 +283,7 @@ Shape heuristic_shape(int which, int ln, bool aligned, int n_vecs) {
     }
     s.k = ceil_div(n_vecs, s.tpr);
     if (s.k == 3 && s.tpr < 64) s.k = 4;     // K = 3 is only compiled for TPR >= 64
-    if (which != kNormBwd) s.block = s.tpr > 256 ? s.tpr : 256;
+    if (which != kNormBwd && which != kFusedBwd) s.block = s.tpr > 256 ? s.tpr : 256;
     else s.block = s.tpr >= 128 ? (s.tpr > 512 ? s.tpr : 512) : 256;
     return s;
 }
@@ -279,7 +314,7 @@ int plan_launch(int which, int ln, bool aligned, int64_t M, int64_t N, int dtype
     int bpc = occupancy(which, dtype, ln, aligned, s);
     // The p-norm families in 256-thread workgroups (rows up to 16 KiB) measured 5-25 % faster with two workgroups
     // per compute unit; everything else with one.
-    const int family_bpc = (which >= kPnormFwd && s.block <= 256) ? 2 : kDefaultBlocksPerCu;
+    const int family_bpc = (which >= kPnormFwd && which <= kNormalizeBwd && s.block <= 256) ? 2 : kDefaultBlocksPerCu;
     const int cap = ov.bpc.load() > 0 ? ov.bpc.load() : family_bpc;
     if (cap < bpc) bpc = cap;
     const int rows_per_block = s.block / s.tpr;
@@ -301,6 +336,115 @@ bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) ==
 
 int64_t partial_pitch(int64_t N) { return (N + 63) / 64 * 64; }
 
+
+bool fusable(int act) { return act == thn::kGelu || act == thn::kGeluTanh || act == thn::kSilu || act == thn::kRelu; }
+
+// thn_norm_fwd (act == kNoAct) and thn_norm_act_fwd.
+int norm_forward(const void* x, int64_t x_row_stride, void* y, int64_t y_row_stride, const void* w, const void* b,
+                 float* mean, float* rstd, int64_t M, int64_t N, float eps, int act, int x_dtype, int w_dtype,
+                 void* stream) {
+    const int bytes = elem_bytes(x_dtype);
+    if (bytes == 0 || ((w != nullptr || b != nullptr) && elem_bytes(w_dtype) == 0)) return THN_E_DTYPE;
+    if (M < 0 || N <= 0) return THN_E_SHAPE;
+    if (N * bytes > kMaxRowBytes) return THN_E_FEATURE_DIM;
+    if (M == 0) return THN_OK;
+    if (x == nullptr || y == nullptr || rstd == nullptr) return THN_E_NULL;
+    const bool ln = mean != nullptr;
+    if (!ln && b != nullptr) return THN_E_SHAPE;          // RMSNorm has no bias (rmsnorm.py:13-22)
+    if (x_row_stride < N || y_row_stride < N) return THN_E_SHAPE;
+
+    const int vec_elems = 16 / bytes;
+    const bool aligned = (N % vec_elems) == 0 && aligned16(x) && aligned16(y) && aligned16(w) && aligned16(b) &&
+                         (x_row_stride * bytes) % 16 == 0 && (y_row_stride * bytes) % 16 == 0;
+    Plan p;
+    const bool fused = act != thn::kNoAct;
+    const int rc = plan_launch(fused ? kFusedFwd : kNormFwd, fused ? ((ln ? 1 : 0) | (act << 1)) : (ln ? 1 : 0), aligned, M, N,
+                               x_dtype, &p);
+    if (rc != THN_OK) return rc;
+
+    FwdArgs a{};
+    a.x = static_cast<const char*>(x);
+    a.y = static_cast<char*>(y);
+    a.w = w;
+    a.b = b;
+    a.mean = mean;
+    a.rstd = rstd;
+    a.x_stride_bytes = x_row_stride * bytes;
+    a.y_stride_bytes = y_row_stride * bytes;
+    a.M = M;
+    a.n_cols = static_cast<int>(N);
+    a.n_vecs = p.n_vecs;
+    a.w_dtype = w_dtype;
+    a.eps = eps;
+    a.inv_n = 1.0f / static_cast<float>(N);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const int lrc = fused ? launch_fused_fwd(x_dtype, (ln ? 1 : 0) | (act << 1), aligned, p.s, a, p.grid, st, nullptr)
+                          : launch_fwd(x_dtype, ln, aligned, p.s, a, p.grid, st, nullptr);
+    if (lrc > 0) return THN_E_SHAPE;
+    return lrc == 0 ? THN_OK : THN_E_LAUNCH;
+}
+
+// thn_norm_bwd_dx_partials (act == kNoAct, b unused) and the first stage of thn_norm_act_bwd.
+int norm_backward_stage1(const void* x, int64_t x_row_stride, const void* dy, int64_t dy_row_stride, void* dx,
+                         int64_t dx_row_stride, const void* w, const void* b, const float* mean, const float* rstd,
+                         int want_dw, int want_db, void* workspace, int64_t workspace_bytes, int32_t* num_partials,
+                         int64_t M, int64_t N, int act, int x_dtype, int w_dtype, void* stream) {
+    const int bytes = elem_bytes(x_dtype);
+    if (bytes == 0 || (w != nullptr && elem_bytes(w_dtype) == 0)) return THN_E_DTYPE;
+    if (M < 0 || N <= 0) return THN_E_SHAPE;
+    if (N * bytes > kMaxRowBytes) return THN_E_FEATURE_DIM;
+    if (num_partials != nullptr) *num_partials = 0;
+    if (M == 0) return THN_OK;
+    if (x == nullptr || dy == nullptr || dx == nullptr || rstd == nullptr) return THN_E_NULL;
+    if (x_row_stride < N || dy_row_stride < N || dx_row_stride < N) return THN_E_SHAPE;
+    const bool ln = mean != nullptr;
+    if (!ln) want_db = 0;
+    const int n_grads = (want_dw ? 1 : 0) + (want_db ? 1 : 0);
+    if (n_grads > 0 && (workspace == nullptr || num_partials == nullptr)) return THN_E_NULL;
+    if (n_grads > 0 && !aligned16(workspace)) return THN_E_WORKSPACE;
+
+    const int vec_elems = 16 / bytes;
+    const bool fused = act != thn::kNoAct;
+    const bool aligned = (N % vec_elems) == 0 && aligned16(x) && aligned16(dy) && aligned16(dx) && aligned16(w) &&
+                         (!fused || aligned16(b)) &&
+                         (x_row_stride * bytes) % 16 == 0 && (dy_row_stride * bytes) % 16 == 0 &&
+                         (dx_row_stride * bytes) % 16 == 0;
+    Plan p;
+    const int variant = fused ? ((ln ? 1 : 0) | (act << 1)) : (ln ? 1 : 0);
+    const int rc = plan_launch(fused ? kFusedBwd : kNormBwd, variant, aligned, M, N, x_dtype, &p);
+    if (rc != THN_OK) return rc;
+    const int64_t pitch = partial_pitch(N);
+    const int64_t need = n_grads * static_cast<int64_t>(p.grid) * pitch * static_cast<int64_t>(sizeof(float));
+    if (workspace_bytes < need) return THN_E_WORKSPACE;
+
+    BwdArgs a{};
+    a.x = static_cast<const char*>(x);
+    a.dy = static_cast<const char*>(dy);
+    a.dx = static_cast<char*>(dx);
+    a.w = w;
+    a.b = fused ? b : nullptr;
+    a.mean = mean;
+    a.rstd = rstd;
+    float* ws = static_cast<float*>(workspace);
+    a.dw_part = want_dw ? ws : nullptr;
+    a.db_part = want_db ? ws + (want_dw ? static_cast<int64_t>(p.grid) * pitch : 0) : nullptr;
+    a.x_stride_bytes = x_row_stride * bytes;
+    a.dy_stride_bytes = dy_row_stride * bytes;
+    a.dx_stride_bytes = dx_row_stride * bytes;
+    a.M = M;
+    a.part_pitch = pitch;
+    a.n_cols = static_cast<int>(N);
+    a.n_vecs = p.n_vecs;
+    a.w_dtype = w_dtype;
+    a.inv_n = 1.0f / static_cast<float>(N);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const int lrc = fused ? launch_fused_bwd(x_dtype, variant, aligned, p.s, a, p.grid, st, nullptr)
+                          : launch_bwd(x_dtype, ln, aligned, p.s, a, p.grid, st, nullptr);
+    if (lrc > 0) return THN_E_SHAPE;
+    if (lrc < 0) return THN_E_LAUNCH;
+    if (num_partials != nullptr) *num_partials = p.grid;
+    return THN_OK;
+}
 
 // ---- row p-norm / normalize ---------------------------------------------------------------------------------
 struct RowProblem {
@@ -514,12 +658,15 @@ int thn_norm_set_launch_override(int which, int vecs_per_thread, int threads_per
 }
 
 int thn_norm_query_launch(int which, int is_layernorm, int64_t M, int64_t N, int x_dtype, int32_t shape[5]) {
-    if (which < 0 || which >= kActFwd || shape == nullptr) return THN_E_SHAPE;    // element-wise kernels have no row shape
+    if (which < 0 || which >= kFamilies || which == kActFwd || which == kActBwd || shape == nullptr) {
+        return THN_E_SHAPE;                                     // the element-wise kernels have no row shape
+    }
     const int bytes = elem_bytes(x_dtype);
     if (bytes == 0) return THN_E_DTYPE;
     Plan p;
     const bool aligned = N > 0 && (N % (16 / bytes)) == 0;
-    const int flavour = which >= kPnormFwd ? static_cast<int>(thn::kP2) : (is_layernorm != 0 ? 1 : 0);
+    int flavour = is_layernorm != 0 ? 1 : 0;
+    if (which >= kPnormFwd && which <= kNormalizeBwd) flavour = thn::kP2;
     const int rc = plan_launch(which, flavour, aligned, M, N, x_dtype, &p);
     if (rc != THN_OK) return rc;
     shape[0] = p.s.k;
@@ -533,41 +680,30 @@ int thn_norm_query_launch(int which, int is_layernorm, int64_t M, int64_t N, int
 int thn_norm_fwd(const void* x, int64_t x_row_stride, void* y, int64_t y_row_stride, const void* w,
                  const void* b, float* mean, float* rstd, int64_t M, int64_t N, float eps, int x_dtype,
                  int w_dtype, void* stream) {
-    const int bytes = elem_bytes(x_dtype);
-    if (bytes == 0 || ((w != nullptr || b != nullptr) && elem_bytes(w_dtype) == 0)) return THN_E_DTYPE;
-    if (M < 0 || N <= 0) return THN_E_SHAPE;
-    if (N * bytes > kMaxRowBytes) return THN_E_FEATURE_DIM;
-    if (M == 0) return THN_OK;
-    if (x == nullptr || y == nullptr || rstd == nullptr) return THN_E_NULL;
-    const bool ln = mean != nullptr;
-    if (!ln && b != nullptr) return THN_E_SHAPE;          // RMSNorm has no bias (rmsnorm.py:13-22)
-    if (x_row_stride < N || y_row_stride < N) return THN_E_SHAPE;
+    return norm_forward(x, x_row_stride, y, y_row_stride, w, b, mean, rstd, M, N, eps, thn::kNoAct, x_dtype, w_dtype,
+                        stream);
+}
 
-    const int vec_elems = 16 / bytes;
-    const bool aligned = (N % vec_elems) == 0 && aligned16(x) && aligned16(y) && aligned16(w) && aligned16(b) &&
-                         (x_row_stride * bytes) % 16 == 0 && (y_row_stride * bytes) % 16 == 0;
-    Plan p;
-    const int rc = plan_launch(kNormFwd, ln, aligned, M, N, x_dtype, &p);
-    if (rc != THN_OK) return rc;
+int thn_norm_act_fwd(const void* x, int64_t x_row_stride, void* y, int64_t y_row_stride, const void* w,
+                     const void* b, float* mean, float* rstd, int64_t M, int64_t N, float eps, int act,
+                     int x_dtype, int w_dtype, void* stream) {
+    if (!fusable(act)) return THN_E_SHAPE;
+    return norm_forward(x, x_row_stride, y, y_row_stride, w, b, mean, rstd, M, N, eps, act, x_dtype, w_dtype, stream);
+}
 
-    FwdArgs a{};
-    a.x = static_cast<const char*>(x);
-    a.y = static_cast<char*>(y);
-    a.w = w;
-    a.b = b;
-    a.mean = mean;
-    a.rstd = rstd;
-    a.x_stride_bytes = x_row_stride * bytes;
-    a.y_stride_bytes = y_row_stride * bytes;
-    a.M = M;
-    a.n_cols = static_cast<int>(N);
-    a.n_vecs = p.n_vecs;
-    a.w_dtype = w_dtype;
-    a.eps = eps;
-    a.inv_n = 1.0f / static_cast<float>(N);
-    const int lrc = launch_fwd(x_dtype, ln, aligned, p.s, a, p.grid, static_cast<hipStream_t>(stream), nullptr);
-    if (lrc > 0) return THN_E_SHAPE;
-    return lrc == 0 ? THN_OK : THN_E_LAUNCH;
+int thn_norm_act_bwd(const void* x, int64_t x_row_stride, const void* dy, int64_t dy_row_stride, void* dx,
+                     int64_t dx_row_stride, const void* w, const void* b, const float* mean, const float* rstd,
+                     void* dw, void* db, void* workspace, int64_t workspace_bytes, int64_t M, int64_t N, int act,
+                     int x_dtype, int w_dtype, void* stream) {
+    if (!fusable(act)) return THN_E_SHAPE;
+    if ((dw != nullptr || db != nullptr || b != nullptr) && elem_bytes(w_dtype) == 0) return THN_E_DTYPE;
+    if (mean == nullptr && (db != nullptr || b != nullptr)) return THN_E_SHAPE;     // RMSNorm has no bias
+    int32_t parts = 0;
+    const int rc = norm_backward_stage1(x, x_row_stride, dy, dy_row_stride, dx, dx_row_stride, w, b, mean, rstd,
+                                        dw != nullptr, db != nullptr, workspace, workspace_bytes, &parts, M, N, act,
+                                        x_dtype, w_dtype, stream);
+    if (rc != THN_OK || M == 0 || (dw == nullptr && db == nullptr)) return rc;
+    return thn_norm_bwd_reduce_partials(workspace, parts, dw, db, N, w_dtype, stream);
 }
 
 int64_t thn_norm_bwd_workspace_bytes(int64_t M, int64_t N, int want_dw, int want_db, int x_dtype) {
@@ -591,55 +727,9 @@ int thn_norm_bwd_dx_partials(const void* x, int64_t x_row_stride, const void* dy
                              const float* rstd, int want_dw, int want_db, void* workspace,
                              int64_t workspace_bytes, int32_t* num_partials, int64_t M, int64_t N,
                              int x_dtype, int w_dtype, void* stream) {
-    const int bytes = elem_bytes(x_dtype);
-    if (bytes == 0 || (w != nullptr && elem_bytes(w_dtype) == 0)) return THN_E_DTYPE;
-    if (M < 0 || N <= 0) return THN_E_SHAPE;
-    if (N * bytes > kMaxRowBytes) return THN_E_FEATURE_DIM;
-    if (num_partials != nullptr) *num_partials = 0;
-    if (M == 0) return THN_OK;
-    if (x == nullptr || dy == nullptr || dx == nullptr || rstd == nullptr) return THN_E_NULL;
-    if (x_row_stride < N || dy_row_stride < N || dx_row_stride < N) return THN_E_SHAPE;
-    const bool ln = mean != nullptr;
-    if (!ln) want_db = 0;
-    const int n_grads = (want_dw ? 1 : 0) + (want_db ? 1 : 0);
-    if (n_grads > 0 && (workspace == nullptr || num_partials == nullptr)) return THN_E_NULL;
-    if (n_grads > 0 && !aligned16(workspace)) return THN_E_WORKSPACE;
-
-    const int vec_elems = 16 / bytes;
-    const bool aligned = (N % vec_elems) == 0 && aligned16(x) && aligned16(dy) && aligned16(dx) && aligned16(w) &&
-                         (x_row_stride * bytes) % 16 == 0 && (dy_row_stride * bytes) % 16 == 0 &&
-                         (dx_row_stride * bytes) % 16 == 0;
-    Plan p;
-    const int rc = plan_launch(kNormBwd, ln, aligned, M, N, x_dtype, &p);
-    if (rc != THN_OK) return rc;
-    const int64_t pitch = partial_pitch(N);
-    const int64_t need = n_grads * static_cast<int64_t>(p.grid) * pitch * static_cast<int64_t>(sizeof(float));
-    if (workspace_bytes < need) return THN_E_WORKSPACE;
-
-    BwdArgs a{};
-    a.x = static_cast<const char*>(x);
-    a.dy = static_cast<const char*>(dy);
-    a.dx = static_cast<char*>(dx);
-    a.w = w;
-    a.mean = mean;
-    a.rstd = rstd;
-    float* ws = static_cast<float*>(workspace);
-    a.dw_part = want_dw ? ws : nullptr;
-    a.db_part = want_db ? ws + (want_dw ? static_cast<int64_t>(p.grid) * pitch : 0) : nullptr;
-    a.x_stride_bytes = x_row_stride * bytes;
-    a.dy_stride_bytes = dy_row_stride * bytes;
-    a.dx_stride_bytes = dx_row_stride * bytes;
-    a.M = M;
-    a.part_pitch = pitch;
-    a.n_cols = static_cast<int>(N);
-    a.n_vecs = p.n_vecs;
-    a.w_dtype = w_dtype;
-    a.inv_n = 1.0f / static_cast<float>(N);
-    const int lrc = launch_bwd(x_dtype, ln, aligned, p.s, a, p.grid, static_cast<hipStream_t>(stream), nullptr);
-    if (lrc > 0) return THN_E_SHAPE;
-    if (lrc < 0) return THN_E_LAUNCH;
-    if (num_partials != nullptr) *num_partials = p.grid;
-    return THN_OK;
+    return norm_backward_stage1(x, x_row_stride, dy, dy_row_stride, dx, dx_row_stride, w, nullptr, mean, rstd, want_dw,
+                                want_db, workspace, workspace_bytes, num_partials, M, N, thn::kNoAct, x_dtype, w_dtype,
+                                stream);
 }
 
 // Workspace layout: dW partial rows first (when wanted), dB partial rows after them.  A caller that wants

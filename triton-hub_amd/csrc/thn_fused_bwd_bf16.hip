@@ -1,0 +1,6 @@
+// Norm backward kernels for an activation epilogue, BF16 storage.
+#include "thn_fused_dispatch.h"
+
+namespace thn {
+THN_DEFINE_FUSED_BWD_LAUNCHER(bf16, BF16)
+}  // namespace thn

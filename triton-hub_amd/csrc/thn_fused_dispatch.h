@@ -1,0 +1,79 @@
+// Norm kernels with an activation epilogue: run-time (dtype, LayerNorm / RMSNorm, activation, shape) -> compiled
+// instance; two translation units per storage type (thn_fused_fwd_<dtype>.hip, thn_fused_bwd_<dtype>.hip).
+#pragma once
+
+#include "thn_dispatch.h"
+
+namespace thn {
+
+// Activations that can ride on a norm kernel: parameter free, and their backward needs only the pre-activation.
+#define THN_FUSED_ACTS(X) X(kGelu) X(kGeluTanh) X(kSilu) X(kRelu)
+
+// X(K, TPR, BLOCK).  Forward: the fewest threads per row with at most 4 vectors each, as the plain forward.
+#define THN_FUSED_FWD_SHAPES(X)                                                      \
+    X(1, 8, 256) X(2, 8, 256) X(4, 8, 256) X(4, 16, 256) X(4, 32, 256)               \
+    X(3, 64, 256) X(4, 64, 256) X(3, 128, 256) X(4, 128, 256)                        \
+    X(3, 256, 256) X(4, 256, 256) X(3, 512, 512) X(4, 512, 512)                      \
+    X(3, 1024, 1024) X(4, 1024, 1024)
+
+// Backward: at most 2 vectors per thread (the bias and the recomputed pre-activation are live too), 512-thread
+// workgroups once a row spans two waves, 3 or 4 vectors only where 1024 threads cannot cover the row otherwise.
+#define THN_FUSED_BWD_SHAPES(X)                                                      \
+    X(1, 8, 256) X(2, 8, 256) X(2, 16, 256) X(2, 32, 256) X(2, 64, 256)              \
+    X(2, 128, 512) X(2, 256, 512) X(2, 512, 512)                                     \
+    X(2, 1024, 1024) X(3, 1024, 1024) X(4, 1024, 1024)
+
+#define THN_DECLARE_FUSED_LAUNCHERS(NAME)                                                                      \
+    int launch_fused_fwd_##NAME(bool ln, int act, bool aligned, Shape s, const FwdArgs& a, int grid,           \
+                                hipStream_t st, int* occupancy);                                               \
+    int launch_fused_bwd_##NAME(bool ln, int act, bool aligned, Shape s, const BwdArgs& a, int grid,           \
+                                hipStream_t st, int* occupancy);
+
+THN_DECLARE_FUSED_LAUNCHERS(f32)
+THN_DECLARE_FUSED_LAUNCHERS(f16)
+THN_DECLARE_FUSED_LAUNCHERS(bf16)
+THN_DECLARE_FUSED_LAUNCHERS(f64)
+
+#define THN_FUSED_ACT_CASE(KERNEL, ARGS_T, AL, K_, TPR_, BLOCK_, A)                                           \
+    if (act == A) {                                                                                            \
+        return ln ? run_kernel<ARGS_T>(KERNEL<T, true, K_, TPR_, BLOCK_, AL, A>, a, grid, BLOCK_, st, occupancy) \
+                  : run_kernel<ARGS_T>(KERNEL<T, false, K_, TPR_, BLOCK_, AL, A>, a, grid, BLOCK_, st, occupancy); \
+    }
+#define THN_FUSED_CASE(KERNEL, ARGS_T, AL, K_, TPR_, BLOCK_)                                                   \
+    if (s.k == K_ && s.tpr == TPR_ && s.block == BLOCK_) {                                                     \
+        THN_FUSED_ACT_CASE(KERNEL, ARGS_T, AL, K_, TPR_, BLOCK_, kGelu)                                        \
+        THN_FUSED_ACT_CASE(KERNEL, ARGS_T, AL, K_, TPR_, BLOCK_, kGeluTanh)                                    \
+        THN_FUSED_ACT_CASE(KERNEL, ARGS_T, AL, K_, TPR_, BLOCK_, kSilu)                                        \
+        THN_FUSED_ACT_CASE(KERNEL, ARGS_T, AL, K_, TPR_, BLOCK_, kRelu)                                        \
+        return 1;                                                                                              \
+    }
+#define THN_FF_AL(K_, TPR_, BLOCK_) THN_FUSED_CASE(norm_fwd_kernel, FwdArgs, true, K_, TPR_, BLOCK_)
+#define THN_FF_SC(K_, TPR_, BLOCK_) THN_FUSED_CASE(norm_fwd_kernel, FwdArgs, false, K_, TPR_, BLOCK_)
+#define THN_FB_AL(K_, TPR_, BLOCK_) THN_FUSED_CASE(norm_bwd_kernel, BwdArgs, true, K_, TPR_, BLOCK_)
+#define THN_FB_SC(K_, TPR_, BLOCK_) THN_FUSED_CASE(norm_bwd_kernel, BwdArgs, false, K_, TPR_, BLOCK_)
+
+#define THN_DEFINE_FUSED_FWD_LAUNCHER(NAME, TYPE)                                                              \
+    int launch_fused_fwd_##NAME(bool ln, int act, bool aligned, Shape s, const FwdArgs& a, int grid,           \
+                                hipStream_t st, int* occupancy) {                                              \
+        using T = TYPE;                                                                                        \
+        if (aligned) {                                                                                         \
+            THN_FUSED_FWD_SHAPES(THN_FF_AL)                                                                    \
+        } else {                                                                                               \
+            THN_SCALAR_SHAPES(THN_FF_SC)                                                                       \
+        }                                                                                                      \
+        return 1;                                                                                              \
+    }
+
+#define THN_DEFINE_FUSED_BWD_LAUNCHER(NAME, TYPE)                                                              \
+    int launch_fused_bwd_##NAME(bool ln, int act, bool aligned, Shape s, const BwdArgs& a, int grid,           \
+                                hipStream_t st, int* occupancy) {                                              \
+        using T = TYPE;                                                                                        \
+        if (aligned) {                                                                                         \
+            THN_FUSED_BWD_SHAPES(THN_FB_AL)                                                                    \
+        } else {                                                                                               \
+            THN_SCALAR_SHAPES(THN_FB_SC)                                                                       \
+        }                                                                                                      \
+        return 1;                                                                                              \
+    }
+
+}  // namespace thn

@@ -1,0 +1,6 @@
+// Norm forward kernels with an activation epilogue, F16 storage.
+#include "thn_fused_dispatch.h"
+
+namespace thn {
+THN_DEFINE_FUSED_FWD_LAUNCHER(f16, F16)
+}  // namespace thn

@@ -1,0 +1,6 @@
+// Norm forward kernels with an activation epilogue, F32 storage.
+#include "thn_fused_dispatch.h"
+
+namespace thn {
+THN_DEFINE_FUSED_FWD_LAUNCHER(f32, F32)
+}  // namespace thn

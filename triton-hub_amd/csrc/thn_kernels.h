@@ -20,9 +20,12 @@
 
 #include <type_traits>
 
+#include "thn_act_math.h"
 #include "thn_device.h"
 
 namespace thn {
+
+constexpr int kNoAct = -1;   // ACT of the norm kernels: no activation epilogue
 
 struct FwdArgs {
     const char* x;
@@ -46,6 +49,7 @@ struct BwdArgs {
     const char* dy;
     char* dx;
     const void* w;      // may be null
+    const void* b;      // may be null; read only by the activation-epilogue instances (to recompute the pre-activation)
     const float* mean;  // null for RMSNorm
     const float* rstd;
     float* dw_part;     // (gridDim.x, part_pitch) float32, may be null
@@ -86,7 +90,9 @@ __device__ __forceinline__ void store_row_vec(char* rowp, int voff, int n_cols, 
 // on registers; carrying delta (the float32 rounding error of mean0) keeps y accurate when |mean| >> std.
 // RMSNorm: rstd = 1/sqrt(sum(x^2)/N + eps); y = x*rstd*w.
 // ---------------------------------------------------------------------------------------------------
-template <typename T, bool LN, int K, int TPR, int BLOCK, bool ALIGNED>
+// ACT != kNoAct: y = act(normalise(x)*w + b) -- the activation (one of the parameter-free, input-saving ones of
+// thn_act_math.h) is applied to the float32 value before the one rounding on store; nothing else changes.
+template <typename T, bool LN, int K, int TPR, int BLOCK, bool ALIGNED, int ACT = kNoAct>
 __global__ void __launch_bounds__(BLOCK) norm_fwd_kernel(const FwdArgs a) {
     constexpr int VEC = T::VEC;
     constexpr int G = BLOCK / TPR;
@@ -186,6 +192,7 @@ __global__ void __launch_bounds__(BLOCK) norm_fwd_kernel(const FwdArgs a) {
             for (int e = 0; e < VEC; ++e) {
                 if constexpr (LN) yf[e] = fmaf((xf[k][e] - delta) * rstd, wr[k][e], br[k][e]);
                 else yf[e] = xf[k][e] * rstd * wr[k][e];
+                if constexpr (ACT != kNoAct) yf[e] = act_fwd<ACT, float>(yf[e], 0.0f, 0.0f);
             }
             store_row_vec<T, ALIGNED>(yrow, voff[k], a.n_cols, yf);
         }
@@ -235,12 +242,19 @@ __device__ __forceinline__ void combine_groups(Acc (&acc)[VEC], Acc* comb, int g
     }
 }
 
-template <typename T, bool LN, int K, int TPR, int BLOCK, bool ALIGNED>
+// ACT != kNoAct: the forward was y = act(z), z = xhat*w + b.  The pre-activation is not stored: the kernel
+// recomputes z from the saved statistics and replaces the upstream gradient by dy * act'(z) before anything else
+// uses it.  z needs the corrected xhat, so LayerNorm takes one more reduction round (sum(u) first); the loop is
+// still bound by memory.
+template <typename T, bool LN, int K, int TPR, int BLOCK, bool ALIGNED, int ACT = kNoAct>
 __global__ void __launch_bounds__(BLOCK) norm_bwd_kernel(const BwdArgs a) {
     constexpr int VEC = T::VEC;
     constexpr int G = BLOCK / TPR;
-    constexpr int NV = LN ? 3 : 1;
+    constexpr bool FUSED = ACT != kNoAct;
+    constexpr int NV = LN ? (FUSED ? 2 : 3) : 1;      // fused LayerNorm: sum(u) has its own round
     static_assert(BLOCK % TPR == 0 && G >= 1, "a workgroup holds whole rows");
+    // (fused LayerNorm calls row_allreduce with 1 value, then with 2, once each per row: the two calls always use
+    // opposite halves of the double buffer, as in the forward kernel, so their different slot strides never overlap)
     __shared__ float red[RedSmem<TPR, G, NV>::kFloats];
     // Column accumulators: float64 for float32 / float64 rows in workgroups that have the registers (a
     // workgroup adds up to M/gridDim.x rows per column; float32 accumulators lose about 10 ulp of the final
@@ -282,6 +296,8 @@ __global__ void __launch_bounds__(BLOCK) norm_bwd_kernel(const BwdArgs a) {
     Acc dw[K][VEC];
     Acc db[LN ? K : 1][VEC];
     load_params_clamped<K, VEC, ALIGNED>(wr, a.w, a.w_dtype, voff, a.n_cols, 1.0f);
+    float br[(FUSED && LN) ? K : 1][VEC];
+    if constexpr (FUSED && LN) load_params_clamped<K, VEC, ALIGNED>(br, a.b, a.w_dtype, voff, a.n_cols, 0.0f);
 #pragma unroll
     for (int k = 0; k < K; ++k) {
 #pragma unroll
@@ -308,36 +324,67 @@ __global__ void __launch_bounds__(BLOCK) norm_bwd_kernel(const BwdArgs a) {
         float s[NV];
 #pragma unroll
         for (int i = 0; i < NV; ++i) s[i] = 0.0f;
+        float dlt_fused = 0.0f;
+        if constexpr (FUSED && LN) {
+            // first round: dlt = sum(u)/N, so that z below is built from the corrected xhat
+            float su[1] = {0.0f};
+#pragma unroll
+            for (int k = 0; k < K; ++k) {
+                T::unpack(cx[k], u[k]);
+                float sk = 0.0f;
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) {
+                    float v = (u[k][e] - c_mean) * c_rstd;
+                    if constexpr (!ALIGNED) v = (voff[k] * VEC + e < a.n_cols) ? v : 0.0f;
+                    u[k][e] = v;
+                    sk += v;
+                }
+                su[0] += own[k] ? sk : 0.0f;
+            }
+            row_allreduce<TPR, G, 1>(su, red, phase, g, t);
+            dlt_fused = su[0] * a.inv_n;
+        }
 #pragma unroll
         for (int k = 0; k < K; ++k) {
-            T::unpack(cx[k], u[k]);
+            if constexpr (!(FUSED && LN)) T::unpack(cx[k], u[k]);
             T::unpack(cg[k], gf[k]);
             float s0 = 0.0f, s1 = 0.0f, s2 = 0.0f;
 #pragma unroll
             for (int e = 0; e < VEC; ++e) {
-                if constexpr (LN) {
+                if constexpr (FUSED && LN) {
+                    float v = u[k][e] - dlt_fused;                      // the corrected xhat
+                    if constexpr (!ALIGNED) v = (voff[k] * VEC + e < a.n_cols) ? v : 0.0f;
+                    u[k][e] = v;
+                } else if constexpr (LN) {
                     float v = (u[k][e] - c_mean) * c_rstd;
                     if constexpr (!ALIGNED) v = (voff[k] * VEC + e < a.n_cols) ? v : 0.0f;
                     u[k][e] = v;
                 } else {
                     u[k][e] *= c_rstd;
                 }
+                if constexpr (FUSED) {
+                    const float z = LN ? fmaf(u[k][e], wr[k][e], br[k][e]) : u[k][e] * wr[k][e];
+                    gf[k][e] = act_bwd<ACT, float>(z, gf[k][e], 0.0f, 0.0f);       // dy * act'(z)
+                }
                 wdy[k][e] = wr[k][e] * gf[k][e];
                 s0 = fmaf(u[k][e], wdy[k][e], s0);
                 if constexpr (LN) {
                     s1 += wdy[k][e];
-                    s2 += u[k][e];
+                    if constexpr (!FUSED) s2 += u[k][e];
                 }
             }
             s[0] += own[k] ? s0 : 0.0f;
             if constexpr (LN) {
                 s[1] += own[k] ? s1 : 0.0f;
-                s[2] += own[k] ? s2 : 0.0f;
+                if constexpr (!FUSED) s[2] += own[k] ? s2 : 0.0f;
             }
         }
         row_allreduce<TPR, G, NV>(s, red, phase, g, t);
         float c1, c2 = 0.0f, dlt = 0.0f;
-        if constexpr (LN) {
+        if constexpr (LN && FUSED) {
+            c2 = s[1] * a.inv_n;                   // u already is the corrected xhat
+            c1 = s[0] * a.inv_n;
+        } else if constexpr (LN) {
             dlt = s[2] * a.inv_n;
             c2 = s[1] * a.inv_n;
             c1 = fmaf(-dlt, c2, s[0] * a.inv_n);
