@@ -40,6 +40,11 @@ WORKLOADS = {
     "rmsnorm_f16_4096x16384_outliers": ("rms", 4096, 16384, "f16"),
     "rmsnorm_f32_4096x16384_outliers": ("rms", 4096, 16384, "f32"),
     "layernorm_f32_200x128_quickstart": ("ln", 200, 128, "f32"),
+    # norm with an activation epilogue (thn_norm_act_fwd + thn_norm_act_bwd): same bytes as the plain norm step
+    "layernorm_gelu_bf16_16384x4096": ("ln+gelu", 16384, 4096, "bf16"),
+    "layernorm_gelu_tanh_bf16_16384x4096": ("ln+gelu_tanh", 16384, 4096, "bf16"),
+    "rmsnorm_silu_bf16_16384x4096": ("rms+silu", 16384, 4096, "bf16"),
+    "layernorm_gelu_f32_16384x4096": ("ln+gelu", 16384, 4096, "f32"),
     # the row-reduction activations next to the norm path (thn_softmax_fwd + thn_softmax_bwd per step)
     "softmax_bf16_16384x4096": ("softmax", 16384, 4096, "bf16"),
     "softmax_f32_16384x4096": ("softmax", 16384, 4096, "f32"),
@@ -121,6 +126,10 @@ def main():
     dev = torch.device("cuda", 0)
     torch.cuda.set_device(dev)
     kind, m, n, dname = WORKLOADS[args.workload]
+    fused_act = -1
+    if "+" in kind:
+        kind, act_name = kind.split("+")
+        fused_act = ["gelu", "gelu_tanh", "silu", "relu"].index(act_name)
     dtype = {"bf16": torch.bfloat16, "f16": torch.float16, "f32": torch.float32}[dname]
     if kind in SOFTMAX_KINDS or kind.startswith(("normalize", "pnorm", "act_")):
         return softmax_main(args, lib, dev, kind, m, n, dname, dtype)
@@ -156,16 +165,26 @@ def main():
     parts = ctypes.c_int32(0)
 
     def forward(b_):
-        rc = lib.thn_norm_fwd(p(b_["x"]), n, p(b_["y"]), n, p(w), p(b), p(b_["mean"]), p(b_["rstd"]), m, n, 1e-6,
-                              code, code, stream)
+        if fused_act >= 0:
+            rc = lib.thn_norm_act_fwd(p(b_["x"]), n, p(b_["y"]), n, p(w), p(b), p(b_["mean"]), p(b_["rstd"]), m, n, 1e-6,
+                                      fused_act, code, code, stream)
+        else:
+            rc = lib.thn_norm_fwd(p(b_["x"]), n, p(b_["y"]), n, p(w), p(b), p(b_["mean"]), p(b_["rstd"]), m, n, 1e-6,
+                                  code, code, stream)
         assert rc == 0, _native.strerror(rc)
 
     def backward(b_):
-        rc = lib.thn_norm_bwd(p(b_["x"]), n, p(b_["dy"]), n, p(b_["dx"]), n, p(w), p(b_["mean"]), p(b_["rstd"]),
-                              p(dw), p(db), p(ws), ws_bytes, m, n, code, code, stream)
+        if fused_act >= 0:
+            rc = lib.thn_norm_act_bwd(p(b_["x"]), n, p(b_["dy"]), n, p(b_["dx"]), n, p(w), p(b), p(b_["mean"]),
+                                      p(b_["rstd"]), p(dw), p(db), p(ws), ws_bytes, m, n, fused_act, code, code, stream)
+        else:
+            rc = lib.thn_norm_bwd(p(b_["x"]), n, p(b_["dy"]), n, p(b_["dx"]), n, p(w), p(b_["mean"]), p(b_["rstd"]),
+                                  p(dw), p(db), p(ws), ws_bytes, m, n, code, code, stream)
         assert rc == 0, _native.strerror(rc)
 
     def backward_stage1(b_):
+        if fused_act >= 0:                 # the fused backward has no separate stage-1 entry point: time the pair
+            return backward(b_)
         rc = lib.thn_norm_bwd_dx_partials(p(b_["x"]), n, p(b_["dy"]), n, p(b_["dx"]), n, p(w), p(b_["mean"]),
                                           p(b_["rstd"]), 1, int(ln), p(ws), ws_bytes, ctypes.byref(parts), m, n,
                                           code, code, stream)
@@ -211,15 +230,20 @@ def main():
 
     fwd_us = avg_launch_us(forward)
     bwd1_us = avg_launch_us(backward_stage1)
+    if fused_act >= 0:
+        parts.value = _launch.query_launch(10, int(ln) | (fused_act << 1), m, n, dtype)[3]
     bwd2_us = avg_launch_us(lambda b_: backward_stage2())
+    if fused_act >= 0:
+        bwd1_us -= bwd2_us                 # the pair minus the second stage alone
     achieved = bwd_bytes / (bwd1_us * 1e-6) / 1e9
     if args.calibration_copy:
         # a plain copy of known size (x -> y: m*n*s bytes read, as many written) for scaling the HBM counters
         for i in range(5):
             sets[i % N_BUFFER_SETS]["y"].copy_(sets[i % N_BUFFER_SETS]["x"])
         torch.cuda.synchronize()
-    fwd_shape = _launch.query_launch(0, ln, m, n, dtype)
-    bwd_shape = _launch.query_launch(1, ln, m, n, dtype)
+    flavour = int(ln) | (fused_act << 1) if fused_act >= 0 else int(ln)
+    fwd_shape = _launch.query_launch(9 if fused_act >= 0 else 0, flavour, m, n, dtype)
+    bwd_shape = _launch.query_launch(10 if fused_act >= 0 else 1, flavour, m, n, dtype)
 
     out = {
         "metric": "fwd+bwd HBM GB/s and % of peak, RMSNorm/LayerNorm bf16 16384x4096",
@@ -235,7 +259,9 @@ def main():
         "dtype": dname,
         "data": "synthetic",
         "config": {"workload": args.workload, "op": "RMSNorm" if kind == "rms" else "LayerNorm", "rows": m,
-                   "hidden": n, "eps": 1e-6, "buffer_sets": N_BUFFER_SETS, "entry_points": "thn_norm_fwd + thn_norm_bwd"},
+                   "hidden": n, "eps": 1e-6, "buffer_sets": N_BUFFER_SETS,
+                   "entry_points": "thn_norm_act_fwd + thn_norm_act_bwd" if fused_act >= 0 else "thn_norm_fwd + thn_norm_bwd",
+                   **({"activation": ["gelu", "gelu_tanh", "silu", "relu"][fused_act]} if fused_act >= 0 else {})},
         "pct_of_hbm_peak": round(100.0 * gbps / HBM_PEAK_GBPS, 2),
         "rows_per_s": round(m / (ms_per_step * 1e-3)),
         "algorithmic_bytes_per_step": step_bytes,
@@ -252,7 +278,7 @@ def main():
                      "algorithmic_bytes_per_launch": bwd_bytes, "avg_launch_us": round(bwd1_us, 2),
                      "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload)},
     }
-    if not args.no_cpu_baseline:
+    if not args.no_cpu_baseline and fused_act < 0:      # (the fused workloads carry no CPU leg)
         out["cpu_baseline"] = cpu_baseline(kind, m, n, dtype, sets[0], w, b, step_bytes)
     print(json.dumps(out), flush=True)
 

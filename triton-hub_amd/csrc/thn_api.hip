@@ -314,7 +314,10 @@ int plan_launch(int which, int ln, bool aligned, int64_t M, int64_t N, int dtype
     int bpc = occupancy(which, dtype, ln, aligned, s);
     // The p-norm families in 256-thread workgroups (rows up to 16 KiB) measured 5-25 % faster with two workgroups
     // per compute unit; everything else with one.
-    const int family_bpc = (which >= kPnormFwd && which <= kNormalizeBwd && s.block <= 256) ? 2 : kDefaultBlocksPerCu;
+    int family_bpc = (which >= kPnormFwd && which <= kNormalizeBwd && s.block <= 256) ? 2 : kDefaultBlocksPerCu;
+    // A GeLU epilogue makes the norm kernels arithmetic-bound (about 30 instruction slots per element): they take
+    // as many workgroups per compute unit as their registers allow, up to four.
+    if ((which == kFusedFwd || which == kFusedBwd) && ((ln >> 1) == thn::kGelu || (ln >> 1) == thn::kGeluTanh)) family_bpc = 4;
     const int cap = ov.bpc.load() > 0 ? ov.bpc.load() : family_bpc;
     if (cap < bpc) bpc = cap;
     const int rows_per_block = s.block / s.tpr;
@@ -667,6 +670,10 @@ int thn_norm_query_launch(int which, int is_layernorm, int64_t M, int64_t N, int
     const bool aligned = N > 0 && (N % (16 / bytes)) == 0;
     int flavour = is_layernorm != 0 ? 1 : 0;
     if (which >= kPnormFwd && which <= kNormalizeBwd) flavour = thn::kP2;
+    if (which == kFusedFwd || which == kFusedBwd) {
+        if (is_layernorm < 0 || !fusable(is_layernorm >> 1)) return THN_E_SHAPE;
+        flavour = is_layernorm;                     // bit 0 = LayerNorm, bits 1.. = activation
+    }
     const int rc = plan_launch(which, flavour, aligned, M, N, x_dtype, &p);
     if (rc != THN_OK) return rc;
     shape[0] = p.s.k;
