@@ -1,0 +1,46 @@
+"""CPU tests of bench.py's command-line contract: the workload table is consistent, more than one GPU is refused
+with a message, and without a GPU the script says so instead of falling back to anything."""
+import os
+import subprocess
+import sys
+
+from conftest import ROOT
+
+sys.path.insert(0, ROOT)
+import bench  # noqa: E402
+
+
+def run(*args):
+    return subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), *args], capture_output=True, text=True,
+                          env={**os.environ, "WORLD_SIZE": "1"})
+
+
+def test_more_than_one_gpu_is_refused_with_a_message():
+    r = run("--gpus", "2")
+    assert r.returncode != 0 and "ONE GPU" in (r.stderr + r.stdout)
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py")], capture_output=True, text=True,
+                       env={**os.environ, "WORLD_SIZE": "4"})
+    assert r.returncode != 0 and "ONE GPU" in (r.stderr + r.stdout)
+
+
+def test_workload_table():
+    assert "rmsnorm_bf16_16384x4096" in bench.WORKLOADS           # the configuration the headline metric is quoted on
+    for name, (kind, m, n, dname) in bench.WORKLOADS.items():
+        assert m > 0 and n > 0 and dname in ("bf16", "f16", "f32"), name
+        s = {"bf16": 2, "f16": 2, "f32": 4}[dname]
+        fwd, bwd = bench.algorithmic_bytes(kind.split("+")[0], m, n, s, s)
+        assert fwd >= m * n * s and bwd >= 2 * m * n * s, name      # at least one read; a read and a write
+    for key in bench.MEASURED_TRAFFIC_BYTES:
+        assert key in bench.WORKLOADS
+    # algorithmic bytes of the default workload: 5*M*N*s + 8*M + 3*N*s
+    f, b = bench.algorithmic_bytes("rms", 16384, 4096, 2, 2)
+    assert f + b == 5 * 16384 * 4096 * 2 + 8 * 16384 + 3 * 4096 * 2
+    f, b = bench.algorithmic_bytes("ln", 16384, 4096, 2, 2)
+    assert f + b == 5 * 16384 * 4096 * 2 + 16 * 16384 + 5 * 4096 * 2
+
+
+def test_profiles_named_by_the_traffic_table_exist():
+    text = open(os.path.join(ROOT, "bench.py")).read()
+    import re
+    for path in re.findall(r"# (profiles/[\w./-]+\.txt)", text):
+        assert os.path.exists(os.path.join(ROOT, path)), path
