@@ -157,7 +157,10 @@ def main():
     b = (0.1 * rand(n)).to(dtype) if ln else None
     dw = torch.empty_like(w)
     db = torch.empty_like(w) if ln else None
-    ws_bytes = lib.thn_norm_bwd_workspace_bytes(m, n, 1, int(ln), code)
+    if fused_act >= 0:
+        ws_bytes = lib.thn_norm_act_bwd_workspace_bytes(m, n, 1, int(ln), fused_act, code)
+    else:
+        ws_bytes = lib.thn_norm_bwd_workspace_bytes(m, n, 1, int(ln), code)
     assert ws_bytes >= 0, ws_bytes
     ws = torch.empty(max(ws_bytes, 16) // 4, device=dev)
     stream = torch.cuda.current_stream(dev).cuda_stream

@@ -70,8 +70,10 @@ int thn_norm_fwd(const void* x, int64_t x_row_stride,
 /*
  * Bytes of scratch thn_norm_bwd() needs for its per-workgroup partial sums of dW / dB: the counterpart of
  * the reference's `_dw` / `_db` (sm_count, N) float32 buffers (layernorm.py:183-184, rmsnorm.py:147).
- * Depends on the current device's compute-unit count.  Returns a negative THN_E_* code on bad arguments,
- * 0 when neither gradient is requested.
+ * One partial row per workgroup the backward can launch: depends on the current device's compute-unit count and
+ * on the blocks_per_cu override in force (thn_norm_set_launch_override; raising it after this query makes the
+ * backward return THN_E_WORKSPACE).  Returns a negative THN_E_* code on bad arguments, 0 when neither gradient is
+ * requested.
  */
 int64_t thn_norm_bwd_workspace_bytes(int64_t M, int64_t N, int want_dw, int want_db, int x_dtype);
 
@@ -245,8 +247,9 @@ int thn_act_bwd(const void* saved, int64_t saved_row_stride,
  * and the backward recomputes the pre-activation z = xhat*w + b from the saved statistics (nothing extra is
  * saved), replaces dy by dy*act'(z) and continues as thn_norm_bwd.  Five passes over the tensor instead of ten.
  * `act`: THN_ACT_GELU, THN_ACT_GELU_TANH, THN_ACT_SILU or THN_ACT_RELU (the parameter-free activations whose
- * backward needs only their input); anything else is THN_E_SHAPE.  All other arguments, the workspace
- * (thn_norm_bwd_workspace_bytes) and the NULL conventions are those of thn_norm_fwd / thn_norm_bwd; `b` is the
+ * backward needs only their input); anything else is THN_E_SHAPE.  All other arguments and the NULL conventions
+ * are those of thn_norm_fwd / thn_norm_bwd; the workspace is sized by thn_norm_act_bwd_workspace_bytes (the
+ * arithmetic-bound GeLU variants run more workgroups, hence more partial rows, than the plain backward); `b` is the
  * forward's bias (NULL when there is none).  Because the intermediate is never rounded to the storage type, the
  * result is closer to exact arithmetic than the chained operators', not bit-identical to them.
  */
@@ -256,6 +259,8 @@ int thn_norm_act_fwd(const void* x, int64_t x_row_stride,
                      float* mean, float* rstd,
                      int64_t M, int64_t N, float eps, int act,
                      int x_dtype, int w_dtype, void* stream);
+
+int64_t thn_norm_act_bwd_workspace_bytes(int64_t M, int64_t N, int want_dw, int want_db, int act, int x_dtype);
 
 int thn_norm_act_bwd(const void* x, int64_t x_row_stride,
                      const void* dy, int64_t dy_row_stride,

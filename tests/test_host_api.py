@@ -25,7 +25,7 @@ def declared_functions():
 
 def test_library_exports_every_declared_symbol():
     names = declared_functions()
-    assert len(names) == 19 and "thn_norm_act_fwd" in names and "thn_norm_act_bwd" in names and "thn_act_fwd" in names and "thn_pnorm_fwd" in names and "thn_normalize_bwd" in names and "thn_norm_fwd" in names and "thn_norm_bwd" in names and "thn_softmax_fwd" in names
+    assert len(names) == 20 and "thn_norm_act_fwd" in names and "thn_norm_act_bwd" in names and "thn_act_fwd" in names and "thn_pnorm_fwd" in names and "thn_normalize_bwd" in names and "thn_norm_fwd" in names and "thn_norm_bwd" in names and "thn_softmax_fwd" in names
     handle = ctypes.CDLL(_native.LIB_PATH)
     for name in names:
         assert hasattr(handle, name), f"{name} is declared in include/thnorm.h but not exported"
@@ -162,6 +162,9 @@ def test_fused_norm_activation_surface_and_argument_checks():
         assert call(4, 32769, _native.ACT_SILU, _native.BF16) == _native.E_FEATURE_DIM
         assert call(0, 128, _native.ACT_RELU, _native.F16) == _native.OK
         assert call(4, 128, _native.ACT_GELU_TANH, _native.F16) == _native.E_NULL
+    assert lib.thn_norm_act_bwd_workspace_bytes(4, 128, 1, 1, _native.ACT_MISH, _native.F32) == _native.E_SHAPE
+    assert lib.thn_norm_act_bwd_workspace_bytes(4, 128, 0, 0, _native.ACT_GELU, _native.F32) == 0
+    assert lib.thn_norm_act_bwd_workspace_bytes(4, 128, 1, 1, _native.ACT_GELU, 8) == _native.E_DTYPE
     assert ACTIVATIONS == {"gelu": 0, "gelu_tanh": 1, "silu": 2, "relu": 3}
     m = LayerNormActivation(48, "gelu_tanh", eps=1e-3, bias=False, dtype=torch.bfloat16)
     assert isinstance(m, LayerNorm) and (m.dim, m.eps, m.activation, m.act) == (48, 1e-3, "gelu_tanh", 1)

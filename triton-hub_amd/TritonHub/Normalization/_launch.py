@@ -195,10 +195,14 @@ def norm_bwd(x: torch.Tensor, dout: torch.Tensor, weight, bias, mean, rstd, laye
         guard = torch.cuda.device(index)
         guard.__enter__()
     try:
-        key = (index, m, n, dw is not None, db is not None, x_code)
+        key = (index, m, n, dw is not None, db is not None, x_code, act)
         nbytes = _workspace_bytes_cache.get(key)
         if nbytes is None:
-            nbytes = int(lib.thn_norm_bwd_workspace_bytes(m, n, int(dw is not None), int(db is not None), x_code))
+            if act < 0:
+                nbytes = int(lib.thn_norm_bwd_workspace_bytes(m, n, int(dw is not None), int(db is not None), x_code))
+            else:
+                nbytes = int(lib.thn_norm_act_bwd_workspace_bytes(m, n, int(dw is not None), int(db is not None), act,
+                                                                  x_code))
             if nbytes < 0:
                 _native.check(nbytes)
             _workspace_bytes_cache[key] = nbytes

@@ -46,6 +46,7 @@ SYMBOLS = {
     'thn_act_fwd': (_i32, [_vp, _i64, _vp, _i64, _i64, _i64, _i32, _f32, _f32, _i32, _vp]),
     'thn_act_bwd': (_i32, [_vp, _i64, _vp, _i64, _vp, _i64, _i64, _i64, _i32, _f32, _f32, _i32, _vp]),
     'thn_norm_act_fwd': (_i32, [_vp, _i64, _vp, _i64, _vp, _vp, _vp, _vp, _i64, _i64, _f32, _i32, _i32, _i32, _vp]),
+    'thn_norm_act_bwd_workspace_bytes': (_i64, [_i64, _i64, _i32, _i32, _i32, _i32]),
     'thn_norm_act_bwd': (_i32, [_vp, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64,
                                 _i32, _i32, _i32, _vp]),
     'thn_norm_set_launch_override': (_i32, [_i32, _i32, _i32, _i32, _i32]),

@@ -187,12 +187,13 @@ int launch_normalize_bwd(int dtype, int mode, bool aligned, Shape s, const Norma
 std::mutex g_occ_mutex;
 std::unordered_map<uint64_t, int> g_occ_cache;
 
-// `ln`: the kernel flavour within the family (LayerNorm / log-softmax: 1; p-norm families: the variant above).
-int occupancy(int which, int dtype, int ln, bool aligned, Shape s) {
+// `flavour`: the kernel variant within the family -- 1 for LayerNorm / log-softmax, 0 for RMSNorm / softmax; the
+// `variant` described above for the p-norm and epilogue families.
+int occupancy(int which, int dtype, int flavour, bool aligned, Shape s) {
     int dev = 0;
     (void)hipGetDevice(&dev);
     const uint64_t key = (static_cast<uint64_t>(dev) << 44) | (static_cast<uint64_t>(which) << 40) |
-                         (static_cast<uint64_t>(dtype) << 36) | (static_cast<uint64_t>(ln) << 32) |
+                         (static_cast<uint64_t>(dtype) << 36) | (static_cast<uint64_t>(flavour) << 32) |
                          (static_cast<uint64_t>(aligned) << 30) | (static_cast<uint64_t>(s.k) << 24) |
                          (static_cast<uint64_t>(s.tpr) << 12) | static_cast<uint64_t>(s.block);
     {
@@ -204,31 +205,31 @@ int occupancy(int which, int dtype, int ln, bool aligned, Shape s) {
     int rc;
     if (which == kNormFwd) {
         FwdArgs dummy{};
-        rc = launch_fwd(dtype, ln, aligned, s, dummy, 0, nullptr, &occ);
+        rc = launch_fwd(dtype, flavour, aligned, s, dummy, 0, nullptr, &occ);
     } else if (which == kNormBwd) {
         BwdArgs dummy{};
-        rc = launch_bwd(dtype, ln, aligned, s, dummy, 0, nullptr, &occ);
+        rc = launch_bwd(dtype, flavour, aligned, s, dummy, 0, nullptr, &occ);
     } else if (which == kSoftmaxFwd) {
         SoftmaxFwdArgs dummy{};
-        rc = launch_softmax_fwd(dtype, ln, aligned, s, dummy, 0, nullptr, &occ);
+        rc = launch_softmax_fwd(dtype, flavour, aligned, s, dummy, 0, nullptr, &occ);
     } else if (which == kSoftmaxBwd) {
         SoftmaxBwdArgs dummy{};
-        rc = launch_softmax_bwd(dtype, ln, aligned, s, dummy, 0, nullptr, &occ);
+        rc = launch_softmax_bwd(dtype, flavour, aligned, s, dummy, 0, nullptr, &occ);
     } else if (which == kFusedFwd) {
         FwdArgs dummy{};
-        rc = launch_fused_fwd(dtype, ln, aligned, s, dummy, 0, nullptr, &occ);
+        rc = launch_fused_fwd(dtype, flavour, aligned, s, dummy, 0, nullptr, &occ);
     } else if (which == kFusedBwd) {
         BwdArgs dummy{};
-        rc = launch_fused_bwd(dtype, ln, aligned, s, dummy, 0, nullptr, &occ);
+        rc = launch_fused_bwd(dtype, flavour, aligned, s, dummy, 0, nullptr, &occ);
     } else if (which == kPnormFwd) {
         PnormFwdArgs dummy{};
-        rc = launch_pnorm_fwd(dtype, ln, aligned, s, dummy, 0, nullptr, &occ);
+        rc = launch_pnorm_fwd(dtype, flavour, aligned, s, dummy, 0, nullptr, &occ);
     } else if (which == kPnormBwd) {
         PnormBwdArgs dummy{};
-        rc = launch_pnorm_bwd(dtype, ln, aligned, s, dummy, 0, nullptr, &occ);
+        rc = launch_pnorm_bwd(dtype, flavour, aligned, s, dummy, 0, nullptr, &occ);
     } else {
         NormalizeBwdArgs dummy{};
-        rc = launch_normalize_bwd(dtype, ln, aligned, s, dummy, 0, nullptr, &occ);
+        rc = launch_normalize_bwd(dtype, flavour, aligned, s, dummy, 0, nullptr, &occ);
     }
     if (rc != 0 || occ <= 0) occ = 1;
     if (occ > kMaxBlocksPerCu) occ = kMaxBlocksPerCu;
@@ -248,21 +249,21 @@ constexpr int kTprList[] = {8, 16, 32, 64, 128, 256, 512, 1024};
 
 // The static replacement of the reference's autotune over num_warps (autotune.py:62-65), fitted to sweeps
 // over (vectors per thread, threads per row, workgroup size, workgroups per compute unit) on MI355X at row
-// widths from 1 KiB to 64 KiB.  HBM throughput peaks when a compute unit keeps about 1024 (forward) to
-// 2048 (backward: two input streams) 16-byte loads in flight and falls off by up to 15 % beyond that, so:
-// one workgroup per compute unit, and
-//   forward : the fewest threads per row with at most 4 vectors each (256-thread workgroups up to 16 KiB rows);
-//   backward: the fewest threads per row with at most 3 vectors each (x, dy, w, dW, dB are live per
-//             element), 4 for rows of at most 2 KiB (they share a wave: the float64 column sums need the
-//             instruction-level parallelism) and for rows that 1024 threads cannot cover otherwise;
-//             512-thread workgroups once a row spans two waves or more, which also halves the number of
-//             partial rows.
+// widths from 1 KiB to 64 KiB.  HBM throughput peaks when a compute unit keeps about 1024 (one input stream) to
+// 2048 (two) 16-byte loads in flight and falls off by up to 15 % beyond that, so, for every row family: the
+// fewest threads per row with at most `kmax` vectors each, and
+//   norm forward, softmax forward, p-norm forward / backward: kmax 4, 256-thread workgroups up to 16 KiB rows;
+//   norm backward: kmax 3 (x, dy, w, dW, dB are live per element), 4 for rows of at most 2 KiB (they share a
+//             wave: the float64 column sums need the instruction-level parallelism) and for rows that 1024
+//             threads cannot cover otherwise; 512-thread workgroups once a row spans two waves or more, which
+//             also halves the number of partial rows;
+//   softmax / normalize / epilogue backward (two or three input streams): kmax 2 up to 32 KiB rows.
+// Workgroups per compute unit: one (kDefaultBlocksPerCu), except where default_blocks_per_cu() says otherwise.
 constexpr int kDefaultBlocksPerCu = 1;
 
 int ceil_div(int a, int b) { return (a + b - 1) / b; }
 
-Shape heuristic_shape(int which, int ln, bool aligned, int n_vecs) {
-    (void)ln;
+Shape heuristic_shape(int which, bool aligned, int n_vecs) {
     int kmax = (aligned && which == kNormBwd && n_vecs > 128) ? 3 : 4;
     // Softmax backward: two input streams and nothing to hold; 2 vectors per thread per stream measured best,
     // except for 2 KiB rows, where one full wave per row (2 x 64) is 8 % slower than half a wave (4 x 32).
@@ -288,7 +289,18 @@ Shape heuristic_shape(int which, int ln, bool aligned, int n_vecs) {
     return s;
 }
 
-int plan_launch(int which, int ln, bool aligned, int64_t M, int64_t N, int dtype, Plan* out) {
+// Upper limit of workgroups per compute unit the library picks by itself (the occupancy may allow fewer).
+int default_blocks_per_cu(int which, int flavour, int block) {
+    // The p-norm families in 256-thread workgroups (rows up to 16 KiB) measured 5-25 % faster with two workgroups
+    // per compute unit.
+    if (which >= kPnormFwd && which <= kNormalizeBwd && block <= 256) return 2;
+    // A GeLU epilogue makes the norm kernels arithmetic-bound (about 30 instruction slots per element): they take
+    // as many workgroups per compute unit as their registers allow, up to four.
+    if ((which == kFusedFwd || which == kFusedBwd) && ((flavour >> 1) == thn::kGelu || (flavour >> 1) == thn::kGeluTanh)) return 4;
+    return kDefaultBlocksPerCu;
+}
+
+int plan_launch(int which, int flavour, bool aligned, int64_t M, int64_t N, int dtype, Plan* out) {
     const int bytes = elem_bytes(dtype);
     if (bytes == 0) return THN_E_DTYPE;
     if (M < 0 || N <= 0) return THN_E_SHAPE;
@@ -298,7 +310,7 @@ int plan_launch(int which, int ln, bool aligned, int64_t M, int64_t N, int dtype
     const int cus = current_cu_count();
     if (cus <= 0) return THN_E_DEVICE;
 
-    Shape s = heuristic_shape(which, ln, aligned, n_vecs);
+    Shape s = heuristic_shape(which, aligned, n_vecs);
     const Override& ov = g_override[which];
     Shape cand = s;
     if (ov.k.load() > 0) cand.k = ov.k.load();
@@ -311,14 +323,8 @@ int plan_launch(int which, int ln, bool aligned, int64_t M, int64_t N, int dtype
     }
     if (!shape_compiled(which, aligned, s)) return THN_E_SHAPE;
 
-    int bpc = occupancy(which, dtype, ln, aligned, s);
-    // The p-norm families in 256-thread workgroups (rows up to 16 KiB) measured 5-25 % faster with two workgroups
-    // per compute unit; everything else with one.
-    int family_bpc = (which >= kPnormFwd && which <= kNormalizeBwd && s.block <= 256) ? 2 : kDefaultBlocksPerCu;
-    // A GeLU epilogue makes the norm kernels arithmetic-bound (about 30 instruction slots per element): they take
-    // as many workgroups per compute unit as their registers allow, up to four.
-    if ((which == kFusedFwd || which == kFusedBwd) && ((ln >> 1) == thn::kGelu || (ln >> 1) == thn::kGeluTanh)) family_bpc = 4;
-    const int cap = ov.bpc.load() > 0 ? ov.bpc.load() : family_bpc;
+    int bpc = occupancy(which, dtype, flavour, aligned, s);
+    const int cap = ov.bpc.load() > 0 ? ov.bpc.load() : default_blocks_per_cu(which, flavour, s.block);
     if (cap < bpc) bpc = cap;
     const int rows_per_block = s.block / s.tpr;
     const int64_t row_blocks = (M + rows_per_block - 1) / rows_per_block;
@@ -339,6 +345,26 @@ bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) ==
 
 int64_t partial_pitch(int64_t N) { return (N + 63) / 64 * 64; }
 
+
+// One float32 partial row per workgroup and gradient.  The backward launches at most
+// cus * max(default, override) workgroups and never more than one per row, whatever shape it picks.
+int64_t bwd_workspace_bytes(int which, int flavour, int64_t M, int64_t N, int want_dw, int want_db, int x_dtype) {
+    const int bytes = elem_bytes(x_dtype);
+    if (bytes == 0) return THN_E_DTYPE;
+    if (M < 0 || N <= 0) return THN_E_SHAPE;
+    if (N * bytes > kMaxRowBytes) return THN_E_FEATURE_DIM;
+    const int n_grads = (want_dw ? 1 : 0) + (want_db ? 1 : 0);
+    if (n_grads == 0 || M == 0) return 0;
+    const int cus = current_cu_count();
+    if (cus <= 0) return THN_E_DEVICE;
+    int bpc = default_blocks_per_cu(which, flavour, 512);
+    const int forced = g_override[which].bpc.load();
+    if (forced > bpc) bpc = forced;
+    if (bpc > kMaxBlocksPerCu) bpc = kMaxBlocksPerCu;
+    int64_t parts = static_cast<int64_t>(cus) * bpc;
+    if (parts > M) parts = M;
+    return n_grads * parts * partial_pitch(N) * static_cast<int64_t>(sizeof(float));
+}
 
 bool fusable(int act) { return act == thn::kGelu || act == thn::kGeluTanh || act == thn::kSilu || act == thn::kRelu; }
 
@@ -714,19 +740,12 @@ int thn_norm_act_bwd(const void* x, int64_t x_row_stride, const void* dy, int64_
 }
 
 int64_t thn_norm_bwd_workspace_bytes(int64_t M, int64_t N, int want_dw, int want_db, int x_dtype) {
-    const int bytes = elem_bytes(x_dtype);
-    if (bytes == 0) return THN_E_DTYPE;
-    if (M < 0 || N <= 0) return THN_E_SHAPE;
-    if (N * bytes > kMaxRowBytes) return THN_E_FEATURE_DIM;
-    const int n_grads = (want_dw ? 1 : 0) + (want_db ? 1 : 0);
-    if (n_grads == 0 || M == 0) return 0;
-    const int cus = current_cu_count();
-    if (cus <= 0) return THN_E_DEVICE;
-    // Upper bound on the number of partial rows for any launch shape: one per workgroup, at most
-    // kMaxBlocksPerCu workgroups per compute unit, never more than one per row.
-    int64_t parts = static_cast<int64_t>(cus) * kMaxBlocksPerCu;
-    if (parts > M) parts = M;
-    return n_grads * parts * partial_pitch(N) * static_cast<int64_t>(sizeof(float));
+    return bwd_workspace_bytes(kNormBwd, 0, M, N, want_dw, want_db, x_dtype);
+}
+
+int64_t thn_norm_act_bwd_workspace_bytes(int64_t M, int64_t N, int want_dw, int want_db, int act, int x_dtype) {
+    if (!fusable(act)) return THN_E_SHAPE;
+    return bwd_workspace_bytes(kFusedBwd, act << 1, M, N, want_dw, want_db, x_dtype);
 }
 
 int thn_norm_bwd_dx_partials(const void* x, int64_t x_row_stride, const void* dy, int64_t dy_row_stride,
