@@ -58,28 +58,10 @@ def _stream_handle(index: int) -> int:
 
 
 def _current_device() -> int:
+    """Index of the current HIP device.  The launches below run with the tensor's device current (the reference
+    wraps its launches in `with torch.cuda.device(x.device.index)`, layernorm.py:73); switching is skipped when it
+    already is."""
     return _get_device() if _get_device is not None else torch.cuda.current_device()
-
-
-class _on_device:
-    """Makes `index` the current HIP device for the duration of a launch; free when it already is
-    (the reference wraps its launches in `with torch.cuda.device(x.device.index)`, layernorm.py:73)."""
-
-    __slots__ = ('index', 'guard')
-
-    def __init__(self, index: int):
-        self.index = index
-        self.guard = None
-
-    def __enter__(self):
-        if _current_device() != self.index:
-            self.guard = torch.cuda.device(self.index)
-            self.guard.__enter__()
-
-    def __exit__(self, *exc):
-        if self.guard is not None:
-            self.guard.__exit__(*exc)
-        return False
 
 
 def _flatten(t: torch.Tensor, what: str):

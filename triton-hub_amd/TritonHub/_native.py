@@ -106,6 +106,3 @@ def require_gpu(t: torch.Tensor) -> None:
         raise RuntimeError('TritonHub.Normalization runs on the GPU only: got a tensor on '
                            f'{t.device}. There is no CPU fallback.')
 
-
-def current_stream(device) -> int:
-    return torch.cuda.current_stream(device).cuda_stream
