@@ -103,6 +103,6 @@ def ptr(t) -> int:
 
 def require_gpu(t: torch.Tensor) -> None:
     if not t.is_cuda:
-        raise RuntimeError('TritonHub.Normalization runs on the GPU only: got a tensor on '
+        raise RuntimeError('this TritonHub build runs on the GPU only: got a tensor on '
                            f'{t.device}. There is no CPU fallback.')
 
