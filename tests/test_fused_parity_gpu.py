@@ -104,6 +104,16 @@ def test_against_composed_oracles(kind, act, dtype):
         run_and_compare(kind, act, x, dy, w, b, 1e-5, f"{kind}+{act} {shape} {dtype}")
 
 
+@pytest.mark.parametrize("dtype,widths", [(torch.bfloat16, (16384, 24576, 32768)), (torch.float32, (12288, 16384))])
+def test_wide_rows_many_per_workgroup(dtype, widths):
+    # rows of 48-64 KiB: the 1024-thread workgroups, with more rows than the grid has workgroups
+    for n in widths:
+        for kind, act in (("ln", "gelu_tanh"), ("rms", "silu")):
+            announce(f"fused wide {kind} {act} {dtype} N={n}")
+            x, dy, w, b = make((520, n), dtype, seed=n, bias=kind == "ln")
+            run_and_compare(kind, act, x, dy, w, b, 1e-5, f"{kind}+{act} wide N={n} {dtype}")
+
+
 @pytest.mark.parametrize("affine,bias", [(True, True), (True, False), (False, False)])
 @pytest.mark.parametrize("kind", ["ln", "rms"])
 def test_constructor_variants_and_hostile_mean(kind, affine, bias):

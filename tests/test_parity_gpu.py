@@ -216,6 +216,26 @@ def test_feature_dim_limit(dtype, n_max):
             mod(over)
 
 
+# ---- rows of 24-64 KiB: the 1024-thread workgroups, several rows per workgroup ----------------------------------
+@pytest.mark.parametrize("dtype,widths", [(torch.bfloat16, (12296, 16384, 20480, 24576, 28680, 32768)),
+                                          (torch.float16, (16384, 24568, 32768)),
+                                          (torch.float32, (6148, 8192, 12288, 16384)),
+                                          (torch.float64, (4096, 8192))])
+def test_wide_rows_many_per_workgroup(dtype, widths):
+    """More rows than the persistent grid has workgroups, so every workgroup walks several rows and the last
+    grid-stride step is only partly filled; parameters in the row's dtype and (16-bit rows) in float32."""
+    g = torch.Generator().manual_seed(31)
+    m = 600
+    for n in widths:
+        announce(f"wide rows {dtype} {m}x{n}")
+        x = (0.5 + torch.randn(m, n, generator=g)).to(dtype); dy = torch.randn(m, n, generator=g).to(dtype)
+        w = 1 + 0.1 * torch.randn(n, generator=g); b = 0.1 * torch.randn(n, generator=g)
+        run_and_compare("ln", x, dy, w.to(dtype), b.to(dtype), 1e-5, f"wide LN N={n}")
+        run_and_compare("rms", x, dy, w.to(dtype), None, 1e-5, f"wide RMS N={n}")
+        if dtype in (torch.bfloat16, torch.float16) and n >= 24576:
+            run_and_compare("ln", x, dy, w, b, 1e-5, f"wide LN N={n}, float32 parameters")
+
+
 # ---- size-independent properties at full BASELINE sizes --------------------------------------------------------
 @pytest.mark.parametrize("name", ["c2_rms_bf16_llm", "c5a_ln_f32_hostile", "c4_ln_f32_small_hidden"])
 def test_properties_at_full_size(name):

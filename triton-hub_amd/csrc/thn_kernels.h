@@ -79,6 +79,56 @@ __device__ __forceinline__ void load_row(u32x4 (&dst)[K], const char* base, int6
 }
 
 template <typename T, bool ALIGNED>
+__device__ __forceinline__ u32x4 load_row_vec(const char* rowp, int voff, int n_cols) {
+    if constexpr (ALIGNED) return ld128(rowp + voff);
+    else return load_vec_elems<T>(rowp, voff, n_cols);
+}
+
+// Workgroups of 1024 threads serve the widest rows (more than 24 KiB of x in the backward, 32 KiB in the
+// forward) and have 128 registers per thread.  Holding a row as float32 next to the packed next row, the
+// parameters and the column accumulators does not always fit there, and a kernel that spills to scratch
+// memory loses more than half of its bandwidth.  Instances that would spill run a leaner form of the row loop,
+// chosen at compile time from three independent savings, in the order of what they cost in speed:
+//   recompute: only the packed 16-byte vectors of the row stay live across a reduction round; every pass
+//              unpacks them again (the same instructions on the same inputs, so the same bits);
+//   lds_dw:    (backward, 16-bit rows) the dW sums of a thread live in LDS, in slots no other thread touches;
+//   !ahead:    the next row is not requested a whole row ahead: vector k of the next row is loaded into the
+//              registers of vector k as soon as that one has been stored (4-16 % slower where the row-ahead
+//              form fits, so it is the last resort).
+struct RowForm {
+    bool recompute, ahead, lds_dw;
+};
+constexpr RowForm kPlainForm{false, true, false};
+
+template <int BYTES, bool LN, int K, int BLOCK, bool FUSED>
+constexpr RowForm fwd_form() {
+    if (BLOCK < 1024) return kPlainForm;
+    if (BYTES == 2 && LN && K == 4) return RowForm{true, true, false};
+    if (FUSED && BYTES == 2 && K == 4) return RowForm{true, true, false};
+    return kPlainForm;
+}
+
+template <int BYTES, bool LN, int K, int BLOCK, bool FUSED>
+constexpr RowForm bwd_form() {
+    if (BLOCK < 1024) return kPlainForm;
+    if (BYTES >= 4) {
+        if (K == 4) return RowForm{true, !LN, false};
+        return (FUSED && LN && K == 3) ? RowForm{true, false, false} : kPlainForm;
+    }
+    if (K == 1) return kPlainForm;
+    if (K == 2) return (LN || FUSED) ? RowForm{true, !(LN && FUSED), false} : kPlainForm;
+    return RowForm{true, !LN, true};     // K = 3, 4: rows of more than 32 KiB
+}
+
+// Makes the compiler forget what it has derived from the packed vectors, so that the next pass really
+// unpacks them again instead of keeping the float32 values of the previous pass in registers.  No instruction.
+template <int K>
+__device__ __forceinline__ void forget_derived(u32x4 (&v)[K]) {
+#pragma unroll
+    for (int k = 0; k < K; ++k) asm volatile("" : "+v"(v[k]));
+}
+
+template <typename T, bool ALIGNED>
 __device__ __forceinline__ void store_row_vec(char* rowp, int voff, int n_cols, const float (&f)[T::VEC]) {
     if constexpr (ALIGNED) st128(rowp + voff, T::pack(f));
     else store_vec_elems<T>(rowp, voff, n_cols, f);
@@ -129,6 +179,96 @@ __global__ void __launch_bounds__(BLOCK) norm_fwd_kernel(const FwdArgs a) {
     if constexpr (LN) load_params_clamped<K, VEC, ALIGNED>(br, a.b, a.w_dtype, voff, a.n_cols, 0.0f);
 
     drain_vector_memory();
+    constexpr RowForm kForm = fwd_form<T::kBytes, LN, K, BLOCK, ACT != kNoAct>();
+    if constexpr (kForm.recompute) {
+        for (int64_t base = static_cast<int64_t>(blockIdx.x) * G; base < a.M; base += rows_per_iter) {
+            const int64_t nrow_raw = row_raw + rows_per_iter;
+            const int64_t nrow = nrow_raw < a.M ? nrow_raw : last_row;
+            const char* nxrow = a.x + nrow * a.x_stride_bytes;
+            u32x4 nxt[kForm.ahead ? K : 1];
+            if constexpr (kForm.ahead) {
+#pragma unroll
+                for (int k = 0; k < K; ++k) nxt[k] = load_row_vec<T, ALIGNED>(nxrow, voff[k], a.n_cols);
+            }
+            float mean0 = 0.0f, mean = 0.0f, rstd, delta = 0.0f;
+            if constexpr (LN) {
+                float s[1] = {0.0f};
+#pragma unroll
+                for (int k = 0; k < K; ++k) {
+                    float xf[VEC];
+                    T::unpack(cur[k], xf);
+                    float sk = 0.0f;
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e) sk += xf[e];
+                    s[0] += own[k] ? sk : 0.0f;
+                }
+                row_allreduce<TPR, G, 1>(s, red, phase, g, t);
+                forget_derived(cur);
+                mean0 = s[0] * a.inv_n;
+                float q[2] = {0.0f, 0.0f};
+#pragma unroll
+                for (int k = 0; k < K; ++k) {
+                    float xf[VEC];
+                    T::unpack(cur[k], xf);
+                    float q0 = 0.0f, q1 = 0.0f;
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e) {
+                        float d = xf[e] - mean0;
+                        if constexpr (!ALIGNED) d = (voff[k] * VEC + e < a.n_cols) ? d : 0.0f;
+                        q0 += d;
+                        q1 = fmaf(d, d, q1);
+                    }
+                    q[0] += own[k] ? q0 : 0.0f;
+                    q[1] += own[k] ? q1 : 0.0f;
+                }
+                row_allreduce<TPR, G, 2>(q, red, phase, g, t);
+                forget_derived(cur);
+                delta = q[0] * a.inv_n;
+                const float var = fmaxf(fmaf(-delta, delta, q[1] * a.inv_n), 0.0f);
+                rstd = rsqrt_refined(var + a.eps);
+                mean = mean0 + delta;
+            } else {
+                float q[1] = {0.0f};
+#pragma unroll
+                for (int k = 0; k < K; ++k) {
+                    float xf[VEC];
+                    T::unpack(cur[k], xf);
+                    float qk = 0.0f;
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e) qk = fmaf(xf[e], xf[e], qk);
+                    q[0] += own[k] ? qk : 0.0f;
+                }
+                row_allreduce<TPR, G, 1>(q, red, phase, g, t);
+                forget_derived(cur);
+                rstd = rsqrt_refined(fmaf(q[0], a.inv_n, a.eps));
+            }
+            char* yrow = a.y + row * a.y_stride_bytes;
+#pragma unroll
+            for (int k = 0; k < K; ++k) {
+                float xf[VEC], yf[VEC];
+                T::unpack(cur[k], xf);
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) {
+                    if constexpr (LN) {
+                        float d = xf[e] - mean0;
+                        if constexpr (!ALIGNED) d = (voff[k] * VEC + e < a.n_cols) ? d : 0.0f;
+                        yf[e] = fmaf((d - delta) * rstd, wr[k][e], br[k][e]);
+                    } else {
+                        yf[e] = xf[e] * rstd * wr[k][e];
+                    }
+                    if constexpr (ACT != kNoAct) yf[e] = act_fwd<ACT, float>(yf[e], 0.0f, 0.0f);
+                }
+                store_row_vec<T, ALIGNED>(yrow, voff[k], a.n_cols, yf);
+                if constexpr (kForm.ahead) cur[k] = nxt[k];
+                else cur[k] = load_row_vec<T, ALIGNED>(nxrow, voff[k], a.n_cols);
+            }
+            if constexpr (LN) a.mean[row] = mean;
+            a.rstd[row] = rstd;
+            row_raw = nrow_raw;
+            row = nrow;
+        }
+        return;
+    }
     for (int64_t base = static_cast<int64_t>(blockIdx.x) * G; base < a.M; base += rows_per_iter) {
         const int64_t nrow_raw = row_raw + rows_per_iter;
         const int64_t nrow = nrow_raw < a.M ? nrow_raw : last_row;
@@ -292,8 +432,15 @@ __global__ void __launch_bounds__(BLOCK) norm_bwd_kernel(const BwdArgs a) {
     float c_mean = LN ? a.mean[row] : 0.0f;
     float c_rstd = a.rstd[row];
 
+    // RowForm::lds_dw: the dW sums of a thread (24 or 32 floats) live in LDS, in slots that only this thread
+    // touches (no barrier), 16 bytes per access.
+    constexpr RowForm kForm = bwd_form<T::kBytes, LN, K, BLOCK, FUSED>();
+    constexpr bool kLdsTotals = kForm.lds_dw;
+    static_assert(!kLdsTotals || (G == 1 && VEC == 8), "one row per workgroup, eight columns per vector");
+    __shared__ f32x4 dw_lds[kLdsTotals ? K * 2 * BLOCK : 1];
+
     float wr[K][VEC];
-    Acc dw[K][VEC];
+    Acc dw[kLdsTotals ? 1 : K][VEC];
     Acc db[LN ? K : 1][VEC];
     load_params_clamped<K, VEC, ALIGNED>(wr, a.w, a.w_dtype, voff, a.n_cols, 1.0f);
     float br[(FUSED && LN) ? K : 1][VEC];
@@ -302,8 +449,12 @@ __global__ void __launch_bounds__(BLOCK) norm_bwd_kernel(const BwdArgs a) {
     for (int k = 0; k < K; ++k) {
 #pragma unroll
         for (int e = 0; e < VEC; ++e) {
-            dw[k][e] = Acc(0);
+            if constexpr (!kLdsTotals) dw[k][e] = Acc(0);
             if constexpr (LN) db[k][e] = Acc(0);
+        }
+        if constexpr (kLdsTotals) {
+            dw_lds[(2 * k) * BLOCK + tid] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+            dw_lds[(2 * k + 1) * BLOCK + tid] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
         }
     }
 
@@ -421,10 +572,162 @@ __global__ void __launch_bounds__(BLOCK) norm_bwd_kernel(const BwdArgs a) {
         row = nrow;
     };
 
+    // The same step in the forms of RowForm::recompute: nothing but the packed vectors of the row lives across
+    // the reduction rounds.
+    auto lean_step = [&](auto masked_tag) {
+        constexpr bool MASKED = decltype(masked_tag)::value;
+        const int64_t nrow_raw = row_raw + rows_per_iter;
+        const int64_t nrow = nrow_raw < a.M ? nrow_raw : last_row;
+        const bool live = !MASKED || row_raw < a.M;
+        const char* nxrow = a.x + nrow * a.x_stride_bytes;
+        const char* ngrow = a.dy + nrow * a.dy_stride_bytes;
+        u32x4 nx[kForm.ahead ? K : 1], ng[kForm.ahead ? K : 1];
+        if constexpr (kForm.ahead) {
+#pragma unroll
+            for (int k = 0; k < K; ++k) nx[k] = load_row_vec<T, ALIGNED>(nxrow, voff[k], a.n_cols);
+#pragma unroll
+            for (int k = 0; k < K; ++k) ng[k] = load_row_vec<T, ALIGNED>(ngrow, voff[k], a.n_cols);
+        }
+        const float n_mean = LN ? a.mean[nrow] : 0.0f;
+        const float n_rstd = a.rstd[nrow];
+
+        // float32 view of vector slot k: u (LayerNorm: before the dlt correction unless `dlt_f` carries it) and
+        // the upstream gradient (times act'(z) with an epilogue)
+        auto expand = [&](int k, float dlt_f, bool corrected, float (&u)[VEC], float (&gf)[VEC]) {
+            T::unpack(cx[k], u);
+            T::unpack(cg[k], gf);
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+                if constexpr (LN) {
+                    float v = (u[e] - c_mean) * c_rstd;
+                    if constexpr (!ALIGNED) v = (voff[k] * VEC + e < a.n_cols) ? v : 0.0f;
+                    if constexpr (FUSED) {
+                        if (corrected) {
+                            v -= dlt_f;
+                            if constexpr (!ALIGNED) v = (voff[k] * VEC + e < a.n_cols) ? v : 0.0f;
+                        }
+                    }
+                    u[e] = v;
+                } else {
+                    u[e] *= c_rstd;
+                }
+                if constexpr (FUSED) {
+                    if (corrected) {
+                        const float z = LN ? fmaf(u[e], wr[k][e], br[k][e]) : u[e] * wr[k][e];
+                        gf[e] = act_bwd<ACT, float>(z, gf[e], 0.0f, 0.0f);
+                    }
+                }
+            }
+        };
+
+        float s[NV];
+#pragma unroll
+        for (int i = 0; i < NV; ++i) s[i] = 0.0f;
+        float dlt_fused = 0.0f;
+        if constexpr (FUSED && LN) {
+            float su[1] = {0.0f};
+#pragma unroll
+            for (int k = 0; k < K; ++k) {
+                float u[VEC], gf[VEC];
+                expand(k, 0.0f, false, u, gf);
+                float sk = 0.0f;
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) sk += u[e];
+                su[0] += own[k] ? sk : 0.0f;
+            }
+            row_allreduce<TPR, G, 1>(su, red, phase, g, t);
+            forget_derived(cx);
+            forget_derived(cg);
+            dlt_fused = su[0] * a.inv_n;
+        }
+#pragma unroll
+        for (int k = 0; k < K; ++k) {
+            float u[VEC], gf[VEC];
+            expand(k, dlt_fused, true, u, gf);
+            float s0 = 0.0f, s1 = 0.0f, s2 = 0.0f;
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+                const float wdy = wr[k][e] * gf[e];
+                s0 = fmaf(u[e], wdy, s0);
+                if constexpr (LN) {
+                    s1 += wdy;
+                    if constexpr (!FUSED) s2 += u[e];
+                }
+            }
+            s[0] += own[k] ? s0 : 0.0f;
+            if constexpr (LN) {
+                s[1] += own[k] ? s1 : 0.0f;
+                if constexpr (!FUSED) s[2] += own[k] ? s2 : 0.0f;
+            }
+        }
+        row_allreduce<TPR, G, NV>(s, red, phase, g, t);
+        forget_derived(cx);
+        forget_derived(cg);
+        float c1, c2 = 0.0f, dlt = 0.0f;
+        if constexpr (LN && FUSED) {
+            c2 = s[1] * a.inv_n;
+            c1 = s[0] * a.inv_n;
+        } else if constexpr (LN) {
+            dlt = s[2] * a.inv_n;
+            c2 = s[1] * a.inv_n;
+            c1 = fmaf(-dlt, c2, s[0] * a.inv_n);
+        } else {
+            c1 = s[0] * a.inv_n;
+        }
+
+        char* dxrow = a.dx + row * a.dx_stride_bytes;
+#pragma unroll
+        for (int k = 0; k < K; ++k) {
+            float u[VEC], gf[VEC], dxf[VEC];
+            expand(k, dlt_fused, true, u, gf);
+            float tot[kLdsTotals ? VEC : 1];
+            if constexpr (kLdsTotals) {
+                const f32x4 lo = dw_lds[(2 * k) * BLOCK + tid], hi = dw_lds[(2 * k + 1) * BLOCK + tid];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) { tot[e] = lo[e]; tot[4 + e] = hi[e]; }
+            }
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+                const float wdy = wr[k][e] * gf[e];
+                float xhat = u[e];
+                if constexpr (LN) {
+                    xhat -= dlt;
+                    if constexpr (!ALIGNED) xhat = (voff[k] * VEC + e < a.n_cols) ? xhat : 0.0f;
+                }
+                dxf[e] = (wdy - fmaf(xhat, c1, c2)) * c_rstd;
+                const float gl = (MASKED && !live) ? 0.0f : gf[e];
+                if constexpr (kLdsTotals) tot[e] = fmaf(gl, xhat, tot[e]);
+                else dw[k][e] = fma(static_cast<Acc>(gl), static_cast<Acc>(xhat), dw[k][e]);
+                if constexpr (LN) db[k][e] += static_cast<Acc>(gl);
+            }
+            if constexpr (kLdsTotals) {
+                dw_lds[(2 * k) * BLOCK + tid] = f32x4{tot[0], tot[1], tot[2], tot[3]};
+                dw_lds[(2 * k + 1) * BLOCK + tid] = f32x4{tot[4], tot[5], tot[6], tot[7]};
+            }
+            store_row_vec<T, ALIGNED>(dxrow, voff[k], a.n_cols, dxf);
+            if constexpr (kForm.ahead) {
+                cx[k] = nx[k];
+                cg[k] = ng[k];
+            } else {
+                cx[k] = load_row_vec<T, ALIGNED>(nxrow, voff[k], a.n_cols);
+                cg[k] = load_row_vec<T, ALIGNED>(ngrow, voff[k], a.n_cols);
+            }
+        }
+        c_mean = n_mean;
+        c_rstd = n_rstd;
+        row_raw = nrow_raw;
+        row = nrow;
+    };
+
     drain_vector_memory();
     int64_t base = static_cast<int64_t>(blockIdx.x) * G;
-    for (; base + G <= a.M; base += rows_per_iter) step(std::false_type{});
-    if (base < a.M) step(std::true_type{});
+    if constexpr (kForm.recompute) {
+        for (; base + G <= a.M; base += rows_per_iter) lean_step(std::false_type{});
+        if (base < a.M) lean_step(std::true_type{});
+    } else {
+        for (; base + G <= a.M; base += rows_per_iter) step(std::false_type{});
+        if (base < a.M) step(std::true_type{});
+    }
 
     // Workgroup partial: tree over the G row groups, then group 0 stores its K vectors of VEC floats.
     // Clamped vector slots hold a copy of their owner's sums and are simply not written.
@@ -432,6 +735,12 @@ __global__ void __launch_bounds__(BLOCK) norm_bwd_kernel(const BwdArgs a) {
     const bool want_db = LN && a.db_part != nullptr;
 #pragma unroll
     for (int k = 0; k < K; ++k) {
+        float dwk[VEC];
+        if constexpr (kLdsTotals) {
+            const f32x4 lo = dw_lds[(2 * k) * BLOCK + tid], hi = dw_lds[(2 * k + 1) * BLOCK + tid];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) { dwk[e] = lo[e]; dwk[4 + e] = hi[e]; }
+        }
         if constexpr (G > 1) {
             if (want_dw) combine_groups<BLOCK, TPR, VEC, Acc>(dw[k], comb, g, t);
             if constexpr (LN) {
@@ -444,7 +753,11 @@ __global__ void __launch_bounds__(BLOCK) norm_bwd_kernel(const BwdArgs a) {
             const int64_t off = static_cast<int64_t>(blockIdx.x) * a.part_pitch + static_cast<int64_t>(v) * VEC;
 #pragma unroll
             for (int e = 0; e < VEC; ++e) {
-                if (want_dw) a.dw_part[off + e] = static_cast<float>(dw[k][e]);
+                if constexpr (kLdsTotals) {
+                    if (want_dw) a.dw_part[off + e] = dwk[e];
+                } else {
+                    if (want_dw) a.dw_part[off + e] = static_cast<float>(dw[k][e]);
+                }
                 if constexpr (LN) {
                     if (want_db) a.db_part[off + e] = static_cast<float>(db[k][e]);
                 }
