@@ -784,8 +784,13 @@ int thn_norm_bwd_reduce_partials(const void* workspace, int32_t num_partials, vo
     r.n_cols = static_cast<int>(N);
     r.n_parts = num_partials;
     r.w_dtype = w_dtype;
-    const dim3 grid(static_cast<unsigned>((N + thn::kReduceCols - 1) / thn::kReduceCols), static_cast<unsigned>(n));
-    hipLaunchKernelGGL(thn::reduce_partials_kernel, grid, dim3(256), 0, static_cast<hipStream_t>(stream), r);
+    if (N >= thn::kReduceWideFrom) {
+        const dim3 grid(static_cast<unsigned>((N + thn::kReduceColsWide - 1) / thn::kReduceColsWide), static_cast<unsigned>(n));
+        hipLaunchKernelGGL(thn::reduce_partials_kernel<thn::kReduceColsWide>, grid, dim3(256), 0, static_cast<hipStream_t>(stream), r);
+    } else {
+        const dim3 grid(static_cast<unsigned>((N + thn::kReduceCols - 1) / thn::kReduceCols), static_cast<unsigned>(n));
+        hipLaunchKernelGGL(thn::reduce_partials_kernel<thn::kReduceCols>, grid, dim3(256), 0, static_cast<hipStream_t>(stream), r);
+    }
     return hipGetLastError() == hipSuccess ? THN_OK : THN_E_LAUNCH;
 }
 

@@ -10,7 +10,9 @@ namespace thn {
 // rounded once to the parameter's storage type.  The stage is pure latency (a few MiB, one dependent launch),
 // so it is cut for parallelism: a workgroup owns 16 columns (4 lanes x float4) and has 64 row slices, each
 // adding every 64th partial row (4 independent loads for 256 partial rows); the slice sums are then added in
-// slice order through LDS.  N / 16 workgroups: every compute unit takes part from N = 4096 on.
+// slice order through LDS.  N / 16 workgroups: every compute unit takes part from N = 4096 on.  From 6144
+// columns on the stage moves 6 MiB and more per gradient and takes 64 columns x 16 slices per workgroup instead
+// (256-byte segments per partial row; measured 2x faster at 16384 columns and more, equal at 8192).
 // blockIdx.y selects dW (0) or dB (1).
 // ---------------------------------------------------------------------------------------------------
 struct ReduceArgs {
@@ -22,13 +24,14 @@ struct ReduceArgs {
     int w_dtype;
 };
 
-#ifndef THN_REDUCE_COLS
-#define THN_REDUCE_COLS 16
-#endif
-constexpr int kReduceCols = THN_REDUCE_COLS;        // columns per workgroup
-constexpr int kReduceSlices = 1024 / kReduceCols;   // row slices per workgroup (256 threads x float4)
+constexpr int kReduceCols = 16;       // columns per workgroup up to kReduceWideFrom columns
+constexpr int kReduceColsWide = 64;   // beyond: 256-byte segments per partial row, still one workgroup or more per compute unit
+constexpr int kReduceWideFrom = 6144;
 
+template <int COLS>
 __global__ void __launch_bounds__(256) reduce_partials_kernel(const ReduceArgs a) {
+    constexpr int kReduceCols = COLS;
+    constexpr int kReduceSlices = 1024 / COLS;     // row slices per workgroup (256 threads x float4)
     __shared__ double acc[kReduceSlices][kReduceCols];
     const int which = blockIdx.y;
     const float* part = a.part[which];
