@@ -289,7 +289,7 @@ int thn_norm_set_launch_override(int which, int vecs_per_thread, int threads_per
 
 /*
  * What the heuristic (or the override) would launch for this problem: fills shape[0..4] with
- * {vecs_per_thread, threads_per_row, block_threads, grid_blocks, vector_path (1) or scalar fallback (0)}.
+ * {vecs_per_thread, threads_per_row, block_threads, grid_blocks, aligned 128-bit path (1) or unaligned-row path (0)}.
  * For the epilogue families (9, 10) `is_layernorm` carries the activation too: bit 0 = LayerNorm, bits 1.. = the
  * thn_act code.
  */

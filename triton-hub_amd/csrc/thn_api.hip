@@ -205,30 +205,39 @@ int occupancy(int which, int dtype, int flavour, bool aligned, Shape s) {
     int rc;
     if (which == kNormFwd) {
         FwdArgs dummy{};
+        dummy.n_cols = 1 << 20;      // the unaligned-window instances, not the ones for rows shorter than a vector
         rc = launch_fwd(dtype, flavour, aligned, s, dummy, 0, nullptr, &occ);
     } else if (which == kNormBwd) {
         BwdArgs dummy{};
+        dummy.n_cols = 1 << 20;      // the unaligned-window instances, not the ones for rows shorter than a vector
         rc = launch_bwd(dtype, flavour, aligned, s, dummy, 0, nullptr, &occ);
     } else if (which == kSoftmaxFwd) {
         SoftmaxFwdArgs dummy{};
+        dummy.n_cols = 1 << 20;      // the unaligned-window instances, not the ones for rows shorter than a vector
         rc = launch_softmax_fwd(dtype, flavour, aligned, s, dummy, 0, nullptr, &occ);
     } else if (which == kSoftmaxBwd) {
         SoftmaxBwdArgs dummy{};
+        dummy.n_cols = 1 << 20;      // the unaligned-window instances, not the ones for rows shorter than a vector
         rc = launch_softmax_bwd(dtype, flavour, aligned, s, dummy, 0, nullptr, &occ);
     } else if (which == kFusedFwd) {
         FwdArgs dummy{};
+        dummy.n_cols = 1 << 20;      // the unaligned-window instances, not the ones for rows shorter than a vector
         rc = launch_fused_fwd(dtype, flavour, aligned, s, dummy, 0, nullptr, &occ);
     } else if (which == kFusedBwd) {
         BwdArgs dummy{};
+        dummy.n_cols = 1 << 20;      // the unaligned-window instances, not the ones for rows shorter than a vector
         rc = launch_fused_bwd(dtype, flavour, aligned, s, dummy, 0, nullptr, &occ);
     } else if (which == kPnormFwd) {
         PnormFwdArgs dummy{};
+        dummy.n_cols = 1 << 20;      // the unaligned-window instances, not the ones for rows shorter than a vector
         rc = launch_pnorm_fwd(dtype, flavour, aligned, s, dummy, 0, nullptr, &occ);
     } else if (which == kPnormBwd) {
         PnormBwdArgs dummy{};
+        dummy.n_cols = 1 << 20;      // the unaligned-window instances, not the ones for rows shorter than a vector
         rc = launch_pnorm_bwd(dtype, flavour, aligned, s, dummy, 0, nullptr, &occ);
     } else {
         NormalizeBwdArgs dummy{};
+        dummy.n_cols = 1 << 20;      // the unaligned-window instances, not the ones for rows shorter than a vector
         rc = launch_normalize_bwd(dtype, flavour, aligned, s, dummy, 0, nullptr, &occ);
     }
     if (rc != 0 || occ <= 0) occ = 1;
@@ -258,7 +267,8 @@ constexpr int kTprList[] = {8, 16, 32, 64, 128, 256, 512, 1024};
 //             threads cannot cover otherwise; 512-thread workgroups once a row spans two waves or more, which
 //             also halves the number of partial rows;
 //   softmax / normalize / epilogue backward (two or three input streams): kmax 2 up to 32 KiB rows.
-// Workgroups per compute unit: one (kDefaultBlocksPerCu), except where default_blocks_per_cu() says otherwise.
+// Workgroups per compute unit: one (kDefaultBlocksPerCu), except where default_blocks_per_cu() or
+// narrow_row_blocks_per_cu() say otherwise.
 constexpr int kDefaultBlocksPerCu = 1;
 
 int ceil_div(int a, int b) { return (a + b - 1) / b; }
@@ -269,7 +279,7 @@ Shape heuristic_shape(int which, bool aligned, int n_vecs) {
     // except for 2 KiB rows, where one full wave per row (2 x 64) is 8 % slower than half a wave (4 x 32).
     if (aligned && which == kSoftmaxBwd && n_vecs <= 2048 && !(n_vecs > 64 && n_vecs <= 128)) kmax = 2;
     if (aligned && which == kNormalizeBwd && n_vecs <= 2048) kmax = 2;    // two or three input streams
-    if (aligned && which == kFusedBwd && n_vecs <= 2048) kmax = 2;        // bias and pre-activation are live too
+    if (aligned && which == kFusedBwd && n_vecs <= 2048) kmax = n_vecs > 128 ? 3 : 2;   // bias and pre-activation are live too
     Shape s{4, 1024, 1024};
     for (int tpr : kTprList) {
         if (static_cast<int64_t>(tpr) * kmax >= n_vecs) {
@@ -282,6 +292,7 @@ Shape heuristic_shape(int which, bool aligned, int n_vecs) {
         s.block = s.tpr > 256 ? s.tpr : 256;
         return s;
     }
+    if (which == kNormBwd && n_vecs > 8 && n_vecs <= 16) s.tpr = 16;      // 256-byte rows: one vector per thread
     s.k = ceil_div(n_vecs, s.tpr);
     if (s.k == 3 && s.tpr < 64) s.k = 4;     // K = 3 is only compiled for TPR >= 64
     if (which != kNormBwd && which != kFusedBwd) s.block = s.tpr > 256 ? s.tpr : 256;
@@ -298,6 +309,22 @@ int default_blocks_per_cu(int which, int flavour, int block) {
     // as many workgroups per compute unit as their registers allow, up to four.
     if ((which == kFusedFwd || which == kFusedBwd) && ((flavour >> 1) == thn::kGelu || (flavour >> 1) == thn::kGeluTanh)) return 4;
     return kDefaultBlocksPerCu;
+}
+
+// Rows of at most 256 bytes: a thread holds one or two vectors, so one workgroup per compute unit keeps too few
+// bytes in flight (measured: bf16 N = 64 forward 3.1 TB/s with one workgroup per compute unit, 5.3 TB/s with
+// four; backward 4.3 -> 6.1 TB/s with two).  Families with one input stream take 4 workgroups up to 128-byte
+// rows and 2 up to 256-byte rows; those with two streams 2 up to 128-byte rows (the norm backward up to 256-byte
+// rows, where it runs one vector per thread: bf16 N = 128 5.2 -> 6.1 TB/s).
+int narrow_row_blocks_per_cu(int which, int n_vecs, bool ragged16) {
+    // 16-bit rows whose width is not a whole number of vectors: the unaligned-window instances spend 2-3 times
+    // the instructions per byte (shifts, per-column masks), and a second workgroup hides their latency
+    // (bf16 N = 4098: forward 2.6 -> 3.6 TB/s, RMSNorm 3.8 -> 4.6; float32 rows do not gain).
+    if (ragged16 && n_vecs > 16) return 2;
+    const bool one_stream = which == kNormFwd || which == kSoftmaxFwd || which == kPnormFwd || which == kFusedFwd;
+    if (n_vecs <= 8) return one_stream ? 4 : 2;
+    if (n_vecs <= 16) return (one_stream || which == kNormBwd) ? 2 : 1;   // norm backward: with one vector per thread
+    return 1;
 }
 
 int plan_launch(int which, int flavour, bool aligned, int64_t M, int64_t N, int dtype, Plan* out) {
@@ -324,7 +351,12 @@ int plan_launch(int which, int flavour, bool aligned, int64_t M, int64_t N, int 
     if (!shape_compiled(which, aligned, s)) return THN_E_SHAPE;
 
     int bpc = occupancy(which, dtype, flavour, aligned, s);
-    const int cap = ov.bpc.load() > 0 ? ov.bpc.load() : default_blocks_per_cu(which, flavour, s.block);
+    int cap = ov.bpc.load();
+    if (cap <= 0) {
+        cap = default_blocks_per_cu(which, flavour, s.block);
+        const int narrow = narrow_row_blocks_per_cu(which, n_vecs, bytes == 2 && N % vec_elems != 0);
+        if (narrow > cap) cap = narrow;
+    }
     if (cap < bpc) bpc = cap;
     const int rows_per_block = s.block / s.tpr;
     const int64_t row_blocks = (M + rows_per_block - 1) / rows_per_block;
@@ -358,6 +390,10 @@ int64_t bwd_workspace_bytes(int which, int flavour, int64_t M, int64_t N, int wa
     const int cus = current_cu_count();
     if (cus <= 0) return THN_E_DEVICE;
     int bpc = default_blocks_per_cu(which, flavour, 512);
+    const int vec_elems = 16 / bytes;
+    const int narrow = narrow_row_blocks_per_cu(which, static_cast<int>((N + vec_elems - 1) / vec_elems),
+                                                bytes == 2 && N % vec_elems != 0);
+    if (narrow > bpc) bpc = narrow;
     const int forced = g_override[which].bpc.load();
     if (forced > bpc) bpc = forced;
     if (bpc > kMaxBlocksPerCu) bpc = kMaxBlocksPerCu;

@@ -65,6 +65,7 @@ __device__ __forceinline__ float rsqrt_refined(float v) {
 // pack() narrows with round-to-nearest-even (v_cvt_pk_bf16_f32 / v_cvt_f16_f32 / v_cvt_f64_f32).
 // ---------------------------------------------------------------------------------------------------
 struct F32 {
+    static constexpr bool kWindowIo = true;   // rows that miss the 16-byte path use unaligned 16-byte windows
     static constexpr int kCode = kF32, kBytes = 4, VEC = 4;
     __device__ static __forceinline__ void unpack(u32x4 v, float (&f)[VEC]) {
         uint32_t a = v[0], b = v[1], c = v[2], d = v[3];
@@ -75,6 +76,11 @@ struct F32 {
         v[0] = as_u32(f[0]); v[1] = as_u32(f[1]); v[2] = as_u32(f[2]); v[3] = as_u32(f[3]);
         return v;
     }
+    using bits_t = uint32_t;
+    __device__ static __forceinline__ bits_t load_bits(const void* p, int64_t i) {
+        return reinterpret_cast<const uint32_t*>(p)[i];
+    }
+    __device__ static __forceinline__ float widen(bits_t u) { return as_f32(u); }
     __device__ static __forceinline__ float load1(const void* p, int64_t i) {
         return reinterpret_cast<const float*>(p)[i];
     }
@@ -84,6 +90,7 @@ struct F32 {
 };
 
 struct F16 {
+    static constexpr bool kWindowIo = true;   // rows that miss the 16-byte path use unaligned 16-byte windows
     static constexpr int kCode = kF16, kBytes = 2, VEC = 8;
     __device__ static __forceinline__ void unpack_pair(uint32_t u, float& lo, float& hi) {
         half2_t h = __builtin_bit_cast(half2_t, u);
@@ -108,6 +115,13 @@ struct F16 {
         }
         return v;
     }
+    using bits_t = uint16_t;
+    __device__ static __forceinline__ bits_t load_bits(const void* p, int64_t i) {
+        return reinterpret_cast<const uint16_t*>(p)[i];
+    }
+    __device__ static __forceinline__ float widen(bits_t u) {
+        return static_cast<float>(__builtin_bit_cast(_Float16, u));
+    }
     __device__ static __forceinline__ float load1(const void* p, int64_t i) {
         return static_cast<float>(reinterpret_cast<const _Float16*>(p)[i]);
     }
@@ -117,6 +131,7 @@ struct F16 {
 };
 
 struct BF16 {
+    static constexpr bool kWindowIo = true;   // rows that miss the 16-byte path use unaligned 16-byte windows
     static constexpr int kCode = kBF16, kBytes = 2, VEC = 8;
     __device__ static __forceinline__ void unpack_pair(uint32_t u, float& lo, float& hi) {
         lo = as_f32(u << 16);
@@ -140,6 +155,11 @@ struct BF16 {
         }
         return v;
     }
+    using bits_t = uint16_t;
+    __device__ static __forceinline__ bits_t load_bits(const void* p, int64_t i) {
+        return reinterpret_cast<const uint16_t*>(p)[i];
+    }
+    __device__ static __forceinline__ float widen(bits_t u) { return as_f32(static_cast<uint32_t>(u) << 16); }
     __device__ static __forceinline__ float load1(const void* p, int64_t i) {
         return as_f32(static_cast<uint32_t>(reinterpret_cast<const uint16_t*>(p)[i]) << 16);
     }
@@ -149,6 +169,7 @@ struct BF16 {
 };
 
 struct F64 {
+    static constexpr bool kWindowIo = true;   // rows that miss the 16-byte path use unaligned 16-byte windows
     static constexpr int kCode = kF64, kBytes = 8, VEC = 2;
     __device__ static __forceinline__ void unpack(u32x4 v, float (&f)[VEC]) {
         uint32_t a = v[0], b = v[1], c = v[2], d = v[3];
@@ -164,6 +185,13 @@ struct F64 {
         v[0] = static_cast<uint32_t>(lo); v[1] = static_cast<uint32_t>(lo >> 32);
         v[2] = static_cast<uint32_t>(hi); v[3] = static_cast<uint32_t>(hi >> 32);
         return v;
+    }
+    using bits_t = uint64_t;
+    __device__ static __forceinline__ bits_t load_bits(const void* p, int64_t i) {
+        return reinterpret_cast<const uint64_t*>(p)[i];
+    }
+    __device__ static __forceinline__ float widen(bits_t u) {
+        return static_cast<float>(__builtin_bit_cast(double, u));
     }
     __device__ static __forceinline__ float load1(const void* p, int64_t i) {
         return static_cast<float>(reinterpret_cast<const double*>(p)[i]);
@@ -223,21 +251,31 @@ __device__ __forceinline__ void load_param_chunk(const void* p, int c0, float (&
 // The K*VEC weight (or bias) elements of a thread's (clamped) vector slots, widened to float32.  The
 // storage type is only known at run time: one uniform branch on it, then independent loads at always valid
 // columns.  voff[k] is the slot's byte offset in a row on the 128-bit path (one wide load per slot), its
-// vector index on the element-wise path (element loads; columns past the row end read as `fill`).
+// vector index on the unaligned path (element loads; columns past the row end read as `fill`).
 template <typename WT, int K, int VEC, int ROW_BYTES_PER_ELEM, bool ALIGNED>
 __device__ __forceinline__ void load_params_as(float (&out)[K][VEC], const void* p, const int (&voff)[K],
                                                int n_cols, float fill) {
+    if constexpr (ALIGNED) {
 #pragma unroll
-    for (int k = 0; k < K; ++k) {
-        if constexpr (ALIGNED) {
-            load_param_chunk<WT, VEC>(p, voff[k] / ROW_BYTES_PER_ELEM, out[k]);
-        } else {
+        for (int k = 0; k < K; ++k) load_param_chunk<WT, VEC>(p, voff[k] / ROW_BYTES_PER_ELEM, out[k]);
+    } else {
+        // Two phases, so that the K*VEC element loads are all in flight before the first one is waited for
+        // (interleaved with their conversions they were issued one by one, each waiting for the previous: tens of
+        // microseconds at the start of every workgroup).
+        typename WT::bits_t raw[K][VEC];
+#pragma unroll
+        for (int k = 0; k < K; ++k) {
 #pragma unroll
             for (int e = 0; e < VEC; ++e) {
                 const int c = voff[k] * VEC + e;
-                const float v = WT::load1(p, c < n_cols ? c : n_cols - 1);
-                out[k][e] = c < n_cols ? v : fill;
+                raw[k][e] = WT::load_bits(p, c < n_cols ? c : n_cols - 1);
             }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int k = 0; k < K; ++k) {
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) out[k][e] = (voff[k] * VEC + e < n_cols) ? WT::widen(raw[k][e]) : fill;
         }
     }
 }
@@ -262,12 +300,72 @@ __device__ __forceinline__ void load_params_clamped(float (&out)[K][VEC], const 
 }
 
 // ---------------------------------------------------------------------------------------------------
-// Element-wise row I/O for rows that cannot use 128-bit accesses (N not a multiple of VEC, or a pointer or
-// row stride that is not a multiple of 16 bytes): the same 16-byte register image is assembled from element
-// loads with a per-column bound, so every other part of the kernels is shared with the 128-bit path.
+// Row I/O for rows that cannot use aligned 128-bit accesses (N not a multiple of VEC, or a pointer or row stride
+// that is not a multiple of 16 bytes): the same 16-byte register image is assembled from an unaligned 16-byte
+// window (rows of at least one vector) or from element loads with a per-column bound (ElemIo<T>: shorter rows),
+// so every other part of the kernels is shared with the 128-bit path.
 // ---------------------------------------------------------------------------------------------------
+// The same storage type, for rows shorter than one vector (N < VEC): every access is a single element.
+template <typename T>
+struct ElemIo : T {
+    static constexpr bool kWindowIo = false;
+};
+
+typedef u32x4 u32x4_unaligned __attribute__((aligned(2)));
+
+// 16-byte accesses at any element-aligned address (the hardware's unaligned access mode, which the HSA stack
+// enables; the compiler emits the same global_load_dwordx4 / global_store_dwordx4 as for aligned ones).
+__device__ __forceinline__ u32x4 ld128u(const void* p) {
+    return __builtin_nontemporal_load(reinterpret_cast<const u32x4_unaligned*>(p));
+}
+__device__ __forceinline__ void st128u(void* p, u32x4 v) {
+    __builtin_nontemporal_store(v, reinterpret_cast<u32x4_unaligned*>(p));
+}
+
+// The 128-bit value w shifted down by `bytes` (0..15, a multiple of 2), zeros shifted in at the top.
+__device__ __forceinline__ u32x4 shift_down_bytes(u32x4 w, int bytes) {
+    const bool by1 = (bytes & 4) != 0, by2 = (bytes & 8) != 0;
+    const uint32_t r = static_cast<uint32_t>(bytes & 3) * 8u;
+    uint32_t e0 = w[0], e1 = w[1], e2 = w[2], e3 = w[3];
+    e0 = by1 ? e1 : e0; e1 = by1 ? e2 : e1; e2 = by1 ? e3 : e2; e3 = by1 ? 0u : e3;
+    e0 = by2 ? e2 : e0; e1 = by2 ? e3 : e1; e2 = by2 ? 0u : e2; e3 = by2 ? 0u : e3;
+    u32x4 out;
+    out[0] = __builtin_amdgcn_alignbit(e1, e0, r);
+    out[1] = __builtin_amdgcn_alignbit(e2, e1, r);
+    out[2] = __builtin_amdgcn_alignbit(e3, e2, r);
+    out[3] = e3 >> r;
+    return out;
+}
+
+// Vector slot `vec` of a row of n_cols >= VEC elements at any element-aligned address, as the 16-byte register
+// image the 128-bit path would hold (columns past the row end read as 0): ONE 16-byte load of the window that
+// ends at the row end at the latest, shifted down when the slot is the ragged last one.  No branch.
+template <typename T>
+__device__ __forceinline__ u32x4 load_vec_window(const char* row, int vec, int n_cols) {
+    const int c0 = vec * T::VEC;
+    const int last = n_cols - T::VEC;
+    const int cw = c0 < last ? c0 : last;
+    return shift_down_bytes(ld128u(row + cw * T::kBytes), (c0 - cw) * T::kBytes);
+}
+
+// Stores slot `vec`: one 16-byte store when the whole slot lies inside the row, element stores for the ragged
+// last slot (one thread per row takes that branch).
+template <typename T>
+__device__ __forceinline__ void store_vec_window(char* row, int vec, int n_cols, const float (&f)[T::VEC]) {
+    const int c0 = vec * T::VEC;
+    if (c0 + T::VEC <= n_cols) {
+        st128u(row + c0 * T::kBytes, T::pack(f));
+    } else {
+#pragma unroll
+        for (int e = 0; e < T::VEC; ++e) {
+            if (c0 + e < n_cols) T::store1(row, c0 + e, f[e]);
+        }
+    }
+}
+
 template <typename T>
 __device__ __forceinline__ u32x4 load_vec_elems(const char* row, int vec, int n_cols) {
+    if constexpr (T::kWindowIo) return load_vec_window<T>(row, vec, n_cols);
     float f[T::VEC];
 #pragma unroll
     for (int e = 0; e < T::VEC; ++e) {
@@ -280,6 +378,10 @@ __device__ __forceinline__ u32x4 load_vec_elems(const char* row, int vec, int n_
 
 template <typename T>
 __device__ __forceinline__ void store_vec_elems(char* row, int vec, int n_cols, const float (&f)[T::VEC]) {
+    if constexpr (T::kWindowIo) {
+        store_vec_window<T>(row, vec, n_cols, f);
+        return;
+    }
 #pragma unroll
     for (int e = 0; e < T::VEC; ++e) {
         const int c = vec * T::VEC + e;

@@ -83,8 +83,11 @@ inline int run_kernel(void (*kern)(const Args), const Args& a, int grid, int blo
         using T = TYPE;                                                                                    \
         if (aligned) {                                                                                     \
             THN_FWD_SHAPES(THN_FWD_AL)                                                                     \
-        } else {                                                                                           \
-            THN_SCALAR_SHAPES(THN_FWD_SC)                                                                  \
+        } else if (a.n_cols >= TYPE::VEC) { \
+            THN_SCALAR_SHAPES(THN_FWD_SC) \
+        } else { \
+            using T = ElemIo<TYPE>; \
+            THN_FWD_SC(4, 8, 256) \
         }                                                                                                  \
         return 1;                                                                                          \
     }
@@ -95,8 +98,11 @@ inline int run_kernel(void (*kern)(const Args), const Args& a, int grid, int blo
         using T = TYPE;                                                                                    \
         if (aligned) {                                                                                     \
             THN_BWD_SHAPES(THN_BWD_AL)                                                                     \
-        } else {                                                                                           \
-            THN_SCALAR_SHAPES(THN_BWD_SC)                                                                  \
+        } else if (a.n_cols >= TYPE::VEC) { \
+            THN_SCALAR_SHAPES(THN_BWD_SC) \
+        } else { \
+            using T = ElemIo<TYPE>; \
+            THN_BWD_SC(4, 8, 256) \
         }                                                                                                  \
         return 1;                                                                                          \
     }

@@ -16,11 +16,13 @@ namespace thn {
     X(3, 256, 256) X(4, 256, 256) X(3, 512, 512) X(4, 512, 512)                      \
     X(3, 1024, 1024) X(4, 1024, 1024)
 
-// Backward: at most 2 vectors per thread (the bias and the recomputed pre-activation are live too), 512-thread
-// workgroups once a row spans two waves, 3 or 4 vectors only where 1024 threads cannot cover the row otherwise.
+// Backward: 2 or 3 vectors per thread (the bias and the recomputed pre-activation are live too; the GeLU
+// variants are arithmetic-bound, so vector slots without work cost their full share: with 3 as well as 2 a row
+// fills at least two thirds of its slots), 512-thread workgroups once a row spans two waves, 4 vectors only
+// where 1024 threads cannot cover the row otherwise.
 #define THN_FUSED_BWD_SHAPES(X)                                                      \
-    X(1, 8, 256) X(2, 8, 256) X(2, 16, 256) X(2, 32, 256) X(2, 64, 256)              \
-    X(2, 128, 512) X(2, 256, 512) X(2, 512, 512)                                     \
+    X(1, 8, 256) X(2, 8, 256) X(2, 16, 256) X(2, 32, 256) X(2, 64, 256) X(3, 64, 256) \
+    X(2, 128, 512) X(3, 128, 512) X(2, 256, 512) X(3, 256, 512) X(2, 512, 512) X(3, 512, 512) \
     X(2, 1024, 1024) X(3, 1024, 1024) X(4, 1024, 1024)
 
 #define THN_DECLARE_FUSED_LAUNCHERS(NAME)                                                                      \
@@ -58,8 +60,11 @@ THN_DECLARE_FUSED_LAUNCHERS(f64)
         using T = TYPE;                                                                                        \
         if (aligned) {                                                                                         \
             THN_FUSED_FWD_SHAPES(THN_FF_AL)                                                                    \
-        } else {                                                                                               \
-            THN_SCALAR_SHAPES(THN_FF_SC)                                                                       \
+        } else if (a.n_cols >= TYPE::VEC) { \
+            THN_SCALAR_SHAPES(THN_FF_SC) \
+        } else { \
+            using T = ElemIo<TYPE>; \
+            THN_FF_SC(4, 8, 256) \
         }                                                                                                      \
         return 1;                                                                                              \
     }
@@ -70,8 +75,11 @@ THN_DECLARE_FUSED_LAUNCHERS(f64)
         using T = TYPE;                                                                                        \
         if (aligned) {                                                                                         \
             THN_FUSED_BWD_SHAPES(THN_FB_AL)                                                                    \
-        } else {                                                                                               \
-            THN_SCALAR_SHAPES(THN_FB_SC)                                                                       \
+        } else if (a.n_cols >= TYPE::VEC) { \
+            THN_SCALAR_SHAPES(THN_FB_SC) \
+        } else { \
+            using T = ElemIo<TYPE>; \
+            THN_FB_SC(4, 8, 256) \
         }                                                                                                      \
         return 1;                                                                                              \
     }

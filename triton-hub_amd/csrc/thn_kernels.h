@@ -66,7 +66,7 @@ struct BwdArgs {
 };
 
 // Loads the K vectors of one row.  `row` is already clamped to a valid row; voff[k] is the byte offset of
-// the (clamped) vector slot k on the 128-bit path and the vector index on the element-wise path.
+// the (clamped) vector slot k on the aligned 128-bit path and the vector index on the unaligned path.
 template <typename T, int K, bool ALIGNED>
 __device__ __forceinline__ void load_row(u32x4 (&dst)[K], const char* base, int64_t stride_bytes, int64_t row,
                                          const int (&voff)[K], int n_cols) {
@@ -286,7 +286,7 @@ __global__ void __launch_bounds__(BLOCK) norm_fwd_kernel(const FwdArgs a) {
             for (int k = 0; k < K; ++k) {
                 float sk = 0.0f;
 #pragma unroll
-                for (int e = 0; e < VEC; ++e) sk += xf[k][e];   // element path: absent columns load as 0
+                for (int e = 0; e < VEC; ++e) sk += xf[k][e];   // unaligned path: absent columns load as 0
                 s[0] += own[k] ? sk : 0.0f;
             }
             row_allreduce<TPR, G, 1>(s, red, phase, g, t);

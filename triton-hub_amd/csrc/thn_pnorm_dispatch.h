@@ -65,8 +65,11 @@ THN_DECLARE_PNORM_LAUNCHERS(f64)
         using T = TYPE;                                                                                         \
         if (aligned) {                                                                                          \
             THN_ROW_SHAPES(THN_PNF_AL)                                                                          \
-        } else {                                                                                                \
-            THN_SCALAR_SHAPES(THN_PNF_SC)                                                                       \
+        } else if (a.n_cols >= TYPE::VEC) { \
+            THN_SCALAR_SHAPES(THN_PNF_SC) \
+        } else { \
+            using T = ElemIo<TYPE>; \
+            THN_PNF_SC(4, 8, 256) \
         }                                                                                                       \
         return 1;                                                                                               \
     }                                                                                                           \
@@ -81,8 +84,11 @@ THN_DECLARE_PNORM_LAUNCHERS(f64)
         using T = TYPE;                                                                                         \
         if (aligned) {                                                                                          \
             THN_ROW_SHAPES(THN_PNB_AL)                                                                          \
-        } else {                                                                                                \
-            THN_SCALAR_SHAPES(THN_PNB_SC)                                                                       \
+        } else if (a.n_cols >= TYPE::VEC) { \
+            THN_SCALAR_SHAPES(THN_PNB_SC) \
+        } else { \
+            using T = ElemIo<TYPE>; \
+            THN_PNB_SC(4, 8, 256) \
         }                                                                                                       \
         return 1;                                                                                               \
     }                                                                                                           \
@@ -91,8 +97,11 @@ THN_DECLARE_PNORM_LAUNCHERS(f64)
         using T = TYPE;                                                                                         \
         if (aligned) {                                                                                          \
             THN_ROW_SHAPES(THN_NZB_AL)                                                                          \
-        } else {                                                                                                \
-            THN_SCALAR_SHAPES(THN_NZB_SC)                                                                       \
+        } else if (a.n_cols >= TYPE::VEC) { \
+            THN_SCALAR_SHAPES(THN_NZB_SC) \
+        } else { \
+            using T = ElemIo<TYPE>; \
+            THN_NZB_SC(4, 8, 256) \
         }                                                                                                       \
         return 1;                                                                                               \
     }                                                                                                           \

@@ -36,10 +36,11 @@ struct SoftmaxBwdArgs {
 // Arithmetic type.  Float32 for 16- and 32-bit storage and for every log-softmax (logsoftmax.py:19, :61-62 widen
 // to float32 explicitly).  The reference's softmax / softmin kernels compute in the type they load
 // (softmax.py:18-23), so float64 rows are computed in float64.
-template <typename T, bool LOG> struct SoftmaxCompute { using type = float; };
-template <> struct SoftmaxCompute<F64, false> { using type = double; };
+template <typename T, bool LOG> struct SoftmaxCompute {
+    using type = typename std::conditional<T::kBytes == 8 && !LOG, double, float>::type;
+};
 
-// load_row for arithmetic type C: the element path of the float32 engine narrows float64 storage on load,
+// load_row for arithmetic type C: the unaligned path of the float32 engine narrows float64 storage on load,
 // which the float64 path must not do.
 template <typename T, typename C, int K, bool ALIGNED>
 __device__ __forceinline__ void load_row_as(u32x4 (&dst)[K], const char* base, int64_t stride_bytes, int64_t row,
@@ -218,7 +219,7 @@ __global__ void __launch_bounds__(BLOCK) softmax_bwd_kernel(const SoftmaxBwdArgs
 #pragma unroll
         for (int k = 0; k < K; ++k) {
             unpack_as<T>(cy[k], yf[k]);
-            unpack_as<T>(cg[k], gf[k]);      // element path: columns past the row end load as 0
+            unpack_as<T>(cg[k], gf[k]);      // unaligned path: columns past the row end load as 0
             C sk = C(0);
 #pragma unroll
             for (int e = 0; e < VEC; ++e) {

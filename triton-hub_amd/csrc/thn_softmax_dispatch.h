@@ -34,8 +34,11 @@ THN_DECLARE_SOFTMAX_LAUNCHERS(f64)
         using T = TYPE;                                                                                         \
         if (aligned) {                                                                                          \
             THN_FWD_SHAPES(THN_SMF_AL)                                                                          \
-        } else {                                                                                                \
-            THN_SCALAR_SHAPES(THN_SMF_SC)                                                                       \
+        } else if (a.n_cols >= TYPE::VEC) { \
+            THN_SCALAR_SHAPES(THN_SMF_SC) \
+        } else { \
+            using T = ElemIo<TYPE>; \
+            THN_SMF_SC(4, 8, 256) \
         }                                                                                                       \
         return 1;                                                                                               \
     }                                                                                                           \
@@ -44,8 +47,11 @@ THN_DECLARE_SOFTMAX_LAUNCHERS(f64)
         using T = TYPE;                                                                                         \
         if (aligned) {                                                                                          \
             THN_FWD_SHAPES(THN_SMB_AL)                                                                          \
-        } else {                                                                                                \
-            THN_SCALAR_SHAPES(THN_SMB_SC)                                                                       \
+        } else if (a.n_cols >= TYPE::VEC) { \
+            THN_SCALAR_SHAPES(THN_SMB_SC) \
+        } else { \
+            using T = ElemIo<TYPE>; \
+            THN_SMB_SC(4, 8, 256) \
         }                                                                                                       \
         return 1;                                                                                               \
     }
