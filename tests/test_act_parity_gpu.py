@@ -165,6 +165,24 @@ def test_strides_views_and_batch_shapes(name, dtype):
         assert y.is_contiguous() and dx.is_contiguous()
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16, torch.float64])
+def test_large_strided_and_misaligned_views(dtype):
+    """Views that take the strided kernel with many rows per workgroup and several steps along a row: ragged and
+    misaligned wide rows, every third row, rows of a few elements."""
+    g = torch.Generator().manual_seed(14)
+    for rows, width, view in ((1500, 2077, lambda t: t[:, 3:2070]), (1500, 2077, lambda t: t[::3, :2048]),
+                              (1500, 2077, lambda t: t[:, 1:2]), (60000, 24, lambda t: t[:, 1:20]),
+                              (7, 70001, lambda t: t[:, 2:69999])):
+        base = (torch.randn(rows, width, generator=g) * 2).to(dtype)
+        gbase = torch.randn(rows, width, generator=g).to(dtype)
+        bg, gg = base.cuda(), gbase.cuda()
+        for name in ("silu", "relu"):
+            announce(f"act large views {name} {dtype} {rows}x{width}")
+            xv, gv = view(base), view(gbase)
+            run_and_compare(name, xv.contiguous(), gv.contiguous(), f"{name} large view {rows}x{width}",
+                            x_gpu=view(bg).detach(), dy_gpu=view(gg))
+
+
 def test_empty_inputs():
     announce("act empty")
     for name in NAMES:

@@ -40,6 +40,7 @@ struct ActArgs {
     int64_t total_elems;  // flat kernels
     int64_t x_stride_bytes, g_stride_bytes, out_stride_bytes;   // row kernels
     int64_t M, N;         // row kernels
+    int lx;               // row kernels: log2 of the threads along a row
     float p0, p1;         // negative_slope | beta, threshold | threshold, value
 };
 
@@ -131,22 +132,64 @@ __global__ void __launch_bounds__(kActBlock) act_flat_kernel(const ActArgs a) {
 }
 
 // ---------------------------------------------------------------------------------------------------
-// Strided rows, or pointers that are not 16-byte aligned: one element per thread and step.  Correct for any
-// layout the reference accepts (unit column stride, arbitrary row strides); not tuned.
+// Strided rows, or pointers that are not 16-byte aligned: the same 16-byte vectors at element-aligned addresses
+// (the memory pipeline runs in unaligned access mode), tiled over (rows, vectors of a row).  A workgroup is
+// 2^lx threads along the row (consecutive lanes take consecutive vectors) by 256 >> lx rows, so rows of any width
+// fill it; every thread takes the same vector slot of U rows per step (all requested before the first is used),
+// walks the slots of a row with stride gridDim.x << lx and the rows with stride gridDim.y.  The elements behind
+// the last whole vector of a row go one by one, in the thread that owns that slot.
 // ---------------------------------------------------------------------------------------------------
 template <typename T, int ACT, bool BWD>
 __global__ void __launch_bounds__(kActBlock) act_rows_kernel(const ActArgs a) {
     using C = typename ActCompute<T, ACT>::type;
+    constexpr int VEC = T::VEC;
+    constexpr int U = BWD ? 2 : 4;
     const C p0 = static_cast<C>(a.p0), p1 = static_cast<C>(a.p1);
-    for (int64_t row = blockIdx.y; row < a.M; row += gridDim.y) {
-        const char* xr = a.x + row * a.x_stride_bytes;
-        const char* gr = BWD ? a.g + row * a.g_stride_bytes : nullptr;
-        char* outr = a.out + row * a.out_stride_bytes;
-        for (int64_t c = static_cast<int64_t>(blockIdx.x) * kActBlock + threadIdx.x; c < a.N;
-             c += static_cast<int64_t>(gridDim.x) * kActBlock) {
-            const C x = load_elem<T, C>(xr, c);
-            if constexpr (BWD) store_elem<T, C>(outr, c, act_bwd<ACT, C>(x, load_elem<T, C>(gr, c), p0, p1));
-            else store_elem<T, C>(outr, c, act_fwd<ACT, C>(x, p0, p1));
+    const int lx = a.lx;
+    const int tx = threadIdx.x & ((1 << lx) - 1);
+    const int ty = threadIdx.x >> lx;
+    const int64_t rows_per_block = kActBlock >> lx;
+    const int64_t slots = (a.N + VEC - 1) / VEC;          // vector slots of a row; the last may be ragged
+    const int64_t whole = a.N / VEC;
+    const int64_t vstep = static_cast<int64_t>(gridDim.x) << lx;
+    for (int64_t row0 = blockIdx.y * rows_per_block * U + ty; row0 < a.M; row0 += gridDim.y * rows_per_block * U) {
+        for (int64_t v = (static_cast<int64_t>(blockIdx.x) << lx) + tx; v < slots; v += vstep) {
+            u32x4 cx[U], cg[BWD ? U : 1];
+            if (v < whole) {
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    const int64_t row = row0 + u * rows_per_block;
+                    if (row < a.M) {
+                        cx[u] = ld128u(a.x + row * a.x_stride_bytes + v * 16);
+                        if constexpr (BWD) cg[u] = ld128u(a.g + row * a.g_stride_bytes + v * 16);
+                    }
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int64_t row = row0 + u * rows_per_block;
+                if (row >= a.M) continue;
+                char* outr = a.out + row * a.out_stride_bytes;
+                if (v < whole) {
+                    C xf[VEC], gf[VEC], of[VEC];
+                    unpack_as<T>(cx[u], xf);
+                    if constexpr (BWD) unpack_as<T>(cg[u], gf);
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e) {
+                        if constexpr (BWD) of[e] = act_bwd<ACT, C>(xf[e], gf[e], p0, p1);
+                        else of[e] = act_fwd<ACT, C>(xf[e], p0, p1);
+                    }
+                    st128u(outr + v * 16, pack_as<T, C>(of));
+                } else {
+                    const char* xr = a.x + row * a.x_stride_bytes;
+                    const char* gr = BWD ? a.g + row * a.g_stride_bytes : nullptr;
+                    for (int64_t c = v * VEC; c < a.N; ++c) {
+                        const C x = load_elem<T, C>(xr, c);
+                        if constexpr (BWD) store_elem<T, C>(outr, c, act_bwd<ACT, C>(x, load_elem<T, C>(gr, c), p0, p1));
+                        else store_elem<T, C>(outr, c, act_fwd<ACT, C>(x, p0, p1));
+                    }
+                }
+            }
         }
     }
 }

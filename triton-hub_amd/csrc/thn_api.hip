@@ -674,9 +674,21 @@ int act_launch(const void* x, int64_t x_row_stride, const void* g, int64_t g_row
         a.x_stride_bytes = x_row_stride * bytes;
         a.g_stride_bytes = g_row_stride * bytes;
         a.out_stride_bytes = out_row_stride * bytes;
-        const int64_t col_blocks = (N + thn::kActBlock - 1) / thn::kActBlock;
-        grid = dim3(static_cast<unsigned>(col_blocks < 1024 ? col_blocks : 1024),
-                    static_cast<unsigned>(M < 65535 ? M : 65535));
+        // Threads along a row: one per vector slot, at most the whole workgroup; a thread takes `vecs` rows per step.
+        const int vecs = bwd ? thn::kActBwdVecs : thn::kActFwdVecs;
+        const int64_t slots = (N + 16 / bytes - 1) / (16 / bytes);
+        int lx = 0;
+        while (lx < 8 && (int64_t{1} << lx) < slots) ++lx;
+        a.lx = lx;
+        const int64_t col_blocks = (slots + (int64_t{1} << lx) - 1) >> lx;
+        const int64_t rows_per_block = static_cast<int64_t>(thn::kActBlock >> lx) * vecs;
+        const int64_t row_blocks = (M + rows_per_block - 1) / rows_per_block;
+        const int64_t cap = static_cast<int64_t>(cus) * (bpc_override > 0 ? bpc_override : 4);
+        int64_t gy = row_blocks < cap ? row_blocks : cap;
+        if (gy > 65535) gy = 65535;
+        int64_t gx = (cap + gy - 1) / gy;           // few rows: spread the slots of a row over workgroups too
+        if (gx > col_blocks) gx = col_blocks;
+        grid = dim3(static_cast<unsigned>(gx), static_cast<unsigned>(gy < 1 ? 1 : gy));
     }
     hipStream_t st = static_cast<hipStream_t>(stream);
     int lrc;
