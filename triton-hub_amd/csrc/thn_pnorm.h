@@ -457,12 +457,14 @@ __global__ void __launch_bounds__(BLOCK) normalize_bwd_kernel(const NormalizeBwd
 }
 
 // ---------------------------------------------------------------------------------------------------
-// Looping kernels: one 256-thread workgroup per row (grid-stride over rows), the row walked in strides of
-// 256 elements as often as the formula needs it (the second walk of a row comes from the L2).  Any row
-// width, any real p in [1, 6] (accurate powf), any alignment.  This is the path of rows wider than 64 KiB
-// and of non-integer p; it is not tuned.
+// Looping kernels: one 256-thread workgroup per row (grid-stride over rows), the row walked as often as the
+// formula needs it (the second walk of a row comes from the L2 or the Infinity Cache).  Any row width, any real
+// p in [1, 6] (accurate powf), any alignment.  This is the path of rows wider than 64 KiB and of non-integer p.
+// A walk moves 16-byte vectors at element-aligned addresses (unaligned access mode), 4 per thread and step, all
+// requested before the first is used; the elements behind the last whole vector go one by one.
 // ---------------------------------------------------------------------------------------------------
 constexpr int kLoopBlock = 256;
+constexpr int kLoopVecs = 4;
 
 // ax^e for ax >= 0; e_int is e when e is an integer in [0, 6], else -1.
 __device__ __forceinline__ float pow_abs_any(float ax, float e, int e_int) {
@@ -472,28 +474,77 @@ __device__ __forceinline__ float pow_abs_any(float ax, float e, int e_int) {
     return powf(ax, e);
 }
 
+// One walk over a row of n elements: fn(in0[c], in1[c], in2[c]) for every column c (absent streams pass 0); its
+// value is stored to out[c] when STORE.  Thread t takes vectors t, t + 256, ... .
+template <typename T, int NIN, bool STORE, typename Fn>
+__device__ __forceinline__ void walk_row(const char* in0, const char* in1, const char* in2, char* out, int64_t n,
+                                         int t, Fn&& fn) {
+    constexpr int VEC = T::VEC;
+    constexpr int U = kLoopVecs;
+    const char* in[3] = {in0, in1, in2};
+    const int64_t whole = n / VEC;
+    for (int64_t v0 = t; v0 < whole; v0 += kLoopBlock * U) {
+        u32x4 raw[U][NIN];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int64_t v = v0 + u * kLoopBlock;
+            if (v < whole) {
+#pragma unroll
+                for (int i = 0; i < NIN; ++i) raw[u][i] = ld128u(in[i] + v * 16);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int64_t v = v0 + u * kLoopBlock;
+            if (v < whole) {
+                float f[3][VEC], o[VEC];
+#pragma unroll
+                for (int i = 0; i < NIN; ++i) T::unpack(raw[u][i], f[i]);
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) o[e] = fn(f[0][e], NIN > 1 ? f[1][e] : 0.0f, NIN > 2 ? f[2][e] : 0.0f);
+                if constexpr (STORE) st128u(out + v * 16, T::pack(o));
+            }
+        }
+    }
+    for (int64_t c = whole * VEC + t; c < n; c += kLoopBlock) {
+        const float o = fn(T::load1(in0, c), NIN > 1 ? T::load1(in1, c) : 0.0f, NIN > 2 ? T::load1(in2, c) : 0.0f);
+        if constexpr (STORE) T::store1(out, c, o);
+    }
+}
+
 template <typename T, bool NORMALIZE>
 __global__ void __launch_bounds__(kLoopBlock) pnorm_fwd_loop_kernel(const PnormFwdArgs a) {
     __shared__ float red[RedSmem<kLoopBlock, 1, 1>::kFloats];
     int phase = 0;
     const int t = threadIdx.x;
+    const int p_int = a.p_int;
+    const float p = a.p;
     for (int64_t row = blockIdx.x; row < a.rows; row += gridDim.x) {
         const char* xrow = a.x + row_offset(a.xmap, a.walk, row);
         float s[1] = {0.0f};
-        for (int64_t c = t; c < a.n_cols64; c += kLoopBlock) {
-            const float x = T::load1(xrow, c);
-            s[0] += a.p_int == 2 ? x * x : pow_abs_any(__builtin_fabsf(x), a.p, a.p_int > 0 ? a.p_int : -1);
+        float acc = 0.0f;
+        if (p_int == 2) {
+            walk_row<T, 1, false>(xrow, nullptr, nullptr, nullptr, a.n_cols64, t, [&](float x, float, float) {
+                acc = __builtin_fmaf(x, x, acc);
+                return 0.0f;
+            });
+        } else {
+            walk_row<T, 1, false>(xrow, nullptr, nullptr, nullptr, a.n_cols64, t, [&](float x, float, float) {
+                acc += pow_abs_any(__builtin_fabsf(x), p, p_int > 0 ? p_int : -1);
+                return 0.0f;
+            });
         }
+        s[0] = acc;
         row_allreduce<kLoopBlock, 1, 1>(s, red, phase, 0, t);
         float n = s[0];
-        if (a.p_int == 2) n = sqrtf(n);
-        else if (a.p_int != 1) n = powf(n, 1.0f / a.p);
+        if (p_int == 2) n = sqrtf(n);
+        else if (p_int != 1) n = powf(n, 1.0f / p);
         n = fmaxf(n, a.eps);
         if (t == 0) T::store1(a.norms, row, n);
         if constexpr (NORMALIZE) {
             const float nr = round_to_storage<T>(n);
             char* yrow = a.y + row_offset(a.ymap, a.walk, row);
-            for (int64_t c = t; c < a.n_cols64; c += kLoopBlock) T::store1(yrow, c, T::load1(xrow, c) / nr);
+            walk_row<T, 1, true>(xrow, nullptr, nullptr, yrow, a.n_cols64, t, [&](float x, float, float) { return x / nr; });
         }
     }
 }
@@ -501,22 +552,26 @@ __global__ void __launch_bounds__(kLoopBlock) pnorm_fwd_loop_kernel(const PnormF
 template <typename T>
 __global__ void __launch_bounds__(kLoopBlock) pnorm_bwd_loop_kernel(const PnormBwdArgs a) {
     const int t = threadIdx.x;
+    const int p_int = a.p_int;
+    const float pm1 = a.p - 1.0f;
+    const int e_int = p_int > 0 ? p_int - 1 : -1;
     for (int64_t row = blockIdx.x; row < a.rows; row += gridDim.x) {
         const char* xrow = a.x + row_offset(a.xmap, a.walk, row);
         char* dxrow = a.dx + row_offset(a.dxmap, a.walk, row);
         const float g = T::load1(a.g, row);
         float den = 1.0f;
-        if (a.p_int != 1) {
+        if (p_int != 1) {
             const float n = T::load1(a.norms, row);
-            den = a.p_int == 2 ? n : pow_abs_any(n, a.p - 1.0f, a.p_int > 0 ? a.p_int - 1 : -1);
+            den = p_int == 2 ? n : pow_abs_any(n, pm1, e_int);
         }
-        for (int64_t c = t; c < a.n_cols64; c += kLoopBlock) {
-            const float x = T::load1(xrow, c);
-            float d;
-            if (a.p_int == 1) d = g * sign_of(x);
-            else if (a.p_int == 2) d = (g * x) / den;
-            else d = (g * sign_of(x) * pow_abs_any(__builtin_fabsf(x), a.p - 1.0f, a.p_int > 0 ? a.p_int - 1 : -1)) / den;
-            T::store1(dxrow, c, d);
+        if (p_int == 1) {
+            walk_row<T, 1, true>(xrow, nullptr, nullptr, dxrow, a.n_cols64, t, [&](float x, float, float) { return g * sign_of(x); });
+        } else if (p_int == 2) {
+            walk_row<T, 1, true>(xrow, nullptr, nullptr, dxrow, a.n_cols64, t, [&](float x, float, float) { return (g * x) / den; });
+        } else {
+            walk_row<T, 1, true>(xrow, nullptr, nullptr, dxrow, a.n_cols64, t, [&](float x, float, float) {
+                return (g * sign_of(x) * pow_abs_any(__builtin_fabsf(x), pm1, e_int)) / den;
+            });
         }
     }
 }
@@ -526,7 +581,9 @@ __global__ void __launch_bounds__(kLoopBlock) normalize_bwd_loop_kernel(const No
     __shared__ float red[RedSmem<kLoopBlock, 1, 1>::kFloats];
     int phase = 0;
     const int t = threadIdx.x;
-    const int e_int = a.p_int > 0 ? a.p_int - 1 : -1;
+    const int p_int = a.p_int;
+    const float pm1 = a.p - 1.0f;
+    const int e_int = p_int > 0 ? p_int - 1 : -1;
     for (int64_t row = blockIdx.x; row < a.rows; row += gridDim.x) {
         const char* xrow = a.x + row_offset(a.xmap, a.walk, row);
         const char* yrow = a.y + row_offset(a.ymap, a.walk, row);
@@ -534,25 +591,21 @@ __global__ void __launch_bounds__(kLoopBlock) normalize_bwd_loop_kernel(const No
         char* dxrow = a.dx + row_offset(a.dxmap, a.walk, row);
         const float n = T::load1(a.norms, row);
         float s[1] = {0.0f};
-        for (int64_t c = t; c < a.n_cols64; c += kLoopBlock) {
-            const float other = a.p_int == 1 ? T::load1(xrow, c) : T::load1(yrow, c);
-            s[0] = __builtin_fmaf(other, T::load1(grow, c), s[0]);
-        }
+        float acc = 0.0f;
+        walk_row<T, 2, false>(p_int == 1 ? xrow : yrow, grow, nullptr, nullptr, a.n_cols64, t, [&](float other, float gg, float) {
+            acc = __builtin_fmaf(other, gg, acc);
+            return 0.0f;
+        });
+        s[0] = acc;
         row_allreduce<kLoopBlock, 1, 1>(s, red, phase, 0, t);
         const float proj = s[0];
-        float coef = 0.0f;
-        if (a.p_int == 1) coef = proj / (n * n);
-        else if (a.p_int != 2) coef = proj / (pow_abs_any(n, a.p - 1.0f, e_int) * n);
-        for (int64_t c = t; c < a.n_cols64; c += kLoopBlock) {
-            const float gg = T::load1(grow, c);
-            float d;
-            if (a.p_int == 2) {
-                d = (gg - T::load1(yrow, c) * proj) / n;
-            } else {
-                const float x = T::load1(xrow, c);
-                d = gg / n - sign_of(x) * pow_abs_any(__builtin_fabsf(x), a.p - 1.0f, e_int) * coef;
-            }
-            T::store1(dxrow, c, d);
+        if (p_int == 2) {
+            walk_row<T, 2, true>(grow, yrow, nullptr, dxrow, a.n_cols64, t, [&](float gg, float y, float) { return (gg - y * proj) / n; });
+        } else {
+            const float coef = p_int == 1 ? proj / (n * n) : proj / (pow_abs_any(n, pm1, e_int) * n);
+            walk_row<T, 2, true>(grow, xrow, nullptr, dxrow, a.n_cols64, t, [&](float gg, float x, float) {
+                return gg / n - sign_of(x) * pow_abs_any(__builtin_fabsf(x), pm1, e_int) * coef;
+            });
         }
     }
 }
