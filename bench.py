@@ -40,6 +40,12 @@ WORKLOADS = {
     "rmsnorm_f16_4096x16384_outliers": ("rms", 4096, 16384, "f16"),
     "rmsnorm_f32_4096x16384_outliers": ("rms", 4096, 16384, "f32"),
     "layernorm_f32_200x128_quickstart": ("ln", 200, 128, "f32"),
+    # rows of 64 KiB (the 1024-thread workgroups) and rows that are not a whole number of 16-byte vectors
+    "layernorm_bf16_4096x32768_wide": ("ln", 4096, 32768, "bf16"),
+    "rmsnorm_bf16_4096x32768_wide": ("rms", 4096, 32768, "bf16"),
+    "layernorm_f32_4096x16384_wide": ("ln", 4096, 16384, "f32"),
+    "layernorm_f32_12279x4099_ragged": ("ln", 12279, 4099, "f32"),
+    "rmsnorm_bf16_24564x4098_ragged": ("rms", 24564, 4098, "bf16"),
     # norm with an activation epilogue (thn_norm_act_fwd + thn_norm_act_bwd): same bytes as the plain norm step
     "layernorm_gelu_bf16_16384x4096": ("ln+gelu", 16384, 4096, "bf16"),
     "layernorm_gelu_tanh_bf16_16384x4096": ("ln+gelu_tanh", 16384, 4096, "bf16"),
