@@ -459,19 +459,40 @@ __global__ void __launch_bounds__(BLOCK) normalize_bwd_kernel(const NormalizeBwd
 // ---------------------------------------------------------------------------------------------------
 // Looping kernels: one 256-thread workgroup per row (grid-stride over rows), the row walked as often as the
 // formula needs it (the second walk of a row comes from the L2 or the Infinity Cache).  Any row width, any real
-// p in [1, 6] (accurate powf), any alignment.  This is the path of rows wider than 64 KiB and of non-integer p.
+// p in [1, 6] (pow_split or, for 16-bit storage, the hardware log2 / exp2), any alignment.  This is the path of
+// rows wider than 64 KiB and of non-integer p.
 // A walk moves 16-byte vectors at element-aligned addresses (unaligned access mode), 4 per thread and step, all
 // requested before the first is used; the elements behind the last whole vector go one by one.
 // ---------------------------------------------------------------------------------------------------
 constexpr int kLoopBlock = 256;
 constexpr int kLoopVecs = 4;
 
-// ax^e for ax >= 0; e_int is e when e is an integer in [0, 6], else -1.
+// ax^e for finite ax > 0 and 0 < e <= 6 to about 3 float32 ulp, at a fifth of the instructions of powf:
+// ax = m * 2^k with m in [0.5, 1), so e*log2(ax) = e*k + e*log2(m).  e*k is kept exactly as a float32 pair (product
+// and fma residual), its integer part goes into the result's exponent, and only the fraction and e*log2(m) --
+// both of magnitude <= 6, so the hardware log2 / exp2 lose a few 2^-24 at most -- pass through exp2.
+__device__ __forceinline__ float pow_split(float ax, float e) {
+    const float m = __builtin_amdgcn_frexp_mantf(ax);
+    const float k = static_cast<float>(__builtin_amdgcn_frexp_expf(ax));
+    const float hi = e * k;
+    const float lo = __builtin_fmaf(e, k, -hi);
+    const float whole = __builtin_rintf(hi);
+    const float frac = (hi - whole) + lo + e * __builtin_amdgcn_logf(m);
+    const float r = __builtin_amdgcn_ldexpf(__builtin_amdgcn_exp2f(frac), static_cast<int>(whole));
+    // 0, infinities and NaN take the library's special cases
+    return (ax > 0.0f && ax < __builtin_inff()) ? r : powf(ax, e);
+}
+
+// ax^e for ax >= 0; e_int is e when e is an integer in [0, 6], else -1.  FAST (16-bit storage): a real exponent
+// goes through the hardware log2 / exp2, whose relative error of about e * |log2(ax)| * 2^-24 (3e-6 at the ends
+// of the float32 range) disappears in the rounding to a 16-bit result; float32 / float64 storage takes pow_split.
+template <bool FAST>
 __device__ __forceinline__ float pow_abs_any(float ax, float e, int e_int) {
     if (e_int == 0) return 1.0f;
     if (e_int == 1) return ax;
     if (e_int >= 2 && e_int <= 6) return pow_small(ax, e_int);
-    return powf(ax, e);
+    if constexpr (FAST) return __builtin_amdgcn_exp2f(e * __builtin_amdgcn_logf(ax));
+    else return pow_split(ax, e);
 }
 
 // One walk over a row of n elements: fn(in0[c], in1[c], in2[c]) for every column c (absent streams pass 0); its
@@ -530,7 +551,7 @@ __global__ void __launch_bounds__(kLoopBlock) pnorm_fwd_loop_kernel(const PnormF
             });
         } else {
             walk_row<T, 1, false>(xrow, nullptr, nullptr, nullptr, a.n_cols64, t, [&](float x, float, float) {
-                acc += pow_abs_any(__builtin_fabsf(x), p, p_int > 0 ? p_int : -1);
+                acc += pow_abs_any<T::kBytes == 2>(__builtin_fabsf(x), p, p_int > 0 ? p_int : -1);
                 return 0.0f;
             });
         }
@@ -562,7 +583,7 @@ __global__ void __launch_bounds__(kLoopBlock) pnorm_bwd_loop_kernel(const PnormB
         float den = 1.0f;
         if (p_int != 1) {
             const float n = T::load1(a.norms, row);
-            den = p_int == 2 ? n : pow_abs_any(n, pm1, e_int);
+            den = p_int == 2 ? n : pow_abs_any<false>(n, pm1, e_int);
         }
         if (p_int == 1) {
             walk_row<T, 1, true>(xrow, nullptr, nullptr, dxrow, a.n_cols64, t, [&](float x, float, float) { return g * sign_of(x); });
@@ -570,7 +591,7 @@ __global__ void __launch_bounds__(kLoopBlock) pnorm_bwd_loop_kernel(const PnormB
             walk_row<T, 1, true>(xrow, nullptr, nullptr, dxrow, a.n_cols64, t, [&](float x, float, float) { return (g * x) / den; });
         } else {
             walk_row<T, 1, true>(xrow, nullptr, nullptr, dxrow, a.n_cols64, t, [&](float x, float, float) {
-                return (g * sign_of(x) * pow_abs_any(__builtin_fabsf(x), pm1, e_int)) / den;
+                return (g * sign_of(x) * pow_abs_any<T::kBytes == 2>(__builtin_fabsf(x), pm1, e_int)) / den;
             });
         }
     }
@@ -602,9 +623,9 @@ __global__ void __launch_bounds__(kLoopBlock) normalize_bwd_loop_kernel(const No
         if (p_int == 2) {
             walk_row<T, 2, true>(grow, yrow, nullptr, dxrow, a.n_cols64, t, [&](float gg, float y, float) { return (gg - y * proj) / n; });
         } else {
-            const float coef = p_int == 1 ? proj / (n * n) : proj / (pow_abs_any(n, pm1, e_int) * n);
+            const float coef = p_int == 1 ? proj / (n * n) : proj / (pow_abs_any<false>(n, pm1, e_int) * n);
             walk_row<T, 2, true>(grow, xrow, nullptr, dxrow, a.n_cols64, t, [&](float gg, float x, float) {
-                return gg / n - sign_of(x) * pow_abs_any(__builtin_fabsf(x), pm1, e_int) * coef;
+                return gg / n - sign_of(x) * pow_abs_any<T::kBytes == 2>(__builtin_fabsf(x), pm1, e_int) * coef;
             });
         }
     }
