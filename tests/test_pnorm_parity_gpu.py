@@ -130,6 +130,23 @@ def test_real_p(p, dtype):
     compare_normalize(x, gy, p, 1e-6, f"normalize p={p}")
 
 
+@pytest.mark.parametrize("dtype,decades", [(torch.float32, 6.0), (torch.float64, 6.0), (torch.bfloat16, 6.0),
+                                           (torch.float16, 1.5)])
+@pytest.mark.parametrize("p", [1.5, 2.5, 3.7])
+def test_real_p_over_many_magnitudes(p, dtype, decades):
+    """|x|^p and |x|^(p-1) with |x| spread over many powers of ten: every binary exponent passes through the
+    exponent-splitting power, and the element-wise relative bound on dx checks each of them."""
+    announce(f"real p={p} {dtype} magnitudes")
+    g = torch.Generator().manual_seed(41)
+    shape = (3, 50, 700)
+    mag = 10.0 ** ((torch.rand(shape, generator=g) * 2 - 1) * decades)
+    x = (torch.randn(shape, generator=g) * mag).to(dtype)
+    gn = torch.rand(shape[:-1], generator=g).to(dtype)
+    gy = torch.randn(shape, generator=g).to(dtype)
+    compare_norm(x, gn, p, 1e-6, f"norm p={p} magnitudes")
+    compare_normalize(x, gy, p, 1e-6, f"normalize p={p} magnitudes")
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16, torch.float64])
 @pytest.mark.parametrize("k", [1, 2, 7, 33, 100, 257, 1000, 4099, 6001])
 def test_ragged_row_widths(k, dtype):

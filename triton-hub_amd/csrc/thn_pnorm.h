@@ -459,7 +459,7 @@ __global__ void __launch_bounds__(BLOCK) normalize_bwd_kernel(const NormalizeBwd
 // ---------------------------------------------------------------------------------------------------
 // Looping kernels: one 256-thread workgroup per row (grid-stride over rows), the row walked as often as the
 // formula needs it (the second walk of a row comes from the L2 or the Infinity Cache).  Any row width, any real
-// p in [1, 6] (pow_split or, for 16-bit storage, the hardware log2 / exp2), any alignment.  This is the path of
+// p in [1, 6] (powf or, for 16-bit storage, the hardware log2 / exp2), any alignment.  This is the path of
 // rows wider than 64 KiB and of non-integer p.
 // A walk moves 16-byte vectors at element-aligned addresses (unaligned access mode), 4 per thread and step, all
 // requested before the first is used; the elements behind the last whole vector go one by one.
@@ -467,32 +467,18 @@ __global__ void __launch_bounds__(BLOCK) normalize_bwd_kernel(const NormalizeBwd
 constexpr int kLoopBlock = 256;
 constexpr int kLoopVecs = 4;
 
-// ax^e for finite ax > 0 and 0 < e <= 6 to about 3 float32 ulp, at a fifth of the instructions of powf:
-// ax = m * 2^k with m in [0.5, 1), so e*log2(ax) = e*k + e*log2(m).  e*k is kept exactly as a float32 pair (product
-// and fma residual), its integer part goes into the result's exponent, and only the fraction and e*log2(m) --
-// both of magnitude <= 6, so the hardware log2 / exp2 lose a few 2^-24 at most -- pass through exp2.
-__device__ __forceinline__ float pow_split(float ax, float e) {
-    const float m = __builtin_amdgcn_frexp_mantf(ax);
-    const float k = static_cast<float>(__builtin_amdgcn_frexp_expf(ax));
-    const float hi = e * k;
-    const float lo = __builtin_fmaf(e, k, -hi);
-    const float whole = __builtin_rintf(hi);
-    const float frac = (hi - whole) + lo + e * __builtin_amdgcn_logf(m);
-    const float r = __builtin_amdgcn_ldexpf(__builtin_amdgcn_exp2f(frac), static_cast<int>(whole));
-    // 0, infinities and NaN take the library's special cases
-    return (ax > 0.0f && ax < __builtin_inff()) ? r : powf(ax, e);
-}
-
 // ax^e for ax >= 0; e_int is e when e is an integer in [0, 6], else -1.  FAST (16-bit storage): a real exponent
 // goes through the hardware log2 / exp2, whose relative error of about e * |log2(ax)| * 2^-24 (3e-6 at the ends
-// of the float32 range) disappears in the rounding to a 16-bit result; float32 / float64 storage takes pow_split.
+// of the float32 range) disappears in the rounding to a 16-bit result; float32 / float64 storage keeps the accurate powf (an
+// exponent-splitting exp2(e*log2) on the hardware functions reached 2-4 ulp, too close to the 4 ulp the results
+// are held to).
 template <bool FAST>
 __device__ __forceinline__ float pow_abs_any(float ax, float e, int e_int) {
     if (e_int == 0) return 1.0f;
     if (e_int == 1) return ax;
     if (e_int >= 2 && e_int <= 6) return pow_small(ax, e_int);
     if constexpr (FAST) return __builtin_amdgcn_exp2f(e * __builtin_amdgcn_logf(ax));
-    else return pow_split(ax, e);
+    else return powf(ax, e);
 }
 
 // One walk over a row of n elements: fn(in0[c], in1[c], in2[c]) for every column c (absent streams pass 0); its
@@ -559,7 +545,14 @@ __global__ void __launch_bounds__(kLoopBlock) pnorm_fwd_loop_kernel(const PnormF
         row_allreduce<kLoopBlock, 1, 1>(s, red, phase, 0, t);
         float n = s[0];
         if (p_int == 2) n = sqrtf(n);
-        else if (p_int != 1) n = powf(n, 1.0f / p);
+        else if (p_int != 1) {
+            // 1/p is rounded to float32, and that rounding is multiplied by ln(n) in the power (8 ulp at n = 2e10):
+            // one Newton step on r^p = n brings the root back to about an ulp (once per row)
+            const float r = powf(n, 1.0f / p);
+            const float rp1 = powf(r, p - 1.0f);
+            const float better = r - (rp1 * r - n) / (p * rp1);
+            n = (r > 0.0f && r < 3.0e38f && rp1 > 0.0f && rp1 < 3.0e38f) ? better : r;
+        }
         n = fmaxf(n, a.eps);
         if (t == 0) T::store1(a.norms, row, n);
         if constexpr (NORMALIZE) {
