@@ -136,8 +136,9 @@ int thn_norm_bwd_reduce_partials(const void* workspace, int32_t num_partials,
  *   THN_SOFTMAX: dx = y*dy - y*sum(y*dy);  THN_SOFTMIN: the negative of that;  THN_LOGSOFTMAX: dx = dy - exp(y)*sum(dy).
  * All tensors share one storage code.  Arithmetic is float32, except softmax / softmin on THN_F64 storage,
  * which run in float64: the reference's softmax kernels compute in the type they load (softmax.py:18-23),
- * its log-softmax kernels widen to float32 (logsoftmax.py:19, :61-62).  Rows wider than 64 KiB are refused with
- * THN_E_FEATURE_DIM (the reference would split such a row into independently normalised chunks).
+ * its log-softmax kernels widen to float32 (logsoftmax.py:19, :61-62).  There is no row-width limit: a row wider
+ * than 64 KiB is one softmax of the whole row, computed by kernels that walk the row twice (the reference splits
+ * such a row into 64 KiB chunks and normalises each chunk by itself, softmax.py:34-40).  N must fit in 31 bits.
  */
 enum thn_softmax_kind { THN_SOFTMAX = 0, THN_SOFTMIN = 1, THN_LOGSOFTMAX = 2 };
 

@@ -77,9 +77,8 @@ def test_softmax_argument_checks_answer_without_a_gpu():
         assert call(4, 128, 0, 5) == _native.E_DTYPE
         assert call(4, 128, 3, _native.F32) == _native.E_SHAPE           # unknown kind
         assert call(4, 0, 0, _native.F32) == _native.E_SHAPE and call(-2, 8, 0, _native.F32) == _native.E_SHAPE
-        assert call(4, 16385, 0, _native.F32) == _native.E_FEATURE_DIM
-        assert call(4, 32769, 2, _native.F16) == _native.E_FEATURE_DIM
-        assert call(4, 8193, 1, _native.F64) == _native.E_FEATURE_DIM
+        assert call(4, 16385, 0, _native.F32) == _native.E_NULL            # no row-width limit: the next check answers
+        assert call(4, 2 ** 31, 0, _native.F32) == _native.E_SHAPE         # the row width must fit in 31 bits
         assert call(0, 128, 0, _native.BF16) == _native.OK
         assert call(4, 128, 0, _native.BF16) == _native.E_NULL
     assert (_native.SOFTMAX, _native.SOFTMIN, _native.LOGSOFTMAX) == (0, 1, 2)   # enum thn_softmax_kind
@@ -227,8 +226,6 @@ def test_package_surface():
         assert issubclass(fn, torch.autograd.Function)
     assert Activations.Softmax().softmax_fn is not None and Activations.Softmin().softmin_fn is not None
     assert Activations.LogSoftmax().logsoftmax_fn is not None
-    with pytest.raises(RuntimeError, match="doesn't support feature dim >= 64KB"):
-        Activations._launch._check_row(16385, 4)
 
 
 @pytest.mark.parametrize("affine,bias", [(True, True), (True, False), (False, True), (False, False)])

@@ -7,7 +7,7 @@ with the same assertion messages -- and then call the C ABI of libthnorm.so on t
 import torch
 
 from .. import _native
-from ..Normalization._launch import FEATURE_DIM_MESSAGE, _current_device, _stream_handle
+from ..Normalization._launch import _current_device, _stream_handle
 
 
 def _rows(t: torch.Tensor) -> torch.Tensor:
@@ -45,13 +45,6 @@ def _call(device, fn_name, *args):
         _native.check(status)
 
 
-def _check_row(n: int, element_size: int) -> None:
-    # The reference launches a second program per row beyond 64 KiB, each normalising its own chunk
-    # (softmax.py:34-36): rows that wide are refused here instead of being computed chunk-wise.
-    if n * element_size > 65536:
-        raise RuntimeError(FEATURE_DIM_MESSAGE)
-
-
 def softmax_fwd(x: torch.Tensor, kind: int) -> torch.Tensor:
     if not x.is_cuda:
         _native.require_gpu(x)
@@ -59,7 +52,6 @@ def softmax_fwd(x: torch.Tensor, kind: int) -> torch.Tensor:
     out = torch.empty((m, n), dtype=x.dtype, device=x.device) if reshaped else torch.empty_like(x)
     assert out.numel() == x2.numel(), 'expect output shape to be the same as input shape'
     assert out.stride(-1) == 1, 'expect output to be row-major'
-    _check_row(n, x.element_size())
     if m > 0:
         _call(x.device, 'thn_softmax_fwd', x2.data_ptr(), x_stride, out.data_ptr(), n, m, n, kind,
               _native.dtype_code(x.dtype))
@@ -77,7 +69,6 @@ def softmax_bwd(y: torch.Tensor, dout: torch.Tensor, kind: int) -> torch.Tensor:
         d2 = d2.to(y2.dtype)
     dx = torch.empty((m, n), dtype=y.dtype, device=y.device) if reshaped else torch.empty_like(y)
     assert dx.stride(-1) == 1, 'expect derivative to be row-major'
-    _check_row(n, y.element_size())
     if m > 0:
         _call(y.device, 'thn_softmax_bwd', y2.data_ptr(), y_stride, d2.data_ptr(), d_stride, dx.data_ptr(), n, m, n, kind,
               _native.dtype_code(y.dtype))

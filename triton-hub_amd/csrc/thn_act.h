@@ -44,24 +44,6 @@ struct ActArgs {
     float p0, p1;         // negative_slope | beta, threshold | threshold, value
 };
 
-template <typename T, typename C>
-__device__ __forceinline__ u32x4 pack_as(const C (&f)[T::VEC]) {
-    if constexpr (std::is_same<C, double>::value) return pack_f64(f);
-    else return T::pack(f);
-}
-
-template <typename T, typename C>
-__device__ __forceinline__ C load_elem(const void* p, int64_t i) {
-    if constexpr (std::is_same<C, double>::value) return reinterpret_cast<const double*>(p)[i];
-    else return T::load1(p, i);
-}
-
-template <typename T, typename C>
-__device__ __forceinline__ void store_elem(void* p, int64_t i, C v) {
-    if constexpr (std::is_same<C, double>::value) reinterpret_cast<double*>(p)[i] = v;
-    else T::store1(p, i, v);
-}
-
 // ---------------------------------------------------------------------------------------------------
 // Contiguous tensors: one flat stream of 16-byte vectors.  A persistent grid; every thread owns U vectors per
 // grid step (vector v0 + u*BLOCK, so a wave touches contiguous 1 KiB segments), requests the next step's

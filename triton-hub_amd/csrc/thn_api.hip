@@ -128,6 +128,28 @@ int launch_softmax_bwd(int dtype, bool is_log, bool aligned, Shape s, const Soft
 }
 
 // `variant` of the fused families: bit 0 = LayerNorm, bits 1.. = the activation code.
+// Workgroup size and workgroups per compute unit of the looping softmax kernels (rows wider than 64 KiB); the
+// launch override of the family (block_threads, blocks_per_cu) replaces them.
+void softmax_loop_launch(int which, int* block, int* bpc);
+
+int launch_softmax_fwd_loop(int dtype, bool is_log, int block, const SoftmaxFwdArgs& a, int grid, hipStream_t st) {
+    switch (dtype) {
+        case THN_F32: return thn::launch_softmax_fwd_loop_f32(is_log, block, a, grid, st);
+        case THN_F16: return thn::launch_softmax_fwd_loop_f16(is_log, block, a, grid, st);
+        case THN_BF16: return thn::launch_softmax_fwd_loop_bf16(is_log, block, a, grid, st);
+        default: return thn::launch_softmax_fwd_loop_f64(is_log, block, a, grid, st);
+    }
+}
+
+int launch_softmax_bwd_loop(int dtype, bool is_log, int block, const SoftmaxBwdArgs& a, int grid, hipStream_t st) {
+    switch (dtype) {
+        case THN_F32: return thn::launch_softmax_bwd_loop_f32(is_log, block, a, grid, st);
+        case THN_F16: return thn::launch_softmax_bwd_loop_f16(is_log, block, a, grid, st);
+        case THN_BF16: return thn::launch_softmax_bwd_loop_bf16(is_log, block, a, grid, st);
+        default: return thn::launch_softmax_bwd_loop_f64(is_log, block, a, grid, st);
+    }
+}
+
 int launch_fused_fwd(int dtype, int variant, bool aligned, Shape s, const FwdArgs& a, int grid, hipStream_t st, int* occ) {
     const bool ln = (variant & 1) != 0;
     const int act = variant >> 1;
@@ -309,6 +331,14 @@ int default_blocks_per_cu(int which, int flavour, int block) {
     // as many workgroups per compute unit as their registers allow, up to four.
     if ((which == kFusedFwd || which == kFusedBwd) && ((flavour >> 1) == thn::kGelu || (flavour >> 1) == thn::kGeluTanh)) return 4;
     return kDefaultBlocksPerCu;
+}
+
+void softmax_loop_launch(int which, int* block, int* bpc) {
+    *block = 1024;      // sweep over {256, 512, 1024} x {1, 2, 4, 8}: 1024 x 2 best or within 2 % of the best at every width
+    *bpc = 2;
+    const int ob = g_override[which].block.load(), oc = g_override[which].bpc.load();
+    if (ob == 256 || ob == 512 || ob == 1024) *block = ob;
+    if (oc > 0) *bpc = oc < kMaxBlocksPerCu ? oc : kMaxBlocksPerCu;
 }
 
 // Rows of at most 256 bytes: a thread holds one or two vectors, so one workgroup per compute unit keeps too few
@@ -863,11 +893,29 @@ int thn_softmax_fwd(const void* x, int64_t x_row_stride, void* y, int64_t y_row_
                     int kind, int dtype, void* stream) {
     const int bytes = elem_bytes(dtype);
     if (bytes == 0) return THN_E_DTYPE;
-    if (M < 0 || N <= 0 || kind < THN_SOFTMAX || kind > THN_LOGSOFTMAX) return THN_E_SHAPE;
-    if (N * bytes > kMaxRowBytes) return THN_E_FEATURE_DIM;
+    if (M < 0 || N <= 0 || N > INT32_MAX || kind < THN_SOFTMAX || kind > THN_LOGSOFTMAX) return THN_E_SHAPE;
     if (M == 0) return THN_OK;
     if (x == nullptr || y == nullptr) return THN_E_NULL;
     if (x_row_stride < N || y_row_stride < N) return THN_E_SHAPE;
+    if (N * bytes > kMaxRowBytes) {                 // rows the row engine cannot hold in registers
+        const int cus = current_cu_count();
+        if (cus <= 0) return THN_E_DEVICE;
+        SoftmaxFwdArgs a{};
+        a.x = static_cast<const char*>(x);
+        a.y = static_cast<char*>(y);
+        a.x_stride_bytes = x_row_stride * bytes;
+        a.y_stride_bytes = y_row_stride * bytes;
+        a.M = M;
+        a.n_cols = static_cast<int>(N);
+        a.sign = kind == THN_SOFTMIN ? -1.0f : 1.0f;
+        int block, bpc;
+        softmax_loop_launch(kSoftmaxFwd, &block, &bpc);
+        const int64_t cap = static_cast<int64_t>(cus) * bpc;
+        const int grid = static_cast<int>(M < cap ? M : cap);
+        const int lrc = launch_softmax_fwd_loop(dtype, kind == THN_LOGSOFTMAX, block, a, grid, static_cast<hipStream_t>(stream));
+        if (lrc > 0) return THN_E_SHAPE;
+        return lrc == 0 ? THN_OK : THN_E_LAUNCH;
+    }
     const int vec_elems = 16 / bytes;
     const bool aligned = (N % vec_elems) == 0 && aligned16(x) && aligned16(y) && (x_row_stride * bytes) % 16 == 0 &&
                          (y_row_stride * bytes) % 16 == 0;
@@ -893,11 +941,31 @@ int thn_softmax_bwd(const void* y, int64_t y_row_stride, const void* dy, int64_t
                     int64_t dx_row_stride, int64_t M, int64_t N, int kind, int dtype, void* stream) {
     const int bytes = elem_bytes(dtype);
     if (bytes == 0) return THN_E_DTYPE;
-    if (M < 0 || N <= 0 || kind < THN_SOFTMAX || kind > THN_LOGSOFTMAX) return THN_E_SHAPE;
-    if (N * bytes > kMaxRowBytes) return THN_E_FEATURE_DIM;
+    if (M < 0 || N <= 0 || N > INT32_MAX || kind < THN_SOFTMAX || kind > THN_LOGSOFTMAX) return THN_E_SHAPE;
     if (M == 0) return THN_OK;
     if (y == nullptr || dy == nullptr || dx == nullptr) return THN_E_NULL;
     if (y_row_stride < N || dy_row_stride < N || dx_row_stride < N) return THN_E_SHAPE;
+    if (N * bytes > kMaxRowBytes) {
+        const int cus = current_cu_count();
+        if (cus <= 0) return THN_E_DEVICE;
+        SoftmaxBwdArgs a{};
+        a.y = static_cast<const char*>(y);
+        a.dy = static_cast<const char*>(dy);
+        a.dx = static_cast<char*>(dx);
+        a.y_stride_bytes = y_row_stride * bytes;
+        a.dy_stride_bytes = dy_row_stride * bytes;
+        a.dx_stride_bytes = dx_row_stride * bytes;
+        a.M = M;
+        a.n_cols = static_cast<int>(N);
+        a.sign = kind == THN_SOFTMIN ? -1.0f : 1.0f;
+        int block, bpc;
+        softmax_loop_launch(kSoftmaxBwd, &block, &bpc);
+        const int64_t cap = static_cast<int64_t>(cus) * bpc;
+        const int grid = static_cast<int>(M < cap ? M : cap);
+        const int lrc = launch_softmax_bwd_loop(dtype, kind == THN_LOGSOFTMAX, block, a, grid, static_cast<hipStream_t>(stream));
+        if (lrc > 0) return THN_E_SHAPE;
+        return lrc == 0 ? THN_OK : THN_E_LAUNCH;
+    }
     const int vec_elems = 16 / bytes;
     const bool aligned = (N % vec_elems) == 0 && aligned16(y) && aligned16(dy) && aligned16(dx) &&
                          (y_row_stride * bytes) % 16 == 0 && (dy_row_stride * bytes) % 16 == 0 &&

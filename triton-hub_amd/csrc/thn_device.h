@@ -6,6 +6,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <type_traits>
+
 namespace thn {
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
@@ -318,6 +320,8 @@ typedef u32x4 u32x4_unaligned __attribute__((aligned(2)));
 __device__ __forceinline__ u32x4 ld128u(const void* p) {
     return __builtin_nontemporal_load(reinterpret_cast<const u32x4_unaligned*>(p));
 }
+// The same load without the non-temporal hint: for data that is read again shortly (it may stay in the caches).
+__device__ __forceinline__ u32x4 ld128u_keep(const void* p) { return *reinterpret_cast<const u32x4_unaligned*>(p); }
 __device__ __forceinline__ void st128u(void* p, u32x4 v) {
     __builtin_nontemporal_store(v, reinterpret_cast<u32x4_unaligned*>(p));
 }
@@ -401,12 +405,32 @@ __device__ __forceinline__ void unpack_as(u32x4 v, double (&f)[T::VEC]) {
     f[1] = __builtin_bit_cast(double, (static_cast<uint64_t>(d) << 32) | c);
 }
 
+
+
 __device__ __forceinline__ u32x4 pack_f64(const double (&f)[2]) {
     const uint64_t lo = __builtin_bit_cast(uint64_t, f[0]), hi = __builtin_bit_cast(uint64_t, f[1]);
     u32x4 v;
     v[0] = static_cast<uint32_t>(lo); v[1] = static_cast<uint32_t>(lo >> 32);
     v[2] = static_cast<uint32_t>(hi); v[3] = static_cast<uint32_t>(hi >> 32);
     return v;
+}
+
+template <typename T, typename C>
+__device__ __forceinline__ u32x4 pack_as(const C (&f)[T::VEC]) {
+    if constexpr (std::is_same<C, double>::value) return pack_f64(f);
+    else return T::pack(f);
+}
+
+template <typename T, typename C>
+__device__ __forceinline__ C load_elem(const void* p, int64_t i) {
+    if constexpr (std::is_same<C, double>::value) return reinterpret_cast<const double*>(p)[i];
+    else return T::load1(p, i);
+}
+
+template <typename T, typename C>
+__device__ __forceinline__ void store_elem(void* p, int64_t i, C v) {
+    if constexpr (std::is_same<C, double>::value) reinterpret_cast<double*>(p)[i] = v;
+    else T::store1(p, i, v);
 }
 
 __device__ __forceinline__ float exp_c(float z) { return __expf(z); }

@@ -19,6 +19,7 @@
 #include <type_traits>
 
 #include "thn_kernels.h"
+#include "thn_walk.h"
 
 namespace thn {
 
@@ -461,11 +462,9 @@ __global__ void __launch_bounds__(BLOCK) normalize_bwd_kernel(const NormalizeBwd
 // formula needs it (the second walk of a row comes from the L2 or the Infinity Cache).  Any row width, any real
 // p in [1, 6] (powf or, for 16-bit storage, the hardware log2 / exp2), any alignment.  This is the path of
 // rows wider than 64 KiB and of non-integer p.
-// A walk moves 16-byte vectors at element-aligned addresses (unaligned access mode), 4 per thread and step, all
-// requested before the first is used; the elements behind the last whole vector go one by one.
+// The walks are walk_row of thn_walk.h.
 // ---------------------------------------------------------------------------------------------------
 constexpr int kLoopBlock = 256;
-constexpr int kLoopVecs = 4;
 
 // ax^e for ax >= 0; e_int is e when e is an integer in [0, 6], else -1.  FAST (16-bit storage): a real exponent
 // goes through the hardware log2 / exp2, whose relative error of about e * |log2(ax)| * 2^-24 (3e-6 at the ends
@@ -481,44 +480,6 @@ __device__ __forceinline__ float pow_abs_any(float ax, float e, int e_int) {
     else return powf(ax, e);
 }
 
-// One walk over a row of n elements: fn(in0[c], in1[c], in2[c]) for every column c (absent streams pass 0); its
-// value is stored to out[c] when STORE.  Thread t takes vectors t, t + 256, ... .
-template <typename T, int NIN, bool STORE, typename Fn>
-__device__ __forceinline__ void walk_row(const char* in0, const char* in1, const char* in2, char* out, int64_t n,
-                                         int t, Fn&& fn) {
-    constexpr int VEC = T::VEC;
-    constexpr int U = kLoopVecs;
-    const char* in[3] = {in0, in1, in2};
-    const int64_t whole = n / VEC;
-    for (int64_t v0 = t; v0 < whole; v0 += kLoopBlock * U) {
-        u32x4 raw[U][NIN];
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-            const int64_t v = v0 + u * kLoopBlock;
-            if (v < whole) {
-#pragma unroll
-                for (int i = 0; i < NIN; ++i) raw[u][i] = ld128u(in[i] + v * 16);
-            }
-        }
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-            const int64_t v = v0 + u * kLoopBlock;
-            if (v < whole) {
-                float f[3][VEC], o[VEC];
-#pragma unroll
-                for (int i = 0; i < NIN; ++i) T::unpack(raw[u][i], f[i]);
-#pragma unroll
-                for (int e = 0; e < VEC; ++e) o[e] = fn(f[0][e], NIN > 1 ? f[1][e] : 0.0f, NIN > 2 ? f[2][e] : 0.0f);
-                if constexpr (STORE) st128u(out + v * 16, T::pack(o));
-            }
-        }
-    }
-    for (int64_t c = whole * VEC + t; c < n; c += kLoopBlock) {
-        const float o = fn(T::load1(in0, c), NIN > 1 ? T::load1(in1, c) : 0.0f, NIN > 2 ? T::load1(in2, c) : 0.0f);
-        if constexpr (STORE) T::store1(out, c, o);
-    }
-}
-
 template <typename T, bool NORMALIZE>
 __global__ void __launch_bounds__(kLoopBlock) pnorm_fwd_loop_kernel(const PnormFwdArgs a) {
     __shared__ float red[RedSmem<kLoopBlock, 1, 1>::kFloats];
@@ -531,12 +492,12 @@ __global__ void __launch_bounds__(kLoopBlock) pnorm_fwd_loop_kernel(const PnormF
         float s[1] = {0.0f};
         float acc = 0.0f;
         if (p_int == 2) {
-            walk_row<T, 1, false>(xrow, nullptr, nullptr, nullptr, a.n_cols64, t, [&](float x, float, float) {
+            walk_row<T, float, kLoopBlock, 1, false, NORMALIZE>(xrow, nullptr, nullptr, nullptr, a.n_cols64, t, [&](float x, float, float) {
                 acc = __builtin_fmaf(x, x, acc);
                 return 0.0f;
             });
         } else {
-            walk_row<T, 1, false>(xrow, nullptr, nullptr, nullptr, a.n_cols64, t, [&](float x, float, float) {
+            walk_row<T, float, kLoopBlock, 1, false, NORMALIZE>(xrow, nullptr, nullptr, nullptr, a.n_cols64, t, [&](float x, float, float) {
                 acc += pow_abs_any<T::kBytes == 2>(__builtin_fabsf(x), p, p_int > 0 ? p_int : -1);
                 return 0.0f;
             });
@@ -558,7 +519,7 @@ __global__ void __launch_bounds__(kLoopBlock) pnorm_fwd_loop_kernel(const PnormF
         if constexpr (NORMALIZE) {
             const float nr = round_to_storage<T>(n);
             char* yrow = a.y + row_offset(a.ymap, a.walk, row);
-            walk_row<T, 1, true>(xrow, nullptr, nullptr, yrow, a.n_cols64, t, [&](float x, float, float) { return x / nr; });
+            walk_row<T, float, kLoopBlock, 1, true>(xrow, nullptr, nullptr, yrow, a.n_cols64, t, [&](float x, float, float) { return x / nr; });
         }
     }
 }
@@ -579,11 +540,11 @@ __global__ void __launch_bounds__(kLoopBlock) pnorm_bwd_loop_kernel(const PnormB
             den = p_int == 2 ? n : pow_abs_any<false>(n, pm1, e_int);
         }
         if (p_int == 1) {
-            walk_row<T, 1, true>(xrow, nullptr, nullptr, dxrow, a.n_cols64, t, [&](float x, float, float) { return g * sign_of(x); });
+            walk_row<T, float, kLoopBlock, 1, true>(xrow, nullptr, nullptr, dxrow, a.n_cols64, t, [&](float x, float, float) { return g * sign_of(x); });
         } else if (p_int == 2) {
-            walk_row<T, 1, true>(xrow, nullptr, nullptr, dxrow, a.n_cols64, t, [&](float x, float, float) { return (g * x) / den; });
+            walk_row<T, float, kLoopBlock, 1, true>(xrow, nullptr, nullptr, dxrow, a.n_cols64, t, [&](float x, float, float) { return (g * x) / den; });
         } else {
-            walk_row<T, 1, true>(xrow, nullptr, nullptr, dxrow, a.n_cols64, t, [&](float x, float, float) {
+            walk_row<T, float, kLoopBlock, 1, true>(xrow, nullptr, nullptr, dxrow, a.n_cols64, t, [&](float x, float, float) {
                 return (g * sign_of(x) * pow_abs_any<T::kBytes == 2>(__builtin_fabsf(x), pm1, e_int)) / den;
             });
         }
@@ -606,7 +567,7 @@ __global__ void __launch_bounds__(kLoopBlock) normalize_bwd_loop_kernel(const No
         const float n = T::load1(a.norms, row);
         float s[1] = {0.0f};
         float acc = 0.0f;
-        walk_row<T, 2, false>(p_int == 1 ? xrow : yrow, grow, nullptr, nullptr, a.n_cols64, t, [&](float other, float gg, float) {
+        walk_row<T, float, kLoopBlock, 2, false, true>(p_int == 1 ? xrow : yrow, grow, nullptr, nullptr, a.n_cols64, t, [&](float other, float gg, float) {
             acc = __builtin_fmaf(other, gg, acc);
             return 0.0f;
         });
@@ -614,10 +575,10 @@ __global__ void __launch_bounds__(kLoopBlock) normalize_bwd_loop_kernel(const No
         row_allreduce<kLoopBlock, 1, 1>(s, red, phase, 0, t);
         const float proj = s[0];
         if (p_int == 2) {
-            walk_row<T, 2, true>(grow, yrow, nullptr, dxrow, a.n_cols64, t, [&](float gg, float y, float) { return (gg - y * proj) / n; });
+            walk_row<T, float, kLoopBlock, 2, true>(grow, yrow, nullptr, dxrow, a.n_cols64, t, [&](float gg, float y, float) { return (gg - y * proj) / n; });
         } else {
             const float coef = p_int == 1 ? proj / (n * n) : proj / (pow_abs_any<false>(n, pm1, e_int) * n);
-            walk_row<T, 2, true>(grow, xrow, nullptr, dxrow, a.n_cols64, t, [&](float gg, float x, float) {
+            walk_row<T, float, kLoopBlock, 2, true>(grow, xrow, nullptr, dxrow, a.n_cols64, t, [&](float gg, float x, float) {
                 return gg / n - sign_of(x) * pow_abs_any<T::kBytes == 2>(__builtin_fabsf(x), pm1, e_int) * coef;
             });
         }

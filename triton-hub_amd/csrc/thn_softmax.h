@@ -6,6 +6,7 @@
 #include <type_traits>
 
 #include "thn_kernels.h"
+#include "thn_walk.h"
 
 namespace thn {
 
@@ -248,6 +249,114 @@ __global__ void __launch_bounds__(BLOCK) softmax_bwd_kernel(const SoftmaxBwdArgs
         for (int k = 0; k < K; ++k) { cy[k] = ny[k]; cg[k] = ng[k]; }
         row_raw = nrow_raw;
         row = nrow;
+    }
+}
+
+// ---------------------------------------------------------------------------------------------------
+// Rows wider than 64 KiB (the reference cuts such a row into 64 KiB chunks and normalises each chunk by itself,
+// softmax.py:34-40 -- which is not a softmax of the row; here the row is one softmax).  One 1024-thread workgroup
+// per row, grid-stride over rows, two walks per row (thn_walk.h); the second comes from the L2 / Infinity Cache.
+//   forward:  walk 1 keeps a running maximum m and sum(exp(x - m)) per thread (the sum is rescaled whenever the
+//             maximum moves: a few times per thread), combined over the workgroup; walk 2 writes y;
+//   backward: walk 1 sum(y*g) (log-softmax: sum(g)); walk 2 writes dx.
+// The row sums are accumulated in float64.
+// ---------------------------------------------------------------------------------------------------
+template <typename T, bool LOG, int kSoftmaxLoopBlock>
+__global__ void __launch_bounds__(kSoftmaxLoopBlock) softmax_fwd_loop_kernel(const SoftmaxFwdArgs a) {
+    using C = typename SoftmaxCompute<T, LOG>::type;
+    __shared__ C red[RedSmem<kSoftmaxLoopBlock, 1, 1>::kFloats];
+    __shared__ double red_sum[RedSmem<kSoftmaxLoopBlock, 1, 1>::kFloats];
+    int phase = 0, phase_sum = 0;
+    const int t = threadIdx.x;
+    const C sign = static_cast<C>(a.sign);
+    const C neg_inf = OpMax::identity<C>();
+    for (int64_t row = blockIdx.x; row < a.M; row += gridDim.x) {
+        const char* xrow = a.x + row * a.x_stride_bytes;
+        char* yrow = a.y + row * a.y_stride_bytes;
+        C m = neg_inf;
+        double acc = 0.0;       // tens of thousands of terms per row: float64 sums keep the row total to an ulp
+        auto one = [&](C x, C, C) {
+            const C v = x * sign;
+            if (v > m) {
+                acc *= static_cast<double>(exp_c(m - v));          // m = -inf: 0
+                m = v;
+            }
+            acc += v > neg_inf ? static_cast<double>(exp_c(v - m)) : 0.0;   // -inf - -inf must not poison the sum
+            return C(0);
+        };
+        walk_row_vec<T, C, kSoftmaxLoopBlock, 1, false, true>(
+            xrow, nullptr, nullptr, nullptr, a.n_cols, t,
+            [&](const C (&f)[3][T::VEC], C (&)[T::VEC]) {
+                C v[T::VEC];
+                C vmax = neg_inf;
+#pragma unroll
+                for (int e = 0; e < T::VEC; ++e) {
+                    v[e] = f[0][e] * sign;
+                    vmax = OpMax::apply(vmax, v[e]);
+                }
+                if (vmax > m) {
+                    acc *= static_cast<double>(exp_c(m - vmax));
+                    m = vmax;
+                }
+                C part = C(0);
+#pragma unroll
+                for (int e = 0; e < T::VEC; ++e) part += v[e] > neg_inf ? exp_c(v[e] - m) : C(0);
+                acc += static_cast<double>(part);
+            },
+            one);
+        C mx[1] = {m};
+        row_allreduce<kSoftmaxLoopBlock, 1, 1, OpMax, C>(mx, red, phase, 0, t);
+        double s[1] = {m > neg_inf ? acc * static_cast<double>(exp_c(m - mx[0])) : 0.0};
+        row_allreduce<kSoftmaxLoopBlock, 1, 1, OpSum, double>(s, red_sum, phase_sum, 0, t);
+        const C row_max = mx[0];
+        C scale;
+        if constexpr (LOG) scale = static_cast<C>(log(s[0]));
+        else scale = static_cast<C>(1.0 / s[0]);
+        walk_row<T, C, kSoftmaxLoopBlock, 1, true>(xrow, nullptr, nullptr, yrow, a.n_cols, t, [&](C x, C, C) {
+            const C z = x * sign - row_max;
+            if constexpr (LOG) return z - scale;
+            else return exp_c(z) * scale;
+        });
+    }
+}
+
+template <typename T, bool LOG, int kSoftmaxLoopBlock>
+__global__ void __launch_bounds__(kSoftmaxLoopBlock) softmax_bwd_loop_kernel(const SoftmaxBwdArgs a) {
+    using C = typename SoftmaxCompute<T, LOG>::type;
+    __shared__ double red_sum[RedSmem<kSoftmaxLoopBlock, 1, 1>::kFloats];
+    int phase_sum = 0;
+    const int t = threadIdx.x;
+    const C sign = static_cast<C>(a.sign);
+    for (int64_t row = blockIdx.x; row < a.M; row += gridDim.x) {
+        const char* yrow = a.y + row * a.y_stride_bytes;
+        const char* grow = a.dy + row * a.dy_stride_bytes;
+        char* dxrow = a.dx + row * a.dx_stride_bytes;
+        double acc = 0.0;
+        walk_row_vec<T, C, kSoftmaxLoopBlock, 2, false, true>(
+            yrow, grow, nullptr, nullptr, a.n_cols, t,
+            [&](const C (&f)[3][T::VEC], C (&)[T::VEC]) {
+                C part = C(0);
+#pragma unroll
+                for (int e = 0; e < T::VEC; ++e) {
+                    if constexpr (LOG) part += f[1][e];
+                    else part = fma(f[0][e], f[1][e], part);
+                }
+                acc += static_cast<double>(part);
+            },
+            [&](C y, C g, C) {
+                if constexpr (LOG) acc += static_cast<double>(g);
+                else acc = fma(static_cast<double>(y), static_cast<double>(g), acc);
+                return C(0);
+            });
+        double s[1] = {acc};
+        row_allreduce<kSoftmaxLoopBlock, 1, 1, OpSum, double>(s, red_sum, phase_sum, 0, t);
+        const C total = static_cast<C>(s[0]);
+        walk_row<T, C, kSoftmaxLoopBlock, 2, true>(yrow, grow, nullptr, dxrow, a.n_cols, t, [&](C y, C g, C) {
+            C d;
+            if constexpr (LOG) d = fma(-exp_c(y), total, g);
+            else d = y * (g - total);
+            return d * sign;
+        });
     }
 }
 

@@ -10,7 +10,9 @@ namespace thn {
     int launch_softmax_fwd_##NAME(bool is_log, bool aligned, Shape s, const SoftmaxFwdArgs& a, int grid,        \
                                   hipStream_t st, int* occupancy);                                              \
     int launch_softmax_bwd_##NAME(bool is_log, bool aligned, Shape s, const SoftmaxBwdArgs& a, int grid,        \
-                                  hipStream_t st, int* occupancy);
+                                  hipStream_t st, int* occupancy);                                              \
+    int launch_softmax_fwd_loop_##NAME(bool is_log, int block, const SoftmaxFwdArgs& a, int grid, hipStream_t st); \
+    int launch_softmax_bwd_loop_##NAME(bool is_log, int block, const SoftmaxBwdArgs& a, int grid, hipStream_t st);
 
 THN_DECLARE_SOFTMAX_LAUNCHERS(f32)
 THN_DECLARE_SOFTMAX_LAUNCHERS(f16)
@@ -26,6 +28,12 @@ THN_DECLARE_SOFTMAX_LAUNCHERS(f64)
 #define THN_SMF_SC(K_, TPR_, BLOCK_) THN_SM_CASE(softmax_fwd_kernel, SoftmaxFwdArgs, false, K_, TPR_, BLOCK_)
 #define THN_SMB_AL(K_, TPR_, BLOCK_) THN_SM_CASE(softmax_bwd_kernel, SoftmaxBwdArgs, true, K_, TPR_, BLOCK_)
 #define THN_SMB_SC(K_, TPR_, BLOCK_) THN_SM_CASE(softmax_bwd_kernel, SoftmaxBwdArgs, false, K_, TPR_, BLOCK_)
+
+#define THN_SM_LOOP_CASE(KERNEL, ARGS_T, TYPE, B)                                                               \
+    if (block == B) {                                                                                           \
+        return is_log ? run_kernel<ARGS_T>(KERNEL<TYPE, true, B>, a, grid, B, st, nullptr)                      \
+                      : run_kernel<ARGS_T>(KERNEL<TYPE, false, B>, a, grid, B, st, nullptr);                    \
+    }
 
 // Both directions use the forward shape list of the norm kernels (no per-column accumulators to hold).
 #define THN_DEFINE_SOFTMAX_LAUNCHERS(NAME, TYPE)                                                                \
@@ -53,6 +61,18 @@ THN_DECLARE_SOFTMAX_LAUNCHERS(f64)
             using T = ElemIo<TYPE>; \
             THN_SMB_SC(4, 8, 256) \
         }                                                                                                       \
+        return 1;                                                                                               \
+    }                                                                                                           \
+    int launch_softmax_fwd_loop_##NAME(bool is_log, int block, const SoftmaxFwdArgs& a, int grid, hipStream_t st) { \
+        THN_SM_LOOP_CASE(softmax_fwd_loop_kernel, SoftmaxFwdArgs, TYPE, 256)                                    \
+        THN_SM_LOOP_CASE(softmax_fwd_loop_kernel, SoftmaxFwdArgs, TYPE, 512)                                    \
+        THN_SM_LOOP_CASE(softmax_fwd_loop_kernel, SoftmaxFwdArgs, TYPE, 1024)                                   \
+        return 1;                                                                                               \
+    }                                                                                                           \
+    int launch_softmax_bwd_loop_##NAME(bool is_log, int block, const SoftmaxBwdArgs& a, int grid, hipStream_t st) { \
+        THN_SM_LOOP_CASE(softmax_bwd_loop_kernel, SoftmaxBwdArgs, TYPE, 256)                                    \
+        THN_SM_LOOP_CASE(softmax_bwd_loop_kernel, SoftmaxBwdArgs, TYPE, 512)                                    \
+        THN_SM_LOOP_CASE(softmax_bwd_loop_kernel, SoftmaxBwdArgs, TYPE, 1024)                                   \
         return 1;                                                                                               \
     }
 
