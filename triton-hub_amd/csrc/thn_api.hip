@@ -316,6 +316,16 @@ Shape heuristic_shape(int which, bool aligned, int n_vecs) {
     }
     if (which == kNormBwd && n_vecs > 8 && n_vecs <= 16) s.tpr = 16;      // 256-byte rows: one vector per thread
     s.k = ceil_div(n_vecs, s.tpr);
+    // The softmax backward prefers 2 vectors per thread, but a row of 3 * 2^k vectors (or a little less) would
+    // leave a quarter to a half of the slots without work: then 3 vectors on half the threads (bf16 N = 1280 /
+    // 2560 / 3072: 5.0 / 5.0 / 5.5 -> 6.0 / 6.4 / 6.3 TB/s; the normalize backward lost 5 % with the same change).
+    if (which == kSoftmaxBwd && s.k == 2 && s.tpr >= 128) {
+        const int half = s.tpr / 2;
+        if (3 * half >= n_vecs) {          // at most three quarters of the 2-vector slots would have work
+            s.tpr = half;
+            s.k = 3;
+        }
+    }
     if (s.k == 3 && s.tpr < 64) s.k = 4;     // K = 3 is only compiled for TPR >= 64
     if (which != kNormBwd && which != kFusedBwd) s.block = s.tpr > 256 ? s.tpr : 256;
     else s.block = s.tpr >= 128 ? (s.tpr > 512 ? s.tpr : 512) : 256;
@@ -386,6 +396,11 @@ int plan_launch(int which, int flavour, bool aligned, int64_t M, int64_t N, int 
         cap = default_blocks_per_cu(which, flavour, s.block);
         const int narrow = narrow_row_blocks_per_cu(which, n_vecs, bytes == 2 && N % vec_elems != 0);
         if (narrow > cap) cap = narrow;
+        // One input stream and fewer than 1024 vectors per workgroup step (3 vectors per thread in 256-thread
+        // workgroups: row widths of 5 * 2^k elements and their neighbours): a second workgroup brings the bytes in
+        // flight back to where HBM throughput peaks (bf16 N = 5120 forward 5.5 -> 6.0 TB/s, N = 1280 5.6 -> 6.1).
+        const bool one_stream = which == kNormFwd || which == kSoftmaxFwd || which == kPnormFwd || which == kFusedFwd;
+        if (one_stream && aligned && s.block * s.k < 1024 && n_vecs > 16 && cap < 2) cap = 2;
     }
     if (cap < bpc) bpc = cap;
     const int rows_per_block = s.block / s.tpr;
