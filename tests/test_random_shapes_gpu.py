@@ -1,0 +1,77 @@
+"""GPU parity on seeded random problems: random family, storage type, row count and row width (log-uniform up to the
+widest row each family accepts), sometimes through a column-offset view.  The per-family tests pin chosen widths;
+this one walks the launch heuristics (vectors per thread, threads per row, workgroups per compute unit, the forms
+for wide, narrow, ragged and misaligned rows) at widths nobody chose.  Same oracles and tolerances as the per-family
+tests, whose comparison helpers it reuses."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import parity_util
+import test_act_parity_gpu as act_t
+import test_fused_parity_gpu as fused_t
+import test_pnorm_parity_gpu as pnorm_t
+import test_softmax_parity_gpu as softmax_t
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [torch.float32, torch.bfloat16, torch.float16, torch.float64]
+FAMILIES = ["ln", "rms", "softmax", "softmin", "logsoftmax", "norm", "normalize", "act", "ln+act", "rms+act"]
+MAX_ELEMS = 3_000_000
+
+
+def log_uniform(rng, lo, hi):
+    return int(round(math.exp(rng.uniform(math.log(lo), math.log(hi)))))
+
+
+def draw(seed):
+    rng = np.random.default_rng(1000 + seed)
+    family = FAMILIES[seed % len(FAMILIES)]
+    dtype = DTYPES[int(rng.integers(len(DTYPES)))]
+    size = torch.empty(0, dtype=dtype).element_size()
+    row_cap = 65536 // size if family in ("ln", "rms", "ln+act", "rms+act") else 200_000
+    n = log_uniform(rng, 1, row_cap)
+    m = max(1, min(log_uniform(rng, 1, 5000), MAX_ELEMS // n))
+    offset = int(rng.integers(0, 4)) if rng.random() < 0.3 else 0       # a view that starts `offset` columns in
+    return family, dtype, m, n, offset, rng
+
+
+@pytest.mark.parametrize("seed", range(200))
+def test_random_problem(seed):
+    family, dtype, m, n, offset, rng = draw(seed)
+    print(f"\n[case] random seed={seed} {family} {dtype} M={m} N={n} offset={offset}", flush=True)
+    g = torch.Generator().manual_seed(seed)
+    pad = offset + int(rng.integers(0, 3)) if offset else 0
+    xb = (torch.randn(m, n + pad, generator=g) * 2).to(dtype)
+    gb = torch.randn(m, n + pad, generator=g).to(dtype)
+    x, dy = xb[:, offset:offset + n].contiguous(), gb[:, offset:offset + n].contiguous()
+    x_gpu = xb.cuda()[:, offset:offset + n] if pad else None
+    dy_gpu = gb.cuda()[:, offset:offset + n] if pad else None
+    what = f"random {seed} {family} {m}x{n}"
+    # Rows of a few elements are often nearly constant; with a tiny eps rstd then reaches hundreds and multiplies the
+    # float32 rounding of (x - mean) beyond any fixed bound, for every implementation that saves a float32 mean.
+    eps = 1e-5 if n >= 16 else 1e-2
+    if family in ("ln", "rms"):
+        w = (1 + 0.1 * torch.randn(n, generator=g)).to(dtype)
+        b = (0.1 * torch.randn(n, generator=g)).to(dtype) if family == "ln" else None
+        parity_util.run_and_compare(family, x, dy, w, b, eps, what)
+    elif family in ("softmax", "softmin", "logsoftmax"):
+        softmax_t.run_and_compare(family, x, dy, what, x_gpu=None if x_gpu is None else x_gpu.detach(), dy_gpu=dy_gpu)
+    elif family == "norm":
+        p = [1, 2, 3, 2.5][int(rng.integers(4))]
+        gn = torch.rand(1, m, generator=g).to(dtype)
+        pnorm_t.compare_norm(x.view(1, m, n), gn, p, 1e-6, f"{what} p={p}")
+    elif family == "normalize":
+        p = [1, 2, 4, 1.5][int(rng.integers(4))]
+        pnorm_t.compare_normalize(x.view(1, m, n), dy.view(1, m, n), p, 1e-6, f"{what} p={p}")
+    elif family == "act":
+        name = ["gelu", "gelu_tanh", "silu", "relu", "sigmoid", "tanh", "mish", "softplus"][int(rng.integers(8))]
+        act_t.run_and_compare(name, x, dy, f"{what} {name}", x_gpu=None if x_gpu is None else x_gpu.detach(), dy_gpu=dy_gpu)
+    else:
+        kind = family.split("+")[0]
+        act = ["gelu", "gelu_tanh", "silu", "relu"][int(rng.integers(4))]
+        w = (1 + 0.2 * torch.randn(n, generator=g)).to(dtype)
+        b = (0.2 * torch.randn(n, generator=g)).to(dtype) if kind == "ln" else None
+        fused_t.run_and_compare(kind, act, x, dy, w, b, eps, f"{what} {act}")
