@@ -400,7 +400,10 @@ int plan_launch(int which, int flavour, bool aligned, int64_t M, int64_t N, int 
         // workgroups: row widths of 5 * 2^k elements and their neighbours): a second workgroup brings the bytes in
         // flight back to where HBM throughput peaks (bf16 N = 5120 forward 5.5 -> 6.0 TB/s, N = 1280 5.6 -> 6.1).
         const bool one_stream = which == kNormFwd || which == kSoftmaxFwd || which == kPnormFwd || which == kFusedFwd;
-        if (one_stream && aligned && s.block * s.k < 1024 && n_vecs > 16 && cap < 2) cap = 2;
+        // (not when that leaves a workgroup fewer than 32 steps: 8192 rows of 6000 fp16 lose 5 % to the second set of
+        // parameter loads and launch ramps)
+        const int64_t steps_with_two = M / (static_cast<int64_t>(s.block / s.tpr) * cus * 2);
+        if (one_stream && aligned && s.block * s.k < 1024 && n_vecs > 16 && steps_with_two >= 32 && cap < 2) cap = 2;
     }
     if (cap < bpc) bpc = cap;
     const int rows_per_block = s.block / s.tpr;
