@@ -58,6 +58,9 @@ WORKLOADS = {
     "softmin_bf16_16384x4096": ("softmin", 16384, 4096, "bf16"),
     "logsoftmax_bf16_8192x32768": ("logsoftmax", 8192, 32768, "bf16"),
     "logsoftmax_f32_16384x4096": ("logsoftmax", 16384, 4096, "f32"),
+    # vocabulary-sized rows, wider than 64 KiB: the looping kernels (two walks per row)
+    "logsoftmax_f32_8192x32000_vocab": ("logsoftmax", 8192, 32000, "f32"),
+    "logsoftmax_bf16_4096x128256_vocab": ("logsoftmax", 4096, 128256, "bf16"),
     # row p-norm / normalize of a (1, rows, K) tensor (thn_normalize_fwd + thn_normalize_bwd, or thn_pnorm_*)
     "normalize_p2_bf16_16384x4096": ("normalize_p2", 16384, 4096, "bf16"),
     "normalize_p2_f32_16384x4096": ("normalize_p2", 16384, 4096, "f32"),

@@ -292,7 +292,8 @@ int thn_norm_set_launch_override(int which, int vecs_per_thread, int threads_per
  * What the heuristic (or the override) would launch for this problem: fills shape[0..4] with
  * {vecs_per_thread, threads_per_row, block_threads, grid_blocks, aligned 128-bit path (1) or unaligned-row path (0)}.
  * For the epilogue families (9, 10) `is_layernorm` carries the activation too: bit 0 = LayerNorm, bits 1.. = the
- * thn_act code.
+ * thn_act code.  Rows wider than 64 KiB of the softmax and p-norm families report their looping kernels:
+ * {vectors per thread and step, block_threads, block_threads, grid_blocks, 0}.
  */
 int thn_norm_query_launch(int which, int is_layernorm, int64_t M, int64_t N, int x_dtype, int32_t shape[5]);
 

@@ -796,6 +796,25 @@ int thn_norm_query_launch(int which, int is_layernorm, int64_t M, int64_t N, int
         if (is_layernorm < 0 || !fusable(is_layernorm >> 1)) return THN_E_SHAPE;
         flavour = is_layernorm;                     // bit 0 = LayerNorm, bits 1.. = activation
     }
+    if (N > 0 && N * bytes > kMaxRowBytes && which >= kSoftmaxFwd && which <= kNormalizeBwd) {
+        // the looping kernels: one workgroup per row
+        const int cus = current_cu_count();
+        if (cus <= 0) return THN_E_DEVICE;
+        if (M < 0) return THN_E_SHAPE;
+        int block = thn::kLoopBlock, grid = loop_grid(M);
+        if (which == kSoftmaxFwd || which == kSoftmaxBwd) {
+            int bpc;
+            softmax_loop_launch(which, &block, &bpc);
+            const int64_t cap = static_cast<int64_t>(cus) * bpc;
+            grid = static_cast<int>(M < cap ? M : cap);
+        }
+        shape[0] = thn::kWalkVecs;
+        shape[1] = block;
+        shape[2] = block;
+        shape[3] = grid;
+        shape[4] = 0;
+        return THN_OK;
+    }
     const int rc = plan_launch(which, flavour, aligned, M, N, x_dtype, &p);
     if (rc != THN_OK) return rc;
     shape[0] = p.s.k;
