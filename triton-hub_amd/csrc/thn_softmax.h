@@ -284,7 +284,7 @@ __global__ void __launch_bounds__(kSoftmaxLoopBlock) softmax_fwd_loop_kernel(con
             acc += v > neg_inf ? static_cast<double>(exp_c(v - m)) : 0.0;   // -inf - -inf must not poison the sum
             return C(0);
         };
-        walk_row_vec<T, C, kSoftmaxLoopBlock, 1, false, true>(
+        walk_row_vec<T, C, kSoftmaxLoopBlock, 1, false, true, true>(
             xrow, nullptr, nullptr, nullptr, a.n_cols, t,
             [&](const C (&f)[3][T::VEC], C (&)[T::VEC]) {
                 C v[T::VEC];
@@ -312,7 +312,7 @@ __global__ void __launch_bounds__(kSoftmaxLoopBlock) softmax_fwd_loop_kernel(con
         C scale;
         if constexpr (LOG) scale = static_cast<C>(log(s[0]));
         else scale = static_cast<C>(1.0 / s[0]);
-        walk_row<T, C, kSoftmaxLoopBlock, 1, true>(xrow, nullptr, nullptr, yrow, a.n_cols, t, [&](C x, C, C) {
+        walk_row<T, C, kSoftmaxLoopBlock, 1, true, false, true>(xrow, nullptr, nullptr, yrow, a.n_cols, t, [&](C x, C, C) {
             const C z = x * sign - row_max;
             if constexpr (LOG) return z - scale;
             else return exp_c(z) * scale;
@@ -332,7 +332,7 @@ __global__ void __launch_bounds__(kSoftmaxLoopBlock) softmax_bwd_loop_kernel(con
         const char* grow = a.dy + row * a.dy_stride_bytes;
         char* dxrow = a.dx + row * a.dx_stride_bytes;
         double acc = 0.0;
-        walk_row_vec<T, C, kSoftmaxLoopBlock, 2, false, true>(
+        walk_row_vec<T, C, kSoftmaxLoopBlock, 2, false, true, true>(
             yrow, grow, nullptr, nullptr, a.n_cols, t,
             [&](const C (&f)[3][T::VEC], C (&)[T::VEC]) {
                 C part = C(0);
@@ -351,7 +351,7 @@ __global__ void __launch_bounds__(kSoftmaxLoopBlock) softmax_bwd_loop_kernel(con
         double s[1] = {acc};
         row_allreduce<kSoftmaxLoopBlock, 1, 1, OpSum, double>(s, red_sum, phase_sum, 0, t);
         const C total = static_cast<C>(s[0]);
-        walk_row<T, C, kSoftmaxLoopBlock, 2, true>(yrow, grow, nullptr, dxrow, a.n_cols, t, [&](C y, C g, C) {
+        walk_row<T, C, kSoftmaxLoopBlock, 2, true, false, true>(yrow, grow, nullptr, dxrow, a.n_cols, t, [&](C y, C g, C) {
             C d;
             if constexpr (LOG) d = fma(-exp_c(y), total, g);
             else d = y * (g - total);
