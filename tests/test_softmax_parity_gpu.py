@@ -169,6 +169,54 @@ def test_large_logits_and_saturated_rows(kind):
             assert float(y[1, hot]) == 1.0 and float(y[1].sum()) == 1.0
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("n", [8, 100, 333, 2048, 4104])
+@pytest.mark.parametrize("kind", ["softmax", "logsoftmax"])
+def test_masked_logits(kind, n, dtype):
+    """Attention-style masks: row i keeps its first i % n + 1 logits and has -inf in the rest; one row is masked
+    completely.  Masked columns come out as exactly 0 (softmax) or -inf (log-softmax) and receive exactly 0 / the
+    upstream gradient; a row without any finite logit is NaN, as exp(-inf - -inf) makes it in the reference
+    (softmax.py:33-37) and in torch; the columns that are kept match the float64 values."""
+    announce(f"masked logits {kind} n={n} {dtype}")
+    rows = min(n, 257) + 3
+    g = torch.Generator().manual_seed(n)
+    x = torch.randn(rows, n, generator=g).to(dtype)
+    dy = torch.randn(rows, n, generator=g).to(dtype)
+    keep = (torch.arange(rows) % n + 1)[:, None]
+    masked = torch.arange(n)[None, :] >= keep
+    x[masked] = float("-inf")
+    x[rows - 2] = float("-inf")
+    dead = torch.zeros(rows, dtype=torch.bool); dead[rows - 2] = True
+    xg = x.cuda().requires_grad_(True)
+    y = MODULE[kind]()(xg)
+    y.backward(dy.cuda())
+    torch.cuda.synchronize()
+    y, dx = y.detach().cpu(), xg.grad.cpu()
+    assert bool(torch.isnan(y[dead]).all()) and bool(torch.isnan(dx[dead]).all())
+    live = ~dead
+    m_live = masked[live]
+    y_l, dx_l, dy_l = y[live], dx[live], dy[live]
+    if kind == "softmax":
+        assert bool((y_l[m_live] == 0).all()) and bool((dx_l[m_live] == 0).all())
+    else:
+        assert bool((y_l[m_live] == float("-inf")).all()) and bool((dx_l[m_live] == dy_l[m_live]).all())
+    xr = x[live].double()
+    fn = torch.softmax if kind == "softmax" else torch.log_softmax
+    yr = fn(xr, -1)
+    ys, gd = y_l.double(), dy_l.double()        # the backward is a function of the saved output (softmax.py:86-97)
+    if kind == "softmax":
+        dxr = ys * (gd - (ys * gd).sum(-1, keepdim=True))
+    else:
+        dxr = gd - torch.exp(ys) * gd.sum(-1, keepdim=True)
+    eps = {torch.float32: 2.0 ** -19, torch.bfloat16: 2.0 ** -7, torch.float16: 2.0 ** -10}[dtype]     # loose: the mask pattern is the point
+    kept = ~m_live
+    for got, ref, what in ((y_l, yr.detach(), "y"), (dx_l, dxr, "dx")):
+        err = (got.double() - ref)[kept].abs()
+        scale = ref[kept].abs() + 1.0
+        assert bool((err <= eps * scale + 1e-30).all()), f"{kind} masked {what}: {float((err / (scale + 1e-30)).max()):.3e}"
+    assert bool(torch.isfinite(y_l[kept]).all()) and bool(torch.isfinite(dx_l).all())
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float64])
 @pytest.mark.parametrize("kind", KINDS)
 def test_strides_views_and_batch_shapes(kind, dtype):
