@@ -200,6 +200,49 @@ def test_empty_and_single_row():
     assert torch.equal(y, torch.zeros(5, 1, device="cuda"))
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("n", [48, 1000, 4096, 12288])
+@pytest.mark.parametrize("kind", ["ln", "rms"])
+def test_non_finite_inputs_stay_in_their_row(kind, n, dtype):
+    """A NaN or an infinity in the input spoils only its own row of y and dx (the statistics are per row) and,
+    through the column sums, every dW entry (xhat of that row is NaN everywhere); dB only sums the upstream
+    gradient and stays finite.  The other rows are bit-identical to a run without the spoiled rows."""
+    announce(f"non-finite {kind} N={n} {dtype}")
+    g = torch.Generator().manual_seed(n)
+    rows = 37
+    x = torch.randn(rows, n, generator=g).to(dtype)
+    dy = torch.randn(rows, n, generator=g).to(dtype)
+    bad = {3: float("nan"), 11: float("inf"), 20: float("-inf")}
+    for r, v in bad.items():
+        x[r, (r * 7) % n] = v
+    make = (lambda: LayerNorm(n, device="cuda", dtype=dtype)) if kind == "ln" else \
+        (lambda: RMSNorm(n, device="cuda", dtype=dtype))
+    mod = make()
+    xg = x.cuda().requires_grad_(True)
+    y = mod(xg)
+    y.backward(dy.cuda())
+    good = torch.ones(rows, dtype=torch.bool)
+    good[list(bad)] = False
+    y, dx = y.detach().cpu(), xg.grad.cpu()
+    assert bool(torch.isnan(dx[~good]).all()) and bool(torch.isnan(y[3]).all())
+    for r in (11, 20):
+        spoiled = torch.zeros(n, dtype=torch.bool)
+        spoiled[(r * 7) % n] = True
+        if kind == "ln":                # mean = +-inf: every x - mean is NaN or infinite, the variance NaN
+            assert bool(torch.isnan(y[r]).all())
+        else:                           # mean(x^2) = inf: rstd = 0, so y = 0 except inf * 0 at the spoiled column
+            assert bool(torch.isnan(y[r][spoiled]).all()) and bool((y[r][~spoiled] == 0).all())
+    assert bool(torch.isfinite(y[good]).all()) and bool(torch.isfinite(dx[good]).all())
+    assert bool(torch.isnan(mod.weight.grad).all())
+    if kind == "ln":
+        assert bool(torch.isfinite(mod.bias.grad).all())
+    ref = make()
+    xr = x[good].cuda().requires_grad_(True)
+    yr = ref(xr)
+    yr.backward(dy[good].cuda())
+    assert torch.equal(yr.detach().cpu(), y[good]) and torch.equal(xr.grad.cpu(), dx[good])
+
+
 # ---- the 64 KiB row limit (layernorm.py:69-72) -----------------------------------------------------------------
 @pytest.mark.parametrize("dtype,n_max", [(torch.float32, 16384), (torch.bfloat16, 32768), (torch.float16, 32768),
                                          (torch.float64, 8192)])

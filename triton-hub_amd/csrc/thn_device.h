@@ -59,7 +59,9 @@ __device__ __forceinline__ float rsqrt_refined(float v) {
     const float h = 0.5f * r;
     const float e = fmaf(-v * r, r, 1.0f);       // 1 - v*r^2
     const float refined = fmaf(h, e, r);          // r + r*e/2
-    return v > 0.0f ? refined : r;                // v == 0 (eps == 0, constant row): +inf, as 1/sqrt(0) is
+    // v == 0 (eps == 0, constant row): +inf, as 1/sqrt(0) is; v == +inf (an infinity in the row): 0, where the
+    // step would make inf * 0 = NaN of it
+    return (v > 0.0f && v < __builtin_inff()) ? refined : r;
 }
 
 // ---------------------------------------------------------------------------------------------------
