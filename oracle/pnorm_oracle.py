@@ -27,7 +27,9 @@ def norm_fwd(x, p=2, eps=1e-6):
         out = np.sqrt((x * x).sum(-1))
     else:
         out = (np.abs(x) ** p).sum(-1) ** (1.0 / p)
-    return np.maximum(out, eps)
+    # tl.maximum with its default NaN handling returns the other operand for a NaN (norm.py:40): a row that
+    # holds a NaN comes out as eps
+    return np.fmax(out, eps)
 
 
 def norm_bwd(x, norms, dnorms, p=2):

@@ -210,6 +210,58 @@ def test_eps_clamp_zero_rows_and_empty_input():
         assert y.shape == shape and e.grad.shape == shape
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("n", [64, 1000, 40000])
+def test_non_finite_and_overflowing_rows(n, dtype):
+    """Rows that hold an infinity, a NaN, only zeros, or entries whose squares overflow float32 (the reference
+    computes these types in float32, norm.py:24): the norm is inf / eps / eps / inf -- eps for the NaN row because
+    tl.maximum(out, eps) returns eps for a NaN (norm.py:40) -- and x / norm follows from the stored norm
+    (normalize.py:30): 0 for a row with an infinite norm (NaN where x itself is infinite), x / eps for the NaN row.
+    For p = 2 the gradients of an overflowed row are 0 (a finite numerator over an infinite norm)."""
+    announce(f"pnorm non-finite N={n} {dtype}")
+    g = torch.Generator().manual_seed(n)
+    x = torch.randn(1, 6, n, generator=g).to(dtype)
+    spoiled = {1: float("inf"), 2: float("nan"), 3: float("-inf")}
+    for r, v in spoiled.items():
+        x[0, r, r * 7] = v
+    x[0, 4] = 0.0
+    x[0, 5] = 1e30
+    eps = 1e-6
+    eps_st = float(torch.tensor(eps).to(dtype))
+    inf = float("inf")
+    for p in (1, 2, 3, 2.5):
+        xg = x.cuda().requires_grad_(True)
+        nrm = norm(p=p, eps=eps)(xg)
+        nrm.backward(torch.ones_like(nrm))
+        got = nrm.detach().float().cpu()[0]
+        assert float(got[1]) == inf and float(got[3]) == inf, f"p={p}: {got}"
+        assert float(got[2]) == eps_st and float(got[4]) == eps_st, f"p={p}: {got}"
+        if p == 1:
+            assert float(got[5]) == pytest.approx(n * 1e30, rel=1e-2)
+        else:
+            assert float(got[5]) == inf
+            if p == 2:                   # p > 2: |x|^(p-1) overflows as well, inf / inf (norm.py:86-90)
+                assert bool((xg.grad[0, 5] == 0).all()), f"p={p}: norm dx of the overflowed row"
+        assert bool(torch.isfinite(got[0])) and bool(torch.isfinite(xg.grad[0, 0]).all())
+        xg = x.cuda().requires_grad_(True)
+        y = normalize(p=p, eps=eps)(xg)
+        y.backward(torch.ones_like(y))
+        yc = y.detach().float().cpu()[0]
+        assert bool((yc[4] == 0).all())
+        for r in (1, 3):
+            hit = torch.zeros(n, dtype=torch.bool); hit[r * 7] = True
+            assert bool(torch.isnan(yc[r][hit]).all()) and bool((yc[r][~hit] == 0).all()), f"p={p} row {r}"
+        hit = torch.zeros(n, dtype=torch.bool); hit[14] = True
+        expect = (x[0, 2].float() / eps_st)[~hit]
+        assert bool(torch.isnan(yc[2][hit]).all())
+        assert torch.allclose(yc[2][~hit], expect.to(dtype).float(), rtol=2.0 ** -6 if dtype == torch.bfloat16 else 1e-5)
+        if p != 1:
+            assert bool((yc[5] == 0).all()), f"p={p}: y of the overflowed row"
+            if p == 2:                   # p > 2: |x|^(p-1) * (0 / inf) = inf * 0 (normalize.py:113)
+                assert bool((xg.grad[0, 5] == 0).all()), f"p={p}: normalize dx of the overflowed row"
+        assert bool(torch.isfinite(yc[0]).all()) and bool(torch.isfinite(xg.grad[0, 0]).all())
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 def test_properties_at_large_size(dtype):
     """Size-independent properties on 16 x 4096 x 4096: unit norm of the output, homogeneity (a power-of-two scale

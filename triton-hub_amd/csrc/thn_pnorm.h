@@ -147,6 +147,10 @@ __device__ __forceinline__ float div_by_row(float num, float den, float rden) {
     const float q = num * rden;
     return __builtin_fmaf(__builtin_fmaf(-q, den, num), rden, q);
 }
+// The `den` to pass to div_by_row: an infinite divisor (a row whose power sum overflowed) becomes 0, so that the
+// residual is num - q*0 instead of the NaN of 0 * inf, and the quotient 0 (NaN for an infinite numerator), as
+// the division gives it.
+__device__ __forceinline__ float residual_divisor(float den) { return den < __builtin_inff() ? den : 0.0f; }
 
 // x rounded to storage type T and widened again.
 template <typename T>
@@ -253,12 +257,13 @@ __global__ void __launch_bounds__(BLOCK) pnorm_fwd_kernel(const PnormFwdArgs a) 
         if constexpr (NORMALIZE) {
             const float nr = round_to_storage<T>(n);
             const float rn = 1.0f / nr;
+            const float nd = residual_divisor(nr);
             char* yrow = a.y + y_off;
 #pragma unroll
             for (int k = 0; k < K; ++k) {
                 float yf[VEC];
 #pragma unroll
-                for (int e = 0; e < VEC; ++e) yf[e] = div_by_row(xf[k][e], nr, rn);
+                for (int e = 0; e < VEC; ++e) yf[e] = div_by_row(xf[k][e], nd, rn);
                 store_row_vec<T, ALIGNED>(yrow, voff[k], a.n_cols, yf);
             }
             y_off = row_offset(a.ymap, ncur);
@@ -321,6 +326,7 @@ __global__ void __launch_bounds__(BLOCK) pnorm_bwd_kernel(const PnormBwdArgs a) 
         float den = c_n;
         if constexpr (MODE == kPInt) den = pow_small(c_n, a.p_int - 1);     // norms^(p-1), norm.py:86-87
         const float rden = 1.0f / den;
+        den = residual_divisor(den);
         char* dxrow = a.dx + dx_off;
         dx_off = row_offset(a.dxmap, ncur);
 #pragma unroll
@@ -421,6 +427,7 @@ __global__ void __launch_bounds__(BLOCK) normalize_bwd_kernel(const NormalizeBwd
         const float proj = s[0];
         const float n = c_n;
         const float rn = 1.0f / n;
+        const float nd = residual_divisor(n);
         float coef = 0.0f;                                                                    // per-row factor of sign(x)*...
         if constexpr (MODE == kP1) coef = proj / (n * n);                                     // normalize.py:106
         if constexpr (MODE == kPInt) coef = proj / (pow_small(n, a.p_int - 1) * n);           // normalize.py:115
@@ -434,12 +441,12 @@ __global__ void __launch_bounds__(BLOCK) normalize_bwd_kernel(const NormalizeBwd
             for (int e = 0; e < VEC; ++e) {
                 const float gg = gf[k][e];
                 if constexpr (MODE == kP2) {
-                    df[e] = div_by_row(gg - yf[k][e] * proj, n, rn);                          // normalize.py:110
+                    df[e] = div_by_row(gg - yf[k][e] * proj, nd, rn);                          // normalize.py:110
                 } else if constexpr (MODE == kP1) {
-                    df[e] = div_by_row(gg, n, rn) - sign_of(xf[k][e]) * coef;
+                    df[e] = div_by_row(gg, nd, rn) - sign_of(xf[k][e]) * coef;
                 } else {
                     const float x = xf[k][e];
-                    df[e] = div_by_row(gg, n, rn) - sign_of(x) * pow_small(__builtin_fabsf(x), a.p_int - 1) * coef;
+                    df[e] = div_by_row(gg, nd, rn) - sign_of(x) * pow_small(__builtin_fabsf(x), a.p_int - 1) * coef;
                 }
             }
             store_row_vec<T, ALIGNED>(dxrow, voff[k], a.n_cols, df);
