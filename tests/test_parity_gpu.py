@@ -122,6 +122,50 @@ def test_rmsnorm_variants(dtype, affine):
     compare_with_oracle("rms", x, dy, mod.weight.detach().cpu() if affine else None, None, 1e-6, out, "variant")
 
 
+@pytest.mark.parametrize("n", [384, 4096, 12288])
+@pytest.mark.parametrize("kind", ["ln", "rms", "ln_gelu"])
+def test_frozen_parameters_skip_their_sums(kind, n):
+    """requires_grad=False on weight and / or bias: that gradient is None, the others and dx are bit-identical to
+    the run with every gradient wanted (the row kernel is the same, only the stores of its sums differ)."""
+    from TritonHub.Normalization.fused import LayerNormActivation
+    announce(f"frozen parameters {kind} N={n}")
+    g = torch.Generator().manual_seed(n)
+    x = torch.randn(300, n, generator=g).bfloat16().cuda()
+    dy = torch.randn(300, n, generator=g).bfloat16().cuda()
+    make = {"ln": lambda: LayerNorm(n, device="cuda", dtype=torch.bfloat16),
+            "rms": lambda: RMSNorm(n, device="cuda", dtype=torch.bfloat16),
+            "ln_gelu": lambda: LayerNormActivation(n, "gelu", device="cuda", dtype=torch.bfloat16)}[kind]
+    full = make()
+    with torch.no_grad():
+        full.weight.copy_(1 + 0.1 * torch.randn(n, generator=g).cuda())
+    xf = x.clone().requires_grad_(True)
+    full(xf).backward(dy)
+    has_bias = kind != "rms"
+    for train_w, train_b in ((False, False), (True, False), (False, True)):
+        if train_b and not has_bias:
+            continue
+        mod = make()
+        mod.load_state_dict(full.state_dict())
+        mod.weight.requires_grad_(train_w)
+        if has_bias:
+            mod.bias.requires_grad_(train_b)
+        xg = x.clone().requires_grad_(True)
+        mod(xg).backward(dy)
+        assert torch.equal(xg.grad, xf.grad)
+        assert (mod.weight.grad is None) == (not train_w)
+        if train_w:
+            assert torch.equal(mod.weight.grad, full.weight.grad)
+        if has_bias:
+            assert (mod.bias.grad is None) == (not train_b)
+            if train_b:
+                assert torch.equal(mod.bias.grad, full.bias.grad)
+    # only the parameters want gradients: the input's is computed and dropped
+    mod = make()
+    mod.load_state_dict(full.state_dict())
+    mod(x).backward(dy)
+    assert torch.equal(mod.weight.grad, full.weight.grad)
+
+
 def test_mixed_parameter_and_activation_dtypes():
     # float32 parameters under bfloat16 activations: dW / dB come back in the parameter dtype (layernorm.py:207-208)
     announce("mixed dtypes")

@@ -140,9 +140,12 @@ def norm_fwd(x: torch.Tensor, weight, bias, eps: float, layernorm: bool, act: in
     return (out.reshape(*x.shape[:-1], n) if reshaped else out), mean, rstd
 
 
-def norm_bwd(x: torch.Tensor, dout: torch.Tensor, weight, bias, mean, rstd, layernorm: bool, act: int = -1):
+def norm_bwd(x: torch.Tensor, dout: torch.Tensor, weight, bias, mean, rstd, layernorm: bool, act: int = -1,
+             need_dw: bool = True, need_db: bool = True):
     """Returns (dx like x, dw or None, db or None); dw/db take the dtype of weight/bias (layernorm.py:207-208).
-    `act` >= 0: the backward of norm_fwd(..., act) (thn_norm_act_bwd)."""
+    `act` >= 0: the backward of norm_fwd(..., act) (thn_norm_act_bwd).  `need_dw` / `need_db` False: that parameter
+    is frozen (autograd's needs_input_grad): its sums are not stored, and with both False the backward is the row
+    kernel alone, without partial sums and without the second stage."""
     if not x.is_cuda:
         _native.require_gpu(x)
     x2, m, n, x_stride, reshaped = _flatten(x, 'input')
@@ -160,11 +163,11 @@ def norm_bwd(x: torch.Tensor, dout: torch.Tensor, weight, bias, mean, rstd, laye
     if n * x.element_size() > 65536:
         raise RuntimeError(FEATURE_DIM_MESSAGE)
     x_code = _native.dtype_code(x.dtype)
-    want_db = layernorm and bias is not None
+    want_db = layernorm and bias is not None and need_db
     mixed = weight is not None and want_db and weight.dtype != bias.dtype
     grad_dtype = weight.dtype if weight is not None else (bias.dtype if want_db else x.dtype)
     w_code = _native.dtype_code(grad_dtype)
-    dw = torch.empty((n,), dtype=grad_dtype, device=device) if weight is not None else None
+    dw = torch.empty((n,), dtype=grad_dtype, device=device) if (weight is not None and need_dw) else None
     db = torch.empty((n,), dtype=grad_dtype, device=device) if want_db else None
     if m == 0:                       # the sum over no rows
         dw = None if dw is None else dw.zero_()

@@ -38,7 +38,9 @@ class layernorm_act(torch.autograd.Function):
     @staticmethod
     def backward(ctx, d_out):
         input, weight, bias, mean, rstd = ctx.saved_tensors
-        grad, dw, db = norm_bwd(input, d_out, weight, bias, mean, rstd, layernorm=True, act=ctx.act)
+        _, need_dw, need_db = ctx.needs_input_grad[:3]
+        grad, dw, db = norm_bwd(input, d_out, weight, bias, mean, rstd, layernorm=True, act=ctx.act, need_dw=need_dw,
+                                need_db=need_db)
         return grad, dw, db, None, None
 
 
@@ -56,7 +58,8 @@ class rmsnorm_act(torch.autograd.Function):
     @staticmethod
     def backward(ctx, d_out):
         input, weight, rstd = ctx.saved_tensors
-        grad, dw, _ = norm_bwd(input, d_out, weight, None, None, rstd, layernorm=False, act=ctx.act)
+        grad, dw, _ = norm_bwd(input, d_out, weight, None, None, rstd, layernorm=False, act=ctx.act,
+                               need_dw=ctx.needs_input_grad[1])
         return grad, dw, None, None
 
 

@@ -22,7 +22,9 @@ class layernorm(torch.autograd.Function):
     @staticmethod
     def backward(ctx, d_out):
         input, weight, bias, mean, rstd = ctx.saved_tensors
-        grad, dw, db = norm_bwd(input, d_out, weight, bias, mean, rstd, layernorm=True)
+        _, need_dw, need_db = ctx.needs_input_grad[:3]        # frozen parameters: their sums are skipped
+        grad, dw, db = norm_bwd(input, d_out, weight, bias, mean, rstd, layernorm=True, need_dw=need_dw,
+                                need_db=need_db)
         return grad, dw, db, None
 
 

@@ -22,7 +22,8 @@ class rmsnorm(torch.autograd.Function):
     @staticmethod
     def backward(ctx, d_out):
         input, weight, rstd = ctx.saved_tensors
-        grad, dw, _ = norm_bwd(input, d_out, weight, None, None, rstd, layernorm=False)
+        grad, dw, _ = norm_bwd(input, d_out, weight, None, None, rstd, layernorm=False,
+                               need_dw=ctx.needs_input_grad[1])           # a frozen weight: no column sums
         return grad, dw, None
 
 
