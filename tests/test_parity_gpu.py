@@ -304,8 +304,8 @@ def test_feature_dim_limit(dtype, n_max):
 
 
 # ---- rows of 24-64 KiB: the 1024-thread workgroups, several rows per workgroup ----------------------------------
-@pytest.mark.parametrize("dtype,widths", [(torch.bfloat16, (12296, 16384, 20480, 24576, 28680, 32768)),
-                                          (torch.float16, (16384, 24568, 32768)),
+@pytest.mark.parametrize("dtype,widths", [(torch.bfloat16, (12296, 16384, 20480, 24576, 26624, 28680, 32768)),
+                                          (torch.float16, (16384, 24568, 28672, 32768)),
                                           (torch.float32, (6148, 8192, 12288, 16384)),
                                           (torch.float64, (4096, 8192))])
 def test_wide_rows_many_per_workgroup(dtype, widths):
@@ -430,7 +430,7 @@ def compiled_shapes():
     bwd = [s for blk in (256, 512) for s in expand("THN_BWD_SHAPES_B", blk)]
     tail = re.search(r"#define THN_BWD_SHAPES\(X\)(.*?)\n\n", text, re.S).group(1)
     bwd += [(int(k), int(t), int(b)) for k, t, b in re.findall(r"X\((\d+), (\d+), (\d+)\)", tail)]
-    return fwd, bwd
+    return fwd, bwd, expand("THN_BWD_SHAPES_LN16")
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
@@ -439,8 +439,10 @@ def test_every_compiled_launch_shape(kind, dtype):
     """Forces each kernel instance in turn through the launch override and checks it against the oracle, at a
     row width that fills the shape exactly and at one that leaves vector slots without work."""
     lib = _native.lib()
-    fwd_shapes, bwd_shapes = compiled_shapes()
-    assert len(fwd_shapes) >= 20 and len(bwd_shapes) >= 40
+    fwd_shapes, bwd_shapes, ln16_shapes = compiled_shapes()
+    assert len(fwd_shapes) >= 20 and len(bwd_shapes) >= 40 and len(ln16_shapes) == 4
+    if kind == "ln" and dtype == torch.bfloat16:
+        bwd_shapes = bwd_shapes + ln16_shapes       # instances that only the LayerNorm backward of 16-bit rows has
     vec = 16 // torch.empty(0, dtype=dtype).element_size()
     g = torch.Generator().manual_seed(23)
     pairs = sorted(set((k, t) for k, t, _ in fwd_shapes + bwd_shapes))

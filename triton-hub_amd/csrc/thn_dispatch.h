@@ -36,6 +36,11 @@ struct Shape {
     X(1, 512, 512) X(2, 512, 512) X(3, 512, 512) X(4, 512, 512)                      \
     X(1, 1024, 1024) X(2, 1024, 1024) X(3, 1024, 1024) X(4, 1024, 1024)
 
+// LayerNorm backward over 16-bit rows of more than 32 KiB: 5 to 8 vectors per thread in 512-thread workgroups,
+// which leave a thread 256 registers for the float32 weights and dB sums of its 40 to 64 columns (the dW sums
+// live in LDS).  A 1024-thread workgroup has half as many and spills at 4 vectors per thread.
+#define THN_BWD_SHAPES_LN16(X) X(5, 512, 512) X(6, 512, 512) X(7, 512, 512) X(8, 512, 512)
+
 // Shapes of the element-wise (unaligned) path: four vectors per thread, any row width.
 #define THN_SCALAR_SHAPES(X)                                                         \
     X(4, 8, 256) X(4, 16, 256) X(4, 32, 256) X(4, 64, 256) X(4, 128, 256)            \
@@ -98,6 +103,11 @@ inline int run_kernel(void (*kern)(const Args), const Args& a, int grid, int blo
         using T = TYPE;                                                                                    \
         if (aligned) {                                                                                     \
             THN_BWD_SHAPES(THN_BWD_AL)                                                                     \
+            if constexpr (TYPE::kBytes == 2) {                                                             \
+                if (ln) {                                                                                  \
+                    THN_BWD_SHAPES_LN16(THN_BWD_AL_LN)                                                     \
+                }                                                                                          \
+            }                                                                                              \
         } else if (a.n_cols >= TYPE::VEC) { \
             THN_SCALAR_SHAPES(THN_BWD_SC) \
         } else { \
@@ -110,6 +120,10 @@ inline int run_kernel(void (*kern)(const Args), const Args& a, int grid, int blo
 #define THN_FWD_AL(K_, TPR_, BLOCK_) THN_CASE(norm_fwd_kernel, FwdArgs, true, K_, TPR_, BLOCK_)
 #define THN_FWD_SC(K_, TPR_, BLOCK_) THN_CASE(norm_fwd_kernel, FwdArgs, false, K_, TPR_, BLOCK_)
 #define THN_BWD_AL(K_, TPR_, BLOCK_) THN_CASE(norm_bwd_kernel, BwdArgs, true, K_, TPR_, BLOCK_)
+#define THN_BWD_AL_LN(K_, TPR_, BLOCK_)                                                                    \
+    if (s.k == K_ && s.tpr == TPR_ && s.block == BLOCK_) {                                                 \
+        return run_kernel<BwdArgs>(norm_bwd_kernel<T, true, K_, TPR_, BLOCK_, true>, a, grid, BLOCK_, st, occupancy); \
+    }
 #define THN_BWD_SC(K_, TPR_, BLOCK_) THN_CASE(norm_bwd_kernel, BwdArgs, false, K_, TPR_, BLOCK_)
 
 }  // namespace thn
