@@ -104,9 +104,11 @@ def test_against_composed_oracles(kind, act, dtype):
         run_and_compare(kind, act, x, dy, w, b, 1e-5, f"{kind}+{act} {shape} {dtype}")
 
 
-@pytest.mark.parametrize("dtype,widths", [(torch.bfloat16, (16384, 24576, 32768)), (torch.float32, (12288, 16384))])
+@pytest.mark.parametrize("dtype,widths", [(torch.bfloat16, (16384, 20480, 24576, 28672, 32768)), (torch.float16, (26632,)),
+                                          (torch.float32, (12288, 16384))])
 def test_wide_rows_many_per_workgroup(dtype, widths):
-    # rows of 48-64 KiB: the 1024-thread workgroups, with more rows than the grid has workgroups
+    # rows of 32-64 KiB (1024-thread workgroups; LayerNorm over 16-bit rows: 512 threads with 5-8 vectors each), with
+    # more rows than the grid has workgroups
     for n in widths:
         for kind, act in (("ln", "gelu_tanh"), ("rms", "silu")):
             announce(f"fused wide {kind} {act} {dtype} N={n}")

@@ -70,7 +70,7 @@ struct Override {
 };
 Override g_override[kFamilies];
 
-// `ln16`: LayerNorm over 16-bit rows (only the norm backward has instances of its own for that).
+// `ln16`: LayerNorm over 16-bit rows (the two norm backwards have instances of their own for that).
 bool shape_compiled(int which, bool aligned, bool ln16, Shape s) {
 #define THN_MATCH(K_, TPR_, BLOCK_) if (s.k == K_ && s.tpr == TPR_ && s.block == BLOCK_) return true;
     if (!aligned) {
@@ -84,6 +84,9 @@ bool shape_compiled(int which, bool aligned, bool ln16, Shape s) {
         THN_FUSED_FWD_SHAPES(THN_MATCH)
     } else if (which == kFusedBwd) {
         THN_FUSED_BWD_SHAPES(THN_MATCH)
+        if (ln16) {
+            THN_FUSED_BWD_SHAPES_LN16(THN_MATCH)
+        }
     } else if (which >= kPnormFwd) {
         THN_ROW_SHAPES(THN_MATCH)
     } else {
@@ -302,8 +305,11 @@ int ceil_div(int a, int b) { return (a + b - 1) / b; }
 Shape heuristic_shape(int which, bool aligned, bool ln16, int n_vecs) {
     // LayerNorm backward over 16-bit rows of more than 32 KiB: 512 threads with 5 to 8 vectors each (256 registers
     // per thread) instead of 1024 threads with 3 or 4 (bf16 N = 20480 / 24576 / 28672 / 32768: 122 / 139 / 183 /
-    // 203 us -> 112 / 131 / 156 / 187 us for 4096 rows).
-    if (which == kNormBwd && aligned && ln16 && n_vecs > 2048) return Shape{ceil_div(n_vecs, 512), 512, 512};
+    // 203 us -> 112 / 131 / 156 / 187 us for 4096 rows; with a GeLU epilogue N = 20480 / 28672: 286 / 518 -> 218 /
+    // 373 us).
+    if ((which == kNormBwd || which == kFusedBwd) && aligned && ln16 && n_vecs > 2048) {
+        return Shape{ceil_div(n_vecs, 512), 512, 512};
+    }
     int kmax = (aligned && which == kNormBwd && n_vecs > 128) ? 3 : 4;
     // Softmax backward: two input streams and nothing to hold; 2 vectors per thread per stream measured best,
     // except for 2 KiB rows, where one full wave per row (2 x 64) is 8 % slower than half a wave (4 x 32).
@@ -385,7 +391,7 @@ int plan_launch(int which, int flavour, bool aligned, int64_t M, int64_t N, int 
     const int cus = current_cu_count();
     if (cus <= 0) return THN_E_DEVICE;
 
-    const bool ln16 = which == kNormBwd && bytes == 2 && (flavour & 1) != 0;
+    const bool ln16 = (which == kNormBwd || which == kFusedBwd) && bytes == 2 && (flavour & 1) != 0;
     Shape s = heuristic_shape(which, aligned, ln16, n_vecs);
     const Override& ov = g_override[which];
     Shape cand = s;

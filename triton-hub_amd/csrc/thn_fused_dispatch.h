@@ -25,6 +25,10 @@ namespace thn {
     X(2, 128, 512) X(3, 128, 512) X(2, 256, 512) X(3, 256, 512) X(2, 512, 512) X(3, 512, 512) \
     X(2, 1024, 1024) X(3, 1024, 1024) X(4, 1024, 1024)
 
+// LayerNorm with an epilogue over 16-bit rows of more than 32 KiB: the 512-thread shapes of the plain LayerNorm
+// backward (bias and weight of 40-64 columns in float32 next to the dB sums; 1024 threads spill 48-284 bytes).
+#define THN_FUSED_BWD_SHAPES_LN16(X) THN_BWD_SHAPES_LN16(X)
+
 #define THN_DECLARE_FUSED_LAUNCHERS(NAME)                                                                      \
     int launch_fused_fwd_##NAME(bool ln, int act, bool aligned, Shape s, const FwdArgs& a, int grid,           \
                                 hipStream_t st, int* occupancy);                                               \
@@ -47,6 +51,16 @@ THN_DECLARE_FUSED_LAUNCHERS(f64)
         THN_FUSED_ACT_CASE(KERNEL, ARGS_T, AL, K_, TPR_, BLOCK_, kGeluTanh)                                    \
         THN_FUSED_ACT_CASE(KERNEL, ARGS_T, AL, K_, TPR_, BLOCK_, kSilu)                                        \
         THN_FUSED_ACT_CASE(KERNEL, ARGS_T, AL, K_, TPR_, BLOCK_, kRelu)                                        \
+        return 1;                                                                                              \
+    }
+#define THN_FUSED_ACT_CASE_LN(AL, K_, TPR_, BLOCK_, A)                                                         \
+    if (act == A) return run_kernel<BwdArgs>(norm_bwd_kernel<T, true, K_, TPR_, BLOCK_, AL, A>, a, grid, BLOCK_, st, occupancy);
+#define THN_FB_AL_LN(K_, TPR_, BLOCK_)                                                                         \
+    if (s.k == K_ && s.tpr == TPR_ && s.block == BLOCK_) {                                                     \
+        THN_FUSED_ACT_CASE_LN(true, K_, TPR_, BLOCK_, kGelu)                                                   \
+        THN_FUSED_ACT_CASE_LN(true, K_, TPR_, BLOCK_, kGeluTanh)                                               \
+        THN_FUSED_ACT_CASE_LN(true, K_, TPR_, BLOCK_, kSilu)                                                   \
+        THN_FUSED_ACT_CASE_LN(true, K_, TPR_, BLOCK_, kRelu)                                                   \
         return 1;                                                                                              \
     }
 #define THN_FF_AL(K_, TPR_, BLOCK_) THN_FUSED_CASE(norm_fwd_kernel, FwdArgs, true, K_, TPR_, BLOCK_)
@@ -75,6 +89,11 @@ THN_DECLARE_FUSED_LAUNCHERS(f64)
         using T = TYPE;                                                                                        \
         if (aligned) {                                                                                         \
             THN_FUSED_BWD_SHAPES(THN_FB_AL)                                                                    \
+            if constexpr (TYPE::kBytes == 2) {                                                                 \
+                if (ln) {                                                                                      \
+                    THN_FUSED_BWD_SHAPES_LN16(THN_FB_AL_LN)                                                    \
+                }                                                                                              \
+            }                                                                                                  \
         } else if (a.n_cols >= TYPE::VEC) { \
             THN_SCALAR_SHAPES(THN_FB_SC) \
         } else { \

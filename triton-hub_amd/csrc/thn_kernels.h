@@ -110,7 +110,7 @@ constexpr RowForm fwd_form() {
 
 template <int BYTES, bool LN, int K, int BLOCK, bool FUSED>
 constexpr RowForm bwd_form() {
-    if (BYTES == 2 && LN && K >= 5 && !FUSED) return RowForm{true, K <= 6, true};      // 512-thread workgroups
+    if (BYTES == 2 && LN && K >= 5) return RowForm{true, K <= 6 && !FUSED, true};      // 512-thread workgroups
     if (BLOCK < 1024) return kPlainForm;
     if (BYTES >= 4) {
         if (K == 4) return RowForm{true, !LN, false};
