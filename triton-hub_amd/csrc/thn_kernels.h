@@ -95,6 +95,8 @@ __device__ __forceinline__ u32x4 load_row_vec(const char* rowp, int voff, int n_
 //   !ahead:    the next row is not requested a whole row ahead: vector k of the next row is loaded into the
 //              registers of vector k as soon as that one has been stored (4-16 % slower where the row-ahead
 //              form fits, so it is the last resort).
+// The LayerNorm backward of 16-bit rows wider than 32 KiB runs in 512-thread workgroups instead (5 to 8 vectors
+// per thread, 256 registers): its weights and dB sums alone take 80 to 128 registers; it uses the same forms.
 struct RowForm {
     bool recompute, ahead, lds_dw;
 };
