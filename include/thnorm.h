@@ -274,6 +274,23 @@ int thn_norm_act_bwd(const void* x, int64_t x_row_stride,
                      int x_dtype, int w_dtype, void* stream);
 
 /*
+ * Dropout over a contiguous tensor of `n` elements (the reference's TritonHub/Layers/dropout.py).  Replaces both
+ * `_dropout_kernel_fwd[grid](x, out, M, p, seed, ...)` (dropout.py:43-48, device code :12-23) and
+ * `_dropout_kernel_bwd[grid](dout, dx, M, p, seed, ...)` (dropout.py:87-92, device code :56-67), which are the same
+ * function: out[i] = rand(seed, i) < p ? 0 : x[i] / (1 - p), in float32 (float64 storage: the float64 quotient by
+ * the float32 1 - p), rounded to the storage type.  rand(seed, i) is what Triton's tl.rand(seed, i) returns --
+ * Philox-4x32-10 on counter (i, 0, 0, 0) and key (seed), first word, mapped to a float32 in [0, 1) -- so a seed
+ * gives the same mask as in the reference, bit for bit.  Element i of the call uses offset first_offset + i (0 for
+ * a whole tensor; a caller that splits a tensor into pieces passes each piece's position); offsets of 2^32 and
+ * more put their high word into the second counter word, as tl.rand does for 64-bit offsets (the reference's
+ * 32-bit `cols` would have wrapped).  0 <= p <= 1.  `x` and `out` need element alignment only and must not overlap
+ * partially (out == x, in place, is fine).  The p == 0 / eval-mode / p == 1 shortcuts of dropout.py:29-32 are the
+ * caller's.
+ */
+int thn_dropout(const void* x, void* out, int64_t n, int64_t first_offset, float p, uint64_t seed, int dtype,
+                void* stream);
+
+/*
  * Launch-shape control for tuning sweeps (the counterpart of the reference's `triton.autotune` over
  * num_warps, autotune.py:62-65, which this library replaces by a fixed heuristic on N and the dtype).
  * `which`: 0 = norm forward, 1 = norm backward, 2 = softmax forward, 3 = softmax backward, 4 = p-norm /

@@ -25,7 +25,7 @@ def declared_functions():
 
 def test_library_exports_every_declared_symbol():
     names = declared_functions()
-    assert len(names) == 20 and "thn_norm_act_fwd" in names and "thn_norm_act_bwd" in names and "thn_act_fwd" in names and "thn_pnorm_fwd" in names and "thn_normalize_bwd" in names and "thn_norm_fwd" in names and "thn_norm_bwd" in names and "thn_softmax_fwd" in names
+    assert len(names) == 21 and "thn_dropout" in names and "thn_norm_act_fwd" in names and "thn_norm_act_bwd" in names and "thn_act_fwd" in names and "thn_pnorm_fwd" in names and "thn_normalize_bwd" in names and "thn_norm_fwd" in names and "thn_norm_bwd" in names and "thn_softmax_fwd" in names
     handle = ctypes.CDLL(_native.LIB_PATH)
     for name in names:
         assert hasattr(handle, name), f"{name} is declared in include/thnorm.h but not exported"
@@ -226,6 +226,38 @@ def test_package_surface():
         assert issubclass(fn, torch.autograd.Function)
     assert Activations.Softmax().softmax_fn is not None and Activations.Softmin().softmin_fn is not None
     assert Activations.LogSoftmax().logsoftmax_fn is not None
+
+
+def test_dropout_surface_and_argument_checks_answer_without_a_gpu():
+    """Layers/dropout.py:95-119: the Function takes (input, p, training) and keeps (p, seed, training); the module is
+    Dropout(p=0.5) and follows train() / eval().  The C entry point checks its arguments before it needs a device."""
+    import random
+    from TritonHub import Layers
+    from TritonHub.Layers.dropout import dropout
+    assert Layers.__all__ == ["Dropout"] and issubclass(dropout, torch.autograd.Function)
+    mod = Layers.Dropout()
+    assert mod.p == 0.5 and mod.training and mod.dropout_fn is not None and not list(mod.parameters())
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        mod(torch.randn(4, 8))
+    # the seed comes from Python's `random`, one draw per forward call, also when nothing is dropped
+    random.seed(5)
+    random.randint(0, 2 ** 16)
+    second = random.randint(0, 2 ** 16)
+    random.seed(5)
+    with pytest.raises(RuntimeError):
+        mod(torch.randn(2, 2))
+    assert random.randint(0, 2 ** 16) == second
+    lib = _native.lib()
+    buf = (ctypes.c_float * 16)()
+    addr = ctypes.addressof(buf)
+    assert lib.thn_dropout(addr, addr, 16, 0, 0.5, 1, 9, None) == _native.E_DTYPE
+    assert lib.thn_dropout(addr, addr, -1, 0, 0.5, 1, _native.F32, None) == _native.E_SHAPE
+    assert lib.thn_dropout(addr, addr, 16, -1, 0.5, 1, _native.F32, None) == _native.E_SHAPE
+    assert lib.thn_dropout(addr, addr, 16, 0, 1.5, 1, _native.F32, None) == _native.E_SHAPE
+    assert lib.thn_dropout(addr, addr, 16, 0, float("nan"), 1, _native.F32, None) == _native.E_SHAPE
+    assert lib.thn_dropout(0, 0, 0, 0, 0.5, 1, _native.F32, None) == 0                  # nothing to do
+    assert lib.thn_dropout(0, addr, 16, 0, 0.5, 1, _native.F32, None) == _native.E_NULL
+    assert lib.thn_dropout(addr + 2, addr, 8, 0, 0.5, 1, _native.F32, None) == _native.E_SHAPE     # element alignment
 
 
 @pytest.mark.parametrize("affine,bias", [(True, True), (True, False), (False, True), (False, False)])

@@ -49,6 +49,7 @@ SYMBOLS = {
     'thn_norm_act_bwd_workspace_bytes': (_i64, [_i64, _i64, _i32, _i32, _i32, _i32]),
     'thn_norm_act_bwd': (_i32, [_vp, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64,
                                 _i32, _i32, _i32, _vp]),
+    'thn_dropout': (_i32, [_vp, _vp, _i64, _i64, _f32, ctypes.c_uint64, _i32, _vp]),
     'thn_norm_set_launch_override': (_i32, [_i32, _i32, _i32, _i32, _i32]),
     'thn_norm_query_launch': (_i32, [_i32, _i32, _i64, _i64, _i32, ctypes.POINTER(ctypes.c_int32)]),
 }

@@ -10,6 +10,7 @@
 #include "thn_fused_dispatch.h"
 #include "thn_reduce.h"
 #include "thn_act_dispatch.h"
+#include "thn_dropout.h"
 #include "thn_pnorm_dispatch.h"
 #include "thn_softmax_dispatch.h"
 
@@ -1167,6 +1168,36 @@ int thn_act_bwd(const void* saved, int64_t saved_row_stride, const void* dy, int
                 void* stream) {
     return act_launch(saved, saved_row_stride, dy, dy_row_stride, dx, dx_row_stride, M, N, act, param0, param1, dtype,
                       true, stream);
+}
+
+int thn_dropout(const void* x, void* out, int64_t n, int64_t first_offset, float p, uint64_t seed, int dtype,
+                void* stream) {
+    const int bytes = elem_bytes(dtype);
+    if (bytes == 0) return THN_E_DTYPE;
+    if (n < 0 || first_offset < 0 || !(p >= 0.0f && p <= 1.0f)) return THN_E_SHAPE;
+    if (n == 0) return THN_OK;
+    if (x == nullptr || out == nullptr) return THN_E_NULL;
+    if ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(out)) % static_cast<uintptr_t>(bytes) != 0) {
+        return THN_E_SHAPE;
+    }
+    const int cus = current_cu_count();
+    if (cus <= 0) return THN_E_DEVICE;
+    thn::DropoutArgs a{};
+    a.x = static_cast<const char*>(x);
+    a.out = static_cast<char*>(out);
+    a.total_elems = n;
+    a.total_vecs = n / (16 / bytes);
+    a.first_offset = first_offset;
+    a.p = p;
+    a.key_lo = static_cast<uint32_t>(seed);
+    a.key_hi = static_cast<uint32_t>(seed >> 32);
+    // Bound by integer arithmetic: as many waves as a compute unit holds (8 workgroups of 256 threads).
+    const int64_t blocks = (a.total_vecs + thn::kDropoutBlock - 1) / thn::kDropoutBlock;
+    const int64_t cap = static_cast<int64_t>(cus) * 8;
+    const int grid = static_cast<int>(blocks < 1 ? 1 : (blocks < cap ? blocks : cap));
+    const int rc = thn::launch_dropout(dtype, a, grid, static_cast<hipStream_t>(stream));
+    if (rc > 0) return THN_E_DTYPE;
+    return rc == 0 ? THN_OK : THN_E_LAUNCH;
 }
 
 }  // extern "C"
