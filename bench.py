@@ -78,6 +78,9 @@ WORKLOADS = {
     "act_mish_bf16_16384x4096": ("act_mish", 16384, 4096, "bf16"),
     "act_softplus_f16_16384x4096": ("act_softplus", 16384, 4096, "f16"),
     "act_sigmoid_f32_16384x4096": ("act_sigmoid", 16384, 4096, "f32"),
+    # Layers.Dropout (thn_dropout on x, then on dy, with the same seed)
+    "dropout_bf16_16384x4096": ("dropout", 16384, 4096, "bf16"),
+    "dropout_f32_16384x4096": ("dropout", 16384, 4096, "f32"),
 }
 ACT_NAMES = ["gelu", "gelu_tanh", "silu", "relu", "leaky_relu", "relu6", "sigmoid", "tanh", "mish", "softplus", "threshold"]
 ACT_PARAMS = {"leaky_relu": (0.01, 0.0), "softplus": (1.0, 20.0), "threshold": (0.1, 20.0)}
@@ -140,6 +143,8 @@ def main():
         kind, act_name = kind.split("+")
         fused_act = ["gelu", "gelu_tanh", "silu", "relu"].index(act_name)
     dtype = {"bf16": torch.bfloat16, "f16": torch.float16, "f32": torch.float32}[dname]
+    if kind == "dropout":
+        return dropout_main(args, lib, dev, m, n, dname, dtype)
     if kind in SOFTMAX_KINDS or kind.startswith(("normalize", "pnorm", "act_")):
         return softmax_main(args, lib, dev, kind, m, n, dname, dtype)
     s = torch.empty(0, dtype=dtype).element_size()
@@ -415,6 +420,98 @@ def softmax_main(args, lib, dev, kind, m, n, dname, dtype):
     if not args.no_cpu_baseline:
         baseline = {None: softmax_cpu_baseline, "act": act_cpu_baseline}.get(row_op, row_op_cpu_baseline)
         out["cpu_baseline"] = baseline(kind, m, n, dtype, sets[0], step_bytes)
+    print(json.dumps(out), flush=True)
+
+
+def dropout_main(args, lib, dev, m, n, dname, dtype):
+    """One step = thn_dropout on x (forward) + thn_dropout on dy with the same seed (backward), p = 0.1, over one of
+    four rotating buffer sets.  Every element costs a Philox-4x32-10 block of its own (the reference draws
+    tl.rand(seed, i) per element): the kernel is bound by 32-bit integer multiplications, and the HBM fraction below
+    says how far that is from the memory roofline, not how good the kernel is."""
+    import torch
+    from TritonHub import _native
+    s = torch.empty(0, dtype=dtype).element_size()
+    code = _native.dtype_code(dtype)
+    gen = torch.Generator(device=dev).manual_seed(0)
+    sets = []
+    for _ in range(N_BUFFER_SETS):
+        x = torch.randn(m, n, device=dev, generator=gen).to(dtype)
+        dy = torch.randn(m, n, device=dev, generator=gen).to(dtype)
+        sets.append(dict(x=x, dy=dy, y=torch.empty_like(x), dx=torch.empty_like(x)))
+    stream = torch.cuda.current_stream(dev).cuda_stream
+    p = _native.ptr
+    mn, prob = m * n, 0.1
+
+    def forward(b_, seed=12345):
+        rc = lib.thn_dropout(p(b_["x"]), p(b_["y"]), mn, 0, prob, seed, code, stream)
+        assert rc == 0, _native.strerror(rc)
+
+    def backward(b_, seed=12345):
+        rc = lib.thn_dropout(p(b_["dy"]), p(b_["dx"]), mn, 0, prob, seed, code, stream)
+        assert rc == 0, _native.strerror(rc)
+
+    def step(i):
+        forward(sets[i % N_BUFFER_SETS], 1000 + i)
+        backward(sets[i % N_BUFFER_SETS], 1000 + i)
+
+    for i in range(args.warmup):
+        step(i)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        step(i)
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    launch_bytes = 2 * mn * s
+    step_bytes = 2 * launch_bytes
+    gbps = step_bytes / (ms_per_step * 1e-3) / 1e9
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    for i in range(args.steps):
+        forward(sets[i % N_BUFFER_SETS])
+    stop.record()
+    torch.cuda.synchronize()
+    fwd_us = start.elapsed_time(stop) * 1e3 / args.steps
+    achieved = launch_bytes / (fwd_us * 1e-6) / 1e9
+    out = {
+        "metric": f"fwd+bwd HBM GB/s and % of peak, dropout {dname} {m}x{n}",
+        "value": round(gbps, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": dname, "data": "synthetic",
+        "config": {"workload": args.workload, "op": "dropout", "rows": m, "row_width": n, "p": prob,
+                   "buffer_sets": N_BUFFER_SETS, "entry_points": "thn_dropout (x) + thn_dropout (dy)"},
+        "pct_of_hbm_peak": round(100.0 * gbps / HBM_PEAK_GBPS, 2),
+        "elements_per_s": round(2 * mn / (ms_per_step * 1e-3)),
+        "algorithmic_bytes_per_step": step_bytes,
+        "kernels_us": {"forward": round(fwd_us, 2)},
+        "roofline": {"bound": "hbm", "kernel": "dropout_flat_kernel", "achieved": round(achieved, 1),
+                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
+                     "algorithmic_bytes_per_launch": launch_bytes, "avg_launch_us": round(fwd_us, 2), "traffic": None,
+                     "note": "limited by the 37 32x32-bit multiplications of one Philox-4x32-10 block per element "
+                             "(quarter-rate instructions), not by memory"},
+    }
+    if not args.no_cpu_baseline:
+        from oracle import dropout_oracle as do
+        rows = min(m, max(16, (1 << 21) // n))
+        x = sets[0]["x"][:rows].float().cpu().numpy()
+        dy = sets[0]["dy"][:rows].float().cpu().numpy()
+
+        def oracle_step():
+            do.dropout(x, prob, 12345)
+            do.dropout(dy, prob, 12345)
+
+        oracle_step()
+        best = float("inf")
+        for _ in range(3):
+            t0 = time.perf_counter()
+            oracle_step()
+            best = min(best, time.perf_counter() - t0)
+        out["cpu_baseline"] = {"value": round(step_bytes * rows / m / best / 1e9, 3), "unit": "GB/s", "cores": 1,
+                               "kind": "port",
+                               "sample": f"first {rows} of {m} rows of the same workload, forward + backward, best of 3 "
+                                         f"passes of oracle/dropout_oracle.py (numpy, one thread; {best * 1e3:.1f} ms "
+                                         "per pass)",
+                               "host_cpu_count": os.cpu_count()}
     print(json.dumps(out), flush=True)
 
 

@@ -55,14 +55,30 @@ __device__ __forceinline__ float dropout_rand(int64_t offset, uint32_t k0, uint3
     return uniform_from_word(philox_first_word(static_cast<uint32_t>(o), static_cast<uint32_t>(o >> 32), k0, k1));
 }
 
+// x / keep for a float32 divisor shared by all elements, correctly rounded like the division it replaces: the
+// float64 product of x and the float64 reciprocal of keep is within 2^-52 of the exact quotient, and a quotient of two
+// float32 values is never closer than 2^-49 (relative) to a point where float32 rounding changes direction, so
+// rounding the product to float32 gives the same value as rounding the quotient itself (infinities, NaN, signed
+// zeros, overflow and subnormal results included).  3 instructions per element instead of the 11 of a division.
+struct KeepDivisor {
+    double rk64;     // float32 storage types
+    double keep64;   // float64 storage
+};
+__device__ __forceinline__ KeepDivisor make_keep_divisor(float keep) {
+    return KeepDivisor{1.0 / static_cast<double>(keep), static_cast<double>(keep)};
+}
+__device__ __forceinline__ float keep_div(float x, const KeepDivisor& d) {
+    return static_cast<float>(static_cast<double>(x) * d.rk64);
+}
+__device__ __forceinline__ double keep_div(double x, const KeepDivisor& d) { return x / d.keep64; }
+
 constexpr int kDropoutBlock = 256;
 
 template <typename T>
 __global__ void __launch_bounds__(kDropoutBlock) dropout_flat_kernel(const DropoutArgs a) {
     using C = typename std::conditional<T::kBytes == 8, double, float>::type;
     constexpr int VEC = T::VEC;
-    const float keep_f = 1.0f - a.p;                // float32, as the reference's `1 - p`
-    const C keep = static_cast<C>(keep_f);
+    const KeepDivisor keep = make_keep_divisor(1.0f - a.p);        // float32 difference, as the reference's `1 - p`
     const int64_t step = static_cast<int64_t>(gridDim.x) * kDropoutBlock;
     for (int64_t v = static_cast<int64_t>(blockIdx.x) * kDropoutBlock + threadIdx.x; v < a.total_vecs; v += step) {
         const u32x4 raw = ld128u(a.x + v * 16);
@@ -72,7 +88,7 @@ __global__ void __launch_bounds__(kDropoutBlock) dropout_flat_kernel(const Dropo
 #pragma unroll
         for (int e = 0; e < VEC; ++e) {
             const float r = dropout_rand(e0 + e, a.key_lo, a.key_hi);
-            of[e] = r < a.p ? C(0) : xf[e] / keep;
+            of[e] = r < a.p ? C(0) : keep_div(xf[e], keep);
         }
         st128u(a.out + v * 16, pack_as<T, C>(of));
     }
@@ -81,7 +97,7 @@ __global__ void __launch_bounds__(kDropoutBlock) dropout_flat_kernel(const Dropo
     if (blockIdx.x == 0 && i < a.total_elems) {
         const C x = load_elem<T, C>(a.x, i);
         const float r = dropout_rand(a.first_offset + i, a.key_lo, a.key_hi);
-        store_elem<T, C>(a.out, i, r < a.p ? C(0) : x / keep);
+        store_elem<T, C>(a.out, i, r < a.p ? C(0) : keep_div(x, keep));
     }
 }
 
