@@ -89,3 +89,22 @@ def test_row_operators_beyond_2_31_elements(name):
         assert torch.equal(edges(y.detach().view(ROWS, N)), ye.detach().view(2 * EDGE, N))
     ye.backward(dye)
     assert torch.equal(edges(xv.grad.view(ROWS, N)), xev.grad.view(2 * EDGE, N))
+
+
+def test_dropout_beyond_2_31_elements():
+    """Element offsets of 2^31 and more: the Philox counter takes the offset as an unsigned 32-bit word (and a high
+    word from 2^32 on); the last rows are compared with the oracle at their true offsets."""
+    import random
+    from oracle import dropout_oracle as do
+    from TritonHub.Layers import Dropout
+    announce("large index dropout")
+    x = big(5)
+    random.seed(3)
+    seed = random.randint(0, 2 ** 16)
+    random.seed(3)
+    y = Dropout(0.25)(x)
+    for r in (0, (1 << 31) // N, (1 << 31) // N + 1, ROWS - 1):
+        ref = do.dropout(x[r].float().cpu().numpy(), 0.25, seed, first_offset=r * N)
+        assert torch.equal(y[r].cpu(), torch.from_numpy(ref).bfloat16()), f"row {r}"
+    rate = float((y == 0).float().mean())
+    assert abs(rate - 0.25) < 1e-3
