@@ -100,3 +100,50 @@ def test_c_abi_calls_replay_from_a_hip_graph():
         torch.cuda.synchronize()
         for name, e, t in zip("y dx dw rstd sm dsm act dact".split(), eager, outputs):
             assert torch.equal(e, t), f"replay {trial}: {name} differs from the eager result"
+
+
+def test_operators_from_several_host_threads():
+    """Four host threads, each on a stream of its own, run different row widths through the operator layer at the same
+    time (the library's launch-plan and occupancy caches and the per-stream workspaces are shared state): every
+    thread's results equal the ones computed alone beforehand."""
+    import threading
+    announce("host threads")
+    torch.manual_seed(1)
+    widths = [384, 1024, 4096, 6000]
+    inputs, expected = [], []
+    for n in widths:
+        x = torch.randn(257, n, device="cuda", dtype=torch.bfloat16)
+        dy = torch.randn(257, n, device="cuda", dtype=torch.bfloat16)
+        mods = [LayerNorm(n, device="cuda", dtype=torch.bfloat16), RMSNorm(n, device="cuda", dtype=torch.bfloat16), Softmax()]
+        outs = []
+        for mod in mods:
+            a = x.clone().requires_grad_(True)
+            y = mod(a); y.backward(dy)
+            outs.append((y.detach().clone(), a.grad.clone()))
+        inputs.append((x, dy, mods))
+        expected.append(outs)
+    torch.cuda.synchronize()
+    errors = []
+
+    def work(i):
+        try:
+            x, dy, mods = inputs[i]
+            stream = torch.cuda.Stream()
+            with torch.cuda.stream(stream):
+                for rep in range(20):
+                    for mod, (ye, ge) in zip(mods, expected[i]):
+                        a = x.clone().requires_grad_(True)
+                        y = mod(a); y.backward(dy)
+                        stream.synchronize()
+                        if not (torch.equal(y.detach(), ye) and torch.equal(a.grad, ge)):
+                            errors.append((i, rep, type(mod).__name__))
+        except Exception as e:                      # surface the failure in the main thread
+            errors.append((i, repr(e)))
+
+    threads = [threading.Thread(target=work, args=(i,)) for i in range(len(widths))]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join(timeout=120)
+    assert not any(t.is_alive() for t in threads), "a worker thread did not finish"
+    assert not errors, errors[:5]
