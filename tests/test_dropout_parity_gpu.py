@@ -179,3 +179,31 @@ def test_properties_at_large_size(dtype):
     for r in rows:
         ref = expected(x[r].cpu(), p, seed, first_offset=r * n)
         assert same_bits(y[r].detach().cpu(), ref), f"row {r}"
+
+
+def test_random_sizes_offsets_seeds_and_alignments():
+    """150 seeded random calls through the C ABI: sizes from 1 to 70000 elements, input and output views that start
+    0-7 elements into their buffers, offsets up to 2^40, seeds up to 2^63, p over (0, 1)."""
+    announce("dropout random C ABI calls")
+    lib = _native.lib()
+    st = torch.cuda.current_stream().cuda_stream
+    rng = np.random.default_rng(2024)
+    for case in range(150):
+        dtype = DTYPES[int(rng.integers(len(DTYPES)))]
+        n = int(np.exp(rng.uniform(0, np.log(70000))))
+        skew_in, skew_out = int(rng.integers(0, 8)), int(rng.integers(0, 8))
+        first = int(rng.integers(0, 2 ** 40)) if rng.random() < 0.5 else int(rng.integers(0, 2 ** 20))
+        seed = int(rng.integers(0, 2 ** 63)) if rng.random() < 0.3 else int(rng.integers(0, 2 ** 16 + 1))
+        p = float(rng.uniform(0.01, 0.99))
+        x = torch.from_numpy(rng.standard_normal(n + skew_in).astype(np.float32)).to(dtype)
+        xg = x.cuda()
+        buf = torch.full((n + skew_out + 8,), 7.0, device="cuda", dtype=dtype)
+        size = x.element_size()
+        rc = lib.thn_dropout(xg.data_ptr() + skew_in * size, buf.data_ptr() + skew_out * size, n, first, p, seed,
+                             _native.dtype_code(dtype), st)
+        assert rc == 0, (case, rc)
+        torch.cuda.synchronize()
+        got = buf.cpu()
+        what = f"case {case}: {dtype} n={n} skew=({skew_in},{skew_out}) first={first} seed={seed} p={p:.3f}"
+        assert same_bits(got[skew_out:skew_out + n].contiguous(), expected(x[skew_in:].contiguous(), p, seed, first)), what
+        assert bool((got[:skew_out] == 7).all()) and bool((got[skew_out + n:] == 7).all()), what + " (wrote outside)"
