@@ -192,6 +192,24 @@ def test_ragged_hidden_sizes(kind, n, dtype):
     run_and_compare(kind, x, dy, w, b, 1e-5, f"ragged N={n}")
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_odd_widths_of_16_bit_rows_reach_every_two_vector_shape(dtype):
+    """LayerNorm backward over 16-bit rows off the 128-bit path runs 2 vectors per thread (its own instances, one per
+    threads-per-row value) up to 2048 vectors and the common 4-vector instance beyond: one odd width for each."""
+    expect = {9: (2, 8), 201: (2, 16), 499: (2, 32), 1001: (2, 64), 1501: (2, 128), 3001: (2, 256), 4099: (2, 512),
+              12289: (2, 1024), 20001: (4, 1024)}
+    g = torch.Generator().manual_seed(77)
+    for n, (k, tpr) in expect.items():
+        announce(f"odd width {n} {dtype}")
+        m = 131
+        assert _launch.query_launch(1, True, m, n, dtype)[:2] == (k, tpr)
+        assert _launch.query_launch(1, False, m, n, dtype)[0] == 4              # RMSNorm keeps the common instances
+        x = (0.5 + torch.randn(m, n, generator=g)).to(dtype); dy = torch.randn(m, n, generator=g).to(dtype)
+        w = (1 + 0.1 * torch.randn(n, generator=g)); b = 0.1 * torch.randn(n, generator=g)
+        run_and_compare("ln", x, dy, w.to(dtype), b.to(dtype), 1e-5, f"odd LN N={n}")
+        run_and_compare("ln", x, dy, w, b, 1e-5, f"odd LN N={n}, float32 parameters")
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_row_strides_and_misaligned_views(dtype):
     announce(f"strides {dtype}")

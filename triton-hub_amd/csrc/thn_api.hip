@@ -76,6 +76,9 @@ bool shape_compiled(int which, bool aligned, bool ln16, Shape s) {
 #define THN_MATCH(K_, TPR_, BLOCK_) if (s.k == K_ && s.tpr == TPR_ && s.block == BLOCK_) return true;
     if (!aligned) {
         THN_SCALAR_SHAPES(THN_MATCH)
+        if (ln16 && which == kNormBwd) {
+            THN_SCALAR_BWD_LN16_SHAPES(THN_MATCH)
+        }
     } else if (which == kNormBwd) {
         THN_BWD_SHAPES(THN_MATCH)
         if (ln16) {
@@ -326,6 +329,17 @@ Shape heuristic_shape(int which, bool aligned, bool ln16, int n_vecs) {
     }
     if (!aligned) {
         s.k = 4;
+        // LayerNorm backward over 16-bit rows: 2 vectors per thread where 1024 threads cover the row (4 vectors are
+        // more than 256 registers of state, one wave per SIMD).
+        if (which == kNormBwd && ln16 && n_vecs <= 2048) {
+            s.k = 2;
+            for (int tpr : kTprList) {
+                if (tpr * 2 >= n_vecs) {
+                    s.tpr = tpr;
+                    break;
+                }
+            }
+        }
         s.block = s.tpr > 256 ? s.tpr : 256;
         return s;
     }
@@ -392,7 +406,8 @@ int plan_launch(int which, int flavour, bool aligned, int64_t M, int64_t N, int 
     const int cus = current_cu_count();
     if (cus <= 0) return THN_E_DEVICE;
 
-    const bool ln16 = (which == kNormBwd || which == kFusedBwd) && bytes == 2 && (flavour & 1) != 0;
+    // (rows shorter than one vector have a single element-wise instance)
+    const bool ln16 = (which == kNormBwd || which == kFusedBwd) && bytes == 2 && (flavour & 1) != 0 && N >= vec_elems;
     Shape s = heuristic_shape(which, aligned, ln16, n_vecs);
     const Override& ov = g_override[which];
     Shape cand = s;

@@ -46,6 +46,12 @@ struct Shape {
     X(4, 8, 256) X(4, 16, 256) X(4, 32, 256) X(4, 64, 256) X(4, 128, 256)            \
     X(4, 256, 256) X(4, 512, 512) X(4, 1024, 1024)
 
+// LayerNorm backward over 16-bit rows off the 128-bit path: 2 vectors per thread (the 4 of THN_SCALAR_SHAPES are 32
+// float32 columns of weights, dW and dB sums per thread: more than 256 registers, one wave per SIMD).
+#define THN_SCALAR_BWD_LN16_SHAPES(X)                                                \
+    X(2, 8, 256) X(2, 16, 256) X(2, 32, 256) X(2, 64, 256) X(2, 128, 256)            \
+    X(2, 256, 256) X(2, 512, 512) X(2, 1024, 1024)
+
 // Return value of the launchers: 0 launched (or occupancy written), 1 no such instance, <0 HIP error.
 // When `occupancy` is not null the kernel is not launched; *occupancy receives the number of workgroups
 // of that instance that fit on one compute unit.
@@ -110,6 +116,11 @@ inline int run_kernel(void (*kern)(const Args), const Args& a, int grid, int blo
             }                                                                                              \
         } else if (a.n_cols >= TYPE::VEC) { \
             THN_SCALAR_SHAPES(THN_BWD_SC) \
+            if constexpr (TYPE::kBytes == 2) { \
+                if (ln) { \
+                    THN_SCALAR_BWD_LN16_SHAPES(THN_BWD_SC_LN) \
+                } \
+            } \
         } else { \
             using T = ElemIo<TYPE>; \
             THN_BWD_SC(4, 8, 256) \
@@ -123,6 +134,10 @@ inline int run_kernel(void (*kern)(const Args), const Args& a, int grid, int blo
 #define THN_BWD_AL_LN(K_, TPR_, BLOCK_)                                                                    \
     if (s.k == K_ && s.tpr == TPR_ && s.block == BLOCK_) {                                                 \
         return run_kernel<BwdArgs>(norm_bwd_kernel<T, true, K_, TPR_, BLOCK_, true>, a, grid, BLOCK_, st, occupancy); \
+    }
+#define THN_BWD_SC_LN(K_, TPR_, BLOCK_)                                                                    \
+    if (s.k == K_ && s.tpr == TPR_ && s.block == BLOCK_) {                                                 \
+        return run_kernel<BwdArgs>(norm_bwd_kernel<T, true, K_, TPR_, BLOCK_, false>, a, grid, BLOCK_, st, occupancy); \
     }
 #define THN_BWD_SC(K_, TPR_, BLOCK_) THN_CASE(norm_bwd_kernel, BwdArgs, false, K_, TPR_, BLOCK_)
 
