@@ -33,10 +33,36 @@ __device__ __forceinline__ float tanh_safe(float u) {
 
 __device__ __forceinline__ float sigmoid_f(float x) { return rcp_fast(1.0f + __expf(-x)); }
 
-// Phi(x) = 0.5*(1 + erf(x/sqrt 2)), the normal distribution function of GeLU, from the complementary error
-// function erfc(z) = t*exp(-z^2 + P(t)), t = 1/(1 + z/2), z >= 0 (Chebyshev fit, relative error below 1.2e-7 for
-// every z, Numerical Recipes 6.2): branch free, a third of the instructions of the library erff, and accurate in
-// the negative tail, where 1 + erf(..) cancels.
+// Phi(x) = 0.5*(1 + erf(x/sqrt 2)), the normal distribution function of GeLU, from the scaled complementary error
+// function: erfc(z) = erfcx(z) * exp(-z^2), and erfcx(z) = t*Q(t) with t = 1/(1 + z/2) in (0, 1] for z >= 0, Q a
+// polynomial of degree 10 (fitted for the smallest relative error of t*Q(t): 1.1e-8; 1.2e-7 after float32 Horner
+// evaluation; Q(0) = 1/(2 sqrt(pi)), the limit of erfcx(z)*z/2).  Branch free, accurate in the negative tail, where
+// 1 + erf(..) cancels, a third of the instructions of the library erff -- and its exponential is exp(-x^2/2), the
+// one the derivative of GeLU needs for the normal density, so the backward evaluates a single exponential.
+struct NormalParts { float cdf, e; };           // e = exp(-x^2/2)
+__device__ __forceinline__ NormalParts normal_parts(float x) {
+    const float z = __builtin_fabsf(x) * 0.70710678118654752440f;
+    const float t = rcp_fast(__builtin_fmaf(0.5f, z, 1.0f));
+    float q = 0.042352267f;
+    q = __builtin_fmaf(q, t, -0.2308562f);
+    q = __builtin_fmaf(q, t, 0.48617613f);
+    q = __builtin_fmaf(q, t, -0.44697466f);
+    q = __builtin_fmaf(q, t, 0.12708776f);
+    q = __builtin_fmaf(q, t, -0.057231836f);
+    q = __builtin_fmaf(q, t, 0.093000434f);
+    q = __builtin_fmaf(q, t, 0.17537685f);
+    q = __builtin_fmaf(q, t, 0.24688059f);
+    q = __builtin_fmaf(q, t, 0.28209385f);
+    q = __builtin_fmaf(q, t, 0.2820948f);
+    NormalParts n;
+    n.e = __expf(-z * z);
+    const float half_erfc = 0.5f * t * q * n.e;
+    n.cdf = x < 0.0f ? half_erfc : 1.0f - half_erfc;
+    return n;
+}
+// The forward needs the distribution function alone: the same t, with erfc(z) = t*exp(-z^2 + P(t)) (Chebyshev fit of
+// Numerical Recipes 6.2, relative error below 1.2e-7 for every z): one multiplication and one fused multiply-add
+// fewer than the product form above.
 __device__ __forceinline__ float normal_cdf(float x) {
     const float z = __builtin_fabsf(x) * 0.70710678118654752440f;
     const float t = rcp_fast(__builtin_fmaf(0.5f, z, 1.0f));
@@ -108,8 +134,9 @@ __device__ __forceinline__ C act_fwd(C x, C p0, C p1) {
 template <int ACT, typename C>
 __device__ __forceinline__ C act_bwd(C s, C g, C p0, C p1) {
     if constexpr (ACT == kGelu) {
-        const float pdf = __expf(-0.5f * s * s) * 0.39894228040143267794f;                 // gelu.py:77-80
-        return g * __builtin_fmaf(s, pdf, normal_cdf(s));
+        const NormalParts n = normal_parts(s);                                             // gelu.py:77-80
+        const float pdf = n.e * 0.39894228040143267794f;
+        return g * __builtin_fmaf(s, pdf, n.cdf);
     } else if constexpr (ACT == kGeluTanh) {
         const float k = 0.79788456080286535588f;                                           // gelu.py:71-75
         const float t = tanh_safe(k * (s + 0.044715f * s * s * s));
