@@ -125,7 +125,10 @@ __device__ __forceinline__ C act_fwd(C x, C p0, C p1) {
         return x * mish_parts(x).t;                                                        // mish.py:19-23
     } else if constexpr (ACT == kSoftplus) {
         if constexpr (std::is_same<C, float>::value) {                                     // softplus.py:21
-            return x * p0 > p1 ? x : __logf(1.0f + __expf(p0 * x)) * rcp_fast(p0);
+            // base-2 hardware exponential and logarithm; the factors log2(e)*beta and ln(2)/beta are the same for every
+            // element (two multiplications fewer per element than exp and log of base e)
+            const float k = p0 * 1.44269504088896341f, inv = 0.69314718055994531f * rcp_fast(p0);
+            return x * p0 > p1 ? x : __builtin_amdgcn_logf(1.0f + __builtin_amdgcn_exp2f(k * x)) * inv;
         } else {
             return x * p0 > p1 ? x : log_c(C(1) + exp_c(p0 * x)) / p0;
         }
@@ -167,7 +170,8 @@ __device__ __forceinline__ C act_bwd(C s, C g, C p0, C p1) {
         return g * (m.t + s * m.one_minus_t2 * m.sig);
     } else if constexpr (ACT == kSoftplus) {
         if constexpr (std::is_same<C, float>::value) {                                     // softplus.py:62
-            return s * p0 > p1 ? g : g * rcp_fast(1.0f + __expf(-p0 * s));
+            const float k = p0 * -1.44269504088896341f;
+            return s * p0 > p1 ? g : g * rcp_fast(1.0f + __builtin_amdgcn_exp2f(k * s));
         } else {
             return s * p0 > p1 ? g : g / (C(1) + exp_c(-p0 * s));
         }
