@@ -33,6 +33,19 @@ __device__ __forceinline__ float tanh_safe(float u) {
 
 __device__ __forceinline__ float sigmoid_f(float x) { return rcp_fast(1.0f + __expf(-x)); }
 
+// The gate of the tanh form of GeLU: 0.5*(1 + tanh(u)) with u = sqrt(2/pi)*(x + 0.044715 x^3) (gelu.py:23-26) is the
+// logistic function of 2u, 1/(1 + exp(-2u)).  One exponential and one reciprocal, no cancellation for negative x
+// (where 1 + tanh(u) loses every digit), no overflow: exp(-2u) = inf gives 0, exp(-2u) = 0 gives 1.
+struct GateParts { float gate, e; };            // e = exp(-2u), gate = 1/(1 + e)
+__device__ __forceinline__ GateParts gelu_tanh_gate_parts(float x) {
+    const float inner = __builtin_fmaf(0.044715f * x * x, x, x);
+    GateParts p;
+    p.e = __builtin_amdgcn_exp2f(-2.302208198144325f * inner);                     // -2*sqrt(2/pi)*log2(e)
+    p.gate = rcp_fast(1.0f + p.e);
+    return p;
+}
+__device__ __forceinline__ float gelu_tanh_gate(float x) { return gelu_tanh_gate_parts(x).gate; }
+
 // Phi(x) = 0.5*(1 + erf(x/sqrt 2)), the normal distribution function of GeLU, from the complementary error function
 // of z = |x|/sqrt 2, in two forms that share t = 1/(1 + z/2) in (0, 1].  Both are branch free, accurate in the
 // negative tail (where 1 + erf(..) cancels) and a third of the instructions of the library erff.  Their
@@ -106,8 +119,7 @@ __device__ __forceinline__ C act_fwd(C x, C p0, C p1) {
     if constexpr (ACT == kGelu) {
         return x * normal_cdf(x);                                                          // gelu.py:28
     } else if constexpr (ACT == kGeluTanh) {
-        const float u = 0.79788456080286535588f * (x + 0.044715f * x * x * x);            // gelu.py:23
-        return 0.5f * x * (1.0f + tanh_safe(u));                                           // gelu.py:26
+        return x * gelu_tanh_gate(x);                                                      // gelu.py:23-26
     } else if constexpr (ACT == kSilu) {
         return x * sigmoid_f(x);                                                           // silu.py:19
     } else if constexpr (ACT == kRelu) {
@@ -145,12 +157,14 @@ __device__ __forceinline__ C act_bwd(C s, C g, C p0, C p1) {
         const float pdf = n.e * 0.39894228040143267794f;
         return g * __builtin_fmaf(s, pdf, n.cdf);
     } else if constexpr (ACT == kGeluTanh) {
-        const float k = 0.79788456080286535588f;                                           // gelu.py:71-75
-        const float t = tanh_safe(k * (s + 0.044715f * s * s * s));
-        const float gp = k * (1.0f + 3.0f * 0.044715f * s * s);
-        const float sech2 = 1.0f - t * t;                          // exactly 0 once |s| > ~6: keeps 0 * inf out for huge |s|
-        const float tail = sech2 == 0.0f ? 0.0f : s * sech2 * gp;
-        return g * (0.5f * (1.0f + t + tail));
+        // gelu.py:71-75 with t = tanh(u) = 2*gate - 1: 0.5*(1 + t) = gate, 0.5*(1 - t^2) = 2*gate*(1 - gate)
+        const GateParts p = gelu_tanh_gate_parts(s);
+        const float gate = p.gate;
+        // 1 - gate = e*gate: taken from whichever side does not cancel (e = inf goes with gate = 0 < 0.5)
+        const float slope = gate * (gate < 0.5f ? 1.0f - gate : p.e * gate);   // gate*(1 - gate) = sech^2(u)/4
+        const float du2 = __builtin_fmaf(3.0f * 0.044715f * 1.59576912160573071f, s * s, 1.59576912160573071f);   // 2*u'
+        const float tail = slope == 0.0f ? 0.0f : s * slope * du2;             // exactly 0 once |s| > ~6: no 0 * inf
+        return g * (gate + tail);
     } else if constexpr (ACT == kSilu) {
         const float sg = sigmoid_f(s);                                                     // silu.py:56-57
         return g * (sg * (1.0f + s * (1.0f - sg)));
