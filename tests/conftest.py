@@ -1,4 +1,4 @@
-"""Shared fixtures: import paths, the `gpu` marker, the BASELINE input generators and the tolerance checks."""
+"""Shared fixtures: import paths, the `gpu` marker, the benchmark input generators and the tolerance checks."""
 import os
 import sys
 
@@ -17,7 +17,7 @@ def pytest_configure(config):
 
 
 # ---------------------------------------------------------------------------------------------------------
-# The five BASELINE configurations.  `rows` lets a test shrink M while keeping N and the data recipe.
+# The five benchmark configurations.  `rows` lets a test shrink M while keeping N and the data recipe.
 # Inputs are generated on the CPU in float32 with a seeded generator, then cast (so the GPU path and the
 # oracle see bit-identical storage values).
 # ---------------------------------------------------------------------------------------------------------

@@ -454,6 +454,25 @@ int plan_launch(int which, int flavour, bool aligned, int64_t M, int64_t N, int 
 
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
+// Whether a norm launch may shift its vector slots onto 128-byte lines (row_line_shift() in thn_kernels.h): rows
+// that start off a line boundary, one row per workgroup at a time, every row a workgroup visits and every stream
+// in the same phase of a line, and room for the up to 7 slots the shift pushes off the left end of the row.
+struct RowStream {
+    const void* base;
+    int64_t stride_bytes;
+};
+bool line_shift_ok(bool aligned, const Shape& s, int grid, int n_vecs, const RowStream* streams, int n_streams) {
+    if (!aligned || s.block != s.tpr || s.k * s.tpr - 7 < n_vecs) return false;
+    const int64_t stride = streams[0].stride_bytes;
+    if (stride % 128 == 0 || (static_cast<int64_t>(grid) * stride) % 128 != 0) return false;
+    const uintptr_t phase = reinterpret_cast<uintptr_t>(streams[0].base) & 127u;
+    for (int i = 1; i < n_streams; ++i) {
+        if ((reinterpret_cast<uintptr_t>(streams[i].base) & 127u) != phase) return false;
+        if ((streams[i].stride_bytes - stride) % 128 != 0) return false;
+    }
+    return true;
+}
+
 int64_t partial_pitch(int64_t N) { return (N + 63) / 64 * 64; }
 
 
@@ -521,6 +540,8 @@ int norm_forward(const void* x, int64_t x_row_stride, void* y, int64_t y_row_str
     a.w_dtype = w_dtype;
     a.eps = eps;
     a.inv_n = 1.0f / static_cast<float>(N);
+    const RowStream streams[2] = {{x, a.x_stride_bytes}, {y, a.y_stride_bytes}};
+    a.line_shift = line_shift_ok(aligned, p.s, p.grid, p.n_vecs, streams, 2) ? 1 : 0;
     hipStream_t st = static_cast<hipStream_t>(stream);
     const int lrc = fused ? launch_fused_fwd(x_dtype, (ln ? 1 : 0) | (act << 1), aligned, p.s, a, p.grid, st, nullptr)
                           : launch_fwd(x_dtype, ln, aligned, p.s, a, p.grid, st, nullptr);
@@ -581,6 +602,8 @@ int norm_backward_stage1(const void* x, int64_t x_row_stride, const void* dy, in
     a.n_vecs = p.n_vecs;
     a.w_dtype = w_dtype;
     a.inv_n = 1.0f / static_cast<float>(N);
+    const RowStream streams[3] = {{x, a.x_stride_bytes}, {dy, a.dy_stride_bytes}, {dx, a.dx_stride_bytes}};
+    a.line_shift = line_shift_ok(aligned, p.s, p.grid, p.n_vecs, streams, 3) ? 1 : 0;
     hipStream_t st = static_cast<hipStream_t>(stream);
     const int lrc = fused ? launch_fused_bwd(x_dtype, variant, aligned, p.s, a, p.grid, st, nullptr)
                           : launch_bwd(x_dtype, ln, aligned, p.s, a, p.grid, st, nullptr);

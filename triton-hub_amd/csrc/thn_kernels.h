@@ -42,6 +42,7 @@ struct FwdArgs {
     int w_dtype;
     float eps;
     float inv_n;
+    int line_shift;     // 1: rows are not 128 bytes apart and the launch may use row_line_shift()
 };
 
 struct BwdArgs {
@@ -63,7 +64,19 @@ struct BwdArgs {
     int n_vecs;
     int w_dtype;
     float inv_n;
+    int line_shift;     // as in FwdArgs
 };
+
+// Rows that are a multiple of 16 but not of 128 bytes apart start in the middle of a 128-byte line, and a wave's
+// 1 KiB request then touches nine lines instead of eight (float32 8192 x 6000: 9 % of the kernel).  Where the
+// host has checked that it may -- one row per workgroup at a time, the same phase for every row the workgroup
+// visits and for every stream, K*TPR - 7 >= n_vecs -- the threads take the vectors `shift` places further left
+// (thread t owns vectors t - shift + k*TPR), which puts every request of a wave on line boundaries; the slots that
+// fall off the left end are clamped onto vector 0 like those off the right end onto the last one.
+__device__ __forceinline__ int row_line_shift(int enabled, const char* base, int64_t stride_bytes, int64_t first_row) {
+    if (!enabled) return 0;
+    return static_cast<int>(((reinterpret_cast<uintptr_t>(base) + static_cast<uint64_t>(first_row * stride_bytes)) & 127u) >> 4);
+}
 
 // Loads the K vectors of one row.  `row` is already clamped to a valid row; voff[k] is the byte offset of
 // the (clamped) vector slot k on the aligned 128-bit path and the vector index on the unaligned path.
@@ -158,14 +171,15 @@ __global__ void __launch_bounds__(BLOCK) norm_fwd_kernel(const FwdArgs a) {
     int phase = 0;
 
     // Per-slot masks (1 = this thread owns real columns there) and clamped offsets.
+    const int shift = (ALIGNED && G == 1) ? row_line_shift(a.line_shift, a.x, a.x_stride_bytes, blockIdx.x) : 0;
     int voff[K];
     bool own[K];
 #pragma unroll
     for (int k = 0; k < K; ++k) {
-        const int v = t + k * TPR;
-        const int vc = v < a.n_vecs ? v : a.n_vecs - 1;
+        const int v = t + k * TPR - shift;
+        const int vc = v < 0 ? 0 : (v < a.n_vecs ? v : a.n_vecs - 1);
         voff[k] = ALIGNED ? vc * 16 : vc;
-        own[k] = v < a.n_vecs;
+        own[k] = v >= 0 && v < a.n_vecs;
     }
 
     const int64_t rows_per_iter = static_cast<int64_t>(gridDim.x) * G;
@@ -432,14 +446,15 @@ __global__ void __launch_bounds__(BLOCK) norm_bwd_kernel(const BwdArgs a) {
     const int t = tid % TPR;
     int phase = 0;
 
+    const int shift = (ALIGNED && G == 1) ? row_line_shift(a.line_shift, a.x, a.x_stride_bytes, blockIdx.x) : 0;
     int voff[K];
     bool own[K];
 #pragma unroll
     for (int k = 0; k < K; ++k) {
-        const int v = t + k * TPR;
-        const int vc = v < a.n_vecs ? v : a.n_vecs - 1;
+        const int v = t + k * TPR - shift;
+        const int vc = v < 0 ? 0 : (v < a.n_vecs ? v : a.n_vecs - 1);
         voff[k] = ALIGNED ? vc * 16 : vc;
-        own[k] = v < a.n_vecs;
+        own[k] = v >= 0 && v < a.n_vecs;
     }
 
     const int64_t rows_per_iter = static_cast<int64_t>(gridDim.x) * G;
@@ -767,8 +782,8 @@ __global__ void __launch_bounds__(BLOCK) norm_bwd_kernel(const BwdArgs a) {
                 if (want_db) combine_groups<BLOCK, TPR, VEC, Acc>(db[k], comb, g, t);
             }
         }
-        const int v = t + k * TPR;
-        if (g == 0 && v < a.n_vecs) {
+        const int v = t + k * TPR - shift;
+        if (g == 0 && own[k]) {
             // part_pitch is a multiple of 64 floats >= n_vecs*VEC, so whole vectors always fit.
             const int64_t off = static_cast<int64_t>(blockIdx.x) * a.part_pitch + static_cast<int64_t>(v) * VEC;
             float pw[VEC], pb[VEC];
