@@ -90,8 +90,8 @@ SOFTMAX_KINDS = ("softmax", "softmin", "logsoftmax")
 # (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch), each scaled by what the same counter reads for a plain
 # copy kernel of known size.  Filled in from the summaries under profiles/; null for workloads not profiled.
 MEASURED_TRAFFIC_BYTES = {
-    # profiles/norm_kernels_rmsnorm_bf16_16384x4096_hbm_counters.txt: 262966 KiB fetched + 135168 KiB written
-    "rmsnorm_bf16_16384x4096": 407689533,
+    # profiles/norm_kernels_rmsnorm_bf16_16384x4096_hbm_counters.txt: 262941 KiB fetched + 135216 KiB written
+    "rmsnorm_bf16_16384x4096": 407712134,
     # profiles/softmax_kernels_softmax_bf16_16384x4096_stats_and_hbm_counters.txt (softmax_bwd_kernel)
     "softmax_bf16_16384x4096": 402815465,
     # profiles/pnorm_kernels_normalize_p2_bf16_16384x4096_stats_and_hbm_counters.txt (normalize_bwd_kernel)
