@@ -18,8 +18,8 @@ CASES = [
     ("rms", torch.float32, 523, 4100),
     ("ln", torch.float32, 300, 6116),      # 1529 vectors = 3 * 512 - 7: the widest row with room for the shift
     ("ln", torch.float32, 300, 6124),      # 1531 vectors: no room, unshifted
-    ("ln", torch.float16, 520, 6000),      # forward shifted (one row per workgroup), backward not (two rows)
-    ("rms", torch.bfloat16, 600, 4104),    # pitch 8208 = 16 mod 128
+    ("ln", torch.float16, 520, 6000),      # 256-thread rows: the backward takes one-row workgroups to shift too
+    ("rms", torch.bfloat16, 600, 4104),    # pitch 8208 = 16 mod 128, 256-thread rows
     ("ln", torch.bfloat16, 600, 4104),
     ("ln", torch.float32, 100, 6000),      # one workgroup per row, 100 * pitch is a multiple of 128
     ("ln", torch.float32, 101, 6000),      # 101 * pitch is not: unshifted
