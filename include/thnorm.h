@@ -59,6 +59,10 @@ const char* thn_strerror(int status);
  *   RMSNorm:   rstd = 1/sqrt(sum(x^2)/N + eps),                         y = x*rstd*w        (b must be NULL)
  * w and b may each be NULL (HAS_WEIGHT / HAS_BIAS false in the reference); both use storage `w_dtype`.
  * x and y use storage `x_dtype`.  mean, rstd: (M,) float32.  M == 0 is a no-op.
+ * A row's results depend on that row alone and are run-to-run identical.  They do not depend on where the row
+ * sits in the tensor when rows are a multiple of 128 bytes apart; at other pitches the order of the row sums
+ * (hence the last bit of the results) can depend on the offset of the row's first byte within a 128-byte line,
+ * and on nothing else.  The same holds for thn_norm_bwd.
  */
 int thn_norm_fwd(const void* x, int64_t x_row_stride,
                  void* y, int64_t y_row_stride,
