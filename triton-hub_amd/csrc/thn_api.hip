@@ -95,6 +95,9 @@ bool shape_compiled(int which, bool aligned, bool ln16, Shape s) {
         THN_ROW_SHAPES(THN_MATCH)
     } else {
         THN_FWD_SHAPES(THN_MATCH)
+        if (which == kNormFwd) {
+            THN_FWD_SHAPES_TWO_ROWS(THN_MATCH)
+        }
     }
 #undef THN_MATCH
     return false;
@@ -358,6 +361,7 @@ Shape heuristic_shape(int which, bool aligned, bool ln16, int n_vecs) {
     if (s.k == 3 && s.tpr < 64) s.k = 4;     // K = 3 is only compiled for TPR >= 64
     if (which != kNormBwd && which != kFusedBwd) s.block = s.tpr > 256 ? s.tpr : 256;
     else s.block = s.tpr >= 128 ? (s.tpr > 512 ? s.tpr : 512) : 256;
+    if (which == kNormFwd && s.k == 3 && s.tpr == 256) s.block = 512;     // THN_FWD_SHAPES_TWO_ROWS
     return s;
 }
 
@@ -396,7 +400,7 @@ int narrow_row_blocks_per_cu(int which, int n_vecs, bool ragged16) {
     return 1;
 }
 
-// `pitch_bytes`: distance between rows of x when the caller knows it (0 otherwise); only the norm backward uses it.
+// `pitch_bytes`: distance between rows of x when the caller knows it (0 otherwise); only the norm kernels use it.
 int plan_launch(int which, int flavour, bool aligned, int64_t M, int64_t N, int dtype, Plan* out,
                 int64_t pitch_bytes = 0) {
     const int bytes = elem_bytes(dtype);
@@ -411,10 +415,11 @@ int plan_launch(int which, int flavour, bool aligned, int64_t M, int64_t N, int 
     // (rows shorter than one vector have a single element-wise instance)
     const bool ln16 = (which == kNormBwd || which == kFusedBwd) && bytes == 2 && (flavour & 1) != 0 && N >= vec_elems;
     Shape s = heuristic_shape(which, aligned, ln16, n_vecs);
-    // Rows that start off 128-byte lines: the backward's two-row workgroups of 256-thread rows cannot put their
-    // requests on line boundaries (the two rows differ in phase, line_shift_ok() below), one-row workgroups can and
-    // are as fast otherwise (fp16 8192 x 6000: 54.8 -> 53.1 us; 8192 x 6016: 52.6 / 52.4 us).
-    if ((which == kNormBwd || which == kFusedBwd) && aligned && pitch_bytes % 128 != 0 && s.tpr >= 256 &&
+    // Rows that start off 128-byte lines: two-row workgroups of 256-thread rows cannot put their requests on line
+    // boundaries (the two rows differ in phase, line_shift_ok() below), one-row workgroups can.  Backward: as fast
+    // otherwise (fp16 8192 x 6000: 54.8 -> 53.1 us; 8192 x 6016: 52.6 / 52.4 us).  Forward (THN_FWD_SHAPES_TWO_ROWS):
+    // float32 16384 x 3000 69.5 -> 67.2 us, 65536 x 3000 290 -> 280 us, bf16 16384 x 6008 71.0 -> 69.1 us.
+    if ((which == kNormBwd || which == kFusedBwd || which == kNormFwd) && aligned && pitch_bytes % 128 != 0 && s.tpr >= 256 &&
         s.block == 2 * s.tpr && s.k * s.tpr - 7 >= n_vecs) {
         Shape one_row = s;
         one_row.block = s.tpr;
@@ -533,7 +538,7 @@ int norm_forward(const void* x, int64_t x_row_stride, void* y, int64_t y_row_str
     Plan p;
     const bool fused = act != thn::kNoAct;
     const int rc = plan_launch(fused ? kFusedFwd : kNormFwd, fused ? ((ln ? 1 : 0) | (act << 1)) : (ln ? 1 : 0), aligned, M, N,
-                               x_dtype, &p);
+                               x_dtype, &p, x_row_stride * bytes);
     if (rc != THN_OK) return rc;
 
     FwdArgs a{};
