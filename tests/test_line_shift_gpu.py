@@ -3,11 +3,12 @@ vector slots so that every wave request starts on a 128-byte line (up to 7 slots
 row's first byte), where one row per workgroup, equal phases of all streams and spare slots allow it.  The cases
 walk every phase (pitches of 16 mod 128 bytes), the two-phase pitch of 6000 columns, the last width that still
 has the spare slots and the first that has not, and row counts whose grid does or does not keep a workgroup on
-one phase.  Same oracle and tolerances as the other norm parity tests."""
+one phase.  The softmax family's row kernels do the same.  Same oracles and tolerances as the other parity tests."""
 import pytest
 import torch
 
 import parity_util
+import test_softmax_parity_gpu as softmax_t
 
 pytestmark = pytest.mark.gpu
 
@@ -36,3 +37,22 @@ def test_rows_off_line_boundaries(kind, dtype, m, n):
     w = (1 + 0.1 * torch.randn(n, generator=g)).to(dtype)
     b = (0.1 * torch.randn(n, generator=g)).to(dtype) if kind == "ln" else None
     parity_util.run_and_compare(kind, x, dy, w, b, 1e-5, f"line shift {kind} {m}x{n}")
+
+
+SOFTMAX_CASES = [
+    ("softmax", torch.float32, 523, 4100),       # 1025 vectors on 512 threads, all eight phases
+    ("logsoftmax", torch.float32, 300, 6000),    # phases 0 / 64
+    ("softmin", torch.bfloat16, 600, 4104),      # 513 vectors on 256 threads
+    ("softmax", torch.float16, 520, 6000),
+    ("logsoftmax", torch.float32, 300, 8180),    # 2045 vectors: 4 x 512 - 7 = 2041 < 2045, unshifted
+    ("softmax", torch.float32, 101, 6000),       # 101 * pitch is not a multiple of 128: unshifted
+]
+
+
+@pytest.mark.parametrize("kind,dtype,m,n", SOFTMAX_CASES)
+def test_softmax_rows_off_line_boundaries(kind, dtype, m, n):
+    print(f"\n[case] line shift {kind} {dtype} M={m} N={n}", flush=True)
+    g = torch.Generator().manual_seed(m * 7919 + n)
+    x = (torch.randn(m, n, generator=g) * 3).to(dtype)
+    dy = torch.randn(m, n, generator=g).to(dtype)
+    softmax_t.run_and_compare(kind, x, dy, f"line shift {kind} {m}x{n}")

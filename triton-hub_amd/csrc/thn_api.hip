@@ -1039,6 +1039,8 @@ int thn_softmax_fwd(const void* x, int64_t x_row_stride, void* y, int64_t y_row_
     a.n_cols = static_cast<int>(N);
     a.n_vecs = p.n_vecs;
     a.sign = kind == THN_SOFTMIN ? -1.0f : 1.0f;
+    const RowStream streams[2] = {{x, a.x_stride_bytes}, {y, a.y_stride_bytes}};
+    a.line_shift = line_shift_ok(aligned, p.s, p.grid, p.n_vecs, streams, 2) ? 1 : 0;
     const int lrc = launch_softmax_fwd(dtype, is_log, aligned, p.s, a, p.grid, static_cast<hipStream_t>(stream), nullptr);
     if (lrc > 0) return THN_E_SHAPE;
     return lrc == 0 ? THN_OK : THN_E_LAUNCH;
@@ -1092,6 +1094,8 @@ int thn_softmax_bwd(const void* y, int64_t y_row_stride, const void* dy, int64_t
     a.n_cols = static_cast<int>(N);
     a.n_vecs = p.n_vecs;
     a.sign = kind == THN_SOFTMIN ? -1.0f : 1.0f;
+    const RowStream streams[3] = {{y, a.y_stride_bytes}, {dy, a.dy_stride_bytes}, {dx, a.dx_stride_bytes}};
+    a.line_shift = line_shift_ok(aligned, p.s, p.grid, p.n_vecs, streams, 3) ? 1 : 0;
     const int lrc = launch_softmax_bwd(dtype, is_log, aligned, p.s, a, p.grid, static_cast<hipStream_t>(stream), nullptr);
     if (lrc > 0) return THN_E_SHAPE;
     return lrc == 0 ? THN_OK : THN_E_LAUNCH;

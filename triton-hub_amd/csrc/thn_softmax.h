@@ -19,6 +19,7 @@ struct SoftmaxFwdArgs {
     int n_cols;
     int n_vecs;
     float sign;      // -1: the input is negated on load (Softmin of x = Softmax of -x)
+    int line_shift;  // as in FwdArgs (row kernels only)
 };
 
 struct SoftmaxBwdArgs {
@@ -32,6 +33,7 @@ struct SoftmaxBwdArgs {
     int n_cols;
     int n_vecs;
     float sign;      // -1: the gradient is negated on store (fused Softmin)
+    int line_shift;  // as in FwdArgs (row kernels only)
 };
 
 // Arithmetic type.  Float32 for 16- and 32-bit storage and for every log-softmax (logsoftmax.py:19, :61-62 widen
@@ -97,14 +99,15 @@ __global__ void __launch_bounds__(BLOCK) softmax_fwd_kernel(const SoftmaxFwdArgs
     const int t = tid % TPR;
     int phase = 0;
 
+    const int shift = (ALIGNED && G == 1) ? row_line_shift(a.line_shift, a.x, a.x_stride_bytes, blockIdx.x) : 0;
     int voff[K];
     bool own[K];
 #pragma unroll
     for (int k = 0; k < K; ++k) {
-        const int v = t + k * TPR;
-        const int vc = v < a.n_vecs ? v : a.n_vecs - 1;
+        const int v = t + k * TPR - shift;
+        const int vc = v < 0 ? 0 : (v < a.n_vecs ? v : a.n_vecs - 1);
         voff[k] = ALIGNED ? vc * 16 : vc;
-        own[k] = v < a.n_vecs;
+        own[k] = v >= 0 && v < a.n_vecs;
     }
     const C sign = static_cast<C>(a.sign);
     const C neg_inf = OpMax::identity<C>();
@@ -188,14 +191,15 @@ __global__ void __launch_bounds__(BLOCK) softmax_bwd_kernel(const SoftmaxBwdArgs
     const int t = tid % TPR;
     int phase = 0;
 
+    const int shift = (ALIGNED && G == 1) ? row_line_shift(a.line_shift, a.y, a.y_stride_bytes, blockIdx.x) : 0;
     int voff[K];
     bool own[K];
 #pragma unroll
     for (int k = 0; k < K; ++k) {
-        const int v = t + k * TPR;
-        const int vc = v < a.n_vecs ? v : a.n_vecs - 1;
+        const int v = t + k * TPR - shift;
+        const int vc = v < 0 ? 0 : (v < a.n_vecs ? v : a.n_vecs - 1);
         voff[k] = ALIGNED ? vc * 16 : vc;
-        own[k] = v < a.n_vecs;
+        own[k] = v >= 0 && v < a.n_vecs;
     }
 
     const int64_t rows_per_iter = static_cast<int64_t>(gridDim.x) * G;
