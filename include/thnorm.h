@@ -143,6 +143,7 @@ int thn_norm_bwd_reduce_partials(const void* workspace, int32_t num_partials,
  * its log-softmax kernels widen to float32 (logsoftmax.py:19, :61-62).  There is no row-width limit: a row wider
  * than 64 KiB is one softmax of the whole row, computed by kernels that walk the row twice (the reference splits
  * such a row into 64 KiB chunks and normalises each chunk by itself, softmax.py:34-40).  N must fit in 31 bits.
+ * What a row's results can depend on is as stated for thn_norm_fwd.
  */
 enum thn_softmax_kind { THN_SOFTMAX = 0, THN_SOFTMIN = 1, THN_LOGSOFTMAX = 2 };
 
