@@ -40,7 +40,7 @@ enum thn_status {
     THN_E_FEATURE_DIM = -2,   /* a row is wider than 64 KiB (the reference's RuntimeError, layernorm.py:71-72) */
     THN_E_NULL = -3,          /* a required pointer is NULL */
     THN_E_SHAPE = -4,         /* M < 0, N <= 0 or a row stride smaller than N */
-    THN_E_WORKSPACE = -5,     /* workspace smaller than thn_norm_bwd_workspace_bytes() asks for */
+    THN_E_WORKSPACE = -5,     /* workspace smaller than thn_norm_bwd_workspace_bytes() asks for, or not 16-byte aligned */
     THN_E_LAUNCH = -6,        /* the HIP runtime refused the launch (hipGetLastError) */
     THN_E_DEVICE = -7         /* no usable current device */
 };
@@ -91,7 +91,8 @@ int64_t thn_norm_bwd_workspace_bytes(int64_t M, int64_t N, int want_dw, int want
  *   c1 = sum(xhat*wdy)/N; c2 = sum(wdy)/N (0 for RMSNorm); dx = (wdy - (xhat*c1 + c2))*rstd;
  *   dW = sum over rows of dy*xhat; dB = sum over rows of dy.
  * dw / db (storage `w_dtype`, (N,)) may each be NULL when that gradient is not wanted; `workspace` may be
- * NULL only when both are.  The two-stage sum has a fixed order: results are run-to-run identical.
+ * NULL only when both are and must be 16-byte aligned otherwise (the partial rows are written 16 bytes at a
+ * time).  The two-stage sum has a fixed order: results are run-to-run identical.
  */
 int thn_norm_bwd(const void* x, int64_t x_row_stride,
                  const void* dy, int64_t dy_row_stride,
