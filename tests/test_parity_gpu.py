@@ -423,6 +423,10 @@ def test_c_abi_direct_calls_and_errors():
     assert lib.thn_norm_bwd(x.data_ptr(), pitch, dy.data_ptr(), pitch, dx.data_ptr(), pitch, w.data_ptr(),
                             mean.data_ptr(), rstd.data_ptr(), dw.data_ptr(), dbias.data_ptr(), ws.data_ptr(), 64,
                             m, n, _native.F32, _native.F32, st) == _native.E_WORKSPACE
+    # a workspace that is not 16-byte aligned is refused before anything is launched
+    assert lib.thn_norm_bwd(x.data_ptr(), pitch, dy.data_ptr(), pitch, dx.data_ptr(), pitch, w.data_ptr(),
+                            mean.data_ptr(), rstd.data_ptr(), dw.data_ptr(), dbias.data_ptr(), ws.data_ptr() + 4,
+                            nbytes - 4, m, n, _native.F32, _native.F32, st) == _native.E_WORKSPACE
     assert lib.thn_norm_bwd(x.data_ptr(), pitch, 0, pitch, dx.data_ptr(), pitch, w.data_ptr(), mean.data_ptr(),
                             rstd.data_ptr(), dw.data_ptr(), dbias.data_ptr(), ws.data_ptr(), nbytes, m, n,
                             _native.F32, _native.F32, st) == _native.E_NULL
