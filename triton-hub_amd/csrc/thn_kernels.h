@@ -78,23 +78,24 @@ __device__ __forceinline__ int row_line_shift(int enabled, const char* base, int
     return static_cast<int>(((reinterpret_cast<uintptr_t>(base) + static_cast<uint64_t>(first_row * stride_bytes)) & 127u) >> 4);
 }
 
-// Loads the K vectors of one row.  `row` is already clamped to a valid row; voff[k] is the byte offset of
+// Loads the K vectors of one row (KEEP: with cache-allocating loads, see ld128_keep).  `row` is already clamped
+// to a valid row; voff[k] is the byte offset of
 // the (clamped) vector slot k on the aligned 128-bit path and the vector index on the unaligned path.
-template <typename T, int K, bool ALIGNED>
+template <typename T, int K, bool ALIGNED, bool KEEP = false>
 __device__ __forceinline__ void load_row(u32x4 (&dst)[K], const char* base, int64_t stride_bytes, int64_t row,
                                          const int (&voff)[K], int n_cols) {
     const char* p = base + row * stride_bytes;
 #pragma unroll
     for (int k = 0; k < K; ++k) {
-        if constexpr (ALIGNED) dst[k] = ld128(p + voff[k]);
-        else dst[k] = load_vec_elems<T>(p, voff[k], n_cols);
+        if constexpr (ALIGNED) dst[k] = KEEP ? ld128_keep(p + voff[k]) : ld128(p + voff[k]);
+        else dst[k] = load_vec_elems<T, KEEP>(p, voff[k], n_cols);
     }
 }
 
-template <typename T, bool ALIGNED>
+template <typename T, bool ALIGNED, bool KEEP = false>
 __device__ __forceinline__ u32x4 load_row_vec(const char* rowp, int voff, int n_cols) {
-    if constexpr (ALIGNED) return ld128(rowp + voff);
-    else return load_vec_elems<T>(rowp, voff, n_cols);
+    if constexpr (ALIGNED) return KEEP ? ld128_keep(rowp + voff) : ld128(rowp + voff);
+    else return load_vec_elems<T, KEEP>(rowp, voff, n_cols);
 }
 
 // Workgroups of 1024 threads serve the widest rows (more than 24 KiB of x in the backward, 32 KiB in the
@@ -162,6 +163,7 @@ template <typename T, bool LN, int K, int TPR, int BLOCK, bool ALIGNED, int ACT 
 __global__ void __launch_bounds__(BLOCK) norm_fwd_kernel(const FwdArgs a) {
     constexpr int VEC = T::VEC;
     constexpr int G = BLOCK / TPR;
+    constexpr bool kKeepX = THN_FWD_X_KEEP != 0;     // x is read again (by the backward): see ld128_keep
     static_assert(BLOCK % TPR == 0 && G >= 1, "a workgroup holds whole rows");
     __shared__ float red[RedSmem<TPR, G, 2>::kFloats];
 
@@ -187,7 +189,7 @@ __global__ void __launch_bounds__(BLOCK) norm_fwd_kernel(const FwdArgs a) {
     int64_t row_raw = static_cast<int64_t>(blockIdx.x) * G + g;
     int64_t row = row_raw < a.M ? row_raw : last_row;
     u32x4 cur[K];
-    load_row<T, K, ALIGNED>(cur, a.x, a.x_stride_bytes, row, voff, a.n_cols);   // first, so it overlaps the params
+    load_row<T, K, ALIGNED, kKeepX>(cur, a.x, a.x_stride_bytes, row, voff, a.n_cols);   // first, so it overlaps the params
 
     // Parameters of the clamped slot, so that a clamped slot reproduces its owner's output bit for bit.
     float wr[K][VEC];
@@ -205,7 +207,7 @@ __global__ void __launch_bounds__(BLOCK) norm_fwd_kernel(const FwdArgs a) {
             u32x4 nxt[kForm.ahead ? K : 1];
             if constexpr (kForm.ahead) {
 #pragma unroll
-                for (int k = 0; k < K; ++k) nxt[k] = load_row_vec<T, ALIGNED>(nxrow, voff[k], a.n_cols);
+                for (int k = 0; k < K; ++k) nxt[k] = load_row_vec<T, ALIGNED, kKeepX>(nxrow, voff[k], a.n_cols);
             }
             float mean0 = 0.0f, mean = 0.0f, rstd, delta = 0.0f;
             if constexpr (LN) {
@@ -277,7 +279,7 @@ __global__ void __launch_bounds__(BLOCK) norm_fwd_kernel(const FwdArgs a) {
                 }
                 store_row_vec<T, ALIGNED>(yrow, voff[k], a.n_cols, yf);
                 if constexpr (kForm.ahead) cur[k] = nxt[k];
-                else cur[k] = load_row_vec<T, ALIGNED>(nxrow, voff[k], a.n_cols);
+                else cur[k] = load_row_vec<T, ALIGNED, kKeepX>(nxrow, voff[k], a.n_cols);
             }
             if constexpr (LN) a.mean[row] = mean;
             a.rstd[row] = rstd;
@@ -290,7 +292,7 @@ __global__ void __launch_bounds__(BLOCK) norm_fwd_kernel(const FwdArgs a) {
         const int64_t nrow_raw = row_raw + rows_per_iter;
         const int64_t nrow = nrow_raw < a.M ? nrow_raw : last_row;
         u32x4 nxt[K];
-        load_row<T, K, ALIGNED>(nxt, a.x, a.x_stride_bytes, nrow, voff, a.n_cols);
+        load_row<T, K, ALIGNED, kKeepX>(nxt, a.x, a.x_stride_bytes, nrow, voff, a.n_cols);
 
         float xf[K][VEC];
 #pragma unroll
