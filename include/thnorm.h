@@ -18,8 +18,15 @@
  *     (a float64 tensor is narrowed on load and widened on store, as the reference does with
  *     `.to(tl.float32)`, layernorm.py:31).  Results are rounded to nearest even on store.
  *   - Return value: THN_OK (0) or a negative THN_E_* code; thn_strerror() names it.  Nothing throws.
- *   - Thread safe.  The only process state is a per-device cache of the compute-unit count and of kernel
- *     occupancies, filled on first use.
+ *   - Outputs must not overlap inputs (nor each other), except where an entry point says that it works in place
+ *     (thn_dropout).  The row kernels keep their loops free of branches by letting a lane without work
+ *     re-load, recompute and re-store the last row or the last vector of its row; with y == x or dx == dy such a
+ *     lane can read a row that another workgroup has already overwritten and store it transformed twice.  (The
+ *     reference's Triton kernels load a whole row before they store it and tolerate in-place use; callers that
+ *     relied on that must pass a separate output here.)
+ *   - Thread safe.  Process state: a per-device cache of the compute-unit count, of kernel occupancies and of the
+ *     address of the static workspace (thn_norm_bwd_static_workspace), filled on first use; and the launch-shape
+ *     override of thn_norm_set_launch_override(), a process-wide tuning switch that is off unless a caller sets it.
  */
 #ifndef THNORM_H_
 #define THNORM_H_
@@ -30,7 +37,7 @@
 extern "C" {
 #endif
 
-#define THN_ABI_VERSION 5
+#define THN_ABI_VERSION 6
 
 enum thn_dtype { THN_F32 = 0, THN_F16 = 1, THN_BF16 = 2, THN_F64 = 3 };
 
@@ -125,6 +132,28 @@ int thn_norm_bwd_dx_partials(const void* x, int64_t x_row_stride,
 int thn_norm_bwd_reduce_partials(const void* workspace, int32_t num_partials,
                                  void* dw, void* db,
                                  int64_t N, int w_dtype, void* stream);
+
+/*
+ * thn_norm_bwd() for callers that cannot allocate device memory or pass a workspace along: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the reference (whose
+ * wrapper allocates its `_dw` / `_db` partial buffers per call, layernorm.py:183-185).  Same arguments and same
+ * results, bit for bit, as thn_norm_bwd(); the partial rows of the two-stage dW / dB sum go to a fixed array of
+ * THN_STATIC_WORKSPACE_BYTES in device memory that belongs to the library (one copy per GPU, held until the
+ * process ends).  The call allocates nothing and frees nothing; the first call on a device looks the array's
+ * address up (hipGetSymbolAddress), so make that one call outside a graph capture.  Problems whose partial rows
+ * need more than THN_STATIC_WORKSPACE_BYTES -- thn_norm_bwd_workspace_bytes() says how much -- return
+ * THN_E_WORKSPACE: bring a workspace and call thn_norm_bwd().  All calls on one GPU share the array: two calls
+ * that may run at the same time (different streams, or graph branches) race on it; calls on one stream are safe.
+ */
+#define THN_STATIC_WORKSPACE_BYTES (16 * 1024 * 1024)
+int thn_norm_bwd_static_workspace(const void* x, int64_t x_row_stride,
+                                  const void* dy, int64_t dy_row_stride,
+                                  void* dx, int64_t dx_row_stride,
+                                  const void* w,
+                                  const float* mean, const float* rstd,
+                                  void* dw, void* db,
+                                  int64_t M, int64_t N,
+                                  int x_dtype, int w_dtype, void* stream);
 
 /*
  * Softmax, Softmin and LogSoftmax over the last dimension (the row-reduction activations next to the norm

@@ -25,7 +25,7 @@ def declared_functions():
 
 def test_library_exports_every_declared_symbol():
     names = declared_functions()
-    assert len(names) == 21 and "thn_dropout" in names and "thn_norm_act_fwd" in names and "thn_norm_act_bwd" in names and "thn_act_fwd" in names and "thn_pnorm_fwd" in names and "thn_normalize_bwd" in names and "thn_norm_fwd" in names and "thn_norm_bwd" in names and "thn_softmax_fwd" in names
+    assert len(names) == 22 and "thn_norm_bwd_static_workspace" in names and "thn_dropout" in names and "thn_norm_act_fwd" in names and "thn_norm_act_bwd" in names and "thn_act_fwd" in names and "thn_pnorm_fwd" in names and "thn_normalize_bwd" in names and "thn_norm_fwd" in names and "thn_norm_bwd" in names and "thn_softmax_fwd" in names
     handle = ctypes.CDLL(_native.LIB_PATH)
     for name in names:
         assert hasattr(handle, name), f"{name} is declared in include/thnorm.h but not exported"

@@ -33,6 +33,7 @@ SYMBOLS = {
     'thn_norm_bwd_workspace_bytes': (_i64, [_i64, _i64, _i32, _i32, _i32]),
     'thn_norm_bwd': (_i32, [_vp, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64,
                             _i32, _i32, _vp]),
+    'thn_norm_bwd_static_workspace': (_i32, [_vp, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i32, _i32, _vp]),
     'thn_norm_bwd_dx_partials': (_i32, [_vp, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _vp, _i32, _i32, _vp, _i64,
                                         ctypes.POINTER(ctypes.c_int32), _i64, _i64, _i32, _i32, _vp]),
     'thn_norm_bwd_reduce_partials': (_i32, [_vp, ctypes.c_int32, _vp, _vp, _i64, _i32, _vp]),

@@ -994,6 +994,61 @@ int thn_norm_bwd(const void* x, int64_t x_row_stride, const void* dy, int64_t dy
     return thn_norm_bwd_reduce_partials(workspace, parts, dw, db, N, w_dtype, stream);
 }
 
+// ---- The backward for callers that cannot allocate -----------------------------------------------------------
+// The partial rows of the two-stage dW / dB sum live in a fixed array in device memory instead of a workspace the
+// caller brings.  Every device the library runs on holds its own copy of the array, at its own address, until the
+// process ends.  In host code the array's name is only a handle for hipGetSymbolAddress(): the address the
+// kernels are given is the one that call returns for the device that is current, looked up once per device.
+constexpr int64_t kStaticWorkspaceBytes = THN_STATIC_WORKSPACE_BYTES;
+static __device__ __align__(256) unsigned char g_static_workspace[kStaticWorkspaceBytes];
+
+namespace {
+std::mutex g_static_ws_mutex;
+void* g_static_ws_ptr[kMaxDevices];          // per device: the device address of g_static_workspace, or null
+bool g_static_ws_known[kMaxDevices];
+
+// The address of the array on the current device; null (and *status set) when it cannot be had.
+void* static_workspace_of_current_device(int* status) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+        (void)hipGetLastError();
+        *status = THN_E_DEVICE;
+        return nullptr;
+    }
+    std::lock_guard<std::mutex> lock(g_static_ws_mutex);
+    if (!g_static_ws_known[dev]) {
+        void* ptr = nullptr;
+        if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(g_static_workspace)) != hipSuccess || ptr == nullptr) {
+            (void)hipGetLastError();
+            *status = THN_E_DEVICE;
+            return nullptr;
+        }
+        g_static_ws_ptr[dev] = ptr;
+        g_static_ws_known[dev] = true;
+    }
+    return g_static_ws_ptr[dev];
+}
+}  // namespace
+
+extern "C" int thn_norm_bwd_static_workspace(const void* x, int64_t x_row_stride, const void* dy, int64_t dy_row_stride,
+                                              void* dx, int64_t dx_row_stride, const void* w, const float* mean,
+                                              const float* rstd, void* dw, void* db, int64_t M, int64_t N, int x_dtype,
+                                              int w_dtype, void* stream) {
+    const int64_t need = thn_norm_bwd_workspace_bytes(M, N, dw != nullptr, db != nullptr, x_dtype);
+    if (need < 0) return static_cast<int>(need);
+    if (need > kStaticWorkspaceBytes) return THN_E_WORKSPACE;      // the caller must bring a workspace: thn_norm_bwd()
+    void* ws = nullptr;
+    if (need > 0) {
+        int status = THN_OK;
+        ws = static_workspace_of_current_device(&status);
+        if (ws == nullptr) return status;
+    }
+    // Every partial row the second stage reads is written in full by the first stage of the same call: nothing in
+    // the array has to be cleared between calls.
+    return thn_norm_bwd(x, x_row_stride, dy, dy_row_stride, dx, dx_row_stride, w, mean, rstd, dw, db, ws, need, M, N,
+                        x_dtype, w_dtype, stream);
+}
+
 // ---- Softmax / Softmin / LogSoftmax -------------------------------------------------------------------------
 
 int thn_softmax_fwd(const void* x, int64_t x_row_stride, void* y, int64_t y_row_stride, int64_t M, int64_t N,
