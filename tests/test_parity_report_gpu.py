@@ -1,0 +1,178 @@
+"""The error report the reference's unit test prints (UnitTests/Normalization/layernorm_unittest.py:44-54: the
+mean / max difference of forward and backward against torch), taken against the float64 oracle and held to the
+LITERAL north-star bounds: float32 max abs error 1e-5 on y, dx, dW, dB; fp16 / bf16 within 1 ulp of the output
+dtype; saved mean / rstd within 1e-6 relative.  For every benchmark configuration and every output it records
+the max abs error, the max error in ulps of the output dtype and how many elements lie outside the literal bound
+-- for this library and, on the same inputs against the same oracle, for torch.nn.functional.layer_norm /
+rms_norm on the GPU.  Where the table shows the literal bound is reachable it is asserted; where it is not (the
+stock op misses it as well: the result does not exist in float32 to that accuracy) the widened bounds of
+conftest.check_* apply, asserted by test_parity_gpu.py.  The table is written to gpurun_out/parity_report.md."""
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from conftest import CONFIGS, ROOT, make_case, f64
+from oracle import c_oracle as co
+from oracle import norm_oracle as no
+from parity_util import gpu_forward_backward
+
+pytestmark = pytest.mark.gpu
+FMT = {torch.float32: "fp32", torch.float16: "fp16", torch.bfloat16: "bf16"}
+REPORT = {}
+
+
+def torch_forward_backward(kind, x, dy, w, b, eps):
+    """The stock operator on the GPU on the same inputs: y, dx, dW, dB and the statistics it saves."""
+    xg = x.cuda().requires_grad_(True)
+    wg = w.cuda().requires_grad_(True)
+    n = x.shape[-1]
+    if kind == "ln":
+        bg = b.cuda().requires_grad_(True)
+        y, mean, rstd = torch.native_layer_norm(xg, [n], wg, bg, eps)
+        y.backward(dy.cuda())
+        stats = dict(mean=mean.detach().reshape(-1).float(), rstd=rstd.detach().reshape(-1).float())
+        return dict(y=y.detach(), dx=xg.grad, dw=wg.grad, db=bg.grad, **stats)
+    y = torch.nn.functional.rms_norm(xg, (n,), wg, eps)
+    y.backward(dy.cuda())
+    return dict(y=y.detach(), dx=xg.grad, dw=wg.grad, db=None, mean=None, rstd=None)
+
+
+class Tally:
+    """Max abs error, max error in ulps of the output format, count outside the literal bound."""
+
+    def __init__(self, fmt, literal):
+        self.fmt, self.literal = fmt, literal          # literal: "abs" (1e-5), "ulp" (1 ulp) or "rel" (1e-6)
+        self.max_abs = self.max_ulp = self.max_rel = 0.0
+        self.over = self.total = 0
+
+    def add(self, got, ref, rel_floor=0.0):
+        got = np.asarray(got, dtype=np.float64)
+        err = np.abs(got - ref)
+        if not err.size:
+            return
+        self.max_abs = max(self.max_abs, float(err.max()))
+        ulps = err / no.ulp(ref, self.fmt)
+        self.max_ulp = max(self.max_ulp, float(ulps.max()))
+        if self.literal == "abs":
+            over = err > 1e-5
+        elif self.literal == "ulp":
+            over = ulps > 1.0
+        else:
+            rel = err / np.maximum(np.abs(ref), rel_floor)
+            self.max_rel = max(self.max_rel, float(rel.max()))
+            over = rel > 1e-6
+        self.over += int(over.sum())
+        self.total += err.size
+
+    def row(self):
+        d = dict(max_abs=self.max_abs, max_ulp=self.max_ulp, over=self.over, total=self.total)
+        if self.literal == "rel":
+            d["max_rel"] = self.max_rel
+        return d
+
+
+def error_table(kind, x, dy, w, b, eps, out, sample_chunks=None, chunk_rows=2048):
+    """Per output: Tally against the float64 oracle (dW / dB and the statistics on every row; y / dx on every row
+    or on `sample_chunks` evenly spread chunks)."""
+    dtype = x.dtype
+    n = x.shape[-1]
+    x2, dy2 = x.reshape(-1, n), dy.reshape(-1, n)
+    m = x2.shape[0]
+    lit = "abs" if dtype == torch.float32 else "ulp"
+    t = dict(y=Tally(FMT[dtype], lit), dx=Tally(FMT[dtype], lit), dw=Tally(FMT[w.dtype], lit), db=Tally(FMT[w.dtype], lit),
+             mean=Tally("fp32", "rel"), rstd=Tally("fp32", "rel"))
+    starts = list(range(0, m, chunk_rows))
+    sampled = set(starts)
+    if sample_chunks is not None and len(starts) > sample_chunks:
+        idx = np.unique(np.linspace(0, len(starts) - 1, sample_chunks).round().astype(int))
+        sampled = {starts[i] for i in idx}
+    dw_ref, db_ref = np.zeros(n), np.zeros(n)
+    y2 = out["y"].reshape(-1, n)
+    dx2 = out["dx"].reshape(-1, n)
+    for s in starts:
+        e = min(s + chunk_rows, m)
+        full = s in sampled
+        if kind == "ln":
+            yo, mean, rstd = co.layernorm_fwd(x2[s:e], w, b, eps, want_y=full)
+            dxo, dwo, dbo = co.layernorm_bwd(x2[s:e], dy2[s:e], w, mean, rstd, has_bias=True, want_dx=full)
+            db_ref += dbo
+            if out.get("mean") is not None:
+                # a mean is measured against the spread of its row (1/rstd): the means of N(0,1) rows are ~0 and
+                # have no relative accuracy of their own
+                t["mean"].add(f64(out["mean"][s:e]), mean, rel_floor=1.0)
+        else:
+            yo, rstd = co.rmsnorm_fwd(x2[s:e], w, eps, want_y=full)
+            dxo, dwo = co.rmsnorm_bwd(x2[s:e], dy2[s:e], w, rstd, want_dx=full)
+        dw_ref += dwo
+        if out.get("rstd") is not None:
+            t["rstd"].add(f64(out["rstd"][s:e]), rstd)
+        if full:
+            t["y"].add(f64(y2[s:e]), yo.reshape(-1, n))
+            t["dx"].add(f64(dx2[s:e]), dxo.reshape(-1, n))
+    t["dw"].add(f64(out["dw"]), dw_ref)
+    if out.get("db") is not None:
+        t["db"].add(f64(out["db"]), db_ref)
+    return {k: v.row() for k, v in t.items() if v.total}
+
+
+# Where the literal bound holds for every element of this library's output (asserted below).  Not listed: outputs
+# whose literal bound no float32-accumulating implementation meets -- the table shows the stock operator over it too:
+#   dW / dB of c4 (2^20 rows: |dW| ~ 1e3, one float32 ulp is 6e-5 > 1e-5) and of the fp32 c5 cases (|dW| ~ 64-90);
+#   y of c5b fp32 (outliers give |y| up to ~130: 1e-5 is 0.7 float32 ulp there);
+#   16-bit y / dx where the result cancels to far below its operands (1 ulp of a tiny bf16 value is below the
+#   float32 rounding of the operands: a few elements in 10^8), and one fp16 dW column of c5b at 1.5 ulp (sum of 4096
+#   float32 terms; the stock operator has two such columns).
+LITERAL_HOLDS = {
+    "c1_ln_f32_quickstart": ["y", "dx", "dw", "db", "mean", "rstd"],
+    "c2_rms_bf16_llm": ["y", "rstd", "dw"],
+    "c3_ln_bf16_wide": ["mean", "rstd", "dw", "db"],
+    "c4_ln_f32_small_hidden": ["y", "dx", "mean", "rstd"],
+    "c5a_ln_f16_hostile": ["dx", "mean", "rstd", "dw", "db"],
+    "c5a_ln_f32_hostile": ["y", "dx", "mean", "rstd"],
+    "c5b_rms_f16_outliers": ["y", "rstd"],
+    "c5b_rms_f32_outliers": ["dx", "rstd"],
+}
+
+
+@pytest.mark.parametrize("name", list(CONFIGS))
+def test_literal_tolerance_report(name):
+    print(f"\n[case] literal-tolerance report {name} shape={CONFIGS[name][1]}", flush=True)
+    c = make_case(name)
+    sample = None if c["x"].numel() <= 80_000_000 else 12
+    ours = gpu_forward_backward(c["kind"], c["x"], c["dy"], c["w"], c["b"], c["eps"])
+    mine = error_table(c["kind"], c["x"], c["dy"], c["w"], c["b"], c["eps"], ours, sample_chunks=sample)
+    del ours
+    torch.cuda.empty_cache()
+    stock = torch_forward_backward(c["kind"], c["x"], c["dy"], c["w"], c["b"], c["eps"])
+    theirs = error_table(c["kind"], c["x"], c["dy"], c["w"], c["b"], c["eps"], stock, sample_chunks=sample)
+    del stock
+    torch.cuda.empty_cache()
+    REPORT[name] = dict(this_library=mine, torch_functional=theirs)
+    for k, v in mine.items():
+        o = theirs.get(k)
+        print(f"  {k:5s} ours: max abs {v['max_abs']:.3e}  max ulp {v['max_ulp']:.3f}  outside literal {v['over']}/{v['total']}"
+              + (f"   | torch: max abs {o['max_abs']:.3e}  max ulp {o['max_ulp']:.3f}  outside {o['over']}/{o['total']}" if o else ""),
+              flush=True)
+    _write_report()
+    for k in LITERAL_HOLDS[name]:
+        assert mine[k]["over"] == 0, f"{name} {k}: {mine[k]['over']} of {mine[k]['total']} outside the literal bound ({mine[k]})"
+
+
+def _write_report():
+    out_dir = os.path.join(ROOT, "gpurun_out")
+    os.makedirs(out_dir, exist_ok=True)
+    with open(os.path.join(out_dir, "parity_report.json"), "w") as f:
+        json.dump(REPORT, f, indent=1)
+    lines = ["| config | output | this library: max abs / max ulp / outside literal | torch.nn.functional on the GPU: max abs / max ulp / outside literal |",
+             "|---|---|---|---|"]
+    for name, r in REPORT.items():
+        for k, v in r["this_library"].items():
+            o = r["torch_functional"].get(k)
+            mine = f"{v['max_abs']:.2e} / {v['max_ulp']:.2f} / {v['over']} of {v['total']}"
+            his = f"{o['max_abs']:.2e} / {o['max_ulp']:.2f} / {o['over']} of {o['total']}" if o else "(not exposed)"
+            lines.append(f"| {name} | {k} | {mine} | {his} |")
+    with open(os.path.join(out_dir, "parity_report.md"), "w") as f:
+        f.write("\n".join(lines) + "\n")
