@@ -10,8 +10,9 @@ Float64 numpy restatement of the reference's row-reduction activation kernels; i
 * ``logsoftmax_bwd``  follows ``TritonHub/Activations/logsoftmax.py:61-67`` (from the saved output y: dy - exp(y)*sum(dy))
 
 For rows within the reference's 64 KiB block the kernels see the whole row; wider rows are split by the
-reference into independently normalised chunks (softmax.py:34-36), which this oracle -- and the product --
-do not imitate: they refuse such rows.
+reference into independently normalised 64 KiB chunks (softmax.py:34-36), which is not a softmax of the row.
+This oracle and the product do not imitate that: both compute ONE softmax over the whole row, whatever its
+width, so for rows wider than 64 KiB they deliberately differ from what the reference would return.
 
 Pinned in tests/test_softmax_oracle_pins.py against torch's float64 CPU softmax / log_softmax and autograd,
 the frozen vectors in tests/golden/softmax_golden.npz, finite differences, closed forms and invariants.

@@ -243,3 +243,28 @@ def test_every_compiled_launch_shape(dtype):
     finally:
         lib.thn_norm_set_launch_override(9, 0, 0, 0, 0)
         lib.thn_norm_set_launch_override(10, 0, 0, 0, 0)
+
+
+def test_frozen_bias_of_another_dtype_without_weight():
+    """layernorm_act.apply(x, None, bias, ...) with 16-bit x and a float32 bias that does not require a gradient:
+    the backward still reads the bias (it rebuilds the pre-activation from it) and must read it as float32.  dx equals
+    the dx of the same call with a trainable bias, bit for bit."""
+    from TritonHub.Normalization.fused import layernorm_act
+    announce("fused LayerNorm, no weight, frozen float32 bias, bf16 rows")
+    g = torch.Generator().manual_seed(11)
+    x = torch.randn(300, 1024, generator=g).to(torch.bfloat16).cuda()
+    dy = torch.randn(300, 1024, generator=g).to(torch.bfloat16).cuda()
+    bias = (0.5 * torch.randn(1024, generator=g)).cuda()                     # float32
+    outs = []
+    for trainable in (True, False):
+        a = x.clone().requires_grad_(True)
+        b = bias.clone().requires_grad_(trainable)
+        y = layernorm_act.apply(a, None, b, 1e-5, _native.ACT_GELU)
+        y.backward(dy)
+        torch.cuda.synchronize()
+        outs.append((y.detach().clone(), a.grad.clone()))
+    assert torch.equal(outs[0][0], outs[1][0]) and torch.equal(outs[0][1], outs[1][1])
+    # and against float64: z = xhat + b, y = gelu(z), dx = layernorm backward of dy * gelu'(z)
+    x64 = f64(x); z, mean, rstd = no.layernorm_fwd(x64, None, f64(bias), 1e-5)
+    dx_ref, _, _ = no.layernorm_bwd(x64, ao.bwd("gelu", z, f64(dy)), None, mean, rstd, has_bias=False)
+    assert np.abs(f64(outs[1][1]) - dx_ref).max() < 0.02                    # bf16 dx of O(1) values: 2-3 ulp at most

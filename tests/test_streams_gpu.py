@@ -147,3 +147,93 @@ def test_operators_from_several_host_threads():
         t.join(timeout=120)
     assert not any(t.is_alive() for t in threads), "a worker thread did not finish"
     assert not errors, errors[:5]
+
+
+def test_two_host_threads_feed_one_stream():
+    """Two host threads run backward passes of different layers on the SAME stream (the autograd engine's worker and
+    a user thread can): the shared per-stream workspace of the two-stage dW / dB sum must never see one call's
+    first stage, the other call's first stage, then a second stage.  Parameter gradients equal the ones computed
+    alone beforehand, bit for bit, on every repetition."""
+    import threading
+    announce("two host threads, one stream")
+    torch.manual_seed(3)
+    stream = torch.cuda.Stream()
+    cases = []
+    for n, rows in ((1024, 4096), (1536, 3000)):
+        x = torch.randn(rows, n, device="cuda", dtype=torch.bfloat16)
+        dy = torch.randn(rows, n, device="cuda", dtype=torch.bfloat16)
+        mod = LayerNorm(n, device="cuda", dtype=torch.bfloat16)
+        a = x.clone().requires_grad_(True)
+        mod(a).backward(dy)
+        cases.append((x, dy, mod, mod.weight.grad.clone(), mod.bias.grad.clone(), a.grad.clone()))
+    torch.cuda.synchronize()
+    errors = []
+
+    def work(i):
+        try:
+            x, dy, mod, dw, db, dx = cases[i]
+            with torch.cuda.stream(stream):
+                for rep in range(200):
+                    a = x.clone().requires_grad_(True)
+                    mod.weight.grad = None
+                    mod.bias.grad = None
+                    mod(a).backward(dy)
+                    got = (mod.weight.grad, mod.bias.grad, a.grad)
+                    if rep % 20 == 19:
+                        stream.synchronize()
+                        if not (torch.equal(got[0], dw) and torch.equal(got[1], db) and torch.equal(got[2], dx)):
+                            errors.append((i, rep))
+        except Exception as e:
+            errors.append((i, repr(e)))
+
+    threads = [threading.Thread(target=work, args=(i,)) for i in range(2)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join(timeout=120)
+    assert not any(t.is_alive() for t in threads), "a worker thread did not finish"
+    assert not errors, errors[:5]
+
+
+def test_operator_layer_backward_under_graph_capture():
+    """The modules captured into a torch graph: the backward then takes a workspace of its own (the graph's) rather
+    than the per-stream one it shares with eager calls, so replays interleaved with eager backward passes of another
+    shape on the same stream still equal the eager result."""
+    announce("operator layer under graph capture")
+    torch.manual_seed(5)
+    n = 2048
+    mod = LayerNorm(n, device="cuda", dtype=torch.bfloat16)
+    other = RMSNorm(768, device="cuda", dtype=torch.bfloat16)
+    xs = torch.randn(1024, n, device="cuda", dtype=torch.bfloat16)
+    dy = torch.randn(1024, n, device="cuda", dtype=torch.bfloat16)
+    xo = torch.randn(5000, 768, device="cuda", dtype=torch.bfloat16)
+
+    def eager(xin):
+        a = xin.clone().requires_grad_(True)
+        mod.weight.grad = None
+        mod.bias.grad = None
+        y = mod(a)
+        y.backward(dy)
+        return y.detach().clone(), a.grad.clone(), mod.weight.grad.clone(), mod.bias.grad.clone()
+
+    eager(xs)                                            # warm-up outside the capture
+    torch.cuda.synchronize()
+    static_x = xs.clone().requires_grad_(True)
+    mod.weight.grad = None
+    mod.bias.grad = None
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        y = mod(static_x)
+        gx, gw, gb = torch.autograd.grad(y, (static_x, mod.weight, mod.bias), dy)
+    for trial in range(3):
+        new_x = torch.randn(1024, n, device="cuda", dtype=torch.bfloat16)
+        expect = eager(new_x)
+        with torch.no_grad():
+            static_x.copy_(new_x)
+        ao = xo.clone().requires_grad_(True)
+        other(ao).backward(torch.ones_like(xo))          # eager work on the shared workspace, enqueued around the replay
+        graph.replay()
+        other(ao).backward(torch.ones_like(xo))
+        torch.cuda.synchronize()
+        for name, e, t in zip(("y", "dx", "dw", "db"), expect, (y, gx, gw, gb)):
+            assert torch.equal(e, t), f"replay {trial}: {name} differs from the eager result"

@@ -9,6 +9,7 @@ call the C ABI of libthnorm.so on the current stream of the input's device.
 from __future__ import annotations
 
 import ctypes
+import threading
 
 import torch
 
@@ -45,8 +46,8 @@ def _check_feature_dim(n: int, element_size: int) -> None:
 
 _raw_stream = getattr(torch._C, '_cuda_getCurrentRawStream', None)
 _get_device = getattr(torch._C, '_cuda_getDevice', None)
-_workspace_bytes_cache = {}
 _workspace_cache = {}           # (device index, stream handle) -> uint8 tensor, grown on demand
+_backward_lock = threading.Lock()   # held from picking the shared workspace until both stages are enqueued
 _F32 = torch.float32
 
 
@@ -78,7 +79,12 @@ def _flatten(t: torch.Tensor, what: str):
 def _workspace(index: int, stream: int, nbytes: int, device) -> torch.Tensor:
     """The counterpart of the reference's per-call `_dw` / `_db` partial buffers (layernorm.py:183-184).  One buffer
     per (device, stream) is kept and grown on demand: both stages of a backward are enqueued on that stream, so a
-    later call on the same stream can only reuse the buffer after they have run."""
+    later call on the same stream can only reuse the buffer after they have run.  The caller holds
+    `_backward_lock` until both stages are enqueued, so two host threads that feed one stream cannot interleave
+    their stages on the buffer.  While the stream is being captured into a graph the call gets a buffer of its
+    own instead (the graph keeps it alive and would replay on the shared one while eager work uses it)."""
+    if torch.cuda.is_current_stream_capturing():
+        return torch.empty((max(nbytes, 16),), dtype=torch.uint8, device=device)
     key = (index, stream)
     ws = _workspace_cache.get(key)
     if ws is None or ws.numel() < nbytes:
@@ -165,7 +171,9 @@ def norm_bwd(x: torch.Tensor, dout: torch.Tensor, weight, bias, mean, rstd, laye
     x_code = _native.dtype_code(x.dtype)
     want_db = layernorm and bias is not None and need_db
     mixed = weight is not None and want_db and weight.dtype != bias.dtype
-    grad_dtype = weight.dtype if weight is not None else (bias.dtype if want_db else x.dtype)
+    # the storage type the kernels read w / b in and write dW / dB in: the weight's, else the bias's -- also when
+    # the bias is frozen, because the fused backward still reads it to rebuild the pre-activation
+    grad_dtype = weight.dtype if weight is not None else (bias.dtype if (layernorm and bias is not None) else x.dtype)
     w_code = _native.dtype_code(grad_dtype)
     dw = torch.empty((n,), dtype=grad_dtype, device=device) if (weight is not None and need_dw) else None
     db = torch.empty((n,), dtype=grad_dtype, device=device) if want_db else None
@@ -176,22 +184,23 @@ def norm_bwd(x: torch.Tensor, dout: torch.Tensor, weight, bias, mean, rstd, laye
     lib = _native.lib()
     index = device.index
     other_device = _current_device() != index
+    locked = False
     if other_device:
         guard = torch.cuda.device(index)
         guard.__enter__()
     try:
-        key = (index, m, n, dw is not None, db is not None, x_code, act)
-        nbytes = _workspace_bytes_cache.get(key)
-        if nbytes is None:
-            if act < 0:
-                nbytes = int(lib.thn_norm_bwd_workspace_bytes(m, n, int(dw is not None), int(db is not None), x_code))
-            else:
-                nbytes = int(lib.thn_norm_act_bwd_workspace_bytes(m, n, int(dw is not None), int(db is not None), act,
-                                                                  x_code))
-            if nbytes < 0:
-                _native.check(nbytes)
-            _workspace_bytes_cache[key] = nbytes
+        # asked on every call: the answer follows the launch shape, which thn_norm_set_launch_override can change
+        if act < 0:
+            nbytes = int(lib.thn_norm_bwd_workspace_bytes(m, n, int(dw is not None), int(db is not None), x_code))
+        else:
+            nbytes = int(lib.thn_norm_act_bwd_workspace_bytes(m, n, int(dw is not None), int(db is not None), act,
+                                                              x_code))
+        if nbytes < 0:
+            _native.check(nbytes)
         stream = _stream_handle(index)
+        locked = nbytes > 0
+        if locked:
+            _backward_lock.acquire()
         workspace = _workspace(index, stream, nbytes, device) if nbytes > 0 else None
         if act < 0:
             status = lib.thn_norm_bwd(
@@ -210,6 +219,8 @@ def norm_bwd(x: torch.Tensor, dout: torch.Tensor, weight, bias, mean, rstd, laye
                 0 if dw is None else dw.data_ptr(), 0 if db is None else db.data_ptr(),
                 0 if workspace is None else workspace.data_ptr(), nbytes, m, n, act, x_code, w_code, stream)
     finally:
+        if locked:
+            _backward_lock.release()
         if other_device:
             guard.__exit__(None, None, None)
     if status != 0:
