@@ -56,6 +56,7 @@ __device__ __forceinline__ void st128(void* p, u32x4 v) {
 #define THN_FWD_X_KEEP 1
 #endif
 __device__ __forceinline__ u32x4 ld128_keep(const void* p) { return *reinterpret_cast<const u32x4*>(p); }
+__device__ __forceinline__ void st128_keep(void* p, u32x4 v) { *reinterpret_cast<u32x4*>(p) = v; }
 
 // s_waitcnt vmcnt(0): every vector-memory operation this wave has issued is complete.  Placed once in front
 // of the row loop so that the loop is entered with nothing outstanding: the compiler derives the loop's own

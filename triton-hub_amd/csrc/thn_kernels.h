@@ -145,9 +145,12 @@ __device__ __forceinline__ void forget_derived(u32x4 (&v)[K]) {
     for (int k = 0; k < K; ++k) asm volatile("" : "+v"(v[k]));
 }
 
-template <typename T, bool ALIGNED>
+// KEEP: an ordinary (cache-allocating) store instead of a streaming one, for an output that the operator's backward
+// reads again (see ld128_keep); on the 128-bit path only.
+template <typename T, bool ALIGNED, bool KEEP = false>
 __device__ __forceinline__ void store_row_vec(char* rowp, int voff, int n_cols, const float (&f)[T::VEC]) {
-    if constexpr (ALIGNED) st128(rowp + voff, T::pack(f));
+    if constexpr (ALIGNED && KEEP) st128_keep(rowp + voff, T::pack(f));
+    else if constexpr (ALIGNED) st128(rowp + voff, T::pack(f));
     else store_vec_elems<T>(rowp, voff, n_cols, f);
 }
 
@@ -402,15 +405,17 @@ __device__ __forceinline__ void combine_groups(Acc (&acc)[VEC], Acc* comb, int g
 }
 
 // One vector slot of a partial row.  The workspace is 16-byte aligned, the partial rows are a multiple of 256
-// bytes apart and a slot starts a multiple of VEC floats into its row: 16-byte streaming stores (the second stage
-// reads the rows once, from another compute unit; plain 4-byte stores left the rows dirty in the L2 until the end
-// of the kernel and cost the LayerNorm backward 2 us at 4096 columns).
+// bytes apart and a slot starts a multiple of VEC floats into its row: 16-byte stores.  They are ordinary
+// (cache-allocating) stores: the second stage reads the rows a few microseconds later, and what is written this way
+// is still in the memory-side cache then (fp16 4096 x 16384, 16 MiB of partial rows: both stages 81.3 -> 78.5 us;
+// bf16 16384 x 4096: step 105.4 -> 104.6 us; as streaming stores the rows went to HBM and came back from there).
+// As 4-byte-per-lane stores they had cost the LayerNorm backward 2 us at 4096 columns, in either form.
 template <int VEC>
 __device__ __forceinline__ void store_partial(float* dst, const float (&f)[VEC]) {
     if constexpr (VEC % 4 == 0) {
 #pragma unroll
         for (int e = 0; e < VEC; e += 4) {
-            st128(dst + e, u32x4{as_u32(f[e]), as_u32(f[e + 1]), as_u32(f[e + 2]), as_u32(f[e + 3])});
+            st128_keep(dst + e, u32x4{as_u32(f[e]), as_u32(f[e + 1]), as_u32(f[e + 2]), as_u32(f[e + 3])});
         }
     } else {
 #pragma unroll

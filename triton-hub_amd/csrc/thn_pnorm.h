@@ -199,6 +199,10 @@ template <typename T, int MODE, bool NORMALIZE, int K, int TPR, int BLOCK, bool 
 __global__ void __launch_bounds__(BLOCK) pnorm_fwd_kernel(const PnormFwdArgs a) {
     constexpr int VEC = T::VEC;
     constexpr int G = BLOCK / TPR;
+    // What the backward reads again stays in the caches (ld128_keep): the norm's backward and the normalize backward
+    // for p = 1 read x, the normalize backward for p = 2 reads y; for the other p it reads both, and x is kept.
+    constexpr bool kKeepY = NORMALIZE && MODE == kP2;
+    constexpr bool kKeepX = !kKeepY;
     static_assert(BLOCK % TPR == 0 && G >= 1, "a workgroup holds whole rows");
     __shared__ float red[RedSmem<TPR, G, 1>::kFloats];
 
@@ -227,7 +231,7 @@ __global__ void __launch_bounds__(BLOCK) pnorm_fwd_kernel(const PnormFwdArgs a) 
     last.init(a.walk, last_row);
     int64_t y_off = NORMALIZE ? row_offset(a.ymap, cursor) : 0;
     u32x4 cur[K];
-    load_row<T, K, ALIGNED>(cur, a.x + row_offset(a.xmap, cursor), 0, 0, voff, a.n_cols);
+    load_row<T, K, ALIGNED, kKeepX>(cur, a.x + row_offset(a.xmap, cursor), 0, 0, voff, a.n_cols);
 
     drain_vector_memory();
     for (int64_t base = static_cast<int64_t>(blockIdx.x) * G; base < a.rows; base += rows_per_iter) {
@@ -237,7 +241,7 @@ __global__ void __launch_bounds__(BLOCK) pnorm_fwd_kernel(const PnormFwdArgs a) 
         cursor.advance(a.walk);
         const RowCursor ncur = clamp_cursor(cursor, last, more);
         u32x4 nxt[K];
-        load_row<T, K, ALIGNED>(nxt, a.x + row_offset(a.xmap, ncur), 0, 0, voff, a.n_cols);
+        load_row<T, K, ALIGNED, kKeepX>(nxt, a.x + row_offset(a.xmap, ncur), 0, 0, voff, a.n_cols);
 
         float xf[K][VEC];
         float s[1] = {0.0f};
@@ -264,7 +268,7 @@ __global__ void __launch_bounds__(BLOCK) pnorm_fwd_kernel(const PnormFwdArgs a) 
                 float yf[VEC];
 #pragma unroll
                 for (int e = 0; e < VEC; ++e) yf[e] = div_by_row(xf[k][e], nd, rn);
-                store_row_vec<T, ALIGNED>(yrow, voff[k], a.n_cols, yf);
+                store_row_vec<T, ALIGNED, kKeepY>(yrow, voff[k], a.n_cols, yf);
             }
             y_off = row_offset(a.ymap, ncur);
         }

@@ -66,15 +66,17 @@ __device__ __forceinline__ void load_row_as(u32x4 (&dst)[K], const char* base, i
     }
 }
 
-template <typename T, bool ALIGNED>
+// KEEP: as store_row_vec.  The softmax family's forward keeps its output: the backward works from the saved y.
+template <typename T, bool ALIGNED, bool KEEP = false>
 __device__ __forceinline__ void store_row_as(char* rowp, int voff, int n_cols, const float (&f)[T::VEC]) {
-    store_row_vec<T, ALIGNED>(rowp, voff, n_cols, f);
+    store_row_vec<T, ALIGNED, KEEP>(rowp, voff, n_cols, f);
 }
-template <typename T, bool ALIGNED>
+template <typename T, bool ALIGNED, bool KEEP = false>
 __device__ __forceinline__ void store_row_as(char* rowp, int voff, int n_cols, const double (&f)[T::VEC]) {
     static_assert(T::kBytes == 8, "float64 arithmetic is for float64 storage only");
     if constexpr (ALIGNED) {
-        st128(rowp + voff, pack_f64(f));
+        if constexpr (KEEP) st128_keep(rowp + voff, pack_f64(f));
+        else st128(rowp + voff, pack_f64(f));
     } else {
 #pragma unroll
         for (int e = 0; e < 2; ++e) {
@@ -165,7 +167,7 @@ __global__ void __launch_bounds__(BLOCK) softmax_fwd_kernel(const SoftmaxFwdArgs
             C yf[VEC];
 #pragma unroll
             for (int e = 0; e < VEC; ++e) yf[e] = LOG ? xf[k][e] - scale : xf[k][e] * scale;
-            store_row_as<T, ALIGNED>(yrow, voff[k], a.n_cols, yf);
+            store_row_as<T, ALIGNED, true>(yrow, voff[k], a.n_cols, yf);
         }
 
 #pragma unroll
