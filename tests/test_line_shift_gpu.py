@@ -56,3 +56,39 @@ def test_softmax_rows_off_line_boundaries(kind, dtype, m, n):
     x = (torch.randn(m, n, generator=g) * 3).to(dtype)
     dy = torch.randn(m, n, generator=g).to(dtype)
     softmax_t.run_and_compare(kind, x, dy, f"line shift {kind} {m}x{n}")
+
+
+# The row p-norm / normalize kernels (thn_pnorm.h) take the same shift when the (B, M, K) tensor folds into one batch
+# of rows.  Same oracle and tolerances as tests/test_pnorm_parity_gpu.py.
+PNORM_CASES = [
+    (2.0, torch.float32, (1, 523, 4100)),     # 1025 vectors on 512 threads, pitch 16 mod 128: all eight phases
+    (2.0, torch.float32, (3, 100, 6000)),     # batches fold (contiguous): phases 0 / 64
+    (1.0, torch.float32, (1, 300, 6000)),
+    (3.0, torch.float32, (2, 150, 6000)),
+    (2.0, torch.bfloat16, (1, 600, 4104)),    # 513 vectors on 256 threads
+    (2.0, torch.float16, (1, 520, 6000)),
+    (2.0, torch.float32, (1, 300, 8180)),     # 2045 vectors: no room for the shift
+    (2.0, torch.float32, (1, 101, 6000)),     # 101 * pitch is not a multiple of 128: unshifted
+]
+
+
+@pytest.mark.parametrize("p,dtype,shape", PNORM_CASES)
+def test_pnorm_rows_off_line_boundaries(p, dtype, shape):
+    import test_pnorm_parity_gpu as pnorm_t
+    print(f"\n[case] line shift pnorm p={p} {dtype} {shape}", flush=True)
+    x, gn, gy = pnorm_t.make(shape, dtype, seed=shape[1] * 31 + shape[2])
+    pnorm_t.compare_norm(x, gn, p, 1e-6, f"line shift norm p={p} {shape}")
+    pnorm_t.compare_normalize(x, gy, p, 1e-6, f"line shift normalize p={p} {shape}")
+
+
+def test_pnorm_strided_batches_do_not_shift():
+    """Batches that do not fold (a batch stride that is not M row strides) keep the unshifted slots: the result must
+    still be right."""
+    import test_pnorm_parity_gpu as pnorm_t
+    print("\n[case] line shift pnorm, batches that do not fold", flush=True)
+    big, _, gbig = pnorm_t.make((3, 140, 6000), torch.float32, seed=77)
+    view = lambda t: t[:, :100, :]                   # batch stride 140 rows, 100 rows used
+    _, gn, _ = pnorm_t.make((3, 100, 8), torch.float32, seed=79)
+    pnorm_t.compare_norm(view(big).contiguous(), gn, 2.0, 1e-6, "non-folding batches norm", x_gpu=view(big.cuda()).detach())
+    pnorm_t.compare_normalize(view(big).contiguous(), view(gbig).contiguous(), 2.0, 1e-6, "non-folding batches normalize",
+                              x_gpu=view(big.cuda()).detach(), gy_gpu=view(gbig.cuda()))

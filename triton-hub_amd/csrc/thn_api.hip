@@ -723,6 +723,9 @@ int pnorm_forward(const void* x, int64_t x_batch_stride, int64_t x_row_stride, v
         if (rc != THN_OK) return rc;
         a.n_vecs = plan.n_vecs;
         a.walk = make_walk(uniform, M, rp.rows, static_cast<int64_t>(plan.grid) * (plan.s.block / plan.s.tpr));
+        // rows of one folded batch sit at r * row stride, which is what the shift's phase test assumes
+        const RowStream streams[2] = {{x, a.xmap.row_stride_bytes}, {y, a.ymap.row_stride_bytes}};
+        a.line_shift = (uniform && line_shift_ok(aligned, plan.s, plan.grid, plan.n_vecs, streams, normalize ? 2 : 1)) ? 1 : 0;
         lrc = launch_pnorm_fwd(dtype, variant, aligned, plan.s, a, plan.grid, st, nullptr);
     } else {
         const int grid = loop_grid(rp.rows);
@@ -969,12 +972,14 @@ int thn_norm_bwd_reduce_partials(const void* workspace, int32_t num_partials, vo
     r.n_cols = static_cast<int>(N);
     r.n_parts = num_partials;
     r.w_dtype = w_dtype;
+    const hipStream_t st = static_cast<hipStream_t>(stream);
+    const auto blocks = [&](int cols) { return dim3(static_cast<unsigned>((N + cols - 1) / cols), static_cast<unsigned>(n)); };
     if (N >= thn::kReduceWideFrom) {
-        const dim3 grid(static_cast<unsigned>((N + thn::kReduceColsWide - 1) / thn::kReduceColsWide), static_cast<unsigned>(n));
-        hipLaunchKernelGGL(thn::reduce_partials_kernel<thn::kReduceColsWide>, grid, dim3(256), 0, static_cast<hipStream_t>(stream), r);
+        hipLaunchKernelGGL(thn::reduce_partials_kernel<thn::kReduceColsWide>, blocks(thn::kReduceColsWide), dim3(256), 0, st, r);
+    } else if (N >= thn::kReduceMidFrom) {
+        hipLaunchKernelGGL(thn::reduce_partials_kernel<thn::kReduceColsMid>, blocks(thn::kReduceColsMid), dim3(256), 0, st, r);
     } else {
-        const dim3 grid(static_cast<unsigned>((N + thn::kReduceCols - 1) / thn::kReduceCols), static_cast<unsigned>(n));
-        hipLaunchKernelGGL(thn::reduce_partials_kernel<thn::kReduceCols>, grid, dim3(256), 0, static_cast<hipStream_t>(stream), r);
+        hipLaunchKernelGGL(thn::reduce_partials_kernel<thn::kReduceCols>, blocks(thn::kReduceCols), dim3(256), 0, st, r);
     }
     return hipGetLastError() == hipSuccess ? THN_OK : THN_E_LAUNCH;
 }
@@ -1200,6 +1205,8 @@ int thn_pnorm_bwd(const void* x, int64_t x_batch_stride, int64_t x_row_stride, c
         if (rc != THN_OK) return rc;
         a.n_vecs = plan.n_vecs;
         a.walk = make_walk(uniform, M, rp.rows, static_cast<int64_t>(plan.grid) * (plan.s.block / plan.s.tpr));
+        const RowStream streams[2] = {{x, a.xmap.row_stride_bytes}, {dx, a.dxmap.row_stride_bytes}};
+        a.line_shift = (uniform && line_shift_ok(aligned, plan.s, plan.grid, plan.n_vecs, streams, 2)) ? 1 : 0;
         lrc = launch_pnorm_bwd(dtype, mode, aligned, plan.s, a, plan.grid, st, nullptr);
     } else {
         const int grid = loop_grid(rp.rows);
@@ -1256,6 +1263,10 @@ int thn_normalize_bwd(const void* x, int64_t x_batch_stride, int64_t x_row_strid
         if (rc != THN_OK) return rc;
         a.n_vecs = plan.n_vecs;
         a.walk = make_walk(uniform, M, rp.rows, static_cast<int64_t>(plan.grid) * (plan.s.block / plan.s.tpr));
+        // (a stream that is not read carries the map of dy: it agrees with dy by construction)
+        const RowStream streams[4] = {{a.g, a.gmap.row_stride_bytes}, {a.dx, a.dxmap.row_stride_bytes},
+                                      {a.x, a.xmap.row_stride_bytes}, {a.y, a.ymap.row_stride_bytes}};
+        a.line_shift = (uniform && line_shift_ok(aligned, plan.s, plan.grid, plan.n_vecs, streams, 4)) ? 1 : 0;
         lrc = launch_normalize_bwd(dtype, mode, aligned, plan.s, a, plan.grid, st, nullptr);
     } else {
         const int grid = loop_grid(rp.rows);

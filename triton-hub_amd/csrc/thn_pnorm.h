@@ -91,6 +91,7 @@ struct PnormFwdArgs {
     int p_int;          // p when it is an integer in [1, 6], else 0
     float p;
     float eps;
+    int line_shift;     // 1: the row kernels may move their vector slots onto 128-byte lines (row_line_shift(), thn_kernels.h)
 };
 
 struct PnormBwdArgs {
@@ -106,6 +107,7 @@ struct PnormBwdArgs {
     int n_vecs;
     int p_int;
     float p;
+    int line_shift;     // as in PnormFwdArgs
 };
 
 struct NormalizeBwdArgs {
@@ -122,6 +124,7 @@ struct NormalizeBwdArgs {
     int n_vecs;
     int p_int;
     float p;
+    int line_shift;     // as in PnormFwdArgs
 };
 
 // a^e for a >= 0 and a launch-uniform integer e in [2, 6], without a branch.
@@ -211,14 +214,17 @@ __global__ void __launch_bounds__(BLOCK) pnorm_fwd_kernel(const PnormFwdArgs a) 
     const int t = tid % TPR;
     int phase = 0;
 
+    // the host sets line_shift only when the rows are one folded batch (row r at r * row stride), every row this
+    // workgroup visits and every stream start in the same phase of a 128-byte line, and the slots have room
+    const int shift = (ALIGNED && G == 1) ? row_line_shift(a.line_shift, a.x, a.xmap.row_stride_bytes, blockIdx.x) : 0;
     int voff[K];
     bool own[K];
 #pragma unroll
     for (int k = 0; k < K; ++k) {
-        const int v = t + k * TPR;
-        const int vc = v < a.n_vecs ? v : a.n_vecs - 1;
+        const int v = t + k * TPR - shift;
+        const int vc = v < 0 ? 0 : (v < a.n_vecs ? v : a.n_vecs - 1);
         voff[k] = ALIGNED ? vc * 16 : vc;
-        own[k] = v < a.n_vecs;
+        own[k] = v >= 0 && v < a.n_vecs;
     }
 
     const int64_t rows_per_iter = static_cast<int64_t>(gridDim.x) * G;
@@ -293,11 +299,12 @@ __global__ void __launch_bounds__(BLOCK) pnorm_bwd_kernel(const PnormBwdArgs a) 
     const int g = tid / TPR;
     const int t = tid % TPR;
 
+    const int shift = (ALIGNED && G == 1) ? row_line_shift(a.line_shift, a.x, a.xmap.row_stride_bytes, blockIdx.x) : 0;
     int voff[K];
 #pragma unroll
     for (int k = 0; k < K; ++k) {
-        const int v = t + k * TPR;
-        const int vc = v < a.n_vecs ? v : a.n_vecs - 1;
+        const int v = t + k * TPR - shift;        // slots off either end repeat their neighbour's vector (same bits)
+        const int vc = v < 0 ? 0 : (v < a.n_vecs ? v : a.n_vecs - 1);
         voff[k] = ALIGNED ? vc * 16 : vc;
     }
 
@@ -374,14 +381,17 @@ __global__ void __launch_bounds__(BLOCK) normalize_bwd_kernel(const NormalizeBwd
     const int t = tid % TPR;
     int phase = 0;
 
+    // the host sets line_shift only when the rows are one folded batch (row r at r * row stride), every row this
+    // workgroup visits and every stream start in the same phase of a 128-byte line, and the slots have room
+    const int shift = (ALIGNED && G == 1) ? row_line_shift(a.line_shift, a.g, a.gmap.row_stride_bytes, blockIdx.x) : 0;
     int voff[K];
     bool own[K];
 #pragma unroll
     for (int k = 0; k < K; ++k) {
-        const int v = t + k * TPR;
-        const int vc = v < a.n_vecs ? v : a.n_vecs - 1;
+        const int v = t + k * TPR - shift;
+        const int vc = v < 0 ? 0 : (v < a.n_vecs ? v : a.n_vecs - 1);
         voff[k] = ALIGNED ? vc * 16 : vc;
-        own[k] = v < a.n_vecs;
+        own[k] = v >= 0 && v < a.n_vecs;
     }
 
     const int64_t rows_per_iter = static_cast<int64_t>(gridDim.x) * G;

@@ -11,8 +11,11 @@ namespace thn {
 // so it is cut for parallelism: a workgroup owns 16 columns (4 lanes x float4) and has 64 row slices, each
 // adding every 64th partial row (4 independent loads for 256 partial rows); the slice sums are then added in
 // slice order through LDS.  N / 16 workgroups: every compute unit takes part from N = 4096 on.  From 6144
-// columns on the stage moves 6 MiB and more per gradient and takes 64 columns x 16 slices per workgroup instead
-// (256-byte segments per partial row; measured 2x faster at 16384 columns and more, equal at 8192).
+// columns on the stage moves 6 MiB and more per gradient and wants longer segments of each partial row: 32 columns
+// x 32 slices (128-byte segments) up to 32768 columns, 64 columns x 16 slices (256-byte segments) from there on
+// (inside a forward + backward step, 32 against 64 columns: fp16 8192 x 6144 89.0 -> 86.6 us, 4096 x 16384
+// 113.3 -> 111.8 us, bf16 32768 x 8192 426.6 -> 425.1 us, 4096 x 32768 257.6 -> 258.6 us; against 16 columns the
+// longer segments are 2x faster at 16384 columns and more).
 // blockIdx.y selects dW (0) or dB (1).
 // ---------------------------------------------------------------------------------------------------
 struct ReduceArgs {
@@ -24,9 +27,11 @@ struct ReduceArgs {
     int w_dtype;
 };
 
-constexpr int kReduceCols = 16;       // columns per workgroup up to kReduceWideFrom columns
-constexpr int kReduceColsWide = 64;   // beyond: 256-byte segments per partial row, still one workgroup or more per compute unit
-constexpr int kReduceWideFrom = 6144;
+constexpr int kReduceCols = 16;       // columns per workgroup up to kReduceMidFrom columns
+constexpr int kReduceColsMid = 32;    // 128-byte segments per partial row, 32 row slices
+constexpr int kReduceColsWide = 64;   // 256-byte segments, 16 row slices
+constexpr int kReduceMidFrom = 6144;
+constexpr int kReduceWideFrom = 32768;
 
 template <int COLS>
 __global__ void __launch_bounds__(256) reduce_partials_kernel(const ReduceArgs a) {
