@@ -223,6 +223,8 @@ class NormBench:
         for i in range(preroll + warmup):
             self.step(i, lag)
         start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()                   # torch creates an event at its first record(): not inside the bracket
+        stop.record()
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         start.record()

@@ -618,6 +618,19 @@ __global__ void __launch_bounds__(BLOCK) norm_bwd_kernel(const BwdArgs a) {
     // the reduction rounds.
     auto lean_step = [&](auto masked_tag) {
         constexpr bool MASKED = decltype(masked_tag)::value;
+        // Byte offset of vector slot k.  The instance with 8 vectors per thread has no register to spare (it spilled
+        // six): it rebuilds the offsets from the lane's position on every row instead of keeping eight of them
+        // (the empty asm keeps the compiler from moving that back out of the row loop).
+        auto vo = [&](int k) -> int {
+            if constexpr (ALIGNED && K >= 8) {
+                int tt = t;
+                asm volatile("" : "+v"(tt));
+                const int v = tt + k * TPR - shift;
+                return (v < 0 ? 0 : (v < a.n_vecs ? v : a.n_vecs - 1)) * 16;
+            } else {
+                return voff[k];
+            }
+        };
         const int64_t nrow_raw = row_raw + rows_per_iter;
         const int64_t nrow = nrow_raw < a.M ? nrow_raw : last_row;
         const bool live = !MASKED || row_raw < a.M;
@@ -626,9 +639,9 @@ __global__ void __launch_bounds__(BLOCK) norm_bwd_kernel(const BwdArgs a) {
         u32x4 nx[kForm.ahead ? K : 1], ng[kForm.ahead ? K : 1];
         if constexpr (kForm.ahead) {
 #pragma unroll
-            for (int k = 0; k < K; ++k) nx[k] = load_row_vec<T, ALIGNED>(nxrow, voff[k], a.n_cols);
+            for (int k = 0; k < K; ++k) nx[k] = load_row_vec<T, ALIGNED>(nxrow, vo(k), a.n_cols);
 #pragma unroll
-            for (int k = 0; k < K; ++k) ng[k] = load_row_vec<T, ALIGNED>(ngrow, voff[k], a.n_cols);
+            for (int k = 0; k < K; ++k) ng[k] = load_row_vec<T, ALIGNED>(ngrow, vo(k), a.n_cols);
         }
         const float n_mean = LN ? a.mean[nrow] : 0.0f;
         const float n_rstd = a.rstd[nrow];
@@ -746,13 +759,13 @@ __global__ void __launch_bounds__(BLOCK) norm_bwd_kernel(const BwdArgs a) {
                 dw_lds[(2 * k) * BLOCK + tid] = f32x4{tot[0], tot[1], tot[2], tot[3]};
                 dw_lds[(2 * k + 1) * BLOCK + tid] = f32x4{tot[4], tot[5], tot[6], tot[7]};
             }
-            store_row_vec<T, ALIGNED>(dxrow, voff[k], a.n_cols, dxf);
+            store_row_vec<T, ALIGNED>(dxrow, vo(k), a.n_cols, dxf);
             if constexpr (kForm.ahead) {
                 cx[k] = nx[k];
                 cg[k] = ng[k];
             } else {
-                cx[k] = load_row_vec<T, ALIGNED>(nxrow, voff[k], a.n_cols);
-                cg[k] = load_row_vec<T, ALIGNED>(ngrow, voff[k], a.n_cols);
+                cx[k] = load_row_vec<T, ALIGNED>(nxrow, vo(k), a.n_cols);
+                cg[k] = load_row_vec<T, ALIGNED>(ngrow, vo(k), a.n_cols);
             }
         }
         c_mean = n_mean;
