@@ -341,6 +341,26 @@ def test_wide_rows_many_per_workgroup(dtype, widths):
             run_and_compare("ln", x, dy, w, b, 1e-5, f"wide LN N={n}, float32 parameters")
 
 
+@pytest.mark.parametrize("dtype,n", [(torch.bfloat16, 32768), (torch.float32, 16384), (torch.float16, 24576)])
+def test_wide_rows_forward_with_more_workgroups_than_the_chip_holds(dtype, n):
+    """From 12 rows of more than 32 KiB per compute unit on, the forward launches up to four times as many workgroups
+    as are resident at once (twice for the 16-bit LayerNorm); below that it does not.  3100 rows leave the last
+    grid-stride step partly filled."""
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    m = 12 * cus + 28
+    grid_rms = _launch.query_launch(0, False, m, n, dtype)[3]
+    grid_ln = _launch.query_launch(0, True, m, n, dtype)[3]
+    assert cus < grid_rms <= 4 * cus and cus < grid_ln <= (2 if dtype != torch.float32 else 4) * cus, (grid_rms, grid_ln)
+    assert _launch.query_launch(0, False, 8 * cus, n, dtype)[3] == cus
+    assert _launch.query_launch(1, False, m, n, dtype)[3] <= cus          # the backward: one partial row per workgroup
+    g = torch.Generator().manual_seed(37)
+    announce(f"wide rows, forward grid {grid_rms} / {grid_ln} workgroups: {dtype} {m}x{n}")
+    x = (0.5 + torch.randn(m, n, generator=g)).to(dtype); dy = torch.randn(m, n, generator=g).to(dtype)
+    w = (1 + 0.1 * torch.randn(n, generator=g)).to(dtype); b = (0.1 * torch.randn(n, generator=g)).to(dtype)
+    run_and_compare("ln", x, dy, w, b, 1e-5, f"LN {m}x{n}")
+    run_and_compare("rms", x, dy, w, None, 1e-5, f"RMS {m}x{n}")
+
+
 # ---- size-independent properties at full benchmark sizes --------------------------------------------------------
 @pytest.mark.parametrize("name", ["c2_rms_bf16_llm", "c5a_ln_f32_hostile", "c4_ln_f32_small_hidden"])
 def test_properties_at_full_size(name):
