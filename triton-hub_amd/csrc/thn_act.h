@@ -77,7 +77,8 @@ __global__ void __launch_bounds__(kActBlock) act_flat_kernel(const ActArgs a) {
             cx[u] = kKeepX ? ld128_keep(a.x + vc) : ld128(a.x + vc);
             if constexpr (BWD) cg[u] = ld128(a.g + vc);
         }
-        drain_vector_memory();
+        if constexpr (BWD) pin_loaded(cg);
+        drain_vector_memory(cx);
         for (int64_t base = static_cast<int64_t>(blockIdx.x) * kActBlock * U; base < a.total_vecs; base += step) {
             const int64_t n0 = v0 + step;
             u32x4 nx[U], ng[BWD ? U : 1];

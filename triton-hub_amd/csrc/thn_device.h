@@ -62,7 +62,22 @@ __device__ __forceinline__ void st128_keep(void* p, u32x4 v) { *reinterpret_cast
 // of the row loop so that the loop is entered with nothing outstanding: the compiler derives the loop's own
 // waits from the number of operations in flight on every path into the loop header, and an entry path with
 // the prologue's loads still pending makes it wait for more than the loop body needs on every trip.
-__device__ __forceinline__ void drain_vector_memory() { __builtin_amdgcn_s_waitcnt(0x0F70); }
+// The wait alone does not hold the prologue's loads in front of it (the compiler is free to issue them after
+// it, and did in the instances whose rows stay inside one wave: their loops then waited for all of the previous
+// row's stores at the top of every trip).  So the values the prologue loaded are passed in and pinned: an empty
+// asm statement takes each as an operand, which makes the compiler have it in registers at this point.
+__device__ __forceinline__ void pin_loaded(float& v) { asm volatile("" : "+v"(v)); }
+__device__ __forceinline__ void pin_loaded(u32x4& v) { asm volatile("" : "+v"(v)); }
+template <typename V, int K>
+__device__ __forceinline__ void pin_loaded(V (&v)[K]) {
+#pragma unroll
+    for (int k = 0; k < K; ++k) pin_loaded(v[k]);
+}
+template <typename... Loaded>
+__device__ __forceinline__ void drain_vector_memory(Loaded&... loaded) {
+    (pin_loaded(loaded), ...);
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+}
 
 // 1/sqrt(v) for v > 0: the hardware estimate (v_rsq_f32, about 1 ulp) refined by one Newton step, which
 // leaves an error of a fraction of an ulp -- well inside the 1e-6 relative bound on the saved rstd -- in 7

@@ -200,7 +200,7 @@ __global__ void __launch_bounds__(BLOCK) norm_fwd_kernel(const FwdArgs a) {
     load_params_clamped<K, VEC, ALIGNED>(wr, a.w, a.w_dtype, voff, a.n_cols, 1.0f);
     if constexpr (LN) load_params_clamped<K, VEC, ALIGNED>(br, a.b, a.w_dtype, voff, a.n_cols, 0.0f);
 
-    drain_vector_memory();
+    drain_vector_memory(cur);
     constexpr RowForm kForm = fwd_form<T::kBytes, LN, K, BLOCK, ACT != kNoAct>();
     if constexpr (kForm.recompute) {
         for (int64_t base = static_cast<int64_t>(blockIdx.x) * G; base < a.M; base += rows_per_iter) {
@@ -622,7 +622,7 @@ __global__ void __launch_bounds__(BLOCK) norm_bwd_kernel(const BwdArgs a) {
         // six): it rebuilds the offsets from the lane's position on every row instead of keeping eight of them
         // (the empty asm keeps the compiler from moving that back out of the row loop).
         auto vo = [&](int k) -> int {
-            if constexpr (ALIGNED && K >= 8) {
+            if constexpr (ALIGNED && (K >= 8 || BLOCK == 1024)) {
                 int tt = t;
                 asm volatile("" : "+v"(tt));
                 const int v = tt + k * TPR - shift;
@@ -774,7 +774,8 @@ __global__ void __launch_bounds__(BLOCK) norm_bwd_kernel(const BwdArgs a) {
         row = nrow;
     };
 
-    drain_vector_memory();
+    if constexpr (LN) pin_loaded(c_mean);
+    drain_vector_memory(cx, cg, c_rstd);
     int64_t base = static_cast<int64_t>(blockIdx.x) * G;
     if constexpr (kForm.recompute) {
         for (; base + G <= a.M; base += rows_per_iter) lean_step(std::false_type{});

@@ -239,7 +239,7 @@ __global__ void __launch_bounds__(BLOCK) pnorm_fwd_kernel(const PnormFwdArgs a) 
     u32x4 cur[K];
     load_row<T, K, ALIGNED, kKeepX>(cur, a.x + row_offset(a.xmap, cursor), 0, 0, voff, a.n_cols);
 
-    drain_vector_memory();
+    drain_vector_memory(cur);
     for (int64_t base = static_cast<int64_t>(blockIdx.x) * G; base < a.rows; base += rows_per_iter) {
         const int64_t nrow_raw = row_raw + rows_per_iter;
         const bool more = nrow_raw < a.rows;
@@ -322,17 +322,20 @@ __global__ void __launch_bounds__(BLOCK) pnorm_bwd_kernel(const PnormBwdArgs a) 
     float c_n = MODE == kP1 ? 1.0f : T::load1(a.norms, row);
     float c_g = T::load1(a.g, row);
 
-    drain_vector_memory();
+    if constexpr (MODE != kP1) pin_loaded(c_n);
+    drain_vector_memory(cur, c_g);
     for (int64_t base = static_cast<int64_t>(blockIdx.x) * G; base < a.rows; base += rows_per_iter) {
         const int64_t nrow_raw = row_raw + rows_per_iter;
         const bool more = nrow_raw < a.rows;
         const int64_t nrow = more ? nrow_raw : last_row;
         cursor.advance(a.walk);
         const RowCursor ncur = clamp_cursor(cursor, last, more);
-        u32x4 nxt[K];
-        load_row<T, K, ALIGNED>(nxt, a.x + row_offset(a.xmap, ncur), 0, 0, voff, a.n_cols);
+        // the next row's scalars first: loads return in issue order, and a wait for a scalar requested after the
+        // row's vectors would be a wait for those vectors
         const float n_n = MODE == kP1 ? 1.0f : T::load1(a.norms, nrow);
         const float n_g = T::load1(a.g, nrow);
+        u32x4 nxt[K];
+        load_row<T, K, ALIGNED>(nxt, a.x + row_offset(a.xmap, ncur), 0, 0, voff, a.n_cols);
 
         float den = c_n;
         if constexpr (MODE == kPInt) den = pow_small(c_n, a.p_int - 1);     // norms^(p-1), norm.py:86-87
@@ -409,18 +412,20 @@ __global__ void __launch_bounds__(BLOCK) normalize_bwd_kernel(const NormalizeBwd
     load_row<T, K, ALIGNED>(cg, a.g + row_offset(a.gmap, cursor), 0, 0, voff, a.n_cols);
     float c_n = T::load1(a.norms, row);
 
-    drain_vector_memory();
+    if constexpr (NEED_X) pin_loaded(cx);
+    if constexpr (NEED_Y) pin_loaded(cy);
+    drain_vector_memory(cg, c_n);
     for (int64_t base = static_cast<int64_t>(blockIdx.x) * G; base < a.rows; base += rows_per_iter) {
         const int64_t nrow_raw = row_raw + rows_per_iter;
         const bool more = nrow_raw < a.rows;
         const int64_t nrow = more ? nrow_raw : last_row;
         cursor.advance(a.walk);
         const RowCursor ncur = clamp_cursor(cursor, last, more);
+        const float n_n = T::load1(a.norms, nrow);      // before the row's vectors, as in pnorm_bwd_kernel
         u32x4 nx[NEED_X ? K : 1], ny[NEED_Y ? K : 1], ng[K];
         if constexpr (NEED_X) load_row<T, K, ALIGNED>(nx, a.x + row_offset(a.xmap, ncur), 0, 0, voff, a.n_cols);
         if constexpr (NEED_Y) load_row<T, K, ALIGNED>(ny, a.y + row_offset(a.ymap, ncur), 0, 0, voff, a.n_cols);
         load_row<T, K, ALIGNED>(ng, a.g + row_offset(a.gmap, ncur), 0, 0, voff, a.n_cols);
-        const float n_n = T::load1(a.norms, nrow);
 
         float xf[NEED_X ? K : 1][VEC], yf[NEED_Y ? K : 1][VEC], gf[K][VEC];
         float s[1] = {0.0f};

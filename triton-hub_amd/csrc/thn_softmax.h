@@ -121,7 +121,7 @@ __global__ void __launch_bounds__(BLOCK) softmax_fwd_kernel(const SoftmaxFwdArgs
     u32x4 cur[K];
     load_row_as<T, C, K, ALIGNED>(cur, a.x, a.x_stride_bytes, row, voff, a.n_cols);
 
-    drain_vector_memory();
+    drain_vector_memory(cur);
     for (int64_t base = static_cast<int64_t>(blockIdx.x) * G; base < a.M; base += rows_per_iter) {
         const int64_t nrow_raw = row_raw + rows_per_iter;
         const int64_t nrow = nrow_raw < a.M ? nrow_raw : last_row;
@@ -213,7 +213,7 @@ __global__ void __launch_bounds__(BLOCK) softmax_bwd_kernel(const SoftmaxBwdArgs
     load_row_as<T, C, K, ALIGNED>(cy, a.y, a.y_stride_bytes, row, voff, a.n_cols);
     load_row_as<T, C, K, ALIGNED>(cg, a.dy, a.dy_stride_bytes, row, voff, a.n_cols);
 
-    drain_vector_memory();
+    drain_vector_memory(cy, cg);
     for (int64_t base = static_cast<int64_t>(blockIdx.x) * G; base < a.M; base += rows_per_iter) {
         const int64_t nrow_raw = row_raw + rows_per_iter;
         const int64_t nrow = nrow_raw < a.M ? nrow_raw : last_row;
