@@ -400,7 +400,7 @@ int narrow_row_blocks_per_cu(int which, int n_vecs, bool ragged16) {
     return 1;
 }
 
-// `pitch_bytes`: distance between rows of x when the caller knows it (0 otherwise); only the norm kernels use it.
+// `pitch_bytes`: distance between rows of x when the caller knows it and every row sits at row * pitch (0 otherwise).
 int plan_launch(int which, int flavour, bool aligned, int64_t M, int64_t N, int dtype, Plan* out,
                 int64_t pitch_bytes = 0) {
     const int bytes = elem_bytes(dtype);
@@ -445,12 +445,31 @@ int plan_launch(int which, int flavour, bool aligned, int64_t M, int64_t N, int 
         if (narrow > cap) cap = narrow;
         // One input stream and fewer than 1024 vectors per workgroup step (3 vectors per thread in 256-thread
         // workgroups: row widths of 5 * 2^k elements and their neighbours): a second workgroup brings the bytes in
-        // flight back to where HBM throughput peaks (bf16 N = 5120 forward 5.5 -> 6.0 TB/s, N = 1280 5.6 -> 6.1).
+        // flight back to where HBM throughput peaks (bf16 N = 1280, LayerNorm / softmax / normalize forward, 2048 to
+        // 32768 rows: 2-10 % faster at every row count; N = 5120 softmax 13.5 / 35.4 / 128.4 -> 11.6 / 34.2 / 125.8 us
+        // at 2048 / 8192 / 32768 rows).  The exception is the one-row workgroup at a pitch off 128-byte lines (its
+        // vectors are shifted onto line boundaries, see line_shift_ok() below), which gains from the second workgroup
+        // only up to 32 rows per compute unit and loses beyond (fp16 N = 6000, LayerNorm forward at 2048 / 4096 /
+        // 8192 / 16384 / 32768 rows: 10.7 / 17.7 / 36.1 / 68.5 / 135.2 us with one, 9.3 / 16.8 / 36.1 / 70.7 / 145.0
+        // with two; softmax and normalize the same way).
         const bool one_stream = which == kNormFwd || which == kSoftmaxFwd || which == kPnormFwd || which == kFusedFwd;
-        // (not when that leaves a workgroup fewer than 32 steps: 8192 rows of 6000 fp16 lose 5 % to the second set of
-        // parameter loads and launch ramps)
-        const int64_t steps_with_two = M / (static_cast<int64_t>(s.block / s.tpr) * cus * 2);
-        if (one_stream && aligned && s.block * s.k < 1024 && n_vecs > 16 && steps_with_two >= 32 && cap < 2) cap = 2;
+        const bool shifted_one_row = pitch_bytes % 128 != 0 && s.block == s.tpr;
+        if (one_stream && aligned && s.block * s.k < 1024 && n_vecs > 16 && cap < 2 &&
+            (!shifted_one_row || M <= 32 * static_cast<int64_t>(cus))) {
+            cap = 2;
+        }
+        // (the normalize forward, which takes two workgroups for every 256-thread shape, follows the same exception:
+        // fp16 N = 6000 at 16384 / 32768 rows 74.9 / 151.9 us with two, 73.8 / 145.2 with one)
+        if (which == kPnormFwd && (flavour & 4) != 0 && aligned && shifted_one_row && n_vecs > 16 && cap == 2 &&
+            M > 32 * static_cast<int64_t>(cus)) {
+            cap = 1;
+        }
+        // The norm forward's two-row workgroups (THN_FWD_SHAPES_TWO_ROWS) with few rows: bf16 N = 5120, 2048 / 4096
+        // rows 8.9 / 14.6 -> 8.3 / 14.0 us with two per compute unit; the same from 8192 rows on.
+        if (which == kNormFwd && aligned && s.k == 3 && s.tpr == 256 && s.block == 512 && cap < 2 &&
+            M <= 24 * static_cast<int64_t>(cus)) {
+            cap = 2;
+        }
     }
     if (cap < bpc) bpc = cap;
     const int rows_per_block = s.block / s.tpr;
@@ -734,7 +753,7 @@ int pnorm_forward(const void* x, int64_t x_batch_stride, int64_t x_row_stride, v
     if (rp.engine) {
         const int variant = mode_of(rp.p_int) | (normalize ? 4 : 0);
         Plan plan;
-        const int rc = plan_launch(kPnormFwd, variant, aligned, rp.rows, K, dtype, &plan);
+        const int rc = plan_launch(kPnormFwd, variant, aligned, rp.rows, K, dtype, &plan, uniform ? a.xmap.row_stride_bytes : 0);
         if (rc != THN_OK) return rc;
         a.n_vecs = plan.n_vecs;
         a.walk = make_walk(uniform, M, rp.rows, static_cast<int64_t>(plan.grid) * (plan.s.block / plan.s.tpr));
@@ -1103,7 +1122,7 @@ int thn_softmax_fwd(const void* x, int64_t x_row_stride, void* y, int64_t y_row_
                          (y_row_stride * bytes) % 16 == 0;
     const bool is_log = kind == THN_LOGSOFTMAX;
     Plan p;
-    const int rc = plan_launch(kSoftmaxFwd, is_log, aligned, M, N, dtype, &p);
+    const int rc = plan_launch(kSoftmaxFwd, is_log, aligned, M, N, dtype, &p, x_row_stride * elem_bytes(dtype));
     if (rc != THN_OK) return rc;
     SoftmaxFwdArgs a{};
     a.x = static_cast<const char*>(x);
