@@ -68,6 +68,11 @@ __device__ __forceinline__ void st128_keep(void* p, u32x4 v) { *reinterpret_cast
 // asm statement takes each as an operand, which makes the compiler have it in registers at this point.
 __device__ __forceinline__ void pin_loaded(float& v) { asm volatile("" : "+v"(v)); }
 __device__ __forceinline__ void pin_loaded(u32x4& v) { asm volatile("" : "+v"(v)); }
+// The raw bits of a scalar load, held where the statement stands: as pin_loaded, and the compiler may not move it
+// across a load or store either (so it stays behind the row's stores when it is written behind them).
+__device__ __forceinline__ void hold_loaded_here(uint16_t& v) { asm volatile("" : "+v"(v) : : "memory"); }
+__device__ __forceinline__ void hold_loaded_here(uint32_t& v) { asm volatile("" : "+v"(v) : : "memory"); }
+__device__ __forceinline__ void hold_loaded_here(uint64_t& v) { asm volatile("" : "+v"(v) : : "memory"); }
 template <typename V, int K>
 __device__ __forceinline__ void pin_loaded(V (&v)[K]) {
 #pragma unroll
@@ -424,6 +429,17 @@ __device__ __forceinline__ void store_vec_elems(char* row, int vec, int n_cols, 
         if (c < n_cols) T::store1(row, c, f[e]);
     }
 }
+
+// A per-row scalar of storage type T (a saved norm, an upstream gradient of one) that the row loop requests one row
+// ahead: load() returns its raw bits, value() widens them.  Between the two the kernel calls hold_loaded_here() at
+// the point up to which the value is not needed.  (The bits stay in their own width: a 16-bit value widened to 32
+// bits before the hold is one more instruction for the compiler to place early.)
+template <typename T>
+struct RowScalar {
+    using bits_t = typename T::bits_t;
+    __device__ static __forceinline__ bits_t load(const void* p, int64_t i) { return T::load_bits(p, i); }
+    __device__ static __forceinline__ float value(bits_t raw) { return T::widen(raw); }
+};
 
 // Unpacking / packing for kernels whose arithmetic type C is float64 on float64 storage (the float32 traits
 // narrow on load).

@@ -330,12 +330,14 @@ __global__ void __launch_bounds__(BLOCK) pnorm_bwd_kernel(const PnormBwdArgs a) 
         const int64_t nrow = more ? nrow_raw : last_row;
         cursor.advance(a.walk);
         const RowCursor ncur = clamp_cursor(cursor, last, more);
-        // the next row's scalars first: loads return in issue order, and a wait for a scalar requested after the
-        // row's vectors would be a wait for those vectors
-        const float n_n = MODE == kP1 ? 1.0f : T::load1(a.norms, nrow);
-        const float n_g = T::load1(a.g, nrow);
         u32x4 nxt[K];
         load_row<T, K, ALIGNED>(nxt, a.x + row_offset(a.xmap, ncur), 0, 0, voff, a.n_cols);
+        // The next row's two scalars are requested here as raw bits and widened at the end of the step (hold_loaded_here
+        // there keeps the compiler from widening them earlier): loads return in issue order, so an earlier use would
+        // wait for the row's vectors in the middle of the step -- or, requested before them, for the previous row's
+        // stores before the vectors are even requested.
+        typename RowScalar<T>::bits_t raw_n = MODE == kP1 ? 0 : RowScalar<T>::load(a.norms, nrow);
+        typename RowScalar<T>::bits_t raw_g = RowScalar<T>::load(a.g, nrow);
 
         float den = c_n;
         if constexpr (MODE == kPInt) den = pow_small(c_n, a.p_int - 1);     // norms^(p-1), norm.py:86-87
@@ -359,8 +361,12 @@ __global__ void __launch_bounds__(BLOCK) pnorm_bwd_kernel(const PnormBwdArgs a) 
 
 #pragma unroll
         for (int k = 0; k < K; ++k) cur[k] = nxt[k];
-        c_n = n_n;
-        c_g = n_g;
+        if constexpr (MODE != kP1) {
+            hold_loaded_here(raw_n);
+            c_n = RowScalar<T>::value(raw_n);
+        }
+        hold_loaded_here(raw_g);
+        c_g = RowScalar<T>::value(raw_g);
         row_raw = nrow_raw;
         row = nrow;
     }
@@ -421,11 +427,11 @@ __global__ void __launch_bounds__(BLOCK) normalize_bwd_kernel(const NormalizeBwd
         const int64_t nrow = more ? nrow_raw : last_row;
         cursor.advance(a.walk);
         const RowCursor ncur = clamp_cursor(cursor, last, more);
-        const float n_n = T::load1(a.norms, nrow);      // before the row's vectors, as in pnorm_bwd_kernel
         u32x4 nx[NEED_X ? K : 1], ny[NEED_Y ? K : 1], ng[K];
         if constexpr (NEED_X) load_row<T, K, ALIGNED>(nx, a.x + row_offset(a.xmap, ncur), 0, 0, voff, a.n_cols);
         if constexpr (NEED_Y) load_row<T, K, ALIGNED>(ny, a.y + row_offset(a.ymap, ncur), 0, 0, voff, a.n_cols);
         load_row<T, K, ALIGNED>(ng, a.g + row_offset(a.gmap, ncur), 0, 0, voff, a.n_cols);
+        typename RowScalar<T>::bits_t raw_n = RowScalar<T>::load(a.norms, nrow);      // widened at the end of the step, as in pnorm_bwd_kernel
 
         float xf[NEED_X ? K : 1][VEC], yf[NEED_Y ? K : 1][VEC], gf[K][VEC];
         float s[1] = {0.0f};
@@ -477,7 +483,8 @@ __global__ void __launch_bounds__(BLOCK) normalize_bwd_kernel(const NormalizeBwd
             if constexpr (NEED_Y) cy[k] = ny[k];
             cg[k] = ng[k];
         }
-        c_n = n_n;
+        hold_loaded_here(raw_n);
+        c_n = RowScalar<T>::value(raw_n);
         row_raw = nrow_raw;
         row = nrow;
     }
