@@ -464,6 +464,17 @@ int plan_launch(int which, int flavour, bool aligned, int64_t M, int64_t N, int 
             M > 32 * static_cast<int64_t>(cus)) {
             cap = 1;
         }
+        // The norm forward's 4-vector 256-thread workgroups (rows of 1024 / G vectors, G rows at a time) with at most
+        // 8 steps each: a second workgroup per compute unit fills the start and the end of so short a kernel (bf16
+        // LayerNorm forward, 4096 rows of 2048 / 4096: 7.2 / 12.1 -> 6.4 / 11.9 us; forward + backward of one batch
+        // 21.7 / 35.0 -> 21.0 / 33.8 us).  From 16 steps on the forward by itself is 1-3 % slower with two (16384 x 4096:
+        // 46.0 -> 46.5 us), although the backward that follows it on the same batch then runs faster by more than that
+        // up to 32 steps (16384 x 4096 forward + backward 109.9 -> 109.4 us, 8192 x 4096 60.7 -> 59.2): with anything
+        // else between a layer's forward and its backward only the forward's loss would be left, so one it stays.
+        if (which == kNormFwd && aligned && s.k == 4 && s.block == 256 && n_vecs > 16 && cap < 2 &&
+            M <= 8 * static_cast<int64_t>(s.block / s.tpr) * cus) {
+            cap = 2;
+        }
         // The norm forward's two-row workgroups (THN_FWD_SHAPES_TWO_ROWS) with few rows: bf16 N = 5120, 2048 / 4096
         // rows 8.9 / 14.6 -> 8.3 / 14.0 us with two per compute unit; the same from 8192 rows on.
         if (which == kNormFwd && aligned && s.k == 3 && s.tpr == 256 && s.block == 512 && cap < 2 &&
