@@ -361,6 +361,32 @@ def test_wide_rows_forward_with_more_workgroups_than_the_chip_holds(dtype, n):
     run_and_compare("rms", x, dy, w, None, 1e-5, f"RMS {m}x{n}")
 
 
+def test_forward_workgroups_per_compute_unit():
+    """The forward's launch rules that depend on the row count: a second workgroup per compute unit for short
+    kernels (4 vectors per thread in 256 threads, at most 8 steps each) and for 3-vector 256-thread shapes -- but
+    for the one-row workgroup at a pitch off 128-byte lines only up to 32 rows per compute unit.  Each case also
+    runs against the oracle at the row count just inside the rule."""
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    bf16, f16 = torch.bfloat16, torch.float16
+    grid = lambda which, ln, m, n, dt: _launch.query_launch(which, ln, m, n, dt)[3]
+    # 4096 bf16 columns: two rows per 256-thread workgroup; 8 steps each = 16 rows per compute unit
+    assert grid(0, True, 16 * cus, 4096, bf16) == 2 * cus
+    assert grid(0, True, 64 * cus, 4096, bf16) == cus
+    assert grid(1, True, 16 * cus, 4096, bf16) == cus                   # the backward: one partial row per compute unit
+    # 1280 bf16 columns (3 vectors x 64 threads, four rows per workgroup): two at every row count
+    assert grid(0, False, 8 * cus, 1280, bf16) == 2 * cus and grid(0, False, 512 * cus, 1280, bf16) == 2 * cus
+    # 6000 fp16 columns: 12000-byte rows, one row per workgroup, vectors shifted onto 128-byte lines
+    assert grid(0, True, 32 * cus, 6000, f16) == 2 * cus
+    assert grid(0, True, 64 * cus, 6000, f16) == cus
+    g = torch.Generator().manual_seed(41)
+    for m, n, dt in ((16 * cus, 4096, bf16), (32 * cus, 6000, f16), (8 * cus + 3, 1280, bf16)):
+        announce(f"forward with two workgroups per compute unit: {dt} {m}x{n}")
+        x = (0.5 + torch.randn(m, n, generator=g)).to(dt); dy = torch.randn(m, n, generator=g).to(dt)
+        w = (1 + 0.1 * torch.randn(n, generator=g)).to(dt); b = (0.1 * torch.randn(n, generator=g)).to(dt)
+        run_and_compare("ln", x, dy, w, b, 1e-5, f"LN {m}x{n}")
+        run_and_compare("rms", x, dy, w, None, 1e-5, f"RMS {m}x{n}")
+
+
 # ---- size-independent properties at full benchmark sizes --------------------------------------------------------
 @pytest.mark.parametrize("name", ["c2_rms_bf16_llm", "c5a_ln_f32_hostile", "c4_ln_f32_small_hidden"])
 def test_properties_at_full_size(name):
