@@ -415,6 +415,13 @@ int plan_launch(int which, int flavour, bool aligned, int64_t M, int64_t N, int 
     // (rows shorter than one vector have a single element-wise instance)
     const bool ln16 = (which == kNormBwd || which == kFusedBwd) && bytes == 2 && (flavour & 1) != 0 && N >= vec_elems;
     Shape s = heuristic_shape(which, aligned, ln16, n_vecs);
+    // The norm forward over rows of 385 to 512 vectors: 2 x 256 vectors, two rows at a time in 512 threads
+    // (THN_FWD_SHAPES_TWO_ROWS), unless the kernel is so short that the 256-thread shape takes two workgroups per
+    // compute unit (below).
+    if (which == kNormFwd && aligned && s.k == 4 && s.tpr == 128 && s.block == 256 && n_vecs > 384 &&
+        M > 16 * static_cast<int64_t>(cus)) {
+        s = Shape{2, 256, 512};
+    }
     // Rows that start off 128-byte lines: two-row workgroups of 256-thread rows cannot put their requests on line
     // boundaries (the two rows differ in phase, line_shift_ok() below), one-row workgroups can.  Backward: as fast
     // otherwise (fp16 8192 x 6000: 54.8 -> 53.1 us; 8192 x 6016: 52.6 / 52.4 us).  Forward (THN_FWD_SHAPES_TWO_ROWS):
