@@ -1028,7 +1028,7 @@ int thn_norm_bwd_reduce_partials(const void* workspace, int32_t num_partials, vo
     const auto blocks = [&](int cols) { return dim3(static_cast<unsigned>((N + cols - 1) / cols), static_cast<unsigned>(n)); };
     if (N >= thn::kReduceWideFrom) {
         hipLaunchKernelGGL(thn::reduce_partials_kernel<thn::kReduceColsWide>, blocks(thn::kReduceColsWide), dim3(256), 0, st, r);
-    } else if (N >= thn::kReduceMidFrom) {
+    } else if (N >= thn::kReduceMidFrom || N * n >= thn::kReduceMidFromBoth) {
         hipLaunchKernelGGL(thn::reduce_partials_kernel<thn::kReduceColsMid>, blocks(thn::kReduceColsMid), dim3(256), 0, st, r);
     } else {
         hipLaunchKernelGGL(thn::reduce_partials_kernel<thn::kReduceCols>, blocks(thn::kReduceCols), dim3(256), 0, st, r);

@@ -15,7 +15,9 @@ namespace thn {
 // x 32 slices (128-byte segments) up to 32768 columns, 64 columns x 16 slices (256-byte segments) from there on
 // (inside a forward + backward step, 32 against 64 columns: fp16 8192 x 6144 89.0 -> 86.6 us, 4096 x 16384
 // 113.3 -> 111.8 us, bf16 32768 x 8192 426.6 -> 425.1 us, 4096 x 32768 257.6 -> 258.6 us; against 16 columns the
-// longer segments are 2x faster at 16384 columns and more).
+// longer segments are 2x faster at 16384 columns and more).  With two gradients the stage has twice the workgroups
+// and moves twice the bytes: the 32-column form from 4096 columns on (bf16 LayerNorm 16384 x 4096: second stage inside
+// the step 4.6 -> 4.2 us; RMSNorm, one gradient, 3.55 -> 4.0 with it and stays at 16 columns).
 // blockIdx.y selects dW (0) or dB (1).
 // ---------------------------------------------------------------------------------------------------
 struct ReduceArgs {
@@ -31,6 +33,7 @@ constexpr int kReduceCols = 16;       // columns per workgroup up to kReduceMidF
 constexpr int kReduceColsMid = 32;    // 128-byte segments per partial row, 32 row slices
 constexpr int kReduceColsWide = 64;   // 256-byte segments, 16 row slices
 constexpr int kReduceMidFrom = 6144;
+constexpr int kReduceMidFromBoth = 8192;   // columns of dW and dB together
 constexpr int kReduceWideFrom = 32768;
 
 template <int COLS>
