@@ -6,7 +6,8 @@ the max abs error, the max error in ulps of the output dtype and how many elemen
 -- for this library and, on the same inputs against the same oracle, for torch.nn.functional.layer_norm /
 rms_norm on the GPU.  Where the table shows the literal bound is reachable it is asserted; where it is not (the
 stock op misses it as well: the result does not exist in float32 to that accuracy) the widened bounds of
-conftest.check_* apply, asserted by test_parity_gpu.py.  The table is written to gpurun_out/parity_report.md."""
+conftest.check_* apply, asserted by test_parity_gpu.py.  The table is written as parity_report.md / .json into the directory
+THN_REPORT_DIR names (default: the run's output folder under the repository root)."""
 import json
 import os
 
@@ -162,7 +163,7 @@ def test_literal_tolerance_report(name):
 
 
 def _write_report():
-    out_dir = os.path.join(ROOT, "gpurun_out")
+    out_dir = os.environ.get("THN_REPORT_DIR") or os.path.join(ROOT, "gpurun_out")
     os.makedirs(out_dir, exist_ok=True)
     with open(os.path.join(out_dir, "parity_report.json"), "w") as f:
         json.dump(REPORT, f, indent=1)
