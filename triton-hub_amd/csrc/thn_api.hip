@@ -297,14 +297,16 @@ constexpr int kTprList[] = {8, 16, 32, 64, 128, 256, 512, 1024};
 // widths from 1 KiB to 64 KiB.  HBM throughput peaks when a compute unit keeps about 1024 (one input stream) to
 // 2048 (two) 16-byte loads in flight and falls off by up to 15 % beyond that, so, for every row family: the
 // fewest threads per row with at most `kmax` vectors each, and
-//   norm forward, softmax forward, p-norm forward / backward: kmax 4, 256-thread workgroups up to 16 KiB rows;
+//   norm forward, softmax forward, p-norm forward / backward: kmax 4, 256-thread workgroups up to 16 KiB rows
+//             (the norm forward takes rows of 3 x 256 and, from 8 steps per workgroup on, of 2 x 256 vectors two
+//             at a time in 512 threads: plan_launch());
 //   norm backward: kmax 3 (x, dy, w, dW, dB are live per element), 4 for rows of at most 2 KiB (they share a
 //             wave: the float64 column sums need the instruction-level parallelism) and for rows that 1024
 //             threads cannot cover otherwise; 512-thread workgroups once a row spans two waves or more, which
 //             also halves the number of partial rows;
 //   softmax / normalize / epilogue backward (two or three input streams): kmax 2 up to 32 KiB rows.
-// Workgroups per compute unit: one (kDefaultBlocksPerCu), except where default_blocks_per_cu() or
-// narrow_row_blocks_per_cu() say otherwise.
+// Workgroups per compute unit: one (kDefaultBlocksPerCu), except where default_blocks_per_cu(),
+// narrow_row_blocks_per_cu() or the row-count dependent rules in plan_launch() say otherwise.
 constexpr int kDefaultBlocksPerCu = 1;
 
 int ceil_div(int a, int b) { return (a + b - 1) / b; }
