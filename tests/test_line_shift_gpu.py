@@ -25,6 +25,10 @@ CASES = [
     ("ln", torch.float32, 100, 6000),      # one workgroup per row, 100 * pitch is a multiple of 128
     ("ln", torch.float32, 101, 6000),      # 101 * pitch is not: unshifted
     ("rms", torch.float64, 300, 3000),     # float64 storage (pitch 24000)
+    ("ln", torch.float32, 3100, 8100),     # 1024-thread rows (2025 vectors, pitch 32400 = 16 mod 128) and enough of them for
+    ("rms", torch.float32, 3100, 8100),    # the forward to launch more workgroups than are resident (a grid that is not a
+                                           # multiple of 8: unshifted); the backward's grid keeps every workgroup on one phase
+    ("ln", torch.float16, 8200, 6000),     # 256-thread one-row forward with two workgroups per compute unit
 ]
 
 
