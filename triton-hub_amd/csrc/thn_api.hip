@@ -1029,11 +1029,11 @@ int thn_norm_bwd_reduce_partials(const void* workspace, int32_t num_partials, vo
     const hipStream_t st = static_cast<hipStream_t>(stream);
     const auto blocks = [&](int cols) { return dim3(static_cast<unsigned>((N + cols - 1) / cols), static_cast<unsigned>(n)); };
     if (N >= thn::kReduceWideFrom) {
-        hipLaunchKernelGGL(thn::reduce_partials_kernel<thn::kReduceColsWide>, blocks(thn::kReduceColsWide), dim3(256), 0, st, r);
+        hipLaunchKernelGGL((thn::reduce_partials_kernel<thn::kReduceColsWide, thn::kReduceAheadWide>), blocks(thn::kReduceColsWide), dim3(256), 0, st, r);
     } else if (N >= thn::kReduceMidFrom || N * n >= thn::kReduceMidFromBoth) {
-        hipLaunchKernelGGL(thn::reduce_partials_kernel<thn::kReduceColsMid>, blocks(thn::kReduceColsMid), dim3(256), 0, st, r);
+        hipLaunchKernelGGL((thn::reduce_partials_kernel<thn::kReduceColsMid, thn::kReduceAheadMid>), blocks(thn::kReduceColsMid), dim3(256), 0, st, r);
     } else {
-        hipLaunchKernelGGL(thn::reduce_partials_kernel<thn::kReduceCols>, blocks(thn::kReduceCols), dim3(256), 0, st, r);
+        hipLaunchKernelGGL((thn::reduce_partials_kernel<thn::kReduceCols, thn::kReduceAhead>), blocks(thn::kReduceCols), dim3(256), 0, st, r);
     }
     return hipGetLastError() == hipSuccess ? THN_OK : THN_E_LAUNCH;
 }
