@@ -93,10 +93,10 @@ SOFTMAX_KINDS = ("softmax", "softmin", "logsoftmax")
 # (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch), each scaled by what the same counter reads for a plain
 # copy kernel of known size.  Filled in from the summaries under profiles/; null for workloads not profiled.
 MEASURED_TRAFFIC_BYTES = {
-    # profiles/norm_kernels_rmsnorm_bf16_16384x4096_hbm_counters.txt: 262955 KiB fetched + 135168 KiB written
-    "rmsnorm_bf16_16384x4096": 407677952,
-    # the same file, LayerNorm rows: 263514 KiB fetched + 139264 KiB written
-    "layernorm_bf16_16384x4096": 412444876,
+    # profiles/norm_kernels_rmsnorm_bf16_16384x4096_hbm_counters.txt: 262958 KiB fetched + 135168 KiB written
+    "rmsnorm_bf16_16384x4096": 407680777,
+    # the same file, LayerNorm rows: 263505 KiB fetched + 139264 KiB written
+    "layernorm_bf16_16384x4096": 412435825,
     # profiles/softmax_kernels_softmax_bf16_16384x4096_stats_and_hbm_counters.txt (softmax_bwd_kernel)
     "softmax_bf16_16384x4096": 402817136,
     # profiles/pnorm_kernels_normalize_p2_bf16_16384x4096_stats_and_hbm_counters.txt (normalize_bwd_kernel)
