@@ -387,6 +387,30 @@ def test_forward_workgroups_per_compute_unit():
         run_and_compare("rms", x, dy, w, None, 1e-5, f"RMS {m}x{n}")
 
 
+def test_backward_over_few_rows_takes_half_the_workgroups():
+    """The backward's launch rule for few rows: when a full grid would visit at most two row blocks per workgroup
+    and the partial rows are a quarter or more of the bytes of x, dy and dx, half the workgroups are launched (half
+    the partial rows for the second stage).  The grids on both sides of the rule, and the oracle at sizes inside it."""
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    bf16, f32 = torch.bfloat16, torch.float32
+    grid = lambda ln, m, n, dt: _launch.query_launch(1, ln, m, n, dt)[3]
+    # 4096 bf16 columns: two rows per workgroup.  2 * cus rows = one row block per workgroup of a full grid
+    assert grid(False, 2 * cus, 4096, bf16) == cus // 2 and grid(True, 2 * cus, 4096, bf16) == cus // 2
+    assert grid(True, 4 * cus, 4096, bf16) == cus // 2          # two gradients: partial rows still a third of the bytes
+    assert grid(False, 4 * cus, 4096, bf16) == cus              # one gradient: a sixth
+    assert grid(True, 8 * cus, 4096, bf16) == cus               # four row blocks per workgroup
+    assert grid(True, cus, 4096, bf16) == cus // 2              # fewer row blocks than compute units: one each
+    assert grid(True, 4 * cus, 4096, f32) == cus                # float32 rows: one row per workgroup, four blocks each
+    g = torch.Generator().manual_seed(43)
+    for m, n, dt in ((2 * cus, 4096, bf16), (4 * cus - 1, 4096, bf16), (cus, 8192, bf16), (2 * cus + 1, 16384, bf16),
+                     (2 * cus, 4096, f32)):
+        announce(f"backward with half the workgroups: {dt} {m}x{n}")
+        x = (0.5 + torch.randn(m, n, generator=g)).to(dt); dy = torch.randn(m, n, generator=g).to(dt)
+        w = (1 + 0.1 * torch.randn(n, generator=g)).to(dt); b = (0.1 * torch.randn(n, generator=g)).to(dt)
+        run_and_compare("ln", x, dy, w, b, 1e-5, f"LN {m}x{n}")
+        run_and_compare("rms", x, dy, w, None, 1e-5, f"RMS {m}x{n}")
+
+
 # ---- size-independent properties at full benchmark sizes --------------------------------------------------------
 @pytest.mark.parametrize("name", ["c2_rms_bf16_llm", "c5a_ln_f32_hostile", "c4_ln_f32_small_hidden"])
 def test_properties_at_full_size(name):

@@ -515,6 +515,17 @@ int plan_launch(int which, int flavour, bool aligned, int64_t M, int64_t N, int 
         const int64_t iters = (row_blocks + grid_max - 1) / grid_max;
         grid = (row_blocks + iters - 1) / iters;      // every workgroup gets the same number of rows (+-1)
     }
+    // The backward over so few rows that a full grid visits at most two row blocks per workgroup and its float32
+    // partial rows are a quarter or more of the bytes of x, dy and dx: half the workgroups write half the partial
+    // rows, and the second stage reads half (bf16, forward + backward of one batch, RMSNorm / LayerNorm: 512 x 4096
+    // 14.6 / 17.5 -> 13.7 / 15.5 us, 1024 x 4096 LayerNorm 19.6 -> 18.6, 256 x 8192 16.3 / 22.0 -> 14.7 / 18.7,
+    // 512 x 16384 25.8 / 32.7 -> 24.7 / 30.8).  With more row blocks per workgroup, or partial rows that are a smaller
+    // part, the lost parallelism costs more (2048 x 4096 LayerNorm 23.7 -> 24.3, 1024 x 8192 26.3 -> 27.5, 4096 x 1024
+    // 19.4 -> 20.5 us); a quarter of the workgroups measured the same as half or slower.
+    if ((which == kNormBwd || which == kFusedBwd) && ov.bpc.load() <= 0 && grid >= cus && row_blocks <= 2 * grid) {
+        const int64_t n_grads = (flavour & 1) != 0 ? 2 : 1;
+        if (grid * 4 * n_grads * 4 >= M * bytes * 3) grid = (grid + 1) / 2;
+    }
     out->s = s;
     out->grid = static_cast<int>(grid);
     out->n_vecs = n_vecs;
