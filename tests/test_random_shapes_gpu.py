@@ -75,3 +75,38 @@ def test_random_problem(seed):
         w = (1 + 0.2 * torch.randn(n, generator=g)).to(dtype)
         b = (0.2 * torch.randn(n, generator=g)).to(dtype) if kind == "ln" else None
         fused_t.run_and_compare(kind, act, x, dy, w, b, eps, f"{what} {act}")
+
+
+def draw_large(seed):
+    """LayerNorm / RMSNorm problems of up to 40 M elements: 200 to 150000 rows, 64 elements to 64 KiB per row; half
+    of the widths whole 16-byte vectors, a quarter whole 128-byte lines."""
+    rng = np.random.default_rng(7000 + seed)
+    dtype = [torch.bfloat16, torch.float16, torch.float32][int(rng.integers(3))]
+    size = torch.empty(0, dtype=dtype).element_size()
+    n = log_uniform(rng, 64, 65536 // size)
+    r = rng.random()
+    if r < 0.5:
+        n = max(8, n // 8 * 8)
+    elif r < 0.75:
+        n = max(64, n // 64 * 64)
+    m = max(1, min(log_uniform(rng, 200, 150000), 40_000_000 // n))
+    kind = "ln" if rng.random() < 0.5 else "rms"
+    return kind, dtype, m, n
+
+
+@pytest.mark.parametrize("seed", range(32))
+def test_random_large_norm_problem(seed):
+    """The launch rules that depend on the row count (workgroups per compute unit, more workgroups than the chip
+    holds for the widest rows, half a grid for few rows, rows off 128-byte lines) at sizes nobody chose."""
+    from TritonHub.Normalization import _launch
+    kind, dtype, m, n = draw_large(seed)
+    fwd = tuple(_launch.query_launch(0, kind == "ln", m, n, dtype))[:4]
+    bwd = tuple(_launch.query_launch(1, kind == "ln", m, n, dtype))[:4]
+    print(f"\n[case] random large seed={seed} {kind} {dtype} M={m} N={n} forward{fwd} backward{bwd}", flush=True)
+    g = torch.Generator().manual_seed(seed)
+    x = (torch.randn(m, n, generator=g) * 2 + 0.5).to(dtype)
+    dy = torch.randn(m, n, generator=g).to(dtype)
+    w = (1 + 0.1 * torch.randn(n, generator=g)).to(dtype)
+    b = (0.1 * torch.randn(n, generator=g)).to(dtype) if kind == "ln" else None
+    parity_util.run_and_compare(kind, x, dy, w, b, 1e-5, f"random large {seed}",
+                                sample_chunks=8 if m * n > 8_000_000 else None)
