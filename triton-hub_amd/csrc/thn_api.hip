@@ -424,6 +424,21 @@ int plan_launch(int which, int flavour, bool aligned, int64_t M, int64_t N, int 
         M > 16 * static_cast<int64_t>(cus)) {
         s = Shape{2, 256, 512};
     }
+    // The norm backward over narrow rows: 2 vectors per thread in 512-thread workgroups -- eight waves per compute
+    // unit instead of the four of a 256-thread workgroup, which a backward step of 16-bit rows (twice the arithmetic
+    // per byte) does not fill a compute unit with.  16-bit rows of 17 to 192 vectors, and the rows of 129 to 192
+    // vectors of every type up to float32 (3 x 64 vectors in 256 threads otherwise).  Forward + backward of 2^26
+    // elements, % of 8 TB/s, RMSNorm / LayerNorm: bf16 N = 256: 76.9 / 73.3 -> 78.3 / 75.3; 640: 66.8 / 62.1 ->
+    // 74.8 / 66.4; 768: 73.1 / 69.0 -> 77.9 / 73.0; 1024: 77.3 / 74.5 -> 78.0 / 75.8; 1280: 72.1 / 66.6 -> 77.4 / 73.3;
+    // 1536: 75.8 / 70.4 -> 77.8 / 75.0; float32 N = 640: 79.2 / 75.0 -> 79.5 / 78.3; 768: 80.4 / 78.1 -> 80.9 / 79.5
+    // (float32 rows of up to 128 vectors are as fast or faster in 4-vector 256-thread workgroups: 80.9-82.0 %).
+    if (which == kNormBwd && aligned && ((bytes == 2 && n_vecs > 16 && n_vecs <= 192) ||
+                                         (bytes <= 4 && n_vecs > 128 && n_vecs <= 192))) {
+        int tpr = 16;
+        while (2 * tpr < n_vecs) tpr *= 2;
+        const Shape narrow{2, tpr, 512};
+        if (shape_compiled(which, aligned, ln16, narrow)) s = narrow;
+    }
     // Rows that start off 128-byte lines: two-row workgroups of 256-thread rows cannot put their requests on line
     // boundaries (the two rows differ in phase, line_shift_ok() below), one-row workgroups can.  Backward: as fast
     // otherwise (fp16 8192 x 6000: 54.8 -> 53.1 us; 8192 x 6016: 52.6 / 52.4 us).  Forward (THN_FWD_SHAPES_TWO_ROWS):
