@@ -43,6 +43,34 @@ def test_rows_off_line_boundaries(kind, dtype, m, n):
     parity_util.run_and_compare(kind, x, dy, w, b, 1e-5, f"line shift {kind} {m}x{n}")
 
 
+def test_two_vector_rows_stay_two_to_a_workgroup():
+    """Rows of 2 x 256 vectors at a pitch off 128-byte lines keep the two-row 512-thread workgroup (unshifted): one
+    such row per 256-thread workgroup would leave a compute unit four waves with two vectors each.  Only the
+    3 x 256-vector shape goes one row at a time to shift.  Also rows of 352-384 vectors and float32 rows of 704-768
+    vectors, which run as 2 vectors per thread on twice the threads."""
+    from TritonHub.Normalization import _launch
+    bf16, f16, f32 = torch.bfloat16, torch.float16, torch.float32
+    shape = lambda which, ln, m, n, dt: tuple(_launch.query_launch(which, ln, m, n, dt))[:3]
+    for which in (0, 1):
+        assert shape(which, False, 16384, 4000, bf16) == (2, 256, 512)       # 500 vectors, pitch 8000
+        assert shape(which, True, 16384, 2000, f32) == (2, 256, 512)
+        assert shape(which, True, 16384, 6000, f16) == (3, 256, 256)         # 750 vectors: one row, shifted
+        assert shape(which, False, 16384, 3072, bf16) == (2, 256, 512)       # 384 vectors
+        assert shape(which, False, 16384, 3072, f32) == (2, 512, 512)        # 768 vectors
+    assert shape(0, True, 16384, 3072, bf16) == (3, 128, 256)                # the 16-bit LayerNorm forward keeps 3 x 128
+    assert shape(1, True, 16384, 3072, bf16) == (2, 256, 512)
+    assert shape(0, False, 16384, 2688, bf16) == (3, 128, 256)               # 336 vectors: too empty for 2 x 256
+    g = torch.Generator().manual_seed(4000)
+    for m, n, dt in ((4200, 4000, bf16), (4200, 2000, f32), (4200, 3000, bf16), (4200, 2816, f16), (4200, 2900, f32)):
+        print(f"\n[case] two-vector rows {dt} M={m} N={n}", flush=True)
+        x = (torch.randn(m, n, generator=g) * 2 + 0.5).to(dt)
+        dy = torch.randn(m, n, generator=g).to(dt)
+        w = (1 + 0.1 * torch.randn(n, generator=g)).to(dt)
+        b = (0.1 * torch.randn(n, generator=g)).to(dt)
+        parity_util.run_and_compare("ln", x, dy, w, b, 1e-5, f"two-vector rows ln {m}x{n}")
+        parity_util.run_and_compare("rms", x, dy, w, None, 1e-5, f"two-vector rows rms {m}x{n}")
+
+
 SOFTMAX_CASES = [
     ("softmax", torch.float32, 523, 4100),       # 1025 vectors on 512 threads, all eight phases
     ("logsoftmax", torch.float32, 300, 6000),    # phases 0 / 64

@@ -424,6 +424,23 @@ int plan_launch(int which, int flavour, bool aligned, int64_t M, int64_t N, int 
         M > 16 * static_cast<int64_t>(cus)) {
         s = Shape{2, 256, 512};
     }
+    // Rows that fill 11/16 or more of a 2-vector shape with twice the threads go there instead of 3 vectors per
+    // thread: 352 to 384 vectors as 2 x 256 (forward and backward; not the 16-bit LayerNorm forward, which is 0-5 %
+    // slower that way), float32 rows of 704 to 768 vectors as 2 x 512.  Forward + backward of 2^26 elements, % of
+    // 8 TB/s, RMSNorm / LayerNorm: float32 N = 1408: 78.8 / 78.2 -> 81.0 / 79.8; 1536: 79.2 / 78.6 -> 81.8 / 80.5;
+    // 3072: 79.6 / 79.2 -> 82.0 / 80.5; bf16 N = 2816: 76.0 / 73.9 -> 77.2 / 74.5; 3072: 76.0 / 74.2 -> 78.4 / 74.7.
+    // Emptier rows lose: float32 N = 1152 forward 92 -> 101 us, bf16 N = 2688 LayerNorm 73.8 -> 70.7 %.
+    {
+        const bool norm_bwd = which == kNormBwd, norm_fwd = which == kNormFwd;
+        const bool ln_fwd16 = norm_fwd && bytes == 2 && (flavour & 1) != 0;
+        Shape two = s;
+        if (n_vecs >= 352 && n_vecs <= 384 && !ln_fwd16) two = Shape{2, 256, 512};
+        if (n_vecs >= 704 && n_vecs <= 768 && bytes == 4) two = Shape{2, 512, 512};
+        if ((norm_bwd || (norm_fwd && M > 16 * static_cast<int64_t>(cus))) && aligned && s.k == 3 &&
+            shape_compiled(which, aligned, ln16, two)) {
+            s = two;
+        }
+    }
     // The norm backward over narrow rows: 2 vectors per thread in 512-thread workgroups -- eight waves per compute
     // unit instead of the four of a 256-thread workgroup, which a backward step of 16-bit rows (twice the arithmetic
     // per byte) does not fill a compute unit with.  16-bit rows of 17 to 192 vectors, and the rows of 129 to 192
@@ -443,8 +460,11 @@ int plan_launch(int which, int flavour, bool aligned, int64_t M, int64_t N, int 
     // boundaries (the two rows differ in phase, line_shift_ok() below), one-row workgroups can.  Backward: as fast
     // otherwise (fp16 8192 x 6000: 54.8 -> 53.1 us; 8192 x 6016: 52.6 / 52.4 us).  Forward (THN_FWD_SHAPES_TWO_ROWS):
     // float32 16384 x 3000 69.5 -> 67.2 us, 65536 x 3000 290 -> 280 us, bf16 16384 x 6008 71.0 -> 69.1 us.
+    // Only the 3-vector shape: one row of 2 x 256 vectors per 256-thread workgroup keeps too little under way (bf16
+    // 16384 x 4000, forward + backward: 116.6 us that way, 107.8 as two unshifted rows per workgroup; LayerNorm 128.3 /
+    // 117.6; float32 16384 x 2000 114.7 / 106.9).
     if ((which == kNormBwd || which == kFusedBwd || which == kNormFwd) && aligned && pitch_bytes % 128 != 0 && s.tpr >= 256 &&
-        s.block == 2 * s.tpr && s.k * s.tpr - 7 >= n_vecs) {
+        s.k == 3 && s.block == 2 * s.tpr && s.k * s.tpr - 7 >= n_vecs) {
         Shape one_row = s;
         one_row.block = s.tpr;
         if (shape_compiled(which, aligned, ln16, one_row)) s = one_row;
