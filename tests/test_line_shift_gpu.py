@@ -60,8 +60,15 @@ def test_two_vector_rows_stay_two_to_a_workgroup():
     assert shape(0, True, 16384, 3072, bf16) == (3, 128, 256)                # the 16-bit LayerNorm forward keeps 3 x 128
     assert shape(1, True, 16384, 3072, bf16) == (2, 256, 512)
     assert shape(0, False, 16384, 2688, bf16) == (3, 128, 256)               # 336 vectors: too empty for 2 x 256
+    # 16-bit forward rows of 769-1024 vectors: 2 x 512 in 512 threads up to 896 vectors, and beyond up to 32 rows per
+    # compute unit; short kernels (two 256-thread workgroups per compute unit) and float32 rows keep 4 x 256
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    assert shape(0, True, 64 * cus, 6656, bf16) == (2, 512, 512) and shape(0, False, 64 * cus, 7168, f16) == (2, 512, 512)
+    assert shape(0, True, 32 * cus, 8192, bf16) == (2, 512, 512) and shape(0, True, 64 * cus, 8192, bf16) == (4, 256, 256)
+    assert shape(0, True, 8 * cus, 6656, bf16) == (4, 256, 256) and shape(0, True, 64 * cus, 3328, f32) == (4, 256, 256)
     g = torch.Generator().manual_seed(4000)
-    for m, n, dt in ((4200, 4000, bf16), (4200, 2000, f32), (4200, 3000, bf16), (4200, 2816, f16), (4200, 2900, f32)):
+    for m, n, dt in ((4200, 4000, bf16), (4200, 2000, f32), (4200, 3000, bf16), (4200, 2816, f16), (4200, 2900, f32),
+                     (2100, 6656, bf16), (2100, 7000, f16), (2100, 8192, bf16)):
         print(f"\n[case] two-vector rows {dt} M={m} N={n}", flush=True)
         x = (torch.randn(m, n, generator=g) * 2 + 0.5).to(dt)
         dy = torch.randn(m, n, generator=g).to(dt)

@@ -441,6 +441,18 @@ int plan_launch(int which, int flavour, bool aligned, int64_t M, int64_t N, int 
             s = two;
         }
     }
+    // The forward over 16-bit rows of 769 to 1024 vectors: one row of 4 x 256 vectors per 256-thread workgroup is one
+    // wave per SIMD, and a row's arithmetic and two reduction rounds then set a floor of 1.3 us per row for LayerNorm
+    // whatever the width (4608 rows: 25 us at every width from 6400 to 8192 columns).  2 x 512 vectors in 512 threads
+    // instead: for rows of up to 896 vectors at every row count, for wider ones up to 32 rows per compute unit (bf16
+    // forward, RMSNorm / LayerNorm: 4608 x 6656 19.1 / 24.9 -> 18.9 / 21.0 us, 16384 x 6656 74.9 / 79.9 -> 72.1 / 74.7,
+    // 32768 x 7168 158.0 / 157.7 -> 156.9 / 156.1, 4608 x 8192 22.8 / 25.4 -> 22.8 / 23.8; from 16384 rows on the
+    // rows of more than 896 vectors are 1-5 % faster as 4 x 256: 16384 x 8192 87.8 / 87.7 against 89.0 / 90.8).
+    // Up to 8 rows per compute unit the 256-thread shape takes two workgroups per compute unit (below) and stays.
+    if (which == kNormFwd && aligned && bytes == 2 && s.k == 4 && s.tpr == 256 && s.block == 256 &&
+        M > 8 * static_cast<int64_t>(cus) && (n_vecs <= 896 || M <= 32 * static_cast<int64_t>(cus))) {
+        s = Shape{2, 512, 512};
+    }
     // The norm backward over narrow rows: 2 vectors per thread in 512-thread workgroups -- eight waves per compute
     // unit instead of the four of a 256-thread workgroup, which a backward step of 16-bit rows (twice the arithmetic
     // per byte) does not fill a compute unit with.  16-bit rows of 17 to 192 vectors, and the rows of 129 to 192
