@@ -57,6 +57,11 @@ def test_two_vector_rows_stay_two_to_a_workgroup():
         assert shape(which, True, 16384, 6000, f16) == (3, 256, 256)         # 750 vectors: one row, shifted
         assert shape(which, False, 16384, 3072, bf16) == (2, 256, 512)       # 384 vectors
         assert shape(which, False, 16384, 3072, f32) == (2, 512, 512)        # 768 vectors
+    # 3 x 256 vectors with a sixth or more of the slots idle: two unshifted rows per workgroup in the forward and in the
+    # 16-bit LayerNorm backward, one shifted row at a time in the other backwards
+    assert shape(0, False, 16384, 4248, bf16) == (3, 256, 512) and shape(0, True, 16384, 2204, f32) == (3, 256, 512)
+    assert shape(1, True, 16384, 4248, bf16) == (3, 256, 512) and shape(1, False, 16384, 4248, bf16) == (3, 256, 256)
+    assert shape(1, True, 16384, 2204, f32) == (3, 256, 256)
     assert shape(0, True, 16384, 3072, bf16) == (3, 128, 256)                # the 16-bit LayerNorm forward keeps 3 x 128
     assert shape(1, True, 16384, 3072, bf16) == (2, 256, 512)
     assert shape(0, False, 16384, 2688, bf16) == (3, 128, 256)               # 336 vectors: too empty for 2 x 256
@@ -68,7 +73,7 @@ def test_two_vector_rows_stay_two_to_a_workgroup():
     assert shape(0, True, 8 * cus, 6656, bf16) == (4, 256, 256) and shape(0, True, 64 * cus, 3328, f32) == (4, 256, 256)
     g = torch.Generator().manual_seed(4000)
     for m, n, dt in ((4200, 4000, bf16), (4200, 2000, f32), (4200, 3000, bf16), (4200, 2816, f16), (4200, 2900, f32),
-                     (2100, 6656, bf16), (2100, 7000, f16), (2100, 8192, bf16)):
+                     (2100, 6656, bf16), (2100, 7000, f16), (2100, 8192, bf16), (2100, 4248, bf16), (2100, 2204, f32)):
         print(f"\n[case] two-vector rows {dt} M={m} N={n}", flush=True)
         x = (torch.randn(m, n, generator=g) * 2 + 0.5).to(dt)
         dy = torch.randn(m, n, generator=g).to(dt)

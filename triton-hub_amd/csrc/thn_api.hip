@@ -477,9 +477,17 @@ int plan_launch(int which, int flavour, bool aligned, int64_t M, int64_t N, int 
     // 117.6; float32 16384 x 2000 114.7 / 106.9).
     if ((which == kNormBwd || which == kFusedBwd || which == kNormFwd) && aligned && pitch_bytes % 128 != 0 && s.tpr >= 256 &&
         s.k == 3 && s.block == 2 * s.tpr && s.k * s.tpr - 7 >= n_vecs) {
+        // ... and only rows that fill the shape: a one-row 256-thread workgroup is one wave per SIMD, and with a sixth
+        // or more of its slots idle the row's arithmetic is no longer covered (bf16 16384 x 4248, 531 vectors, forward
+        // RMSNorm / LayerNorm 55.5 / 62.4 us one row at a time, 48.3 / 50.0 two unshifted rows; 4760 columns 58.2 /
+        // 63.2 against 55.8 / 58.5; 5336 columns, 667 vectors, the same both ways; float32 16384 x 2204 55.7 / 57.8
+        // against 50.3 / 50.8).  The 16-bit LayerNorm backward likewise up to 704 vectors (16384 x 4248 forward +
+        // backward 143.8 -> 131.2 us, 4760: 148.0 -> 139.6, 5336: 153.4 -> 149.3; fp16 8192 x 6000, 750 vectors: 86.7
+        // one row at a time, 88.7 two); the other backwards are 1-3 % faster one row at a time at every fill.
+        const bool too_empty = (which == kNormFwd && n_vecs <= 640) || (which == kNormBwd && ln16 && n_vecs <= 704);
         Shape one_row = s;
         one_row.block = s.tpr;
-        if (shape_compiled(which, aligned, ln16, one_row)) s = one_row;
+        if (!too_empty && shape_compiled(which, aligned, ln16, one_row)) s = one_row;
     }
     const Override& ov = g_override[which];
     Shape cand = s;
