@@ -343,14 +343,20 @@ def test_wide_rows_many_per_workgroup(dtype, widths):
 
 @pytest.mark.parametrize("dtype,n", [(torch.bfloat16, 32768), (torch.float32, 16384), (torch.float16, 24576)])
 def test_wide_rows_forward_with_more_workgroups_than_the_chip_holds(dtype, n):
-    """From 12 rows of more than 32 KiB per compute unit on, the forward launches up to four times as many workgroups
-    as are resident at once (twice for the 16-bit LayerNorm); below that it does not.  3100 rows leave the last
-    grid-stride step partly filled."""
+    """From 12 rows of more than 48 KiB (4 x 1024 vectors) per compute unit on, the forward launches up to four times as
+    many workgroups as are resident at once (twice for the 16-bit LayerNorm) when that makes whole rounds of them;
+    rows of 3 x 1024 vectors and row counts that would leave a round half empty keep one workgroup per compute unit.
+    The oracle comparison runs 16 * cus - 3 rows, which leave the last grid-stride step partly filled."""
     cus = torch.cuda.get_device_properties(0).multi_processor_count
-    m = 12 * cus + 28
-    grid_rms = _launch.query_launch(0, False, m, n, dtype)[3]
-    grid_ln = _launch.query_launch(0, True, m, n, dtype)[3]
-    assert cus < grid_rms <= 4 * cus and cus < grid_ln <= (2 if dtype != torch.float32 else 4) * cus, (grid_rms, grid_ln)
+    grid_rms = _launch.query_launch(0, False, 16 * cus, n, dtype)[3]
+    grid_ln = _launch.query_launch(0, True, 16 * cus, n, dtype)[3]
+    m = 16 * cus - 3
+    if _launch.query_launch(0, False, m, n, dtype)[0] == 4:
+        assert grid_rms == 4 * cus and grid_ln == (2 if dtype != torch.float32 else 4) * cus, (grid_rms, grid_ln)
+        assert _launch.query_launch(0, False, m, n, dtype)[3] == 2 * cus               # two whole rounds, the last rows short
+        assert _launch.query_launch(0, False, 12 * cus + 128, n, dtype)[3] <= cus      # 2.5 rounds of workgroups: not taken
+    else:
+        assert grid_rms <= cus and grid_ln <= cus, (grid_rms, grid_ln)
     assert _launch.query_launch(0, False, 8 * cus, n, dtype)[3] == cus
     assert _launch.query_launch(1, False, m, n, dtype)[3] <= cus          # the backward: one partial row per workgroup
     g = torch.Generator().manual_seed(37)

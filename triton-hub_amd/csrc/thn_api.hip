@@ -560,10 +560,20 @@ int plan_launch(int which, int flavour, bool aligned, int64_t M, int64_t N, int 
     // gained (2048 rows in 512 workgroups: 46.8 -> 47.0, LayerNorm 47.7 -> 48.5; 3072 rows in 768: 70.9 -> 70.4);
     // narrower rows measured the same or slower this way at any row count, and the backward would pay for it with
     // more partial rows.
-    if (which == kNormFwd && aligned && s.block == 1024 && ov.bpc.load() <= 0) {
+    // Rows of 4 x 1024 vectors only: with 3 vectors per thread the larger grids are 1-6 % slower (float32 3584 x 9080
+    // 44.9 -> 47.8 us, 3072 x 10240 42.9 -> 44.0, bf16 3584 x 20480 50.4 -> 51.6).  And only grids that are whole
+    // rounds of workgroups, or close to four of them: 3200 rows of 64 KiB in 640 workgroups (two and a half rounds)
+    // took 73.9 us against 72.4 in 247.
+    if (which == kNormFwd && aligned && s.block == 1024 && s.k == 4 && ov.bpc.load() <= 0 && row_blocks >= 12 * grid_max) {
         const int64_t most = (bytes == 2 && (flavour & 1) != 0) ? 2 : 4;
-        const int64_t fits = row_blocks >= 12 * grid_max ? row_blocks / (4 * grid_max) : 1;
-        grid_max *= fits < most ? fits : most;
+        int64_t f = row_blocks / (4 * grid_max);
+        if (f > most) f = most;
+        for (; f > 1; --f) {
+            const int64_t iters = (row_blocks + grid_max * f - 1) / (grid_max * f);
+            const int64_t g = (row_blocks + iters - 1) / iters;
+            if (g % grid_max == 0 || 4 * g >= 15 * grid_max) break;
+        }
+        if (f > 1) grid_max *= f;
     }
     int64_t grid = row_blocks;
     if (grid > grid_max) {
