@@ -364,6 +364,11 @@ Shape heuristic_shape(int which, bool aligned, bool ln16, int n_vecs) {
     if (which != kNormBwd && which != kFusedBwd) s.block = s.tpr > 256 ? s.tpr : 256;
     else s.block = s.tpr >= 128 ? (s.tpr > 512 ? s.tpr : 512) : 256;
     if (which == kNormFwd && s.k == 3 && s.tpr == 256) s.block = 512;     // THN_FWD_SHAPES_TWO_ROWS
+    // The norm backward over rows of up to 16 vectors (one vector per thread): 512-thread workgroups, two per compute
+    // unit (forward + backward of 2^26 elements, % of 8 TB/s, RMSNorm / LayerNorm: bf16 N = 96 68.8 / 66.1 ->
+    // 75.0 / 72.9, N = 128 75.9 / 74.1 -> 78.3 / 76.3, N = 64 71.1 / 68.1 -> 72.1 / 68.9; float32 N = 64 79.5 / 76.0 ->
+    // 80.3 / 78.4).
+    if (which == kNormBwd && aligned && n_vecs <= 16 && s.k == 1) s.block = 512;
     return s;
 }
 
