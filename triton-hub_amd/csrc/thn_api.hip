@@ -305,6 +305,11 @@ constexpr int kTprList[] = {8, 16, 32, 64, 128, 256, 512, 1024};
 //             threads cannot cover otherwise; 512-thread workgroups once a row spans two waves or more, which
 //             also halves the number of partial rows;
 //   softmax / normalize / epilogue backward (two or three input streams): kmax 2 up to 32 KiB rows.
+// A second finding runs through the norm rules of plan_launch(): a compute unit wants eight waves of a row kernel,
+// not four.  One 256-thread workgroup per compute unit (one wave per SIMD) leaves a row's arithmetic and reduction
+// rounds uncovered -- the 16-bit LayerNorm forward then takes 1.3 us per row at any width -- so the backward of
+// narrow rows, the rows that fill most of a 2-vector shape and the 16-bit forward rows of 769 to 1024 vectors run in
+// 512-thread workgroups, and one-row-at-a-time workgroups (the line shift) are kept for rows that fill their shape.
 // Workgroups per compute unit: one (kDefaultBlocksPerCu), except where default_blocks_per_cu(),
 // narrow_row_blocks_per_cu() or the row-count dependent rules in plan_launch() say otherwise.
 constexpr int kDefaultBlocksPerCu = 1;
