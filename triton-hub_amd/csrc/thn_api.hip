@@ -590,6 +590,14 @@ int plan_launch(int which, int flavour, bool aligned, int64_t M, int64_t N, int 
         const int64_t iters = (row_blocks + grid_max - 1) / grid_max;
         grid = (row_blocks + iters - 1) / iters;      // every workgroup gets the same number of rows (+-1)
     }
+    // More than one workgroup per compute unit: a grid between whole multiples of the compute units would leave some
+    // of them one workgroup more than others (384 workgroups of 3 row blocks on 256 compute units: half of them work
+    // twice as long), so it is rounded up to the next multiple, where the row blocks differ by one at most (bf16
+    // RMSNorm forward, 9216 x 1024: 7.16 -> 6.91 us; 2304 x 3072: 6.14 -> 5.78).
+    if (grid > cus && grid % cus != 0) {
+        const int64_t up = (grid + cus - 1) / cus * cus;
+        if (up <= grid_max && up <= row_blocks) grid = up;
+    }
     // The backward over so few rows that a full grid visits at most two row blocks per workgroup and its float32
     // partial rows are a quarter or more of the bytes of x, dy and dx: half the workgroups write half the partial
     // rows, and the second stage reads half (bf16, forward + backward of one batch, RMSNorm / LayerNorm: 512 x 4096
