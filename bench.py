@@ -561,59 +561,6 @@ def ceiling_main(args, lib, dev):
         "thn_act_fwd on 1 row": round(timed(lambda b_: act_fwd(b_, 1), 400), 2),
         "torch copy_ of 8 elements": round(timed(lambda b_: b_["y"][0, :8].copy_(b_["x"][0, :8]), 400), 2)}
 
-    # ---- the probes of libthnprobe.so (triton-hub_amd/csrc/thn_probe.hip): the norm kernels' row loop without its
-    # arithmetic, with the time every workgroup finished; empty launches; device-scope atomics on one address ----
-    probe_path = os.path.join(ROOT, "triton-hub_amd", "TritonHub", "libthnprobe.so")
-    if not os.path.exists(probe_path):
-        sys.exit(f"bench.py --ceiling: {probe_path} is missing (make -C triton-hub_amd/csrc)")
-    probe = ctypes.CDLL(probe_path)
-    vp, i64 = ctypes.c_void_p, ctypes.c_int64
-    probe.thnp_empty.argtypes = [ctypes.c_int, ctypes.c_int, vp]
-    probe.thnp_copy.argtypes = [vp, vp, i64, vp, vp]
-    probe.thnp_atomic_burst.argtypes = [vp, ctypes.c_int, vp]
-    probe.thnp_atomic_chain.argtypes = [vp, vp, ctypes.c_int, vp]
-    tick_us = 1e3 / probe.thnp_wall_clock_khz()
-    out["probe_empty_launch_us"] = {
-        "1 workgroup x 64 threads": round(timed(lambda b_: probe.thnp_empty(1, 64, stream), 2000), 2),
-        "256 workgroups x 256 threads": round(timed(lambda b_: probe.thnp_empty(256, 256, stream), 2000), 2),
-        "256 workgroups x 1024 threads": round(timed(lambda b_: probe.thnp_empty(256, 1024, stream), 2000), 2)}
-    nbytes = 16384 * n * s
-    pts = [(m_, timed(lambda b_, m_=m_: probe.thnp_copy(p(b_["x"]), p(b_["y"]), m_ * n * s, 0, stream), 40)) for m_ in rows_list]
-    a0, slope = fit(pts)
-    out["streams"]["probe copy: the norm kernels' row loop without arithmetic (1 read + 1 write)"] = {
-        "us_per_launch": {str(m_): round(t, 2) for m_, t in pts},
-        "GBps_at_16384_rows": round(2 * nbytes / dict(pts)[16384] / 1e3, 1),
-        "fit_intercept_us": round(a0, 2), "fit_slope_GBps": round(2 * n * s / slope / 1e3, 1)}
-    ts = torch.zeros(256 * 4, dtype=torch.int64, device=dev)
-    ends, starts, drained = [], [], []
-    for rep in range(8):
-        b_ = sets[rep % N_BUFFER_SETS]
-        assert probe.thnp_copy(p(b_["x"]), p(b_["y"]), nbytes, p(ts), stream) == 0
-        torch.cuda.synchronize()
-        t = ts.cpu().reshape(256, 4).double() * tick_us
-        t0 = float(t[:, 0].min())
-        starts.append(sorted((t[:, 0] - t0).tolist()))
-        ends.append(sorted((t[:, 2] - t0).tolist()))
-        drained.append(float((t[:, 3] - t0).max()))
-    med = lambda v: sorted(v)[len(v) // 2]
-    out["probe_copy_timeline_us"] = {
-        "what": "128 MiB copied by 256 workgroups with equal shares, 8 launches: when the workgroups left their loops, "
-                "in microseconds after the first workgroup started (median over the launches)",
-        "last_workgroup_started": round(med([v[-1] for v in starts]), 2),
-        "loop_end_first": round(med([v[0] for v in ends]), 2), "loop_end_median": round(med([v[128] for v in ends]), 2),
-        "loop_end_last": round(med([v[-1] for v in ends]), 2), "last_store_acknowledged": round(med(drained), 2)}
-    ctr = torch.zeros(64, dtype=torch.int32, device=dev)
-    t8 = timed(lambda b_: probe.thnp_atomic_burst(p(ctr), 8, stream), 50)
-    t32 = timed(lambda b_: probe.thnp_atomic_burst(p(ctr), 32, stream), 50)
-    ticks = torch.zeros(2, dtype=torch.int64, device=dev)
-    assert probe.thnp_atomic_chain(p(ctr), p(ticks), 500, stream) == 0
-    torch.cuda.synchronize()
-    out["probe_device_scope_atomics"] = {
-        "ns_per_atomic_on_one_address": round((t32 - t8) * 1e3 / (24 * 256), 1),
-        "what": "256 workgroups x 8 and x 32 relaxed device-scope fetch-adds on ONE counter: (t32 - t8) / (24 * 256); a "
-                "ticket per workgroup and row step of the forward would be 8192 of them in 44 us",
-        "us_per_launch_8_each": round(t8, 2), "us_per_launch_32_each": round(t32, 2),
-        "round_trip_us_idle_gpu": round(float(ticks[0]) * tick_us / 500, 3)}
     print(json.dumps(out), flush=True)
 
 
