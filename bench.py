@@ -89,25 +89,47 @@ ACT_NAMES = ["gelu", "gelu_tanh", "silu", "relu", "leaky_relu", "relu6", "sigmoi
 ACT_PARAMS = {"leaky_relu": (0.01, 0.0), "softplus": (1.0, 20.0), "threshold": (0.1, 20.0)}
 SOFTMAX_KINDS = ("softmax", "softmin", "logsoftmax")
 
-# HBM bytes per launch of the backward dx / partial-sum kernel, from two rocprofv3 --pmc runs of this script
-# (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch), each scaled by what the same counter reads for a plain
-# copy kernel of known size.  Filled in from the summaries under profiles/; null for workloads not profiled.
-MEASURED_TRAFFIC_BYTES = {
-    # profiles/norm_kernels_rmsnorm_bf16_16384x4096_hbm_counters.txt: 262958 KiB fetched + 135168 KiB written
-    "rmsnorm_bf16_16384x4096": 407680777,
-    # the same file, LayerNorm rows: 263505 KiB fetched + 139264 KiB written
-    "layernorm_bf16_16384x4096": 412435825,
-    # profiles/softmax_kernels_softmax_bf16_16384x4096_stats_and_hbm_counters.txt (softmax_bwd_kernel)
-    "softmax_bf16_16384x4096": 402817136,
-    # profiles/pnorm_kernels_normalize_p2_bf16_16384x4096_stats_and_hbm_counters.txt (normalize_bwd_kernel)
-    "normalize_p2_bf16_16384x4096": 403137354,
-    # profiles/act_kernels_gelu_tanh_bf16_16384x4096_stats_and_hbm_counters.txt (act_flat_kernel backward)
-    "act_gelu_tanh_bf16_16384x4096": 402671069,
-}
+# HBM bytes per launch of a workload's dominant kernel: not a figure of this run (counters need rocprofv3), but the
+# one the named summary under profiles/ holds, read from that file when the line is printed.  A summary carries
+# it as a line
+#     bench.traffic <workload> <kernel> <bytes per launch> <cache policy of the run>
+# (from two rocprofv3 --pmc runs of this script, FETCH_SIZE then WRITE_SIZE, each scaled by what the same counter
+# reads for a plain copy of known size); a workload without such a line reports null.
+PROFILES_DIR = os.path.join(ROOT, "profiles")
+
+
+def traffic_from_profiles(workload):
+    """{"bytes": ..., "kernel": ..., "cache_policy": ..., "source": "profiles/<file>"} or None."""
+    try:
+        names = sorted(os.listdir(PROFILES_DIR))
+    except OSError:
+        return None
+    for name in names:
+        if not name.endswith((".txt", ".md")):
+            continue
+        try:
+            with open(os.path.join(PROFILES_DIR, name)) as fh:
+                for line in fh:
+                    parts = line.split()
+                    if len(parts) >= 4 and parts[0] == "bench.traffic" and parts[1] == workload:
+                        return {"bytes": int(parts[3]), "kernel": parts[2],
+                                "cache_policy": parts[4] if len(parts) > 4 else None, "source": "profiles/" + name}
+        except (OSError, ValueError):
+            continue
+    return None
 
 
 # Untimed steps of the norm workloads before the W warm-up steps (see the timed region of the norm bench).
 PREROLL_STEPS = 150
+
+
+def traffic_fields(workload):
+    """`traffic` of the roofline object and where it comes from."""
+    t = traffic_from_profiles(workload)
+    if t is None:
+        return {"traffic": None}
+    return {"traffic": t["bytes"], "traffic_source": f"{t['source']} (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of {t['kernel']}, "
+                                                     f"cache policy {t['cache_policy']}; not counted in this run)"}
 
 
 def algorithmic_bytes(kind, m, n, s, sw):
@@ -132,6 +154,7 @@ class NormBench:
         self.torch, self.lib, self.native = torch, lib, _native
         kind, m, n, dname = WORKLOADS[workload]
         self.workload, self.fused_act = workload, -1
+        self.x_flag = _native.X_KEEP          # this bench's forward calls say how they read x: see set_policy()
         if "+" in kind:
             kind, act_name = kind.split("+")
             self.fused_act = FUSED_ACTS.index(act_name)
@@ -172,15 +195,19 @@ class NormBench:
         self.fwd_bytes, self.bwd_bytes = algorithmic_bytes(kind, m, n, self.s, self.s)
         self.step_bytes = self.fwd_bytes + self.bwd_bytes
 
+    def set_policy(self, policy):
+        """'keep': the forward leaves x in the caches for the backward (THN_X_KEEP); 'stream': it does not."""
+        self.x_flag = {"keep": self.native.X_KEEP, "stream": self.native.X_STREAM}[policy]
+
     # ---- the launches ----
     def forward(self, b_):
         p, lib, m, n, code = self.native.ptr, self.lib, self.m, self.n, self.code
         if self.fused_act >= 0:
             rc = lib.thn_norm_act_fwd(p(b_["x"]), n, p(b_["y"]), n, p(self.w), p(self.b), p(b_["mean"]), p(b_["rstd"]),
-                                      m, n, 1e-6, self.fused_act, code, code, self.stream)
+                                      m, n, 1e-6, self.fused_act, code | self.x_flag, code, self.stream)
         else:
             rc = lib.thn_norm_fwd(p(b_["x"]), n, p(b_["y"]), n, p(self.w), p(self.b), p(b_["mean"]), p(b_["rstd"]),
-                                  m, n, 1e-6, code, code, self.stream)
+                                  m, n, 1e-6, code | self.x_flag, code, self.stream)
         assert rc == 0, self.native.strerror(rc)
 
     def backward(self, b_):
@@ -292,43 +319,88 @@ class NormBench:
 
 
 FUSED_ACTS = ["gelu", "gelu_tanh", "silu", "relu"]
-REUSE_NOTE = ("one step = forward and backward of the SAME batch, back to back: the backward re-reads the x its forward "
-              "has just read, and a part of it is still in the 256 MB Infinity Cache (the forward loads x with "
-              "cache-allocating loads; everything else streams). 'no_reuse' is the same step with the backward working on "
-              "the batch whose forward ran two steps earlier (four batches, 2.1 GB, in rotation): nothing of its "
-              "operands is left in any cache.")
+STEP_NOTE = ("one step = forward and backward of the SAME batch, back to back, the forward under the 'keep' cache policy "
+             "(THN_X_KEEP: x is loaded with cache-allocating loads, everything else streams): the backward re-reads the x "
+             "its forward has just read, and a part of it is still in the 256 MB Infinity Cache.")
+NO_REUSE_NOTE = ("the same step with the backward working on the batch whose forward ran two steps earlier (four batches "
+                 "in rotation: 1.3 GB of other traffic lie between the two reads of an x, nothing of a backward's operands is "
+                 "left in any cache -- what a training step sees when the rest of the network runs between a layer's forward "
+                 "and its backward), the forward under the 'stream' cache policy (THN_X_STREAM)")
+
+# The other configurations of the benchmark contract, measured after the headline on the default run.
+CONTRACT_CONFIGS = ["layernorm_bf16_32768x8192", "layernorm_f32_1048576x256", "layernorm_f16_8192x6000_hostile",
+                    "layernorm_f32_8192x6000_hostile", "rmsnorm_f16_4096x16384_outliers", "rmsnorm_f32_4096x16384_outliers",
+                    "layernorm_f32_200x128_quickstart"]
 
 
-def measure_norm(bench, args, full):
-    """The numbers of one norm workload.  `full`: also the no-reuse step and the isolated launches."""
-    ms_per_step, ms_events = bench.timed_steps(args.steps, args.warmup, preroll=PREROLL_STEPS)
+def measure_norm(bench, args, policy="keep", lag=0, preroll=PREROLL_STEPS, with_kernels=True):
+    """The step of one norm workload under one cache policy; lag = 0: the backward of the batch just forwarded,
+    lag = 2: of the batch forwarded two steps earlier."""
+    bench.set_policy(policy)
+    ms_per_step, ms_events = bench.timed_steps(args.steps, args.warmup, lag=lag, preroll=preroll)
     gbps = bench.step_bytes / (ms_per_step * 1e-3) / 1e9
     res = {"ms_per_step": round(ms_per_step, 5), "GBps": round(gbps, 1),
            "pct_of_hbm_peak": round(100.0 * gbps / HBM_PEAK_GBPS, 2),
            "ms_per_step_by_hip_events": round(ms_events, 5),
-           "pct_of_hbm_peak_by_hip_events": round(100.0 * bench.step_bytes / (ms_events * 1e-3) / 1e9 / HBM_PEAK_GBPS, 2)}
-
-    def kernels(ms_step, lag):
+           "pct_of_hbm_peak_by_hip_events": round(100.0 * bench.step_bytes / (ms_events * 1e-3) / 1e9 / HBM_PEAK_GBPS, 2),
+           "rows_per_s": round(bench.m / (ms_per_step * 1e-3))}
+    if with_kernels:
         # An event between two kernels keeps the second from starting the moment the first ends: the three
         # intervals of an instrumented step add up to more than the plain step.  That surplus is the events' own
         # cost; it is taken off the three intervals in equal parts (rocprofv3's kernel durations of the same run
         # agree with the result to half a microsecond).
         k = bench.kernels_in_step(args.steps, lag)
-        if k is None:
-            return None
-        cost = (sum(k) - ms_step * 1e3) / 3.0
-        return {"forward": round(k[0] - cost, 2), "backward_dx_partials": round(k[1] - cost, 2),
-                "backward_reduce_partials": round(k[2] - cost, 2), "event_cost_taken_off_each": round(cost, 2)}
-
-    k = kernels(ms_per_step, 0)
-    if k is not None:
-        res["kernels_us"] = k
-    if full and bench.fused_act < 0:
-        ms_nr, _ = bench.timed_steps(args.steps, min(args.warmup, 5), lag=2)
-        res["no_reuse"] = {"ms_per_step": round(ms_nr, 5),
-                           "pct_of_hbm_peak": round(100.0 * bench.step_bytes / (ms_nr * 1e-3) / 1e9 / HBM_PEAK_GBPS, 2),
-                           "kernels_us": kernels(ms_nr, 2)}
+        if k is not None:
+            cost = (sum(k) - ms_per_step * 1e3) / 3.0
+            res["kernels_us"] = {"forward": round(k[0] - cost, 2), "backward_dx_partials": round(k[1] - cost, 2),
+                                 "backward_reduce_partials": round(k[2] - cost, 2),
+                                 "event_cost_taken_off_each": round(cost, 2)}
     return res
+
+
+def norm_roofline(bench, cold, warm):
+    """The dominant kernel -- the backward dx / partial-sum kernel -- against the HBM roofline.  `achieved` is taken
+    from the kernel on a batch that no cache holds (the no-reuse step): only then are the algorithmic bytes HBM
+    bytes.  Inside the same-batch step a part of x comes from the Infinity Cache; that figure is reported beside it
+    and is not an HBM fraction."""
+    roofline = {"bound": "hbm", "kernel": "norm_bwd_kernel (backward dx + dW/dB partials)", "peak": HBM_PEAK_GBPS,
+                "unit": "GB/s", "algorithmic_bytes_per_launch": bench.bwd_bytes, **traffic_fields(bench.workload)}
+    if cold is not None and "kernels_us" in cold:
+        us = cold["kernels_us"]["backward_dx_partials"]
+        achieved = bench.bwd_bytes / (us * 1e-6) / 1e9
+        roofline.update({"achieved": round(achieved, 1), "frac": round(achieved / HBM_PEAK_GBPS, 4), "avg_launch_us": us,
+                         "measured": "HIP events on the launch stream around the kernel inside the no-reuse step (its "
+                                     "operands in no cache), less the events' own cost"})
+    if warm is not None and "kernels_us" in warm:
+        us = warm["kernels_us"]["backward_dx_partials"]
+        ach = bench.bwd_bytes / (us * 1e-6) / 1e9
+        roofline["in_step_cache_assisted"] = {
+            "avg_launch_us": us, "algorithmic_GBps": round(ach, 1), "frac_of_hbm_peak": round(ach / HBM_PEAK_GBPS, 4),
+            "note": "inside the same-batch step part of x is served by the Infinity Cache: algorithmic bytes per second, "
+                    "not HBM bytes per second"}
+        if "achieved" not in roofline:
+            roofline.update({"achieved": round(ach, 1), "frac": round(ach / HBM_PEAK_GBPS, 4), "avg_launch_us": us,
+                             "measured": "HIP events around the kernel inside the same-batch step (cache-assisted)"})
+    return roofline
+
+
+def config_summary(lib, dev, workload, args):
+    """One more configuration of the benchmark contract: the step as defined, the no-reuse step, the kernels."""
+    bench = NormBench(lib, dev, workload)
+    short = argparse.Namespace(steps=args.steps, warmup=min(args.warmup, 5))
+    warm = measure_norm(bench, short, "keep", 0, preroll=min(PREROLL_STEPS, 30))
+    cold = measure_norm(bench, short, "stream", 2, preroll=0)
+    fwd_shape, bwd_shape = bench.shapes()
+    out = {"op": "LayerNorm" if bench.ln else "RMSNorm", "rows": bench.m, "hidden": bench.n, "dtype": bench.dname,
+           "algorithmic_bytes_per_step": bench.step_bytes,
+           "ms_per_step": warm["ms_per_step"], "GBps": warm["GBps"], "pct_of_hbm_peak": warm["pct_of_hbm_peak"],
+           "rows_per_s": warm["rows_per_s"], "kernels_us": warm.get("kernels_us"),
+           "no_reuse_ms_per_step": cold["ms_per_step"], "no_reuse_pct": cold["pct_of_hbm_peak"],
+           "no_reuse_kernels_us": cold.get("kernels_us"),
+           "launch": {"forward": fwd_shape, "backward": bwd_shape},
+           "bwd_kernel_frac_of_hbm_peak_no_reuse": norm_roofline(bench, cold, None).get("frac")}
+    bench.free()
+    return out
 
 
 def main():
@@ -338,14 +410,27 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="rmsnorm_bf16_16384x4096", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-configs", action="store_true",
+                    help="skip the other configurations of the benchmark contract (default run only)")
     ap.add_argument("--steps-only", action="store_true",
                     help="only the step itself (timed, then once more with events): every launch a profiler sees is "
                          "one of the step's")
+    ap.add_argument("--policy", choices=("keep", "stream"), default="keep",
+                    help="cache policy of the forward's read of x for --steps-only runs")
+    ap.add_argument("--lag", type=int, default=0,
+                    help="--steps-only: the backward works on the batch forwarded this many steps earlier (2 = no reuse)")
     ap.add_argument("--calibration-copy", action="store_true",
                     help="append five plain tensor copies of known size (reference points for rocprofv3 counters)")
     ap.add_argument("--ceiling", action="store_true",
                     help="instead of a workload: what plain streams reach on this GPU (copy, 2 reads + 1 write, empty "
                          "launches) and the launch intercept / slope of the norm kernels over 8192 ... 32768 rows")
+    ap.add_argument("--scan", action="store_true",
+                    help="instead of a workload: forward + backward of RMSNorm and LayerNorm over a grid of row widths "
+                         "and row counts per storage type, % of HBM peak per cell (the table the launch heuristic is "
+                         "fitted against)")
+    ap.add_argument("--host", action="store_true",
+                    help="instead of a workload: the host cost of the module path (per-call microseconds of the Python "
+                         "layer) and where forward + backward through the modules turns host-bound")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         sys.exit("bench.py: this path runs on ONE GPU: rows are independent and nothing here uses a second device; "
@@ -361,6 +446,10 @@ def main():
     torch.cuda.set_device(dev)
     if args.ceiling:
         return ceiling_main(args, lib, dev)
+    if args.scan:
+        return scan_main(args, lib, dev)
+    if args.host:
+        return host_main(args, lib, dev)
     kind, m, n, dname = WORKLOADS[args.workload]
     dtype = {"bf16": torch.bfloat16, "f16": torch.float16, "f32": torch.float32}[dname]
     if kind == "dropout":
@@ -369,32 +458,25 @@ def main():
         return softmax_main(args, lib, dev, kind, m, n, dname, dtype)
 
     bench = NormBench(lib, dev, args.workload)
-    full = not args.steps_only
-    res = measure_norm(bench, args, full)
+    headline = args.workload == "rmsnorm_bf16_16384x4096"
+    if args.steps_only:
+        res = measure_norm(bench, args, args.policy, args.lag)
+        cold = res if args.lag > 0 else None
+        warm = res if args.lag == 0 else None
+    else:
+        res = warm = measure_norm(bench, args, "keep", 0)
+        cold = measure_norm(bench, args, "stream", 2, preroll=0) if bench.fused_act < 0 else None
     kern = res.get("kernels_us")
     fwd_shape, bwd_shape = bench.shapes()
-
-    # The dominant kernel: the backward dx / partial-sum kernel, as it runs inside the step.
-    roofline = {"bound": "hbm", "kernel": "norm_bwd_kernel (backward dx + dW/dB partials)", "peak": HBM_PEAK_GBPS,
-                "unit": "GB/s", "algorithmic_bytes_per_launch": bench.bwd_bytes,
-                "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload)}
-    if kern is not None:
-        achieved = bench.bwd_bytes / (kern["backward_dx_partials"] * 1e-6) / 1e9
-        roofline.update({"achieved": round(achieved, 1), "frac": round(achieved / HBM_PEAK_GBPS, 4),
-                         "avg_launch_us": kern["backward_dx_partials"],
-                         "measured": "HIP events on the launch stream around the kernel inside the step, less the "
-                                     "events' own cost (kernels_us.event_cost_taken_off_each)"})
-        if "no_reuse" in res:
-            us = res["no_reuse"]["kernels_us"]["backward_dx_partials"]
-            roofline["no_reuse"] = {"avg_launch_us": us, "achieved": round(bench.bwd_bytes / (us * 1e-6) / 1e9, 1),
-                                    "frac": round(bench.bwd_bytes / (us * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4)}
-    else:
+    roofline = norm_roofline(bench, cold, warm)
+    if "achieved" not in roofline:             # the fused backward has no separate stage entry points
         pair = bench.isolated_launch_us(bench.backward, args.steps, args.warmup)
         achieved = bench.bwd_bytes / (pair * 1e-6) / 1e9
         roofline.update({"achieved": round(achieved, 1), "frac": round(achieved / HBM_PEAK_GBPS, 4),
                          "avg_launch_us": round(pair, 2),
                          "measured": "HIP events around back-to-back launches of the fused backward (both stages)"})
 
+    op = "RMSNorm" if kind.startswith("rms") else "LayerNorm"
     out = {
         "metric": "fwd+bwd HBM GB/s and % of peak, RMSNorm/LayerNorm bf16 16384x4096",
         "value": res["GBps"],
@@ -410,28 +492,35 @@ def main():
         "vs_baseline": None,
         "dtype": dname,
         "data": "synthetic",
-        "config": {"workload": args.workload, "op": "RMSNorm" if kind.startswith("rms") else "LayerNorm", "rows": m,
+        "config": {"workload": args.workload, "op": op, "rows": m,
                    "hidden": n, "eps": 1e-6, "buffer_sets": N_BUFFER_SETS, "preroll_steps": PREROLL_STEPS,
                    "entry_points": "thn_norm_act_fwd + thn_norm_act_bwd" if bench.fused_act >= 0 else "thn_norm_fwd + thn_norm_bwd",
                    **({"activation": FUSED_ACTS[bench.fused_act]} if bench.fused_act >= 0 else {}),
-                   "step": REUSE_NOTE},
+                   "cache_policy": (args.policy if args.steps_only else "keep") + "_x",
+                   "backward_lag_steps": args.lag if args.steps_only else 0,
+                   "step": STEP_NOTE if not (args.steps_only and (args.lag or args.policy == "stream")) else NO_REUSE_NOTE},
         "pct_of_hbm_peak": res["pct_of_hbm_peak"],
-        "rows_per_s": round(m / (res["ms_per_step"] * 1e-3)),
+        "rows_per_s": res["rows_per_s"],
         "algorithmic_bytes_per_step": bench.step_bytes,
         "kernels_us": kern,
         "launch": {"forward": fwd_shape, "backward": bwd_shape},
         "roofline": roofline,
     }
-    if "no_reuse" in res:
-        out["no_reuse"] = res["no_reuse"]
-    if full and bench.fused_act < 0:
+    strip = lambda r: {k_: v for k_, v in r.items() if k_ != "GBps"} | {"value": r["GBps"], "unit": "GB/s"}
+    if cold is not None and not args.steps_only:
+        # first-class beside `value`: the no-reuse step under the stream policy, for both operators on the headline
+        out["no_reuse"] = {"cache_policy": "stream_x", "what": NO_REUSE_NOTE, op.lower(): strip(cold)}
+    if not args.steps_only and bench.fused_act < 0:
         # each kernel on its own: K back-to-back launches of that kernel alone
         iso_steps = min(args.steps, 50)
-        out["isolated_kernels_us"] = {
-            "forward": round(bench.isolated_launch_us(bench.forward, iso_steps, args.warmup), 2),
-            "backward_dx_partials": round(bench.isolated_launch_us(bench.backward_stage1, iso_steps, args.warmup), 2),
-            "backward_reduce_partials": round(bench.isolated_launch_us(lambda b_: bench.backward_stage2(), iso_steps,
-                                                                       args.warmup), 2)}
+        iso = {}
+        for pol in ("keep", "stream"):
+            bench.set_policy(pol)
+            iso["forward_" + pol + "_x"] = round(bench.isolated_launch_us(bench.forward, iso_steps, args.warmup), 2)
+        iso["backward_dx_partials"] = round(bench.isolated_launch_us(bench.backward_stage1, iso_steps, args.warmup), 2)
+        iso["backward_reduce_partials"] = round(bench.isolated_launch_us(lambda b_: bench.backward_stage2(), iso_steps,
+                                                                         args.warmup), 2)
+        out["isolated_kernels_us"] = iso
     if args.calibration_copy:
         # a plain copy of known size (x -> y: m*n*s bytes read, as many written) for scaling the HBM counters
         for i in range(5):
@@ -442,16 +531,176 @@ def main():
     bench.free()
 
     # The metric names both operators: on the default workload the LayerNorm step of the same shape is measured
-    # the same way and reported beside it (`value` stays the RMSNorm step).
-    if args.workload == "rmsnorm_bf16_16384x4096":
+    # the same way and reported beside it (`value` stays the RMSNorm step), and the other configurations of the
+    # benchmark contract follow.
+    if headline and not args.steps_only:
         other = NormBench(lib, dev, "layernorm_bf16_16384x4096")
-        r2 = measure_norm(other, args, full)
-        out["layernorm_same_shape"] = {"workload": "layernorm_bf16_16384x4096", "value": r2["GBps"], "unit": "GB/s",
-                                       "algorithmic_bytes_per_step": other.step_bytes,
-                                       **{k_: v for k_, v in r2.items() if k_ != "GBps"}}
+        r2 = measure_norm(other, args, "keep", 0)
+        c2 = measure_norm(other, args, "stream", 2, preroll=0)
+        out["layernorm_same_shape"] = {"workload": "layernorm_bf16_16384x4096",
+                                       "algorithmic_bytes_per_step": other.step_bytes, **strip(r2),
+                                       "roofline": norm_roofline(other, c2, r2)}
+        out["no_reuse"]["layernorm"] = strip(c2)
         other.free()
+        if not args.no_configs:
+            short = argparse.Namespace(steps=min(args.steps, 50), warmup=args.warmup)
+            out["configs"] = {w_: config_summary(lib, dev, w_, short) for w_ in CONTRACT_CONFIGS}
     if not args.no_cpu_baseline and not args.steps_only and bench.fused_act < 0:      # (the fused workloads carry no CPU leg)
         out["cpu_baseline"] = cpu_baseline(*cpu_args)
+    print(json.dumps(out), flush=True)
+
+
+SCAN_WIDTHS = [64, 72, 96, 120, 128, 192, 200, 248, 256, 320, 384, 512, 640, 768, 896, 1024, 1152, 1280, 1408, 1536, 1600, 1792,
+               2048, 2304, 2560, 2816, 3072, 3584, 4000, 4096, 4098, 4104, 4608, 5120, 5632, 6000, 6144, 6656, 7168, 8192,
+               9216, 10240, 12288, 14336, 16384, 20480, 24576, 28672, 32768]
+
+
+def scan_main(args, lib, dev):
+    """Forward + backward of one batch (same batch, 'keep' policy) for RMSNorm and LayerNorm over a grid of row widths
+    and two row-count classes per storage type, in % of the HBM peak on the algorithmic bytes: the table the launch
+    heuristic (plan_launch in thn_api.hip) was fitted against, regenerated for the build and the GPU at hand.
+    Prints a text table, one line per (storage type, width)."""
+    import torch
+    from TritonHub import _native
+    from TritonHub.Normalization import _launch
+    p = _native.ptr
+    stream = torch.cuda.current_stream(dev).cuda_stream
+    total = 1 << 26                                       # elements per tensor in the long class
+    steps = min(args.steps, 30)
+    gen = torch.Generator(device=dev).manual_seed(0)
+    props = torch.cuda.get_device_properties(dev)
+    print(f"# bench.py --scan: forward + backward of one batch, % of {HBM_PEAK_GBPS:.0f} GB/s on the algorithmic bytes; "
+          f"{props.name}, {props.multi_processor_count} compute units; {steps} timed steps per cell, four buffer sets")
+    print("# classes: long = 2^26 elements per tensor; short = 16 rows per compute unit (omitted where that is the long class "
+          "or more)")
+    print("# launch = forward KxTPR/BLOCK@grid | backward KxTPR/BLOCK@grid of the long class (LayerNorm)")
+    print(f"{'dtype':5} {'N':>6} {'rows':>8} | {'RMS long':>8} {'LN long':>8} | {'rows':>6} {'RMS short':>9} {'LN short':>9} | launch")
+    for dname in ("bf16", "f32", "f16"):
+        dtype = {"bf16": torch.bfloat16, "f16": torch.float16, "f32": torch.float32}[dname]
+        s = torch.empty(0, dtype=dtype).element_size()
+        code = _native.dtype_code(dtype)
+        pool = [{k: (torch.randn(total, device=dev, generator=gen).to(dtype) if k in ("x", "dy")
+                     else torch.empty(total, device=dev, dtype=dtype)) for k in ("x", "dy", "y", "dx")}
+                for _ in range(N_BUFFER_SETS)]
+        for n in SCAN_WIDTHS:
+            if n * s > 65536:
+                continue
+            w = (1.0 + 0.1 * torch.randn(n, device=dev, generator=gen)).to(dtype)
+            b = (0.1 * torch.randn(n, device=dev, generator=gen)).to(dtype)
+            dw, db = torch.empty_like(w), torch.empty_like(w)
+            cells = {}
+            m_long = total // n
+            m_short = 16 * props.multi_processor_count
+            for cls, m in (("long", m_long), ("short", m_short)):
+                if cls == "short" and m_short >= m_long:
+                    continue
+                mean = torch.empty(m, device=dev)
+                rstd = torch.empty(m, device=dev)
+                ws_bytes = lib.thn_norm_bwd_workspace_bytes(m, n, 1, 1, code)
+                ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=dev)
+                for ln in (False, True):
+                    def step(i):
+                        b_ = pool[i % N_BUFFER_SETS]
+                        rc = lib.thn_norm_fwd(p(b_["x"]), n, p(b_["y"]), n, p(w), p(b) if ln else 0, p(mean) if ln else 0,
+                                              p(rstd), m, n, 1e-6, code | _native.X_KEEP, code, stream)
+                        assert rc == 0, _native.strerror(rc)
+                        rc = lib.thn_norm_bwd(p(b_["x"]), n, p(b_["dy"]), n, p(b_["dx"]), n, p(w), p(mean) if ln else 0,
+                                              p(rstd), p(dw), p(db) if ln else 0, p(ws), ws_bytes, m, n, code, code, stream)
+                        assert rc == 0, _native.strerror(rc)
+                    for i in range(8):
+                        step(i)
+                    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                    best = float("inf")
+                    for _ in range(2):
+                        start.record()
+                        for i in range(steps):
+                            step(i)
+                        stop.record()
+                        torch.cuda.synchronize()
+                        best = min(best, start.elapsed_time(stop) / steps)
+                    f_, b__ = algorithmic_bytes("ln" if ln else "rms", m, n, s, s)
+                    cells[(cls, ln)] = 100.0 * (f_ + b__) / (best * 1e-3) / 1e9 / HBM_PEAK_GBPS
+            f = _launch.query_launch(0, True, m_long, n, dtype)
+            g = _launch.query_launch(1, True, m_long, n, dtype)
+            launch = f"{f[0]}x{f[1]}/{f[2]}@{f[3]} | {g[0]}x{g[1]}/{g[2]}@{g[3]}" + ("" if f[4] else "  (off the 128-bit path)")
+            short = (f"{m_short:6d} {cells[('short', False)]:9.1f} {cells[('short', True)]:9.1f}" if ("short", False) in cells
+                     else f"{'':6} {'':9} {'':9}")
+            print(f"{dname:5} {n:6d} {m_long:8d} | {cells[('long', False)]:8.1f} {cells[('long', True)]:8.1f} | {short} | {launch}",
+                  flush=True)
+        del pool
+        torch.cuda.empty_cache()
+
+
+def host_main(args, lib, dev):
+    """What the Python layer costs on the host, and where the module path turns host-bound: bfloat16 rows of 4096."""
+    import torch
+    from TritonHub.Normalization import LayerNorm, RMSNorm, _launch
+    n, dtype = 4096, torch.bfloat16
+    out = {"what": "host cost of the operator layer (autograd Function + launch wrapper + C ABI) per call, and forward + "
+                   "backward through the modules against the same step through the C ABI; bfloat16 rows of 4096",
+           "host_us_per_call": {}, "module_path": {}}
+    # host cost: so few rows that the GPU never holds the host up; the clock runs over enqueueing only
+    x = torch.randn(8, n, device=dev).to(dtype)
+    dy = torch.randn(8, n, device=dev).to(dtype)
+    w = torch.ones(n, device=dev, dtype=dtype)
+    b = torch.zeros(n, device=dev, dtype=dtype)
+    reps = 2000
+
+    def host_us(fn):
+        for _ in range(200):
+            fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            fn()
+        t = (time.perf_counter() - t0) * 1e6 / reps
+        torch.cuda.synchronize()
+        return round(t, 2)
+
+    for ln in (False, True):
+        name = "layernorm" if ln else "rmsnorm"
+        _, mean, rstd = _launch.norm_fwd(x, w, b if ln else None, 1e-6, ln)
+        out["host_us_per_call"][name] = {
+            "_launch.norm_fwd": host_us(lambda: _launch.norm_fwd(x, w, b if ln else None, 1e-6, ln)),
+            "_launch.norm_bwd": host_us(lambda: _launch.norm_bwd(x, dy, w, b if ln else None, mean, rstd, ln))}
+        mod = (LayerNorm if ln else RMSNorm)(n, eps=1e-6, device=dev, dtype=dtype)
+        xg = x.clone().requires_grad_(True)
+
+        def fb():
+            mod(xg).backward(dy)
+        out["host_us_per_call"][name]["module forward + backward (autograd included)"] = host_us(fb)
+        with torch.no_grad():
+            out["host_us_per_call"][name]["module forward under no_grad"] = host_us(lambda: mod(x))
+    # module path against the C ABI over row counts
+    for ln in (False, True):
+        name = "layernorm" if ln else "rmsnorm"
+        rows_out = {}
+        for m in (256, 1024, 2048, 4096, 8192, 16384):
+            bench = NormBench(lib, dev, "layernorm_bf16_16384x4096" if ln else "rmsnorm_bf16_16384x4096")
+            bench.m = m
+            short = argparse.Namespace(steps=min(args.steps, 100), warmup=10)
+            abi = measure_norm(bench, short, "keep", 0, preroll=20, with_kernels=False)
+            mod = (LayerNorm if ln else RMSNorm)(n, eps=1e-6, device=dev, dtype=dtype)
+            xs = [bench.sets[i]["x"][:m].requires_grad_(True) for i in range(N_BUFFER_SETS)]
+            dys = [bench.sets[i]["dy"][:m] for i in range(N_BUFFER_SETS)]
+
+            def step(i):
+                xi = xs[i % N_BUFFER_SETS]
+                xi.grad = None
+                mod(xi).backward(dys[i % N_BUFFER_SETS])
+            for i in range(20):
+                step(i)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for i in range(short.steps):
+                step(i)
+            torch.cuda.synchronize()
+            mod_us = (time.perf_counter() - t0) * 1e6 / short.steps
+            rows_out[str(m)] = {"c_abi_us_per_step": round(abi["ms_per_step"] * 1e3, 2), "module_us_per_step": round(mod_us, 2),
+                                "host_bound": bool(mod_us > 1.15 * abi["ms_per_step"] * 1e3)}
+            bench.free()
+            del xs, dys
+        out["module_path"][name] = rows_out
     print(json.dumps(out), flush=True)
 
 
@@ -679,7 +928,7 @@ def softmax_main(args, lib, dev, kind, m, n, dname, dtype):
         "roofline": {"bound": "hbm", "kernel": bwd_kernel, "achieved": round(achieved, 1),
                      "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
                      "algorithmic_bytes_per_launch": bwd_bytes, "avg_launch_us": round(bwd_us, 2),
-                     "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload)},
+                     **traffic_fields(args.workload)},
     }
     if not args.no_cpu_baseline:
         baseline = {None: softmax_cpu_baseline, "act": act_cpu_baseline}.get(row_op, row_op_cpu_baseline)

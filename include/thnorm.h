@@ -19,14 +19,16 @@
  *     `.to(tl.float32)`, layernorm.py:31).  Results are rounded to nearest even on store.
  *   - Return value: THN_OK (0) or a negative THN_E_* code; thn_strerror() names it.  Nothing throws.
  *   - Outputs must not overlap inputs (nor each other), except where an entry point says that it works in place
- *     (thn_dropout).  The row kernels keep their loops free of branches by letting a lane without work
+ *     (thn_dropout).  A call whose output tensor (y, dx) overlaps the address range of one of its input tensors
+ *     returns THN_E_SHAPE and launches nothing.  The row kernels keep their loops free of branches by letting a lane without work
  *     re-load, recompute and re-store the last row or the last vector of its row; with y == x or dx == dy such a
  *     lane can read a row that another workgroup has already overwritten and store it transformed twice.  (The
  *     reference's Triton kernels load a whole row before they store it and tolerate in-place use; callers that
  *     relied on that must pass a separate output here.)
  *   - Thread safe.  Process state: a per-device cache of the compute-unit count, of kernel occupancies and of the
- *     address of the static workspace (thn_norm_bwd_static_workspace), filled on first use; and the launch-shape
- *     override of thn_norm_set_launch_override(), a process-wide tuning switch that is off unless a caller sets it.
+ *     address of the static workspace (thn_norm_bwd_static_workspace), filled on first use; the launch-shape
+ *     override of thn_norm_set_launch_override(), a process-wide tuning switch that is off unless a caller sets it;
+ *     and the default cache policy of thn_norm_set_cache_policy().
  */
 #ifndef THNORM_H_
 #define THNORM_H_
@@ -37,7 +39,7 @@
 extern "C" {
 #endif
 
-#define THN_ABI_VERSION 6
+#define THN_ABI_VERSION 7
 
 enum thn_dtype { THN_F32 = 0, THN_F16 = 1, THN_BF16 = 2, THN_F64 = 3 };
 
@@ -46,7 +48,7 @@ enum thn_status {
     THN_E_DTYPE = -1,         /* unknown storage code */
     THN_E_FEATURE_DIM = -2,   /* a row is wider than 64 KiB (the reference's RuntimeError, layernorm.py:71-72) */
     THN_E_NULL = -3,          /* a required pointer is NULL */
-    THN_E_SHAPE = -4,         /* M < 0, N <= 0 or a row stride smaller than N */
+    THN_E_SHAPE = -4,         /* M < 0, N <= 0, a row stride smaller than N, or an output that overlaps an input */
     THN_E_WORKSPACE = -5,     /* workspace smaller than thn_norm_bwd_workspace_bytes() asks for, or not 16-byte aligned */
     THN_E_LAUNCH = -6,        /* the HIP runtime refused the launch (hipGetLastError) */
     THN_E_DEVICE = -7         /* no usable current device */
@@ -77,6 +79,27 @@ int thn_norm_fwd(const void* x, int64_t x_row_stride,
                  float* mean, float* rstd,
                  int64_t M, int64_t N, float eps,
                  int x_dtype, int w_dtype, void* stream);
+
+/*
+ * Cache policy of the forward's read of x (no counterpart in the reference; Triton chooses for it).  x is the one
+ * tensor of a norm step that is read twice: by the forward, and again by the backward, which rebuilds xhat from it.
+ *   THN_CACHE_KEEP_X    the forward loads x with ordinary loads, which leave it in the L2 and in the 256 MB
+ *                       memory-side cache: a backward that follows its forward closely finds part of x there
+ *                       (bfloat16 16384 x 4096: the backward kernel takes 57 us instead of 65); the forward itself is
+ *                       2-3 % slower than with streaming loads.  For forward + backward of one batch back to back.
+ *   THN_CACHE_STREAM_X  streaming (non-temporal) loads, like every other access of the step.  For inference, and for
+ *                       training steps in which so much other work runs between a layer's forward and its backward
+ *                       that nothing of x would be left in any cache.
+ * Results are bit-identical under both.  thn_norm_set_cache_policy() sets the process-wide default (initially
+ * THN_CACHE_KEEP_X) that thn_norm_fwd() and thn_norm_act_fwd() follow; one call can choose for itself by or-ing
+ * THN_X_KEEP or THN_X_STREAM into its `x_dtype` argument (THN_BF16 | THN_X_STREAM), which overrides the default for
+ * that call and touches no shared state.  The flags are accepted by these two entry points only.
+ */
+enum thn_cache_policy { THN_CACHE_KEEP_X = 0, THN_CACHE_STREAM_X = 1 };
+#define THN_X_KEEP 0x100
+#define THN_X_STREAM 0x200
+int thn_norm_set_cache_policy(int policy);      /* THN_E_SHAPE for an unknown policy */
+int thn_norm_get_cache_policy(void);
 
 /*
  * Bytes of scratch thn_norm_bwd() needs for its per-workgroup partial sums of dW / dB: the counterpart of
@@ -140,9 +163,10 @@ int thn_norm_bwd_reduce_partials(const void* workspace, int32_t num_partials,
  * results, bit for bit, as thn_norm_bwd(); the partial rows of the two-stage dW / dB sum go to a fixed array of
  * THN_STATIC_WORKSPACE_BYTES in device memory that belongs to the library (one copy per GPU, held until the
  * process ends).  The call allocates nothing and frees nothing; the first call on a device looks the array's
- * address up (hipGetSymbolAddress), so make that one call outside a graph capture.  Problems whose partial rows
- * need more than THN_STATIC_WORKSPACE_BYTES -- thn_norm_bwd_workspace_bytes() says how much -- return
- * THN_E_WORKSPACE: bring a workspace and call thn_norm_bwd().  All calls on one GPU share the array: two calls
+ * address up (hipGetSymbolAddress), so make that one call outside a graph capture: a first call on a stream that
+ * is being captured returns THN_E_DEVICE.  Problems whose partial rows -- one per workgroup of the grid the
+ * backward launches, at most what thn_norm_bwd_workspace_bytes() says -- need more than THN_STATIC_WORKSPACE_BYTES
+ * return THN_E_WORKSPACE: bring a workspace and call thn_norm_bwd().  All calls on one GPU share the array: two calls
  * that may run at the same time (different streams, or graph branches) race on it; calls on one stream are safe.
  */
 #define THN_STATIC_WORKSPACE_BYTES (16 * 1024 * 1024)

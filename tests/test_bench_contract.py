@@ -30,8 +30,6 @@ def test_workload_table():
         s = {"bf16": 2, "f16": 2, "f32": 4}[dname]
         fwd, bwd = bench.algorithmic_bytes(kind.split("+")[0], m, n, s, s)
         assert fwd >= m * n * s and bwd >= 2 * m * n * s, name      # at least one read; a read and a write
-    for key in bench.MEASURED_TRAFFIC_BYTES:
-        assert key in bench.WORKLOADS
     # algorithmic bytes of the default workload: 5*M*N*s + 8*M + 3*N*s
     f, b = bench.algorithmic_bytes("rms", 16384, 4096, 2, 2)
     assert f + b == 5 * 16384 * 4096 * 2 + 8 * 16384 + 3 * 4096 * 2
@@ -39,8 +37,19 @@ def test_workload_table():
     assert f + b == 5 * 16384 * 4096 * 2 + 16 * 16384 + 5 * 4096 * 2
 
 
-def test_profiles_named_by_the_traffic_table_exist():
-    text = open(os.path.join(ROOT, "bench.py")).read()
-    import re
-    for path in re.findall(r"# (profiles/[\w./-]+\.txt)", text):
-        assert os.path.exists(os.path.join(ROOT, path)), path
+def test_traffic_comes_from_the_profile_summaries():
+    """roofline.traffic is read from `bench.traffic` lines of the summaries under profiles/: every such line names a
+    workload of the table, and the headline workload has one."""
+    seen = set()
+    for name in sorted(os.listdir(os.path.join(ROOT, "profiles"))):
+        for line in open(os.path.join(ROOT, "profiles", name)):
+            parts = line.split()
+            if parts[:1] == ["bench.traffic"]:
+                assert len(parts) >= 5 and parts[1] in bench.WORKLOADS and int(parts[3]) > 0, (name, line)
+                seen.add(parts[1])
+    assert "rmsnorm_bf16_16384x4096" in seen and "layernorm_bf16_16384x4096" in seen
+    t = bench.traffic_from_profiles("rmsnorm_bf16_16384x4096")
+    f, b = bench.algorithmic_bytes("rms", 16384, 4096, 2, 2)
+    assert t is not None and t["source"].startswith("profiles/") and b <= t["bytes"] < 1.1 * b
+    assert bench.traffic_from_profiles("layernorm_f32_200x128_quickstart") is None
+    assert bench.traffic_fields("no_such_workload") == {"traffic": None}

@@ -25,7 +25,7 @@ def declared_functions():
 
 def test_library_exports_every_declared_symbol():
     names = declared_functions()
-    assert len(names) == 22 and "thn_norm_bwd_static_workspace" in names and "thn_dropout" in names and "thn_norm_act_fwd" in names and "thn_norm_act_bwd" in names and "thn_act_fwd" in names and "thn_pnorm_fwd" in names and "thn_normalize_bwd" in names and "thn_norm_fwd" in names and "thn_norm_bwd" in names and "thn_softmax_fwd" in names
+    assert len(names) == 24 and "thn_norm_set_cache_policy" in names and "thn_norm_bwd_static_workspace" in names and "thn_dropout" in names and "thn_norm_act_fwd" in names and "thn_norm_act_bwd" in names and "thn_act_fwd" in names and "thn_pnorm_fwd" in names and "thn_normalize_bwd" in names and "thn_norm_fwd" in names and "thn_norm_bwd" in names and "thn_softmax_fwd" in names
     handle = ctypes.CDLL(_native.LIB_PATH)
     for name in names:
         assert hasattr(handle, name), f"{name} is declared in include/thnorm.h but not exported"
@@ -67,6 +67,81 @@ def test_argument_checks_answer_without_a_gpu():
         _native.check(_native.E_FEATURE_DIM)
     with pytest.raises(RuntimeError, match="workspace"):
         _native.check(_native.E_WORKSPACE)
+
+
+def test_cache_policy_switch_and_per_call_flags():
+    lib = _native.lib()
+    assert lib.thn_norm_get_cache_policy() == 0                              # THN_CACHE_KEEP_X is the default
+    assert lib.thn_norm_set_cache_policy(1) == _native.OK and lib.thn_norm_get_cache_policy() == 1
+    assert lib.thn_norm_set_cache_policy(2) == _native.E_SHAPE and lib.thn_norm_get_cache_policy() == 1
+    assert lib.thn_norm_set_cache_policy(0) == _native.OK and lib.thn_norm_get_cache_policy() == 0
+    fwd = lambda xd: lib.thn_norm_fwd(0, 128, 0, 128, 0, 0, 0, 0, 4, 128, 1e-5, xd, 0, 0)
+    afwd = lambda xd: lib.thn_norm_act_fwd(0, 128, 0, 128, 0, 0, 0, 0, 4, 128, 1e-5, _native.ACT_SILU, xd, 0, 0)
+    for call in (fwd, afwd):
+        # the flag rides on the storage code: the code underneath is still checked, then the pointers
+        assert call(_native.BF16 | _native.X_STREAM) == _native.E_NULL
+        assert call(_native.F32 | _native.X_KEEP) == _native.E_NULL
+        assert call(7 | _native.X_STREAM) == _native.E_DTYPE
+        assert call(_native.BF16 | _native.X_KEEP | _native.X_STREAM) == _native.E_DTYPE     # both: contradictory
+    # no other entry point takes the flags
+    assert lib.thn_norm_bwd_workspace_bytes(4, 128, 1, 1, _native.BF16 | _native.X_STREAM) == _native.E_DTYPE
+    assert lib.thn_softmax_fwd(0, 128, 0, 128, 4, 128, 0, _native.BF16 | _native.X_STREAM, 0) == _native.E_DTYPE
+    # the Python switch
+    assert _launch.get_cache_policy() == "auto"
+    assert _launch._x_policy_flag(True) == _native.X_KEEP and _launch._x_policy_flag(False) == _native.X_STREAM
+    try:
+        _launch.set_cache_policy("stream")
+        assert _launch._x_policy_flag(True) == _native.X_STREAM
+        _launch.set_cache_policy("keep")
+        assert _launch._x_policy_flag(False) == _native.X_KEEP
+        with pytest.raises(ValueError):
+            _launch.set_cache_policy("sometimes")
+        assert Normalization.get_cache_policy() == "keep"
+    finally:
+        _launch.set_cache_policy("auto")
+    assert "set_cache_policy" not in Normalization.__all__                    # the reference's surface is unchanged
+
+
+def test_outputs_that_overlap_inputs_are_refused_on_the_host():
+    """The address ranges alone decide: no kernel is launched, so fake addresses do."""
+    lib = _native.lib()
+    s = 2                                              # bf16
+    base, m, n = 1 << 20, 16, 128
+    size = m * n * s
+    fwd = lambda x, y, ys=n: lib.thn_norm_fwd(x, n, y, ys, 0, 0, 0, 4096, m, n, 1e-5, _native.BF16, 0, 0)
+    assert fwd(base, base) == _native.E_SHAPE                                   # in place
+    assert fwd(base, base + size - 2) == _native.E_SHAPE                        # last element of x is first of y
+    assert fwd(base + size - 2, base) == _native.E_SHAPE
+    assert fwd(base, base + n * s, 2 * n) == _native.E_SHAPE                    # different pitches: the ranges decide
+    # two column blocks of one buffer (the same pitch, rows that do not touch) may interleave; shifted by less than a row not
+    fwd2 = lambda x, y: lib.thn_norm_fwd(x, 2 * n, y, 2 * n, 0, 0, 0, 4096, m, n, 1e-5, _native.BF16, 0, 0)
+    assert fwd2(base, base + n * s - 2) == _native.E_SHAPE and fwd2(base + 2, base + n * s) == _native.E_SHAPE
+    assert fwd2(base + n * s - 2, base) == _native.E_SHAPE
+    if not torch.cuda.is_available():
+        assert fwd2(base, base + n * s) == _native.E_DEVICE and fwd2(base + n * s, base) == _native.E_DEVICE
+    not_refused = (_native.OK, _native.E_DEVICE, _native.E_LAUNCH)
+    if not torch.cuda.is_available():
+        assert fwd(base, base + size) == _native.E_DEVICE                       # adjacent is fine: the next check answers
+    bwd = lambda x, dy, dx: lib.thn_norm_bwd_dx_partials(x, n, dy, n, dx, n, 0, 0, 4096, 0, 0, 0, 0, None, m, n,
+                                                          _native.BF16, 0, 0)
+    assert bwd(base, base + size, base) == _native.E_SHAPE and bwd(base, base + size, base + size + 64) == _native.E_SHAPE
+    sm = lambda x, y: lib.thn_softmax_fwd(x, n, y, n, m, n, 0, _native.BF16, 0)
+    smb = lambda y, dy, dx: lib.thn_softmax_bwd(y, n, dy, n, dx, n, m, n, 0, _native.BF16, 0)
+    assert sm(base, base + 2) == _native.E_SHAPE and smb(base, base + size, base + size) == _native.E_SHAPE
+    act = lambda x, y: lib.thn_act_fwd(x, n, y, n, m, n, _native.ACT_RELU, 0.0, 0.0, _native.BF16, 0)
+    actb = lambda x, g, dx: lib.thn_act_bwd(x, n, g, n, dx, n, m, n, _native.ACT_RELU, 0.0, 0.0, _native.BF16, 0)
+    assert act(base, base) == _native.E_SHAPE and actb(base, base + size, base + size) == _native.E_SHAPE
+    k = n
+    nz = lambda x, y: lib.thn_normalize_fwd(x, m * k, k, y, m * k, k, 4096, 1, m, k, 2.0, 1e-6, _native.BF16, 0)
+    assert nz(base, base) == _native.E_SHAPE
+    pb = lambda x, dx: lib.thn_pnorm_bwd(x, m * k, k, 4096, 8192, dx, m * k, k, 1, m, k, 2.0, _native.BF16, 0)
+    assert pb(base, base + 16) == _native.E_SHAPE
+    nb = lambda y, dy, dx: lib.thn_normalize_bwd(0, m * k, k, y, m * k, k, 4096, dy, m * k, k, dx, m * k, k, 1, m, k,
+                                                 2.0, _native.BF16, 0)
+    assert nb(base, base + size, base + size + 2) == _native.E_SHAPE and nb(base, base + size, base) == _native.E_SHAPE
+    if not torch.cuda.is_available():
+        for rc in (sm(base, base + size), act(base, base + size), nz(base, base + size), pb(base, base + size)):
+            assert rc in not_refused
 
 
 def test_softmax_argument_checks_answer_without_a_gpu():

@@ -517,6 +517,65 @@ def test_c_abi_direct_calls_and_errors():
     assert torch.equal(dx2, dx[:, :n])
 
 
+# ---- cache policy of the forward's read of x ------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32, torch.float16])
+def test_cache_policies_give_the_same_bits(dtype):
+    """The keep-x and stream-x forwards differ in a hint on their loads of x and in nothing else: y, mean and rstd
+    must be bit-identical, through the per-call flag, through the process-wide default and through the modules
+    (training keeps, torch.no_grad() streams, set_cache_policy forces)."""
+    announce(f"cache policies {dtype}")
+    lib = _native.lib()
+    p = _native.ptr
+    code = _native.dtype_code(dtype)
+    st = torch.cuda.current_stream().cuda_stream
+    g = torch.Generator().manual_seed(5)
+    # 128-bit path (several launch shapes), rows off it, rows shorter than a vector, an activation epilogue
+    for m, n in ((3000, 4096), (777, 6000), (5000, 256), (64, 16384), (1500, 4099), (300, 3), (900, 1288)):
+        x = (torch.randn(m, n, generator=g) * 2 + 0.5).to(dtype).cuda()
+        w = (1 + 0.1 * torch.randn(n, generator=g)).to(dtype).cuda()
+        b = (0.1 * torch.randn(n, generator=g)).to(dtype).cuda()
+        for ln in (True, False):
+            for act in (-1, _native.ACT_SILU):
+                outs = []
+                for how in ("keep flag", "stream flag", "default keep", "default stream"):
+                    y = torch.full_like(x, 9.0)
+                    mean = torch.full((m,), 9.0, device="cuda") if ln else None
+                    rstd = torch.full((m,), 9.0, device="cuda")
+                    flag = {"keep flag": _native.X_KEEP, "stream flag": _native.X_STREAM}.get(how, 0)
+                    assert lib.thn_norm_set_cache_policy(1 if how == "default stream" else 0) == 0
+                    try:
+                        if act < 0:
+                            rc = lib.thn_norm_fwd(p(x), n, p(y), n, p(w), p(b) if ln else 0, p(mean), p(rstd), m, n, 1e-6,
+                                                  code | flag, code, st)
+                        else:
+                            rc = lib.thn_norm_act_fwd(p(x), n, p(y), n, p(w), p(b) if ln else 0, p(mean), p(rstd), m, n,
+                                                      1e-6, act, code | flag, code, st)
+                    finally:
+                        lib.thn_norm_set_cache_policy(0)
+                    assert rc == 0, (_native.strerror(rc), how, m, n, ln, act)
+                    torch.cuda.synchronize()
+                    outs.append((y, mean, rstd))
+                for y, mean, rstd in outs[1:]:
+                    assert torch.equal(y.view(torch.uint8), outs[0][0].view(torch.uint8)), (m, n, ln, act)
+                    assert torch.equal(rstd, outs[0][2]) and (not ln or torch.equal(mean, outs[0][1]))
+                assert not bool((outs[0][2] == 9.0).any())
+    # the modules: the same bits whichever policy the Python layer picks
+    x = torch.randn(4, 500, 2048, generator=g).to(dtype).cuda()
+    for mod in (LayerNorm(2048, device="cuda", dtype=dtype), RMSNorm(2048, device="cuda", dtype=dtype)):
+        ys = []
+        with torch.no_grad():
+            ys.append(mod(x))                                 # 'auto': no backward follows, x is streamed
+        ys.append(mod(x.clone().requires_grad_(True)).detach())    # 'auto': x is kept
+        for forced in ("keep", "stream"):
+            _launch.set_cache_policy(forced)
+            try:
+                ys.append(mod(x.clone().requires_grad_(True)).detach())
+            finally:
+                _launch.set_cache_policy("auto")
+        for y in ys[1:]:
+            assert torch.equal(y.view(torch.uint8), ys[0].view(torch.uint8))
+
+
 # ---- every compiled kernel shape ---------------------------------------------------------------------------------
 def compiled_shapes():
     import os, re

@@ -2,6 +2,8 @@
 go to a fixed array in device memory that the library owns.  It must give the bits of thn_norm_bwd (the same
 kernels with a caller-supplied workspace) on two calls in a row, the second one smaller than the first, and refuse
 problems whose partial rows do not fit the array.  Collected last: the file name sorts behind every other test."""
+import ctypes
+
 import pytest
 import torch
 
@@ -72,6 +74,42 @@ def test_static_workspace_backward_matches_the_workspace_backward_twice_in_a_row
     _both_backwards("ln", 64, 256, torch.float32, 5, want_dw=False, want_db=False)   # no gradient: the array is not touched
 
 
+def test_static_workspace_is_sized_by_the_grid_the_backward_launches():
+    """512 rows of 16384 bf16 columns: the upper bound of thn_norm_bwd_workspace_bytes (one partial row per compute
+    unit and gradient: 32 MiB) does not fit the array, but the backward over so few rows launches half the
+    workgroups, and what those write does."""
+    announce("static workspace: LayerNorm bf16 512 x 16384 (upper bound 32 MiB, 128 partial rows per gradient)")
+    lib = _native.lib()
+    m, n = 512, 16384
+    shape = (ctypes.c_int32 * 5)()
+    assert lib.thn_norm_query_launch(1, 1, m, n, _native.BF16, shape) == 0
+    need = 2 * shape[3] * n * 4
+    upper = lib.thn_norm_bwd_workspace_bytes(m, n, 1, 1, _native.BF16)
+    if not (need <= STATIC_BYTES < upper):
+        pytest.skip(f"this device launches {shape[3]} workgroups here: {need} bytes of {upper}")
+    p = _native.ptr
+    st = torch.cuda.current_stream().cuda_stream
+    x, dy, w, b = _case("ln", m, n, torch.bfloat16, 6)
+    y, mean, rstd = torch.empty_like(x), torch.empty(m, device="cuda"), torch.empty(m, device="cuda")
+    code = _native.BF16
+    assert lib.thn_norm_fwd(p(x), n, p(y), n, p(w), p(b), p(mean), p(rstd), m, n, 1e-6, code, code, st) == 0
+    outs = []
+    for static in (False, True):
+        dx, dw, db = torch.full_like(x, 3.0), torch.full_like(w, 3.0), torch.full_like(w, 3.0)
+        if static:
+            rc = lib.thn_norm_bwd_static_workspace(p(x), n, p(dy), n, p(dx), n, p(w), p(mean), p(rstd), p(dw), p(db), m, n,
+                                                   code, code, st)
+        else:
+            ws = torch.empty(upper, dtype=torch.uint8, device="cuda")
+            rc = lib.thn_norm_bwd(p(x), n, p(dy), n, p(dx), n, p(w), p(mean), p(rstd), p(dw), p(db), p(ws), upper, m, n,
+                                  code, code, st)
+        assert rc == 0, _native.strerror(rc)
+        torch.cuda.synchronize()
+        outs.append((dx, dw, db))
+    for a, c in zip(*outs):
+        assert torch.equal(a, c) and not bool((c == 3.0).all())
+
+
 def test_static_workspace_refuses_what_does_not_fit():
     announce("static workspace: limits")
     lib = _native.lib()
@@ -80,10 +118,11 @@ def test_static_workspace_refuses_what_does_not_fit():
     m, n = 4096, 16384                                          # float32 LayerNorm: 2 x 256 partial rows of 64 KiB = 32 MiB
     need = lib.thn_norm_bwd_workspace_bytes(m, n, 1, 1, _native.F32)
     assert need > STATIC_BYTES
-    x = torch.zeros(8, n, device="cuda")                        # never read: the call returns before any launch
+    # never read or written: the call returns before any launch (full size: the argument checks look at the spans)
+    x, g, d = (torch.empty(m, n, device="cuda") for _ in range(3))
     v = torch.zeros(n, device="cuda")
     r = torch.zeros(m, device="cuda")
-    rc = lib.thn_norm_bwd_static_workspace(p(x), n, p(x), n, p(x), n, p(v), p(r), p(r), p(v), p(v), m, n, _native.F32,
+    rc = lib.thn_norm_bwd_static_workspace(p(x), n, p(g), n, p(d), n, p(v), p(r), p(r), p(v), p(v), m, n, _native.F32,
                                            _native.F32, st)
     assert rc == _native.E_WORKSPACE
     # the same errors as thn_norm_bwd for bad arguments

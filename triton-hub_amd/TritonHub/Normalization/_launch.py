@@ -44,6 +44,34 @@ def _check_feature_dim(n: int, element_size: int) -> None:
         raise RuntimeError(FEATURE_DIM_MESSAGE)
 
 
+# How the forward reads x (include/thnorm.h, thn_cache_policy): 'keep' leaves x in the caches for the backward,
+# 'stream' does not; 'auto' keeps it exactly when autograd will run a backward for the call.
+_CACHE_POLICIES = ('auto', 'keep', 'stream')
+_cache_policy = 'auto'
+
+
+def set_cache_policy(policy: str) -> None:
+    """'auto' (default): the forward keeps x in the caches when a backward will follow (some input of the autograd
+    Function requires a gradient) and streams it otherwise (inference); 'keep' / 'stream': always.  Choose 'stream'
+    for training loops in which so much other work runs between a layer's forward and its backward that nothing of
+    x would still be cached: the forward alone is 2-3 % faster that way.  Results are bit-identical under all three."""
+    global _cache_policy
+    if policy not in _CACHE_POLICIES:
+        raise ValueError(f'cache policy must be one of {_CACHE_POLICIES}, got {policy!r}')
+    _cache_policy = policy
+
+
+def get_cache_policy() -> str:
+    return _cache_policy
+
+
+def _x_policy_flag(backward_follows: bool) -> int:
+    policy = _cache_policy
+    if policy == 'auto':
+        return _native.X_KEEP if backward_follows else _native.X_STREAM
+    return _native.X_KEEP if policy == 'keep' else _native.X_STREAM
+
+
 _raw_stream = getattr(torch._C, '_cuda_getCurrentRawStream', None)
 _get_device = getattr(torch._C, '_cuda_getDevice', None)
 _workspace_cache = {}           # (device index, stream handle) -> uint8 tensor, grown on demand
@@ -93,9 +121,10 @@ def _workspace(index: int, stream: int, nbytes: int, device) -> torch.Tensor:
     return ws
 
 
-def norm_fwd(x: torch.Tensor, weight, bias, eps: float, layernorm: bool, act: int = -1):
+def norm_fwd(x: torch.Tensor, weight, bias, eps: float, layernorm: bool, act: int = -1, backward_follows: bool = True):
     """Returns (y like x, mean (M,) float32 or None, rstd (M,) float32).  `act` >= 0: the activation with that
-    code is applied in the same pass (thn_norm_act_fwd)."""
+    code is applied in the same pass (thn_norm_act_fwd).  `backward_follows`: whether autograd will run a backward
+    for this call (it decides the cache policy of the read of x under set_cache_policy('auto'))."""
     if not x.is_cuda:
         _native.require_gpu(x)
     x2, m, n, x_stride, reshaped = _flatten(x, 'input')
@@ -114,6 +143,7 @@ def norm_fwd(x: torch.Tensor, weight, bias, eps: float, layernorm: bool, act: in
     if m == 0:                       # nothing to launch (and empty tensors have no address to pass)
         return (out.reshape(*x.shape[:-1], n) if reshaped else out), mean, rstd
     w_code = x_code
+    x_code |= _x_policy_flag(backward_follows)
     if weight is not None:
         w_code = _native.dtype_code(weight.dtype)
         if bias is not None and weight.dtype != bias.dtype:

@@ -29,7 +29,7 @@ class layernorm_act(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, input, weight, bias, eps, act):
-        output, mean, rstd = norm_fwd(input, weight, bias, eps, layernorm=True, act=act)
+        output, mean, rstd = norm_fwd(input, weight, bias, eps, layernorm=True, act=act, backward_follows=any(ctx.needs_input_grad))
         ctx.save_for_backward(input, weight, bias, mean, rstd)
         ctx.eps = eps
         ctx.act = act
@@ -49,7 +49,7 @@ class rmsnorm_act(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, input, weight, eps, act):
-        output, _, rstd = norm_fwd(input, weight, None, eps, layernorm=False, act=act)
+        output, _, rstd = norm_fwd(input, weight, None, eps, layernorm=False, act=act, backward_follows=any(ctx.needs_input_grad))
         ctx.save_for_backward(input, weight, rstd)
         ctx.eps = eps
         ctx.act = act

@@ -14,7 +14,7 @@ class layernorm(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, input, weight, bias, eps):
-        output, mean, rstd = norm_fwd(input, weight, bias, eps, layernorm=True)
+        output, mean, rstd = norm_fwd(input, weight, bias, eps, layernorm=True, backward_follows=any(ctx.needs_input_grad))
         ctx.save_for_backward(input, weight, bias, mean, rstd)
         ctx.eps = eps
         return output

@@ -14,7 +14,7 @@ class rmsnorm(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, input, weight, eps):
-        output, _, rstd = norm_fwd(input, weight, None, eps, layernorm=False)
+        output, _, rstd = norm_fwd(input, weight, None, eps, layernorm=False, backward_follows=any(ctx.needs_input_grad))
         ctx.save_for_backward(input, weight, rstd)
         ctx.eps = eps
         return output

@@ -21,6 +21,9 @@ SOFTMAX, SOFTMIN, LOGSOFTMAX = 0, 1, 2
  ACT_THRESHOLD) = range(11)
 DTYPE_CODES = {torch.float32: F32, torch.float16: F16, torch.bfloat16: BF16, torch.float64: F64}
 
+# or-ed into the x_dtype argument of thn_norm_fwd / thn_norm_act_fwd: this call's cache policy for its read of x
+X_KEEP, X_STREAM = 0x100, 0x200
+
 OK = 0
 E_DTYPE, E_FEATURE_DIM, E_NULL, E_SHAPE, E_WORKSPACE, E_LAUNCH, E_DEVICE = -1, -2, -3, -4, -5, -6, -7
 
@@ -52,6 +55,8 @@ SYMBOLS = {
                                 _i32, _i32, _i32, _vp]),
     'thn_dropout': (_i32, [_vp, _vp, _i64, _i64, _f32, ctypes.c_uint64, _i32, _vp]),
     'thn_norm_set_launch_override': (_i32, [_i32, _i32, _i32, _i32, _i32]),
+    'thn_norm_set_cache_policy': (_i32, [_i32]),
+    'thn_norm_get_cache_policy': (_i32, []),
     'thn_norm_query_launch': (_i32, [_i32, _i32, _i64, _i64, _i32, ctypes.POINTER(ctypes.c_int32)]),
 }
 

@@ -3,6 +3,7 @@
 #include "thnorm.h"
 
 #include <atomic>
+#include <initializer_list>
 #include <mutex>
 #include <unordered_map>
 
@@ -70,6 +71,10 @@ struct Override {
     std::atomic<int> k{0}, tpr{0}, block{0}, bpc{0};
 };
 Override g_override[kFamilies];
+
+// Default cache policy of the forward's read of x (thn_norm_set_cache_policy).
+std::atomic<int> g_cache_policy{THN_CACHE_KEEP_X};
+constexpr int kPolicyFlags = THN_X_KEEP | THN_X_STREAM;
 
 // `ln16`: LayerNorm over 16-bit rows (the two norm backwards have instances of their own for that).
 bool shape_compiled(int which, bool aligned, bool ln16, Shape s) {
@@ -241,6 +246,7 @@ int occupancy(int which, int dtype, int flavour, bool aligned, Shape s) {
     int rc;
     if (which == kNormFwd) {
         FwdArgs dummy{};
+        dummy.keep_x = 1;
         dummy.n_cols = 1 << 20;      // the unaligned-window instances, not the ones for rows shorter than a vector
         rc = launch_fwd(dtype, flavour, aligned, s, dummy, 0, nullptr, &occ);
     } else if (which == kNormBwd) {
@@ -257,6 +263,7 @@ int occupancy(int which, int dtype, int flavour, bool aligned, Shape s) {
         rc = launch_softmax_bwd(dtype, flavour, aligned, s, dummy, 0, nullptr, &occ);
     } else if (which == kFusedFwd) {
         FwdArgs dummy{};
+        dummy.keep_x = 1;
         dummy.n_cols = 1 << 20;      // the unaligned-window instances, not the ones for rows shorter than a vector
         rc = launch_fused_fwd(dtype, flavour, aligned, s, dummy, 0, nullptr, &occ);
     } else if (which == kFusedBwd) {
@@ -606,6 +613,8 @@ int plan_launch(int which, int flavour, bool aligned, int64_t M, int64_t N, int 
     // part, the lost parallelism costs more (2048 x 4096 LayerNorm 23.7 -> 24.3, 1024 x 8192 26.3 -> 27.5, 4096 x 1024
     // 19.4 -> 20.5 us); a quarter of the workgroups measured the same as half or slower.
     if ((which == kNormBwd || which == kFusedBwd) && ov.bpc.load() <= 0 && grid >= cus && row_blocks <= 2 * grid) {
+        // (two gradients for LayerNorm whichever of them the caller asks for: the grid decides which rows meet in a
+        // partial row, and dW must not depend on whether dB is requested as well)
         const int64_t n_grads = (flavour & 1) != 0 ? 2 : 1;
         if (grid * 4 * n_grads * 4 >= M * bytes * 3) grid = (grid + 1) / 2;
     }
@@ -617,6 +626,39 @@ int plan_launch(int which, int flavour, bool aligned, int64_t M, int64_t N, int 
 }
 
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// The bytes a (rows, row_bytes) operand with the given row pitch spans, as a half-open address range, with the
+// pitch and the row width kept for the row-level test below (pitch 0: not a plain stack of rows).
+struct ByteRange {
+    uintptr_t lo, hi;
+    int64_t pitch, row_bytes;
+};
+ByteRange span_of(const void* p, int64_t rows, int64_t pitch_bytes, int64_t row_bytes) {
+    const uintptr_t lo = reinterpret_cast<uintptr_t>(p);
+    if (p == nullptr || rows <= 0) return ByteRange{lo, lo, 0, 0};
+    return ByteRange{lo, lo + static_cast<uintptr_t>((rows - 1) * pitch_bytes + row_bytes), rows > 1 ? pitch_bytes : 0,
+                     row_bytes};
+}
+// Outputs must not overlap inputs: lanes without work re-load and re-store the last row or vector, so an aliased
+// call would store rows transformed twice.  Checked on the host, on the addresses alone: the two address ranges
+// must be disjoint, except that two stacks of rows with the SAME pitch may interleave (x = buf[:, :n], y = buf[:, n:]
+// of one buffer) as long as no row of one touches a row of the other.
+bool overlaps(ByteRange a, ByteRange b) {
+    if (!(a.lo < b.hi && b.lo < a.hi)) return false;
+    if (a.pitch > 0 && a.pitch == b.pitch) {
+        const int64_t p = a.pitch;
+        const int64_t d = static_cast<int64_t>((b.lo >= a.lo ? b.lo - a.lo : p - (a.lo - b.lo) % p) % p);   // (b - a) mod p
+        // a row of b starts d bytes behind a row of a (and p - d bytes in front of the next one)
+        return d < a.row_bytes || p - d < b.row_bytes;
+    }
+    return true;
+}
+bool overlaps_any(ByteRange out, std::initializer_list<ByteRange> ins) {
+    for (const ByteRange& in : ins) {
+        if (overlaps(out, in)) return true;
+    }
+    return false;
+}
 
 // Whether a norm launch may shift its vector slots onto 128-byte lines (row_line_shift() in thn_kernels.h): rows
 // that start off a line boundary, one row per workgroup at a time, every row a workgroup visits and every stream
@@ -670,6 +712,11 @@ bool fusable(int act) { return act == thn::kGelu || act == thn::kGeluTanh || act
 int norm_forward(const void* x, int64_t x_row_stride, void* y, int64_t y_row_stride, const void* w, const void* b,
                  float* mean, float* rstd, int64_t M, int64_t N, float eps, int act, int x_dtype, int w_dtype,
                  void* stream) {
+    // the caller's choice for this call rides on the storage code (THN_X_KEEP / THN_X_STREAM)
+    const int policy_flags = x_dtype & kPolicyFlags;
+    if (policy_flags == kPolicyFlags) return THN_E_DTYPE;
+    x_dtype &= ~kPolicyFlags;
+    const bool keep_x = policy_flags != 0 ? policy_flags == THN_X_KEEP : g_cache_policy.load() == THN_CACHE_KEEP_X;
     const int bytes = elem_bytes(x_dtype);
     if (bytes == 0 || ((w != nullptr || b != nullptr) && elem_bytes(w_dtype) == 0)) return THN_E_DTYPE;
     if (M < 0 || N <= 0) return THN_E_SHAPE;
@@ -679,6 +726,9 @@ int norm_forward(const void* x, int64_t x_row_stride, void* y, int64_t y_row_str
     const bool ln = mean != nullptr;
     if (!ln && b != nullptr) return THN_E_SHAPE;          // RMSNorm has no bias (rmsnorm.py:13-22)
     if (x_row_stride < N || y_row_stride < N) return THN_E_SHAPE;
+    if (overlaps(span_of(y, M, y_row_stride * bytes, N * bytes), span_of(x, M, x_row_stride * bytes, N * bytes))) {
+        return THN_E_SHAPE;
+    }
 
     const int vec_elems = 16 / bytes;
     const bool aligned = (N % vec_elems) == 0 && aligned16(x) && aligned16(y) && aligned16(w) && aligned16(b) &&
@@ -706,6 +756,7 @@ int norm_forward(const void* x, int64_t x_row_stride, void* y, int64_t y_row_str
     a.inv_n = 1.0f / static_cast<float>(N);
     const RowStream streams[2] = {{x, a.x_stride_bytes}, {y, a.y_stride_bytes}};
     a.line_shift = line_shift_ok(aligned, p.s, p.grid, p.n_vecs, streams, 2) ? 1 : 0;
+    a.keep_x = keep_x ? 1 : 0;
     hipStream_t st = static_cast<hipStream_t>(stream);
     const int lrc = fused ? launch_fused_fwd(x_dtype, (ln ? 1 : 0) | (act << 1), aligned, p.s, a, p.grid, st, nullptr)
                           : launch_fwd(x_dtype, ln, aligned, p.s, a, p.grid, st, nullptr);
@@ -726,6 +777,10 @@ int norm_backward_stage1(const void* x, int64_t x_row_stride, const void* dy, in
     if (M == 0) return THN_OK;
     if (x == nullptr || dy == nullptr || dx == nullptr || rstd == nullptr) return THN_E_NULL;
     if (x_row_stride < N || dy_row_stride < N || dx_row_stride < N) return THN_E_SHAPE;
+    if (overlaps_any(span_of(dx, M, dx_row_stride * bytes, N * bytes),
+                     {span_of(x, M, x_row_stride * bytes, N * bytes), span_of(dy, M, dy_row_stride * bytes, N * bytes)})) {
+        return THN_E_SHAPE;
+    }
     const bool ln = mean != nullptr;
     if (!ln) want_db = 0;
     const int n_grads = (want_dw ? 1 : 0) + (want_db ? 1 : 0);
@@ -829,6 +884,13 @@ thn::RowWalk make_walk(bool uniform, int64_t M, int64_t rows, int64_t rows_per_i
     return w;
 }
 
+// The span of a (B, M, K) operand with non-negative batch and row strides in elements.
+ByteRange span_of_bmk(const void* p, int64_t B, int64_t M, int64_t K, int64_t batch_stride, int64_t row_stride, int bytes) {
+    const uintptr_t lo = reinterpret_cast<uintptr_t>(p);
+    if (p == nullptr || B <= 0 || M <= 0 || batch_stride < 0 || row_stride < 0) return ByteRange{lo, lo, 0, 0};
+    return ByteRange{lo, lo + static_cast<uintptr_t>(((B - 1) * batch_stride + (M - 1) * row_stride + K) * bytes), 0, 0};
+}
+
 int mode_of(int p_int) { return p_int == 1 ? thn::kP1 : (p_int == 2 ? thn::kP2 : thn::kPInt); }
 
 int loop_grid(int64_t rows) {
@@ -846,6 +908,10 @@ int pnorm_forward(const void* x, int64_t x_batch_stride, int64_t x_row_stride, v
     if (!(eps >= 0.0f)) return THN_E_SHAPE;                      // "eps must be non-negative" (Ops/norm.py:149)
     if (done) return THN_OK;
     if (x == nullptr || norms == nullptr || (normalize && y == nullptr)) return THN_E_NULL;
+    if (normalize && overlaps(span_of_bmk(y, B, M, K, y_batch_stride, y_row_stride, rp.bytes),
+                              span_of_bmk(x, B, M, K, x_batch_stride, x_row_stride, rp.bytes))) {
+        return THN_E_SHAPE;
+    }
     if (current_cu_count() <= 0) return THN_E_DEVICE;
     PnormFwdArgs a{};
     bool aligned = rp.aligned, uniform = true;
@@ -911,6 +977,11 @@ int act_launch(const void* x, int64_t x_row_stride, const void* g, int64_t g_row
     if (M == 0) return THN_OK;
     if (x == nullptr || out == nullptr || (bwd && g == nullptr)) return THN_E_NULL;
     if (M > 1 && (x_row_stride < N || out_row_stride < N || (bwd && g_row_stride < N))) return THN_E_SHAPE;
+    if (overlaps_any(span_of(out, M, out_row_stride * bytes, N * bytes),
+                     {span_of(x, M, x_row_stride * bytes, N * bytes),
+                      span_of(bwd ? g : nullptr, M, g_row_stride * bytes, N * bytes)})) {
+        return THN_E_SHAPE;
+    }
     const int cus = current_cu_count();
     if (cus <= 0) return THN_E_DEVICE;
     const int which = bwd ? kActBwd : kActFwd;
@@ -1002,6 +1073,14 @@ int thn_norm_set_launch_override(int which, int vecs_per_thread, int threads_per
     ov.bpc.store(blocks_per_cu);
     return THN_OK;
 }
+
+int thn_norm_set_cache_policy(int policy) {
+    if (policy != THN_CACHE_KEEP_X && policy != THN_CACHE_STREAM_X) return THN_E_SHAPE;
+    g_cache_policy.store(policy);
+    return THN_OK;
+}
+
+int thn_norm_get_cache_policy(void) { return g_cache_policy.load(); }
 
 int thn_norm_query_launch(int which, int is_layernorm, int64_t M, int64_t N, int x_dtype, int32_t shape[5]) {
     if (which < 0 || which >= kFamilies || which == kActFwd || which == kActBwd || shape == nullptr) {
@@ -1122,12 +1201,16 @@ int thn_norm_bwd_reduce_partials(const void* workspace, int32_t num_partials, vo
     r.w_dtype = w_dtype;
     const hipStream_t st = static_cast<hipStream_t>(stream);
     const auto blocks = [&](int cols) { return dim3(static_cast<unsigned>((N + cols - 1) / cols), static_cast<unsigned>(n)); };
-    if (N >= thn::kReduceWideFrom) {
-        hipLaunchKernelGGL((thn::reduce_partials_kernel<thn::kReduceColsWide, thn::kReduceAheadWide>), blocks(thn::kReduceColsWide), dim3(256), 0, st, r);
-    } else if (N >= thn::kReduceMidFrom || N * n >= thn::kReduceMidFromBoth) {
-        hipLaunchKernelGGL((thn::reduce_partials_kernel<thn::kReduceColsMid, thn::kReduceAheadMid>), blocks(thn::kReduceColsMid), dim3(256), 0, st, r);
+    // The row slices -- the order of the additions -- follow from N alone; the column width of a workgroup is free.
+    const int slices = thn::reduce_slices(N);
+    if (slices == 16) {
+        hipLaunchKernelGGL((thn::reduce_partials_kernel<64, 16, 1>), blocks(64), dim3(256), 0, st, r);
+    } else if (slices == 32) {
+        hipLaunchKernelGGL((thn::reduce_partials_kernel<32, 32, 4>), blocks(32), dim3(256), 0, st, r);
+    } else if (N * n >= thn::kReduceMidFromBoth) {
+        hipLaunchKernelGGL((thn::reduce_partials_kernel<32, 64, 4>), blocks(32), dim3(512), 0, st, r);
     } else {
-        hipLaunchKernelGGL((thn::reduce_partials_kernel<thn::kReduceCols, thn::kReduceAhead>), blocks(thn::kReduceCols), dim3(256), 0, st, r);
+        hipLaunchKernelGGL((thn::reduce_partials_kernel<16, 64, 1>), blocks(16), dim3(256), 0, st, r);
     }
     return hipGetLastError() == hipSuccess ? THN_OK : THN_E_LAUNCH;
 }
@@ -1161,7 +1244,7 @@ void* g_static_ws_ptr[kMaxDevices];          // per device: the device address o
 bool g_static_ws_known[kMaxDevices];
 
 // The address of the array on the current device; null (and *status set) when it cannot be had.
-void* static_workspace_of_current_device(int* status) {
+void* static_workspace_of_current_device(hipStream_t stream, int* status) {
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
         (void)hipGetLastError();
@@ -1170,6 +1253,17 @@ void* static_workspace_of_current_device(int* status) {
     }
     std::lock_guard<std::mutex> lock(g_static_ws_mutex);
     if (!g_static_ws_known[dev]) {
+        // The lookup is not a stream operation and must not happen while the caller's stream is being captured
+        // into a graph: the first call on a device belongs outside a capture.
+        hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing(stream, &capturing) != hipSuccess) {
+            (void)hipGetLastError();
+            capturing = hipStreamCaptureStatusNone;
+        }
+        if (capturing != hipStreamCaptureStatusNone) {
+            *status = THN_E_DEVICE;
+            return nullptr;
+        }
         void* ptr = nullptr;
         if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(g_static_workspace)) != hipSuccess || ptr == nullptr) {
             (void)hipGetLastError();
@@ -1187,19 +1281,22 @@ extern "C" int thn_norm_bwd_static_workspace(const void* x, int64_t x_row_stride
                                               void* dx, int64_t dx_row_stride, const void* w, const float* mean,
                                               const float* rstd, void* dw, void* db, int64_t M, int64_t N, int x_dtype,
                                               int w_dtype, void* stream) {
-    const int64_t need = thn_norm_bwd_workspace_bytes(M, N, dw != nullptr, db != nullptr, x_dtype);
-    if (need < 0) return static_cast<int>(need);
-    if (need > kStaticWorkspaceBytes) return THN_E_WORKSPACE;      // the caller must bring a workspace: thn_norm_bwd()
+    // bad arguments are reported as thn_norm_bwd() reports them
+    const int64_t upper = thn_norm_bwd_workspace_bytes(M, N, dw != nullptr, db != nullptr, x_dtype);
+    if (upper < 0) return static_cast<int>(upper);
     void* ws = nullptr;
-    if (need > 0) {
+    if (upper > 0) {
         int status = THN_OK;
-        ws = static_workspace_of_current_device(&status);
+        ws = static_workspace_of_current_device(static_cast<hipStream_t>(stream), &status);
         if (ws == nullptr) return status;
     }
+    // The first stage compares what its launch really writes -- one partial row per workgroup of the grid it picks,
+    // which can be fewer than the upper bound above -- with the size of the array and returns THN_E_WORKSPACE when
+    // that does not fit: the caller must then bring a workspace (thn_norm_bwd()).
     // Every partial row the second stage reads is written in full by the first stage of the same call: nothing in
     // the array has to be cleared between calls.
-    return thn_norm_bwd(x, x_row_stride, dy, dy_row_stride, dx, dx_row_stride, w, mean, rstd, dw, db, ws, need, M, N,
-                        x_dtype, w_dtype, stream);
+    return thn_norm_bwd(x, x_row_stride, dy, dy_row_stride, dx, dx_row_stride, w, mean, rstd, dw, db, ws,
+                        upper > 0 ? kStaticWorkspaceBytes : 0, M, N, x_dtype, w_dtype, stream);
 }
 
 // ---- Softmax / Softmin / LogSoftmax -------------------------------------------------------------------------
@@ -1212,6 +1309,9 @@ int thn_softmax_fwd(const void* x, int64_t x_row_stride, void* y, int64_t y_row_
     if (M == 0) return THN_OK;
     if (x == nullptr || y == nullptr) return THN_E_NULL;
     if (x_row_stride < N || y_row_stride < N) return THN_E_SHAPE;
+    if (overlaps(span_of(y, M, y_row_stride * bytes, N * bytes), span_of(x, M, x_row_stride * bytes, N * bytes))) {
+        return THN_E_SHAPE;
+    }
     if (N * bytes > kMaxRowBytes) {                 // rows the row engine cannot hold in registers
         const int cus = current_cu_count();
         if (cus <= 0) return THN_E_DEVICE;
@@ -1262,6 +1362,10 @@ int thn_softmax_bwd(const void* y, int64_t y_row_stride, const void* dy, int64_t
     if (M == 0) return THN_OK;
     if (y == nullptr || dy == nullptr || dx == nullptr) return THN_E_NULL;
     if (y_row_stride < N || dy_row_stride < N || dx_row_stride < N) return THN_E_SHAPE;
+    if (overlaps_any(span_of(dx, M, dx_row_stride * bytes, N * bytes),
+                     {span_of(y, M, y_row_stride * bytes, N * bytes), span_of(dy, M, dy_row_stride * bytes, N * bytes)})) {
+        return THN_E_SHAPE;
+    }
     if (N * bytes > kMaxRowBytes) {
         const int cus = current_cu_count();
         if (cus <= 0) return THN_E_DEVICE;
@@ -1330,6 +1434,10 @@ int thn_pnorm_bwd(const void* x, int64_t x_batch_stride, int64_t x_row_stride, c
     if (crc != THN_OK) return crc;
     if (done) return THN_OK;
     if (x == nullptr || dnorms == nullptr || dx == nullptr || (norms == nullptr && p != 1.0f)) return THN_E_NULL;
+    if (overlaps(span_of_bmk(dx, B, M, K, dx_batch_stride, dx_row_stride, rp.bytes),
+                 span_of_bmk(x, B, M, K, x_batch_stride, x_row_stride, rp.bytes))) {
+        return THN_E_SHAPE;
+    }
     if (current_cu_count() <= 0) return THN_E_DEVICE;
     PnormBwdArgs a{};
     bool aligned = rp.aligned, uniform = true;
@@ -1382,6 +1490,12 @@ int thn_normalize_bwd(const void* x, int64_t x_batch_stride, int64_t x_row_strid
     const bool need_x = p != 2.0f, need_y = p != 1.0f;
     if (norms == nullptr || dy == nullptr || dx == nullptr || (need_x && x == nullptr) || (need_y && y == nullptr)) {
         return THN_E_NULL;
+    }
+    if (overlaps_any(span_of_bmk(dx, B, M, K, dx_batch_stride, dx_row_stride, rp.bytes),
+                     {span_of_bmk(need_x ? x : nullptr, B, M, K, x_batch_stride, x_row_stride, rp.bytes),
+                      span_of_bmk(need_y ? y : nullptr, B, M, K, y_batch_stride, y_row_stride, rp.bytes),
+                      span_of_bmk(dy, B, M, K, dy_batch_stride, dy_row_stride, rp.bytes)})) {
+        return THN_E_SHAPE;
     }
     if (current_cu_count() <= 0) return THN_E_DEVICE;
     NormalizeBwdArgs a{};

@@ -45,16 +45,14 @@ __device__ __forceinline__ void st128(void* p, u32x4 v) {
 }
 
 // The same load without the non-temporal hint: the lines are allocated in the L2 and in the 256 MB memory-side
-// cache behind it.  The norm forward reads x this way (THN_FWD_X_KEEP): x is the one tensor of the step that is
-// read again -- by the backward, which needs x to rebuild xhat -- and a backward that follows its forward closely
-// then finds a part of x in that cache.  Measured on MI355X, bfloat16 16384 x 4096, forward + backward on the same
-// batch, four batches in rotation: RMSNorm 113.8 -> 105.4 us, LayerNorm 117.0 -> 109.9 us; 32768 x 8192 (x is twice
-// the cache) 450 -> 434 us.  The forward on its own is 2-3 % slower for it (44.1 -> 44.9 us): the streaming loads
-// leave the L2 alone.  Everything that is touched once (y, dy, dx; x in the backward) stays non-temporal; keeping
-// any of those as well made the step slower again.
-#ifndef THN_FWD_X_KEEP
-#define THN_FWD_X_KEEP 1
-#endif
+// cache behind it.  The norm forward reads x this way under the "keep" cache policy (the KEEPX instances of
+// norm_fwd_kernel): x is the one tensor of the step that is read again -- by the backward, which needs x to rebuild
+// xhat -- and a backward that follows its forward closely then finds a part of x in that cache.  Measured on MI355X,
+// bfloat16 16384 x 4096, forward + backward on the same batch, four batches in rotation: RMSNorm 113.8 -> 105.4 us,
+// LayerNorm 117.0 -> 109.9 us; 32768 x 8192 (x is twice the cache) 450 -> 434 us.  The forward on its own is 2-3 %
+// slower for it (44.1 -> 44.9 us): the streaming loads leave the L2 alone, which is why a forward that no backward
+// follows takes the streaming instances.  Everything that is touched once (y, dy, dx; x in the backward) stays
+// non-temporal; keeping any of those as well made the step slower again.
 __device__ __forceinline__ u32x4 ld128_keep(const void* p) { return *reinterpret_cast<const u32x4*>(p); }
 __device__ __forceinline__ void st128_keep(void* p, u32x4 v) { *reinterpret_cast<u32x4*>(p) = v; }
 

@@ -140,8 +140,18 @@ inline int run_kernel(void (*kern)(const Args), const Args& a, int grid, int blo
         return 1;                                                                                          \
     }
 
-#define THN_FWD_AL(K_, TPR_, BLOCK_) THN_CASE(norm_fwd_kernel, FwdArgs, true, K_, TPR_, BLOCK_)
-#define THN_FWD_SC(K_, TPR_, BLOCK_) THN_CASE(norm_fwd_kernel, FwdArgs, false, K_, TPR_, BLOCK_)
+// The forward has two instances per shape: x kept in the caches for the backward, or streamed (FwdArgs::keep_x).
+#define THN_FWD_CASE(AL, K_, TPR_, BLOCK_)                                                                 \
+    if (s.k == K_ && s.tpr == TPR_ && s.block == BLOCK_) {                                                 \
+        if (a.keep_x) {                                                                                    \
+            return ln ? run_kernel<FwdArgs>(norm_fwd_kernel<T, true, K_, TPR_, BLOCK_, AL, kNoAct, true>, a, grid, BLOCK_, st, occupancy) \
+                      : run_kernel<FwdArgs>(norm_fwd_kernel<T, false, K_, TPR_, BLOCK_, AL, kNoAct, true>, a, grid, BLOCK_, st, occupancy); \
+        }                                                                                                  \
+        return ln ? run_kernel<FwdArgs>(norm_fwd_kernel<T, true, K_, TPR_, BLOCK_, AL, kNoAct, false>, a, grid, BLOCK_, st, occupancy) \
+                  : run_kernel<FwdArgs>(norm_fwd_kernel<T, false, K_, TPR_, BLOCK_, AL, kNoAct, false>, a, grid, BLOCK_, st, occupancy); \
+    }
+#define THN_FWD_AL(K_, TPR_, BLOCK_) THN_FWD_CASE(true, K_, TPR_, BLOCK_)
+#define THN_FWD_SC(K_, TPR_, BLOCK_) THN_FWD_CASE(false, K_, TPR_, BLOCK_)
 #define THN_BWD_AL(K_, TPR_, BLOCK_) THN_CASE(norm_bwd_kernel, BwdArgs, true, K_, TPR_, BLOCK_)
 #define THN_BWD_AL_LN(K_, TPR_, BLOCK_)                                                                    \
     if (s.k == K_ && s.tpr == TPR_ && s.block == BLOCK_) {                                                 \

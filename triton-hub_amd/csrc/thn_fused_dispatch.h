@@ -63,8 +63,27 @@ THN_DECLARE_FUSED_LAUNCHERS(f64)
         THN_FUSED_ACT_CASE_LN(true, K_, TPR_, BLOCK_, kRelu)                                                   \
         return 1;                                                                                              \
     }
-#define THN_FF_AL(K_, TPR_, BLOCK_) THN_FUSED_CASE(norm_fwd_kernel, FwdArgs, true, K_, TPR_, BLOCK_)
-#define THN_FF_SC(K_, TPR_, BLOCK_) THN_FUSED_CASE(norm_fwd_kernel, FwdArgs, false, K_, TPR_, BLOCK_)
+// The forward on the 128-bit path has a streaming-x instance next to the one that keeps x for the backward
+// (FwdArgs::keep_x); rows off that path always keep x.
+#define THN_FUSED_FWD_ACT_CASE(AL, K_, TPR_, BLOCK_, A)                                                        \
+    if (act == A) {                                                                                            \
+        if (AL && !a.keep_x) {                                                                                 \
+            return ln ? run_kernel<FwdArgs>(norm_fwd_kernel<T, true, K_, TPR_, BLOCK_, AL, A, !AL>, a, grid, BLOCK_, st, occupancy) \
+                      : run_kernel<FwdArgs>(norm_fwd_kernel<T, false, K_, TPR_, BLOCK_, AL, A, !AL>, a, grid, BLOCK_, st, occupancy); \
+        }                                                                                                      \
+        return ln ? run_kernel<FwdArgs>(norm_fwd_kernel<T, true, K_, TPR_, BLOCK_, AL, A, true>, a, grid, BLOCK_, st, occupancy) \
+                  : run_kernel<FwdArgs>(norm_fwd_kernel<T, false, K_, TPR_, BLOCK_, AL, A, true>, a, grid, BLOCK_, st, occupancy); \
+    }
+#define THN_FUSED_FWD_CASE(AL, K_, TPR_, BLOCK_)                                                               \
+    if (s.k == K_ && s.tpr == TPR_ && s.block == BLOCK_) {                                                     \
+        THN_FUSED_FWD_ACT_CASE(AL, K_, TPR_, BLOCK_, kGelu)                                                    \
+        THN_FUSED_FWD_ACT_CASE(AL, K_, TPR_, BLOCK_, kGeluTanh)                                                \
+        THN_FUSED_FWD_ACT_CASE(AL, K_, TPR_, BLOCK_, kSilu)                                                    \
+        THN_FUSED_FWD_ACT_CASE(AL, K_, TPR_, BLOCK_, kRelu)                                                    \
+        return 1;                                                                                              \
+    }
+#define THN_FF_AL(K_, TPR_, BLOCK_) THN_FUSED_FWD_CASE(true, K_, TPR_, BLOCK_)
+#define THN_FF_SC(K_, TPR_, BLOCK_) THN_FUSED_FWD_CASE(false, K_, TPR_, BLOCK_)
 #define THN_FB_AL(K_, TPR_, BLOCK_) THN_FUSED_CASE(norm_bwd_kernel, BwdArgs, true, K_, TPR_, BLOCK_)
 #define THN_FB_SC(K_, TPR_, BLOCK_) THN_FUSED_CASE(norm_bwd_kernel, BwdArgs, false, K_, TPR_, BLOCK_)
 

@@ -43,6 +43,7 @@ struct FwdArgs {
     float eps;
     float inv_n;
     int line_shift;     // 1: rows are not 128 bytes apart and the launch may use row_line_shift()
+    int keep_x;         // host side only: selects the KEEPX instance (thn_norm_set_cache_policy)
 };
 
 struct BwdArgs {
@@ -162,11 +163,14 @@ __device__ __forceinline__ void store_row_vec(char* rowp, int voff, int n_cols, 
 // ---------------------------------------------------------------------------------------------------
 // ACT != kNoAct: y = act(normalise(x)*w + b) -- the activation (one of the parameter-free, input-saving ones of
 // thn_act_math.h) is applied to the float32 value before the one rounding on store; nothing else changes.
-template <typename T, bool LN, int K, int TPR, int BLOCK, bool ALIGNED, int ACT = kNoAct>
+// KEEPX: x is loaded with ordinary (cache-allocating) loads because the operator's backward reads it again (see
+// ld128_keep); false: with streaming loads, for a forward that no backward follows closely.  The two forms differ in
+// that hint on the load instructions and in nothing else: same arithmetic, same bits.
+template <typename T, bool LN, int K, int TPR, int BLOCK, bool ALIGNED, int ACT = kNoAct, bool KEEPX = true>
 __global__ void __launch_bounds__(BLOCK) norm_fwd_kernel(const FwdArgs a) {
     constexpr int VEC = T::VEC;
     constexpr int G = BLOCK / TPR;
-    constexpr bool kKeepX = THN_FWD_X_KEEP != 0;     // x is read again (by the backward): see ld128_keep
+    constexpr bool kKeepX = KEEPX;
     static_assert(BLOCK % TPR == 0 && G >= 1, "a workgroup holds whole rows");
     __shared__ float red[RedSmem<TPR, G, 2>::kFloats];
 
