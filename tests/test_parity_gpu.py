@@ -194,20 +194,25 @@ def test_ragged_hidden_sizes(kind, n, dtype):
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_odd_widths_of_16_bit_rows_reach_every_two_vector_shape(dtype):
-    """LayerNorm backward over 16-bit rows off the 128-bit path runs 2 vectors per thread (its own instances, one per
-    threads-per-row value) up to 2048 vectors and the common 4-vector instance beyond: one odd width for each."""
-    expect = {9: (2, 8), 201: (2, 16), 499: (2, 32), 1001: (2, 64), 1501: (2, 128), 3001: (2, 256), 4099: (2, 512),
-              12289: (2, 1024), 20001: (4, 1024)}
+    """Rows off the 128-bit path run in the same slot shapes as rows on it.  The LayerNorm backward over 16-bit rows
+    keeps to 2 vectors per thread up to 2048 vectors (more would leave one wave per SIMD): one odd width for each
+    threads-per-row value, and one beyond."""
+    expect = {9: (1, 8), 121: (1, 16), 201: (2, 16), 499: (2, 32), 1001: (2, 64), 1501: (2, 128), 3001: (2, 256),
+              4099: (2, 512), 12289: (2, 1024), 20001: (3, 1024)}
     g = torch.Generator().manual_seed(77)
     for n, (k, tpr) in expect.items():
         announce(f"odd width {n} {dtype}")
         m = 131
         assert _launch.query_launch(1, True, m, n, dtype)[:2] == (k, tpr)
-        assert _launch.query_launch(1, False, m, n, dtype)[0] == 4              # RMSNorm keeps the common instances
+        for which, ln in ((0, True), (0, False), (1, False)):
+            kk, tt, _, _, vector_path = _launch.query_launch(which, ln, m, n, dtype)
+            n_vecs = (n + 7) // 8
+            assert vector_path == 0 and kk * tt >= n_vecs and (kk - 1) * tt < n_vecs    # no emptier than it has to be
         x = (0.5 + torch.randn(m, n, generator=g)).to(dtype); dy = torch.randn(m, n, generator=g).to(dtype)
         w = (1 + 0.1 * torch.randn(n, generator=g)); b = 0.1 * torch.randn(n, generator=g)
         run_and_compare("ln", x, dy, w.to(dtype), b.to(dtype), 1e-5, f"odd LN N={n}")
         run_and_compare("ln", x, dy, w, b, 1e-5, f"odd LN N={n}, float32 parameters")
+        run_and_compare("rms", x, dy, w.to(dtype), None, 1e-5, f"odd RMS N={n}")
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
@@ -610,9 +615,14 @@ def test_every_compiled_launch_shape(kind, dtype):
     pairs = sorted(set((k, t) for k, t, _ in fwd_shapes + bwd_shapes))
     try:
         for k, tpr in pairs:
+            widths = []
             for n_vecs in sorted({k * tpr, max((k - 1) * tpr + 1, k * tpr - tpr // 2 - 1)}):
-                n = n_vecs * vec
-                if n * (16 // vec) > 65536:
+                widths.append(n_vecs * vec)
+                # ... and the same number of slots off the 128-bit path: the last one ragged, its window overlapping
+                # the slot before it by 1 to vec - 1 columns
+                widths.append(n_vecs * vec - 1 - n_vecs % (vec - 1))
+            for n in widths:
+                if n * (16 // vec) > 65536 or n < vec or (n % vec and k >= 5):      # (5 to 8 vectors: 128-bit path only)
                     continue
                 f_blocks = [b for kk, tt, b in fwd_shapes if (kk, tt) == (k, tpr)]
                 b_blocks = [b for kk, tt, b in bwd_shapes if (kk, tt) == (k, tpr)]

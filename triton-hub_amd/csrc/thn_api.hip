@@ -79,11 +79,10 @@ constexpr int kPolicyFlags = THN_X_KEEP | THN_X_STREAM;
 // `ln16`: LayerNorm over 16-bit rows (the two norm backwards have instances of their own for that).
 bool shape_compiled(int which, bool aligned, bool ln16, Shape s) {
 #define THN_MATCH(K_, TPR_, BLOCK_) if (s.k == K_ && s.tpr == TPR_ && s.block == BLOCK_) return true;
-    if (!aligned) {
+    if (!aligned && which != kNormFwd && which != kNormBwd) {
         THN_SCALAR_SHAPES(THN_MATCH)
-        if (ln16 && which == kNormBwd) {
-            THN_SCALAR_BWD_LN16_SHAPES(THN_MATCH)
-        }
+    } else if (!aligned && which == kNormBwd) {
+        THN_BWD_SHAPES(THN_MATCH)
     } else if (which == kNormBwd) {
         THN_BWD_SHAPES(THN_MATCH)
         if (ln16) {
@@ -331,7 +330,12 @@ Shape heuristic_shape(int which, bool aligned, bool ln16, int n_vecs) {
     if ((which == kNormBwd || which == kFusedBwd) && aligned && ln16 && n_vecs > 2048) {
         return Shape{ceil_div(n_vecs, 512), 512, 512};
     }
-    int kmax = (aligned && which == kNormBwd && n_vecs > 128) ? 3 : 4;
+    // (the plain norm kernels take the same shapes off the 128-bit path as on it)
+    const bool norm_plain = which == kNormFwd || which == kNormBwd;
+    int kmax = ((aligned || norm_plain) && which == kNormBwd && n_vecs > 128) ? 3 : 4;
+    // LayerNorm backward over 16-bit rows off the 128-bit path: 2 vectors per thread where 1024 threads cover the row
+    // (with 3 or 4 the float32 weights, dW and dB sums of 24-32 columns leave one wave per SIMD).
+    if (!aligned && which == kNormBwd && ln16 && n_vecs <= 2048) kmax = 2;
     // Softmax backward: two input streams and nothing to hold; 2 vectors per thread per stream measured best,
     // except for 2 KiB rows, where one full wave per row (2 x 64) is 8 % slower than half a wave (4 x 32).
     if (aligned && which == kSoftmaxBwd && n_vecs <= 2048 && !(n_vecs > 64 && n_vecs <= 128)) kmax = 2;
@@ -344,19 +348,8 @@ Shape heuristic_shape(int which, bool aligned, bool ln16, int n_vecs) {
             break;
         }
     }
-    if (!aligned) {
+    if (!aligned && !norm_plain) {
         s.k = 4;
-        // LayerNorm backward over 16-bit rows: 2 vectors per thread where 1024 threads cover the row (4 vectors are
-        // more than 256 registers of state, one wave per SIMD).
-        if (which == kNormBwd && ln16 && n_vecs <= 2048) {
-            s.k = 2;
-            for (int tpr : kTprList) {
-                if (tpr * 2 >= n_vecs) {
-                    s.tpr = tpr;
-                    break;
-                }
-            }
-        }
         s.block = s.tpr > 256 ? s.tpr : 256;
         return s;
     }
@@ -485,6 +478,27 @@ int plan_launch(int which, int flavour, bool aligned, int64_t M, int64_t N, int 
         const Shape narrow{2, tpr, 512};
         if (shape_compiled(which, aligned, ln16, narrow)) s = narrow;
     }
+    // Narrow rows (17 to 64 vectors) whose pitch is not a multiple of 128 bytes: with 8 or 16 threads per row a
+    // wave's request is eight or four separate 128- or 256-byte pieces, each across two or three lines; with 16 to 32
+    // threads per row and one or two vectors each the pieces are longer and a wave touches about a third fewer lines.
+    // Forward: 2 vectors per thread in 256-thread workgroups, two per compute unit; backward: 1 vector per thread up
+    // to 32 vectors, 2 beyond, in 512-thread workgroups.  Kernels alone at 2^25 elements, before -> after: float32
+    // N = 72 forward 53.7 -> 49.1 us, backward 96.7 -> 71 us; N = 120 47.4 -> 45.5, 81.3 -> 69.7; N = 200 45.9 -> 45.5,
+    // 74.1 -> 70.3; bfloat16 N = 200 forward 24.0 -> 22.2, backward 41.1 -> 39.7; N = 248 23.6 -> 22.1, 40.5 -> 39.0.
+    // 16-bit rows of 17 to 32 vectors gain the same way at every pitch (N = 256: forward 22.3 -> 21.7, LayerNorm
+    // 23.6 -> 22.6); float32 rows on 128-byte lines do not (N = 128 forward 44.2 -> 44.8) and keep their shapes.
+    bool narrow_forward_pair = false;
+    if ((which == kNormFwd || which == kNormBwd) && aligned && n_vecs > 16 && n_vecs <= 64 &&
+        (pitch_bytes % 128 != 0 || (bytes == 2 && n_vecs <= 32))) {
+        const int k = (which == kNormFwd || n_vecs > 32) ? 2 : 1;
+        int tpr = 8;
+        while (k * tpr < n_vecs) tpr *= 2;
+        const Shape narrow{k, tpr, which == kNormFwd ? 256 : 512};
+        if (shape_compiled(which, aligned, ln16, narrow)) {
+            s = narrow;
+            narrow_forward_pair = which == kNormFwd;
+        }
+    }
     // Rows that start off 128-byte lines: two-row workgroups of 256-thread rows cannot put their requests on line
     // boundaries (the two rows differ in phase, line_shift_ok() below), one-row workgroups can.  Backward: as fast
     // otherwise (fp16 8192 x 6000: 54.8 -> 53.1 us; 8192 x 6016: 52.6 / 52.4 us).  Forward (THN_FWD_SHAPES_TWO_ROWS):
@@ -516,6 +530,8 @@ int plan_launch(int which, int flavour, bool aligned, int64_t M, int64_t N, int 
         shape_compiled(which, aligned, ln16, cand)) {
         s = cand;
     }
+    // rows shorter than one vector have a single element-wise instance per kernel
+    if (!aligned && N < vec_elems) s = Shape{4, 8, 256};
     if (!shape_compiled(which, aligned, ln16, s)) return THN_E_SHAPE;
 
     int bpc = occupancy(which, dtype, flavour, aligned, s);
@@ -562,6 +578,7 @@ int plan_launch(int which, int flavour, bool aligned, int64_t M, int64_t N, int 
             M <= 24 * static_cast<int64_t>(cus)) {
             cap = 2;
         }
+        if (narrow_forward_pair && cap < 2) cap = 2;
     }
     if (cap < bpc) bpc = cap;
     const int rows_per_block = s.block / s.tpr;

@@ -247,10 +247,17 @@ __device__ __forceinline__ void store_param(void* p, int dtype, int64_t i, float
     }
 }
 
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef u32x4 u32x4_param_unaligned __attribute__((aligned(2)));
+typedef u32x2 u32x2_param_unaligned __attribute__((aligned(2)));
+typedef uint32_t u32_param_unaligned __attribute__((aligned(2)));
+
 // VEC consecutive parameter elements of storage type WT starting at column c0, widened to float32, fetched
-// with the widest loads their size allows (the 128-bit path guarantees that the chunk is inside the vector
-// and naturally aligned: the parameter pointer is 16-byte aligned and c0 is a multiple of VEC).
-template <typename WT, int VEC>
+// with the widest loads their size allows.  UNALIGNED false: the 128-bit path guarantees that the chunk is
+// naturally aligned (the parameter pointer is 16-byte aligned and c0 is a multiple of VEC).  UNALIGNED true: the
+// chunk starts at any element (rows off the 128-bit path: the hardware's unaligned access mode serves the same
+// instructions at element-aligned addresses).
+template <typename WT, int VEC, bool UNALIGNED = false>
 __device__ __forceinline__ void load_param_chunk(const void* p, int c0, float (&out)[VEC]) {
     constexpr int BYTES = VEC * WT::kBytes;
     const char* src = static_cast<const char*>(p) + static_cast<int64_t>(c0) * WT::kBytes;
@@ -259,7 +266,10 @@ __device__ __forceinline__ void load_param_chunk(const void* p, int c0, float (&
         constexpr int EPP = WT::VEC;            // elements per 16-byte piece
         u32x4 raw[PIECES];
 #pragma unroll
-        for (int i = 0; i < PIECES; ++i) raw[i] = *reinterpret_cast<const u32x4*>(src + 16 * i);
+        for (int i = 0; i < PIECES; ++i) {
+            if constexpr (UNALIGNED) raw[i] = *reinterpret_cast<const u32x4_param_unaligned*>(src + 16 * i);
+            else raw[i] = *reinterpret_cast<const u32x4*>(src + 16 * i);
+        }
 #pragma unroll
         for (int i = 0; i < PIECES; ++i) {
             float f[EPP];
@@ -268,17 +278,23 @@ __device__ __forceinline__ void load_param_chunk(const void* p, int c0, float (&
             for (int j = 0; j < EPP; ++j) out[i * EPP + j] = f[j];
         }
     } else if constexpr (WT::kBytes == 4) {       // two float32 (VEC == 2)
-        const uint2 raw = *reinterpret_cast<const uint2*>(src);
-        out[0] = as_f32(raw.x);
-        out[1] = as_f32(raw.y);
+        u32x2 raw;
+        if constexpr (UNALIGNED) raw = *reinterpret_cast<const u32x2_param_unaligned*>(src);
+        else raw = *reinterpret_cast<const u32x2*>(src);
+        out[0] = as_f32(raw[0]);
+        out[1] = as_f32(raw[1]);
     } else {                                      // 16-bit parameters under a wider row type: 4 or 8 bytes
         static_assert(WT::kBytes == 2 && (VEC == 2 || VEC == 4), "chunk shape");
         if constexpr (VEC == 4) {
-            const uint2 raw = *reinterpret_cast<const uint2*>(src);
-            WT::unpack_pair(raw.x, out[0], out[1]);
-            WT::unpack_pair(raw.y, out[2], out[3]);
+            u32x2 raw;
+            if constexpr (UNALIGNED) raw = *reinterpret_cast<const u32x2_param_unaligned*>(src);
+            else raw = *reinterpret_cast<const u32x2*>(src);
+            WT::unpack_pair(raw[0], out[0], out[1]);
+            WT::unpack_pair(raw[1], out[2], out[3]);
         } else {
-            const uint32_t raw = *reinterpret_cast<const uint32_t*>(src);
+            uint32_t raw;
+            if constexpr (UNALIGNED) raw = *reinterpret_cast<const u32_param_unaligned*>(src);
+            else raw = *reinterpret_cast<const uint32_t*>(src);
             WT::unpack_pair(raw, out[0], out[1]);
         }
     }
@@ -332,6 +348,33 @@ __device__ __forceinline__ void load_params_clamped(float (&out)[K][VEC], const 
         case kF16: load_params_as<F16, K, VEC, RB, ALIGNED>(out, p, voff, n_cols, fill); break;
         case kBF16: load_params_as<BF16, K, VEC, RB, ALIGNED>(out, p, voff, n_cols, fill); break;
         default: load_params_as<F64, K, VEC, RB, ALIGNED>(out, p, voff, n_cols, fill); break;
+    }
+}
+
+// The same for the overlapped-window slots of rows off the 128-bit path (norm kernels): slot k covers the VEC
+// columns that start at byte offset woff[k] of a row, all of them inside the row, at any element.
+template <typename WT, int K, int VEC>
+__device__ __forceinline__ void load_params_window_as(float (&out)[K][VEC], const void* p, const int (&woff)[K]) {
+    constexpr int RB = 16 / VEC;    // bytes per row element: byte offset / RB = column
+#pragma unroll
+    for (int k = 0; k < K; ++k) load_param_chunk<WT, VEC, true>(p, woff[k] / RB, out[k]);
+}
+
+template <int K, int VEC>
+__device__ __forceinline__ void load_params_window(float (&out)[K][VEC], const void* p, int dtype, const int (&woff)[K],
+                                                   float fill) {
+    if (p == nullptr) {
+#pragma unroll
+        for (int k = 0; k < K; ++k)
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) out[k][e] = fill;
+        return;
+    }
+    switch (dtype) {
+        case kF32: load_params_window_as<F32, K, VEC>(out, p, woff); break;
+        case kF16: load_params_window_as<F16, K, VEC>(out, p, woff); break;
+        case kBF16: load_params_window_as<BF16, K, VEC>(out, p, woff); break;
+        default: load_params_window_as<F64, K, VEC>(out, p, woff); break;
     }
 }
 

@@ -52,16 +52,13 @@ struct Shape {
 // live in LDS).  A 1024-thread workgroup has half as many and spills at 4 vectors per thread.
 #define THN_BWD_SHAPES_LN16(X) X(5, 512, 512) X(6, 512, 512) X(7, 512, 512) X(8, 512, 512)
 
-// Shapes of the element-wise (unaligned) path: four vectors per thread, any row width.
+// Rows off the 128-bit path (N not a whole number of 16-byte vectors, or a pointer or stride off 16 bytes) run the
+// plain norm kernels in the same shapes as rows on it (their slots are 16-byte windows at element-aligned
+// addresses, the ragged last one overlapping its neighbour).  The other families and the norm kernels with an
+// activation epilogue keep one shape per row width there: four vectors per thread.
 #define THN_SCALAR_SHAPES(X)                                                         \
     X(4, 8, 256) X(4, 16, 256) X(4, 32, 256) X(4, 64, 256) X(4, 128, 256)            \
     X(4, 256, 256) X(4, 512, 512) X(4, 1024, 1024)
-
-// LayerNorm backward over 16-bit rows off the 128-bit path: 2 vectors per thread (the 4 of THN_SCALAR_SHAPES are 32
-// float32 columns of weights, dW and dB sums per thread: more than 256 registers, one wave per SIMD).
-#define THN_SCALAR_BWD_LN16_SHAPES(X)                                                \
-    X(2, 8, 256) X(2, 16, 256) X(2, 32, 256) X(2, 64, 256) X(2, 128, 256)            \
-    X(2, 256, 256) X(2, 512, 512) X(2, 1024, 1024)
 
 // Return value of the launchers: 0 launched (or occupancy written), 1 no such instance, <0 HIP error.
 // When `occupancy` is not null the kernel is not launched; *occupancy receives the number of workgroups
@@ -106,11 +103,12 @@ inline int run_kernel(void (*kern)(const Args), const Args& a, int grid, int blo
         if (aligned) {                                                                                     \
             THN_FWD_SHAPES(THN_FWD_AL)                                                                     \
             THN_FWD_SHAPES_TWO_ROWS(THN_FWD_AL)                                                            \
-        } else if (a.n_cols >= TYPE::VEC) { \
-            THN_SCALAR_SHAPES(THN_FWD_SC) \
-        } else { \
-            using T = ElemIo<TYPE>; \
-            THN_FWD_SC(4, 8, 256) \
+        } else if (a.n_cols >= TYPE::VEC) {                                                                \
+            THN_FWD_SHAPES(THN_FWD_SC)                                                                     \
+            THN_FWD_SHAPES_TWO_ROWS(THN_FWD_SC)                                                            \
+        } else {                                                                                           \
+            using T = ElemIo<TYPE>;                                                                        \
+            THN_FWD_SC(4, 8, 256)                                                                          \
         }                                                                                                  \
         return 1;                                                                                          \
     }
@@ -126,16 +124,11 @@ inline int run_kernel(void (*kern)(const Args), const Args& a, int grid, int blo
                     THN_BWD_SHAPES_LN16(THN_BWD_AL_LN)                                                     \
                 }                                                                                          \
             }                                                                                              \
-        } else if (a.n_cols >= TYPE::VEC) { \
-            THN_SCALAR_SHAPES(THN_BWD_SC) \
-            if constexpr (TYPE::kBytes == 2) { \
-                if (ln) { \
-                    THN_SCALAR_BWD_LN16_SHAPES(THN_BWD_SC_LN) \
-                } \
-            } \
-        } else { \
-            using T = ElemIo<TYPE>; \
-            THN_BWD_SC(4, 8, 256) \
+        } else if (a.n_cols >= TYPE::VEC) {                                                                \
+            THN_BWD_SHAPES(THN_BWD_SC)                                                                     \
+        } else {                                                                                           \
+            using T = ElemIo<TYPE>;                                                                        \
+            THN_BWD_SC(4, 8, 256)                                                                          \
         }                                                                                                  \
         return 1;                                                                                          \
     }
@@ -156,10 +149,6 @@ inline int run_kernel(void (*kern)(const Args), const Args& a, int grid, int blo
 #define THN_BWD_AL_LN(K_, TPR_, BLOCK_)                                                                    \
     if (s.k == K_ && s.tpr == TPR_ && s.block == BLOCK_) {                                                 \
         return run_kernel<BwdArgs>(norm_bwd_kernel<T, true, K_, TPR_, BLOCK_, true>, a, grid, BLOCK_, st, occupancy); \
-    }
-#define THN_BWD_SC_LN(K_, TPR_, BLOCK_)                                                                    \
-    if (s.k == K_ && s.tpr == TPR_ && s.block == BLOCK_) {                                                 \
-        return run_kernel<BwdArgs>(norm_bwd_kernel<T, true, K_, TPR_, BLOCK_, false>, a, grid, BLOCK_, st, occupancy); \
     }
 #define THN_BWD_SC(K_, TPR_, BLOCK_) THN_CASE(norm_bwd_kernel, BwdArgs, false, K_, TPR_, BLOCK_)
 

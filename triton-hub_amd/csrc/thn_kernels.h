@@ -99,6 +99,75 @@ __device__ __forceinline__ u32x4 load_row_vec(const char* rowp, int voff, int n_
     else return load_vec_elems<T, KEEP>(rowp, voff, n_cols);
 }
 
+// Vector slots of the norm kernels.  Three I/O modes, fixed at compile time:
+//   ALIGNED                      the 128-bit path: slot v is bytes [16 v, 16 v + 16) of the row;
+//   !ALIGNED, T::kWindowIo       rows off that path that hold at least one vector: slot v is the 16-byte window of
+//                                VEC columns that starts at column min(v * VEC, N - VEC) -- whole inside the row, at
+//                                any element-aligned address.  Only the ragged last slot of a row is moved: its
+//                                window ends at the row end and OVERLAPS the slot before it by `lead` columns.  Those
+//                                columns are loaded, computed and stored a second time -- the same inputs through the
+//                                same instructions, so the same bits to the same bytes as their owner writes -- and
+//                                only left out of the row sums and of the dW / dB sums.  No shifting of registers, no
+//                                branch around the ragged store: the loop keeps its exact s_waitcnt, like the
+//                                128-bit path;
+//   !ALIGNED, !T::kWindowIo      rows shorter than one vector (ElemIo<T>): element accesses with a column bound.
+// voff is the slot's byte offset in a row in the first two modes and its vector index in the third.
+template <typename T, bool ALIGNED, bool KEEP = false>
+__device__ __forceinline__ u32x4 slot_load(const char* rowp, int voff, int n_cols) {
+    if constexpr (ALIGNED) return KEEP ? ld128_keep(rowp + voff) : ld128(rowp + voff);
+    else if constexpr (T::kWindowIo) return KEEP ? ld128u_keep(rowp + voff) : ld128u(rowp + voff);
+    else return load_vec_elems<T, KEEP>(rowp, voff, n_cols);
+}
+
+template <typename T, int K, bool ALIGNED, bool KEEP = false>
+__device__ __forceinline__ void slot_load_row(u32x4 (&dst)[K], const char* base, int64_t stride_bytes, int64_t row,
+                                              const int (&voff)[K], int n_cols) {
+    const char* p = base + row * stride_bytes;
+#pragma unroll
+    for (int k = 0; k < K; ++k) dst[k] = slot_load<T, ALIGNED, KEEP>(p, voff[k], n_cols);
+}
+
+template <typename T, bool ALIGNED>
+__device__ __forceinline__ void slot_store(char* rowp, int voff, int n_cols, const float (&f)[T::VEC]) {
+    if constexpr (ALIGNED) st128(rowp + voff, T::pack(f));
+    else if constexpr (T::kWindowIo) st128u(rowp + voff, T::pack(f));
+    else store_vec_elems<T>(rowp, voff, n_cols, f);
+}
+
+// Offset, overlap and ownership of vector slot v of a row (v may lie outside [0, n_vecs): a slot without work is
+// clamped onto the nearest one and mirrors it).
+template <typename T, bool ALIGNED>
+__device__ __forceinline__ void slot_place(int v, int n_vecs, int n_cols, int& voff, int& lead, bool& own) {
+    const int vc = v < 0 ? 0 : (v < n_vecs ? v : n_vecs - 1);
+    own = v >= 0 && v < n_vecs;
+    lead = 0;
+    if constexpr (ALIGNED) {
+        voff = vc * 16;
+    } else if constexpr (T::kWindowIo) {
+        const int c0 = vc * T::VEC, last = n_cols - T::VEC;
+        const int cw = c0 < last ? c0 : last;
+        voff = cw * T::kBytes;
+        lead = c0 - cw;
+    } else {
+        voff = vc;
+    }
+}
+
+// Whether element e of a slot is a column that this slot owns (and therefore counts in sums).
+template <typename T, bool ALIGNED>
+__device__ __forceinline__ bool slot_counts(int voff, int lead, int e, int n_cols) {
+    if constexpr (ALIGNED) return true;
+    else if constexpr (T::kWindowIo) return e >= lead;
+    else return voff * T::VEC + e < n_cols;
+}
+
+template <typename T, int K, bool ALIGNED>
+__device__ __forceinline__ void slot_params(float (&out)[K][T::VEC], const void* p, int dtype, const int (&voff)[K],
+                                            int n_cols, float fill) {
+    if constexpr (!ALIGNED && T::kWindowIo) load_params_window<K, T::VEC>(out, p, dtype, voff, fill);
+    else load_params_clamped<K, T::VEC, ALIGNED>(out, p, dtype, voff, n_cols, fill);
+}
+
 // Workgroups of 1024 threads serve the widest rows (more than 24 KiB of x in the backward, 32 KiB in the
 // forward) and have 128 registers per thread.  Holding a row as float32 next to the packed next row, the
 // parameters and the column accumulators does not always fit there, and a kernel that spills to scratch
@@ -181,28 +250,25 @@ __global__ void __launch_bounds__(BLOCK) norm_fwd_kernel(const FwdArgs a) {
 
     // Per-slot masks (1 = this thread owns real columns there) and clamped offsets.
     const int shift = (ALIGNED && G == 1) ? row_line_shift(a.line_shift, a.x, a.x_stride_bytes, blockIdx.x) : 0;
-    int voff[K];
+    int voff[K], lead[K];
     bool own[K];
 #pragma unroll
-    for (int k = 0; k < K; ++k) {
-        const int v = t + k * TPR - shift;
-        const int vc = v < 0 ? 0 : (v < a.n_vecs ? v : a.n_vecs - 1);
-        voff[k] = ALIGNED ? vc * 16 : vc;
-        own[k] = v >= 0 && v < a.n_vecs;
-    }
+    for (int k = 0; k < K; ++k) slot_place<T, ALIGNED>(t + k * TPR - shift, a.n_vecs, a.n_cols, voff[k], lead[k], own[k]);
+    // element e of slot k counts in the row sums (always true on the 128-bit path)
+    auto counts = [&](int k, int e) -> bool { return slot_counts<T, ALIGNED>(voff[k], lead[k], e, a.n_cols); };
 
     const int64_t rows_per_iter = static_cast<int64_t>(gridDim.x) * G;
     const int64_t last_row = a.M - 1;
     int64_t row_raw = static_cast<int64_t>(blockIdx.x) * G + g;
     int64_t row = row_raw < a.M ? row_raw : last_row;
     u32x4 cur[K];
-    load_row<T, K, ALIGNED, kKeepX>(cur, a.x, a.x_stride_bytes, row, voff, a.n_cols);   // first, so it overlaps the params
+    slot_load_row<T, K, ALIGNED, kKeepX>(cur, a.x, a.x_stride_bytes, row, voff, a.n_cols);   // first, so it overlaps the params
 
     // Parameters of the clamped slot, so that a clamped slot reproduces its owner's output bit for bit.
     float wr[K][VEC];
     float br[LN ? K : 1][VEC];
-    load_params_clamped<K, VEC, ALIGNED>(wr, a.w, a.w_dtype, voff, a.n_cols, 1.0f);
-    if constexpr (LN) load_params_clamped<K, VEC, ALIGNED>(br, a.b, a.w_dtype, voff, a.n_cols, 0.0f);
+    slot_params<T, K, ALIGNED>(wr, a.w, a.w_dtype, voff, a.n_cols, 1.0f);
+    if constexpr (LN) slot_params<T, K, ALIGNED>(br, a.b, a.w_dtype, voff, a.n_cols, 0.0f);
 
     drain_vector_memory(cur);
     constexpr RowForm kForm = fwd_form<T::kBytes, LN, K, BLOCK, ACT != kNoAct>();
@@ -214,7 +280,7 @@ __global__ void __launch_bounds__(BLOCK) norm_fwd_kernel(const FwdArgs a) {
             u32x4 nxt[kForm.ahead ? K : 1];
             if constexpr (kForm.ahead) {
 #pragma unroll
-                for (int k = 0; k < K; ++k) nxt[k] = load_row_vec<T, ALIGNED, kKeepX>(nxrow, voff[k], a.n_cols);
+                for (int k = 0; k < K; ++k) nxt[k] = slot_load<T, ALIGNED, kKeepX>(nxrow, voff[k], a.n_cols);
             }
             float mean0 = 0.0f, mean = 0.0f, rstd, delta = 0.0f;
             if constexpr (LN) {
@@ -225,7 +291,7 @@ __global__ void __launch_bounds__(BLOCK) norm_fwd_kernel(const FwdArgs a) {
                     T::unpack(cur[k], xf);
                     float sk = 0.0f;
 #pragma unroll
-                    for (int e = 0; e < VEC; ++e) sk += xf[e];
+                    for (int e = 0; e < VEC; ++e) sk += counts(k, e) ? xf[e] : 0.0f;
                     s[0] += own[k] ? sk : 0.0f;
                 }
                 row_allreduce<TPR, G, 1>(s, red, phase, g, t);
@@ -240,7 +306,7 @@ __global__ void __launch_bounds__(BLOCK) norm_fwd_kernel(const FwdArgs a) {
 #pragma unroll
                     for (int e = 0; e < VEC; ++e) {
                         float d = xf[e] - mean0;
-                        if constexpr (!ALIGNED) d = (voff[k] * VEC + e < a.n_cols) ? d : 0.0f;
+                        d = counts(k, e) ? d : 0.0f;
                         q0 += d;
                         q1 = fmaf(d, d, q1);
                     }
@@ -261,7 +327,10 @@ __global__ void __launch_bounds__(BLOCK) norm_fwd_kernel(const FwdArgs a) {
                     T::unpack(cur[k], xf);
                     float qk = 0.0f;
 #pragma unroll
-                    for (int e = 0; e < VEC; ++e) qk = fmaf(xf[e], xf[e], qk);
+                    for (int e = 0; e < VEC; ++e) {
+                        const float xm = counts(k, e) ? xf[e] : 0.0f;
+                        qk = fmaf(xm, xm, qk);
+                    }
                     q[0] += own[k] ? qk : 0.0f;
                 }
                 row_allreduce<TPR, G, 1>(q, red, phase, g, t);
@@ -276,17 +345,16 @@ __global__ void __launch_bounds__(BLOCK) norm_fwd_kernel(const FwdArgs a) {
 #pragma unroll
                 for (int e = 0; e < VEC; ++e) {
                     if constexpr (LN) {
-                        float d = xf[e] - mean0;
-                        if constexpr (!ALIGNED) d = (voff[k] * VEC + e < a.n_cols) ? d : 0.0f;
+                        const float d = xf[e] - mean0;       // every column of the slot is stored: none is masked here
                         yf[e] = fmaf((d - delta) * rstd, wr[k][e], br[k][e]);
                     } else {
                         yf[e] = xf[e] * rstd * wr[k][e];
                     }
                     if constexpr (ACT != kNoAct) yf[e] = act_fwd<ACT, float>(yf[e], 0.0f, 0.0f);
                 }
-                store_row_vec<T, ALIGNED>(yrow, voff[k], a.n_cols, yf);
+                slot_store<T, ALIGNED>(yrow, voff[k], a.n_cols, yf);
                 if constexpr (kForm.ahead) cur[k] = nxt[k];
-                else cur[k] = load_row_vec<T, ALIGNED, kKeepX>(nxrow, voff[k], a.n_cols);
+                else cur[k] = slot_load<T, ALIGNED, kKeepX>(nxrow, voff[k], a.n_cols);
             }
             if constexpr (LN) a.mean[row] = mean;
             a.rstd[row] = rstd;
@@ -306,7 +374,7 @@ __global__ void __launch_bounds__(BLOCK) norm_fwd_kernel(const FwdArgs a) {
         // 3-5 % with the same wait from 8192 rows on, the other forward shapes +-1 %, and the backward shapes with one
         // row per workgroup lose 2-6 %.
         if constexpr (G == 1 && ALIGNED && K == 4 && BLOCK == 256) __builtin_amdgcn_s_waitcnt(0x0F70);
-        load_row<T, K, ALIGNED, kKeepX>(nxt, a.x, a.x_stride_bytes, nrow, voff, a.n_cols);
+        slot_load_row<T, K, ALIGNED, kKeepX>(nxt, a.x, a.x_stride_bytes, nrow, voff, a.n_cols);
 
         float xf[K][VEC];
 #pragma unroll
@@ -319,7 +387,7 @@ __global__ void __launch_bounds__(BLOCK) norm_fwd_kernel(const FwdArgs a) {
             for (int k = 0; k < K; ++k) {
                 float sk = 0.0f;
 #pragma unroll
-                for (int e = 0; e < VEC; ++e) sk += xf[k][e];   // unaligned path: absent columns load as 0
+                for (int e = 0; e < VEC; ++e) sk += counts(k, e) ? xf[k][e] : 0.0f;
                 s[0] += own[k] ? sk : 0.0f;
             }
             row_allreduce<TPR, G, 1>(s, red, phase, g, t);
@@ -330,11 +398,11 @@ __global__ void __launch_bounds__(BLOCK) norm_fwd_kernel(const FwdArgs a) {
                 float q0 = 0.0f, q1 = 0.0f;
 #pragma unroll
                 for (int e = 0; e < VEC; ++e) {
-                    float d = xf[k][e] - mean0;
-                    if constexpr (!ALIGNED) d = (voff[k] * VEC + e < a.n_cols) ? d : 0.0f;
-                    xf[k][e] = d;
-                    q0 += d;
-                    q1 = fmaf(d, d, q1);
+                    const float d = xf[k][e] - mean0;
+                    xf[k][e] = d;                                   // kept for the output of every column of the slot
+                    const float dm = counts(k, e) ? d : 0.0f;
+                    q0 += dm;
+                    q1 = fmaf(dm, dm, q1);
                 }
                 q[0] += own[k] ? q0 : 0.0f;
                 q[1] += own[k] ? q1 : 0.0f;
@@ -350,7 +418,10 @@ __global__ void __launch_bounds__(BLOCK) norm_fwd_kernel(const FwdArgs a) {
             for (int k = 0; k < K; ++k) {
                 float qk = 0.0f;
 #pragma unroll
-                for (int e = 0; e < VEC; ++e) qk = fmaf(xf[k][e], xf[k][e], qk);
+                for (int e = 0; e < VEC; ++e) {
+                    const float xm = counts(k, e) ? xf[k][e] : 0.0f;
+                    qk = fmaf(xm, xm, qk);
+                }
                 q[0] += own[k] ? qk : 0.0f;
             }
             row_allreduce<TPR, G, 1>(q, red, phase, g, t);
@@ -367,7 +438,7 @@ __global__ void __launch_bounds__(BLOCK) norm_fwd_kernel(const FwdArgs a) {
                 else yf[e] = xf[k][e] * rstd * wr[k][e];
                 if constexpr (ACT != kNoAct) yf[e] = act_fwd<ACT, float>(yf[e], 0.0f, 0.0f);
             }
-            store_row_vec<T, ALIGNED>(yrow, voff[k], a.n_cols, yf);
+            slot_store<T, ALIGNED>(yrow, voff[k], a.n_cols, yf);
         }
         // Every thread of the row stores the same two words to the same address (one request per wave): a
         // store under "if (t == 0)" would be a branch, see the note on branches at the top of this file.
@@ -465,23 +536,20 @@ __global__ void __launch_bounds__(BLOCK) norm_bwd_kernel(const BwdArgs a) {
     int phase = 0;
 
     const int shift = (ALIGNED && G == 1) ? row_line_shift(a.line_shift, a.x, a.x_stride_bytes, blockIdx.x) : 0;
-    int voff[K];
+    int voff[K], lead[K];
     bool own[K];
 #pragma unroll
-    for (int k = 0; k < K; ++k) {
-        const int v = t + k * TPR - shift;
-        const int vc = v < 0 ? 0 : (v < a.n_vecs ? v : a.n_vecs - 1);
-        voff[k] = ALIGNED ? vc * 16 : vc;
-        own[k] = v >= 0 && v < a.n_vecs;
-    }
+    for (int k = 0; k < K; ++k) slot_place<T, ALIGNED>(t + k * TPR - shift, a.n_vecs, a.n_cols, voff[k], lead[k], own[k]);
+    // element e of slot k counts in the row sums and in dW / dB (always true on the 128-bit path)
+    auto counts = [&](int k, int e) -> bool { return slot_counts<T, ALIGNED>(voff[k], lead[k], e, a.n_cols); };
 
     const int64_t rows_per_iter = static_cast<int64_t>(gridDim.x) * G;
     const int64_t last_row = a.M - 1;
     int64_t row_raw = static_cast<int64_t>(blockIdx.x) * G + g;
     int64_t row = row_raw < a.M ? row_raw : last_row;
     u32x4 cx[K], cg[K];
-    load_row<T, K, ALIGNED>(cx, a.x, a.x_stride_bytes, row, voff, a.n_cols);    // first, so they overlap the params
-    load_row<T, K, ALIGNED>(cg, a.dy, a.dy_stride_bytes, row, voff, a.n_cols);
+    slot_load_row<T, K, ALIGNED>(cx, a.x, a.x_stride_bytes, row, voff, a.n_cols);    // first, so they overlap the params
+    slot_load_row<T, K, ALIGNED>(cg, a.dy, a.dy_stride_bytes, row, voff, a.n_cols);
     float c_mean = LN ? a.mean[row] : 0.0f;
     float c_rstd = a.rstd[row];
 
@@ -495,9 +563,9 @@ __global__ void __launch_bounds__(BLOCK) norm_bwd_kernel(const BwdArgs a) {
     float wr[K][VEC];
     Acc dw[kLdsTotals ? 1 : K][VEC];
     Acc db[LN ? K : 1][VEC];
-    load_params_clamped<K, VEC, ALIGNED>(wr, a.w, a.w_dtype, voff, a.n_cols, 1.0f);
+    slot_params<T, K, ALIGNED>(wr, a.w, a.w_dtype, voff, a.n_cols, 1.0f);
     float br[(FUSED && LN) ? K : 1][VEC];
-    if constexpr (FUSED && LN) load_params_clamped<K, VEC, ALIGNED>(br, a.b, a.w_dtype, voff, a.n_cols, 0.0f);
+    if constexpr (FUSED && LN) slot_params<T, K, ALIGNED>(br, a.b, a.w_dtype, voff, a.n_cols, 0.0f);
 #pragma unroll
     for (int k = 0; k < K; ++k) {
 #pragma unroll
@@ -518,12 +586,14 @@ __global__ void __launch_bounds__(BLOCK) norm_bwd_kernel(const BwdArgs a) {
         const int64_t nrow_raw = row_raw + rows_per_iter;
         const int64_t nrow = nrow_raw < a.M ? nrow_raw : last_row;
         u32x4 nx[K], ng[K];
-        load_row<T, K, ALIGNED>(nx, a.x, a.x_stride_bytes, nrow, voff, a.n_cols);
-        load_row<T, K, ALIGNED>(ng, a.dy, a.dy_stride_bytes, nrow, voff, a.n_cols);
+        slot_load_row<T, K, ALIGNED>(nx, a.x, a.x_stride_bytes, nrow, voff, a.n_cols);
+        slot_load_row<T, K, ALIGNED>(ng, a.dy, a.dy_stride_bytes, nrow, voff, a.n_cols);
         const float n_mean = LN ? a.mean[nrow] : 0.0f;
         const float n_rstd = a.rstd[nrow];
         const bool live = !MASKED || row_raw < a.M;
 
+        // u, gf, wdy hold every column of a slot as it is needed for dx (also the columns of an overlapped window that
+        // the slot does not own); whatever enters a sum goes through counts().
         float u[K][VEC], gf[K][VEC], wdy[K][VEC];
         float s[NV];
 #pragma unroll
@@ -538,10 +608,9 @@ __global__ void __launch_bounds__(BLOCK) norm_bwd_kernel(const BwdArgs a) {
                 float sk = 0.0f;
 #pragma unroll
                 for (int e = 0; e < VEC; ++e) {
-                    float v = (u[k][e] - c_mean) * c_rstd;
-                    if constexpr (!ALIGNED) v = (voff[k] * VEC + e < a.n_cols) ? v : 0.0f;
+                    const float v = (u[k][e] - c_mean) * c_rstd;
                     u[k][e] = v;
-                    sk += v;
+                    sk += counts(k, e) ? v : 0.0f;
                 }
                 su[0] += own[k] ? sk : 0.0f;
             }
@@ -556,13 +625,9 @@ __global__ void __launch_bounds__(BLOCK) norm_bwd_kernel(const BwdArgs a) {
 #pragma unroll
             for (int e = 0; e < VEC; ++e) {
                 if constexpr (FUSED && LN) {
-                    float v = u[k][e] - dlt_fused;                      // the corrected xhat
-                    if constexpr (!ALIGNED) v = (voff[k] * VEC + e < a.n_cols) ? v : 0.0f;
-                    u[k][e] = v;
+                    u[k][e] -= dlt_fused;                               // the corrected xhat
                 } else if constexpr (LN) {
-                    float v = (u[k][e] - c_mean) * c_rstd;
-                    if constexpr (!ALIGNED) v = (voff[k] * VEC + e < a.n_cols) ? v : 0.0f;
-                    u[k][e] = v;
+                    u[k][e] = (u[k][e] - c_mean) * c_rstd;
                 } else {
                     u[k][e] *= c_rstd;
                 }
@@ -571,10 +636,12 @@ __global__ void __launch_bounds__(BLOCK) norm_bwd_kernel(const BwdArgs a) {
                     gf[k][e] = act_bwd<ACT, float>(z, gf[k][e], 0.0f, 0.0f);       // dy * act'(z)
                 }
                 wdy[k][e] = wr[k][e] * gf[k][e];
-                s0 = fmaf(u[k][e], wdy[k][e], s0);
+                const bool in = counts(k, e);
+                const float wdy_in = in ? wdy[k][e] : 0.0f;
+                s0 = fmaf(u[k][e], wdy_in, s0);
                 if constexpr (LN) {
-                    s1 += wdy[k][e];
-                    if constexpr (!FUSED) s2 += u[k][e];
+                    s1 += wdy_in;
+                    if constexpr (!FUSED) s2 += in ? u[k][e] : 0.0f;
                 }
             }
             s[0] += own[k] ? s0 : 0.0f;
@@ -603,18 +670,15 @@ __global__ void __launch_bounds__(BLOCK) norm_bwd_kernel(const BwdArgs a) {
 #pragma unroll
             for (int e = 0; e < VEC; ++e) {
                 float xhat = u[k][e];
-                if constexpr (LN) {
-                    xhat -= dlt;
-                    if constexpr (!ALIGNED) xhat = (voff[k] * VEC + e < a.n_cols) ? xhat : 0.0f;
-                }
+                if constexpr (LN) xhat -= dlt;
                 // subtract first, scale by rstd last: when dx cancels to (almost) nothing -- rstd is huge for a
                 // near-constant row -- the rounding error stays relative to the small difference
                 dxf[e] = (wdy[k][e] - fmaf(xhat, c1, c2)) * c_rstd;
-                const float gl = (MASKED && !live) ? 0.0f : gf[k][e];
+                const float gl = ((MASKED && !live) || !counts(k, e)) ? 0.0f : gf[k][e];
                 dw[k][e] = fma(static_cast<Acc>(gl), static_cast<Acc>(xhat), dw[k][e]);
                 if constexpr (LN) db[k][e] += static_cast<Acc>(gl);
             }
-            store_row_vec<T, ALIGNED>(dxrow, voff[k], a.n_cols, dxf);
+            slot_store<T, ALIGNED>(dxrow, voff[k], a.n_cols, dxf);
         }
 
 #pragma unroll
@@ -650,15 +714,15 @@ __global__ void __launch_bounds__(BLOCK) norm_bwd_kernel(const BwdArgs a) {
         u32x4 nx[kForm.ahead ? K : 1], ng[kForm.ahead ? K : 1];
         if constexpr (kForm.ahead) {
 #pragma unroll
-            for (int k = 0; k < K; ++k) nx[k] = load_row_vec<T, ALIGNED>(nxrow, vo(k), a.n_cols);
+            for (int k = 0; k < K; ++k) nx[k] = slot_load<T, ALIGNED>(nxrow, vo(k), a.n_cols);
 #pragma unroll
-            for (int k = 0; k < K; ++k) ng[k] = load_row_vec<T, ALIGNED>(ngrow, vo(k), a.n_cols);
+            for (int k = 0; k < K; ++k) ng[k] = slot_load<T, ALIGNED>(ngrow, vo(k), a.n_cols);
         }
         const float n_mean = LN ? a.mean[nrow] : 0.0f;
         const float n_rstd = a.rstd[nrow];
 
         // float32 view of vector slot k: u (LayerNorm: before the dlt correction unless `dlt_f` carries it) and
-        // the upstream gradient (times act'(z) with an epilogue)
+        // the upstream gradient (times act'(z) with an epilogue); every column of the slot, masked nowhere
         auto expand = [&](int k, float dlt_f, bool corrected, float (&u)[VEC], float (&gf)[VEC]) {
             T::unpack(cx[k], u);
             T::unpack(cg[k], gf);
@@ -666,12 +730,8 @@ __global__ void __launch_bounds__(BLOCK) norm_bwd_kernel(const BwdArgs a) {
             for (int e = 0; e < VEC; ++e) {
                 if constexpr (LN) {
                     float v = (u[e] - c_mean) * c_rstd;
-                    if constexpr (!ALIGNED) v = (voff[k] * VEC + e < a.n_cols) ? v : 0.0f;
                     if constexpr (FUSED) {
-                        if (corrected) {
-                            v -= dlt_f;
-                            if constexpr (!ALIGNED) v = (voff[k] * VEC + e < a.n_cols) ? v : 0.0f;
-                        }
+                        if (corrected) v -= dlt_f;
                     }
                     u[e] = v;
                 } else {
@@ -698,7 +758,7 @@ __global__ void __launch_bounds__(BLOCK) norm_bwd_kernel(const BwdArgs a) {
                 expand(k, 0.0f, false, u, gf);
                 float sk = 0.0f;
 #pragma unroll
-                for (int e = 0; e < VEC; ++e) sk += u[e];
+                for (int e = 0; e < VEC; ++e) sk += counts(k, e) ? u[e] : 0.0f;
                 su[0] += own[k] ? sk : 0.0f;
             }
             row_allreduce<TPR, G, 1>(su, red, phase, g, t);
@@ -713,11 +773,12 @@ __global__ void __launch_bounds__(BLOCK) norm_bwd_kernel(const BwdArgs a) {
             float s0 = 0.0f, s1 = 0.0f, s2 = 0.0f;
 #pragma unroll
             for (int e = 0; e < VEC; ++e) {
-                const float wdy = wr[k][e] * gf[e];
-                s0 = fmaf(u[e], wdy, s0);
+                const bool in = counts(k, e);
+                const float wdy_in = in ? wr[k][e] * gf[e] : 0.0f;
+                s0 = fmaf(u[e], wdy_in, s0);
                 if constexpr (LN) {
-                    s1 += wdy;
-                    if constexpr (!FUSED) s2 += u[e];
+                    s1 += wdy_in;
+                    if constexpr (!FUSED) s2 += in ? u[e] : 0.0f;
                 }
             }
             s[0] += own[k] ? s0 : 0.0f;
@@ -756,12 +817,9 @@ __global__ void __launch_bounds__(BLOCK) norm_bwd_kernel(const BwdArgs a) {
             for (int e = 0; e < VEC; ++e) {
                 const float wdy = wr[k][e] * gf[e];
                 float xhat = u[e];
-                if constexpr (LN) {
-                    xhat -= dlt;
-                    if constexpr (!ALIGNED) xhat = (voff[k] * VEC + e < a.n_cols) ? xhat : 0.0f;
-                }
+                if constexpr (LN) xhat -= dlt;
                 dxf[e] = (wdy - fmaf(xhat, c1, c2)) * c_rstd;
-                const float gl = (MASKED && !live) ? 0.0f : gf[e];
+                const float gl = ((MASKED && !live) || !counts(k, e)) ? 0.0f : gf[e];
                 if constexpr (kLdsTotals) tot[e] = fmaf(gl, xhat, tot[e]);
                 else dw[k][e] = fma(static_cast<Acc>(gl), static_cast<Acc>(xhat), dw[k][e]);
                 if constexpr (LN) db[k][e] += static_cast<Acc>(gl);
@@ -770,13 +828,13 @@ __global__ void __launch_bounds__(BLOCK) norm_bwd_kernel(const BwdArgs a) {
                 dw_lds[(2 * k) * BLOCK + tid] = f32x4{tot[0], tot[1], tot[2], tot[3]};
                 dw_lds[(2 * k + 1) * BLOCK + tid] = f32x4{tot[4], tot[5], tot[6], tot[7]};
             }
-            store_row_vec<T, ALIGNED>(dxrow, vo(k), a.n_cols, dxf);
+            slot_store<T, ALIGNED>(dxrow, vo(k), a.n_cols, dxf);
             if constexpr (kForm.ahead) {
                 cx[k] = nx[k];
                 cg[k] = ng[k];
             } else {
-                cx[k] = load_row_vec<T, ALIGNED>(nxrow, vo(k), a.n_cols);
-                cg[k] = load_row_vec<T, ALIGNED>(ngrow, vo(k), a.n_cols);
+                cx[k] = slot_load<T, ALIGNED>(nxrow, vo(k), a.n_cols);
+                cg[k] = slot_load<T, ALIGNED>(ngrow, vo(k), a.n_cols);
             }
         }
         c_mean = n_mean;
@@ -814,10 +872,13 @@ __global__ void __launch_bounds__(BLOCK) norm_bwd_kernel(const BwdArgs a) {
                 if (want_db) combine_groups<BLOCK, TPR, VEC, Acc>(db[k], comb, g, t);
             }
         }
-        const int v = t + k * TPR - shift;
         if (g == 0 && own[k]) {
-            // part_pitch is a multiple of 64 floats >= n_vecs*VEC, so whole vectors always fit.
-            const int64_t off = static_cast<int64_t>(blockIdx.x) * a.part_pitch + static_cast<int64_t>(v) * VEC;
+            // The slot's first column: a multiple of VEC floats into the partial row on the 128-bit path (the pitch is a
+            // multiple of 64 floats >= n_vecs*VEC, so whole vectors fit and the 16-byte stores are aligned), any column
+            // for the overlapped window of a ragged last slot, whose first `lead` columns belong to the slot before it.
+            const int col0 = ALIGNED ? (t + k * TPR - shift) * VEC
+                                     : (T::kWindowIo ? voff[k] / T::kBytes : voff[k] * VEC);
+            const int64_t off = static_cast<int64_t>(blockIdx.x) * a.part_pitch + col0;
             float pw[VEC], pb[VEC];
 #pragma unroll
             for (int e = 0; e < VEC; ++e) {
@@ -825,8 +886,18 @@ __global__ void __launch_bounds__(BLOCK) norm_bwd_kernel(const BwdArgs a) {
                 else pw[e] = static_cast<float>(dw[k][e]);
                 pb[e] = LN ? static_cast<float>(db[LN ? k : 0][e]) : 0.0f;
             }
-            if (want_dw) store_partial<VEC>(a.dw_part + off, pw);
-            if (want_db) store_partial<VEC>(a.db_part + off, pb);
+            if (lead[k] == 0) {
+                if (want_dw) store_partial<VEC>(a.dw_part + off, pw);
+                if (want_db) store_partial<VEC>(a.db_part + off, pb);
+            } else {
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) {
+                    if (e >= lead[k]) {
+                        if (want_dw) a.dw_part[off + e] = pw[e];
+                        if (want_db) a.db_part[off + e] = pb[e];
+                    }
+                }
+            }
         }
     }
 }
