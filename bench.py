@@ -388,7 +388,7 @@ def config_summary(lib, dev, workload, args):
     """One more configuration of the benchmark contract: the step as defined, the no-reuse step, the kernels."""
     bench = NormBench(lib, dev, workload)
     short = argparse.Namespace(steps=args.steps, warmup=min(args.warmup, 5))
-    warm = measure_norm(bench, short, "keep", 0, preroll=min(PREROLL_STEPS, 30))
+    warm = measure_norm(bench, short, "keep", 0)
     cold = measure_norm(bench, short, "stream", 2, preroll=0)
     fwd_shape, bwd_shape = bench.shapes()
     out = {"op": "LayerNorm" if bench.ln else "RMSNorm", "rows": bench.m, "hidden": bench.n, "dtype": bench.dname,
@@ -547,6 +547,25 @@ def main():
             out["configs"] = {w_: config_summary(lib, dev, w_, short) for w_ in CONTRACT_CONFIGS}
     if not args.no_cpu_baseline and not args.steps_only and bench.fused_act < 0:      # (the fused workloads carry no CPU leg)
         out["cpu_baseline"] = cpu_baseline(*cpu_args)
+    if headline and not args.steps_only:
+        # The figures of the whole line once more, short, as its last key (a reader who keeps only the end of the line
+        # still has every workload), and as plain numbers inside `config`.
+        def row(r, cold_):
+            k = r.get("kernels_us") or {}
+            return [r["pct_of_hbm_peak"], cold_["pct_of_hbm_peak"] if cold_ else None, round(r["ms_per_step"] * 1e3, 1),
+                    [k.get("forward"), k.get("backward_dx_partials"), k.get("backward_reduce_partials")]]
+        digest = {"columns": ["% of 8 TB/s, same-batch step, keep_x", "% of 8 TB/s, no-reuse step, stream_x", "us per step",
+                              "us forward | backward dx+partials | second stage, inside the step"],
+                  "rmsnorm_bf16_16384x4096": row(res, cold),
+                  "layernorm_bf16_16384x4096": row(out["layernorm_same_shape"], out["no_reuse"]["layernorm"])}
+        for w_, c in out.get("configs", {}).items():
+            k = c.get("kernels_us") or {}
+            digest[w_] = [c["pct_of_hbm_peak"], c["no_reuse_pct"], round(c["ms_per_step"] * 1e3, 1),
+                          [k.get("forward"), k.get("backward_dx_partials"), k.get("backward_reduce_partials")]]
+        out["config"].update({"layernorm_same_shape_pct_of_hbm_peak": out["layernorm_same_shape"]["pct_of_hbm_peak"],
+                              "no_reuse_stream_x_rmsnorm_pct_of_hbm_peak": cold["pct_of_hbm_peak"],
+                              "no_reuse_stream_x_layernorm_pct_of_hbm_peak": out["no_reuse"]["layernorm"]["pct_of_hbm_peak"]})
+        out["digest"] = digest
     print(json.dumps(out), flush=True)
 
 

@@ -333,9 +333,6 @@ Shape heuristic_shape(int which, bool aligned, bool ln16, int n_vecs) {
     // (the plain norm kernels take the same shapes off the 128-bit path as on it)
     const bool norm_plain = which == kNormFwd || which == kNormBwd;
     int kmax = ((aligned || norm_plain) && which == kNormBwd && n_vecs > 128) ? 3 : 4;
-    // LayerNorm backward over 16-bit rows off the 128-bit path: 2 vectors per thread where 1024 threads cover the row
-    // (with 3 or 4 the float32 weights, dW and dB sums of 24-32 columns leave one wave per SIMD).
-    if (!aligned && which == kNormBwd && ln16 && n_vecs <= 2048) kmax = 2;
     // Softmax backward: two input streams and nothing to hold; 2 vectors per thread per stream measured best,
     // except for 2 KiB rows, where one full wave per row (2 x 64) is 8 % slower than half a wave (4 x 32).
     if (aligned && which == kSoftmaxBwd && n_vecs <= 2048 && !(n_vecs > 64 && n_vecs <= 128)) kmax = 2;
@@ -402,10 +399,12 @@ void softmax_loop_launch(int which, int* block, int* bpc) {
 // rows and 2 up to 256-byte rows; those with two streams 2 up to 128-byte rows (the norm backward up to 256-byte
 // rows, where it runs one vector per thread: bf16 N = 128 5.2 -> 6.1 TB/s).
 int narrow_row_blocks_per_cu(int which, int n_vecs, bool ragged16) {
-    // 16-bit rows whose width is not a whole number of vectors: the unaligned-window instances spend 2-3 times
-    // the instructions per byte (shifts, per-column masks), and a second workgroup hides their latency
-    // (bf16 N = 4098: forward 2.6 -> 3.6 TB/s, RMSNorm 3.8 -> 4.6; float32 rows do not gain).
-    if (ragged16 && n_vecs > 16) return 2;
+    // 16-bit rows whose width is not a whole number of vectors, in the families whose unaligned-window instances
+    // shift the ragged vector in registers: 2-3 times the instructions per byte (shifts, per-column masks), and a
+    // second workgroup hides their latency (bf16 N = 4098 softmax: 2.6 -> 3.6 TB/s; float32 rows do not gain).  The
+    // norm kernels' overlapped windows cost no more than aligned vectors and lose 5-7 % with a second workgroup
+    // (bf16 24564 x 4098 forward 69.1 us with one, 73.4 with two; fp16 8192 x 12289 81.6 / 85.0).
+    if (ragged16 && n_vecs > 16 && which != kNormFwd && which != kNormBwd) return 2;
     const bool one_stream = which == kNormFwd || which == kSoftmaxFwd || which == kPnormFwd || which == kFusedFwd;
     if (n_vecs <= 8) return one_stream ? 4 : 2;
     if (n_vecs <= 16) return (one_stream || which == kNormBwd) ? 2 : 1;   // norm backward: with one vector per thread
@@ -463,40 +462,47 @@ int plan_launch(int which, int flavour, bool aligned, int64_t M, int64_t N, int 
         M > 8 * static_cast<int64_t>(cus) && (n_vecs <= 896 || M <= 32 * static_cast<int64_t>(cus))) {
         s = Shape{2, 512, 512};
     }
-    // The norm backward over narrow rows: 2 vectors per thread in 512-thread workgroups -- eight waves per compute
-    // unit instead of the four of a 256-thread workgroup, which a backward step of 16-bit rows (twice the arithmetic
-    // per byte) does not fill a compute unit with.  16-bit rows of 17 to 192 vectors, and the rows of 129 to 192
-    // vectors of every type up to float32 (3 x 64 vectors in 256 threads otherwise).  Forward + backward of 2^26
-    // elements, % of 8 TB/s, RMSNorm / LayerNorm: bf16 N = 256: 76.9 / 73.3 -> 78.3 / 75.3; 640: 66.8 / 62.1 ->
-    // 74.8 / 66.4; 768: 73.1 / 69.0 -> 77.9 / 73.0; 1024: 77.3 / 74.5 -> 78.0 / 75.8; 1280: 72.1 / 66.6 -> 77.4 / 73.3;
-    // 1536: 75.8 / 70.4 -> 77.8 / 75.0; float32 N = 640: 79.2 / 75.0 -> 79.5 / 78.3; 768: 80.4 / 78.1 -> 80.9 / 79.5
-    // (float32 rows of up to 128 vectors are as fast or faster in 4-vector 256-thread workgroups: 80.9-82.0 %).
-    if (which == kNormBwd && aligned && ((bytes == 2 && n_vecs > 16 && n_vecs <= 192) ||
-                                         (bytes <= 4 && n_vecs > 128 && n_vecs <= 192))) {
+    // The norm backward over narrow rows (17 to 192 vectors, every storage type, on and off the 128-bit path): 2
+    // vectors per thread in 512-thread workgroups -- eight waves per compute unit instead of the four of a 256-thread
+    // workgroup, which a backward step does not fill a compute unit with, and twice the threads per row of the
+    // 4-vector shapes, so that a wave's request is made of fewer, longer pieces (at a pitch that is not a multiple of
+    // 128 bytes every piece starts and ends inside a line).  The LayerNorm backward over 16-bit rows of up to 96
+    // vectors goes one step further: 1 vector per thread, two workgroups per compute unit.  Forward + backward of
+    // 2^26 elements with only the backward's shape changed, % of 8 TB/s, 4 x TPR / 256 -> 2 x TPR / 512 (-> 1 x TPR /
+    // 512, two per compute unit): float32 RMSNorm N = 72: 62.4 -> 75.7; 96: 78.2 -> 79.6; 136: 68.8 -> 75.6; 200:
+    // 77.3 -> 79.9; 256: 82.0 -> 81.9; 384: 79.0 -> 80.0; 512: 81.9 -> 81.9; bfloat16 RMSNorm N = 200: 65.3 -> 73.4;
+    // 256: 74.8 -> 77.3; 640: 65.5 -> 74.4; 1000: 75.1 -> 76.4; bfloat16 LayerNorm N = 160: 59.6 -> 69.2 -> 71.3; 200:
+    // 65.0 -> 70.9 -> 72.6; 256: 70.6 -> 74.3 -> 77.0; 384: 66.6 -> 71.4 -> 73.3; 640: 60.4 -> 67.4 -> 70.7 (1 vector per
+    // thread and ONE workgroup per compute unit keeps too little under way: 136 columns 52.9, 200 columns 68.0).
+    bool narrow_backward_pair = false;
+    // (float32 / float64 rows that fill a 4-vector shape exactly stay there: N = 256 on 2^20 rows 75.6 against 74.5)
+    const bool fills_four = bytes >= 4 && n_vecs <= 128 && (n_vecs & (n_vecs - 1)) == 0;
+    if (which == kNormBwd && N >= vec_elems && n_vecs > 16 && n_vecs <= 192 && !fills_four) {
+        const bool one_each = ln16 && n_vecs <= 96;
+        const int k = one_each ? 1 : 2;
         int tpr = 16;
-        while (2 * tpr < n_vecs) tpr *= 2;
-        const Shape narrow{2, tpr, 512};
-        if (shape_compiled(which, aligned, ln16, narrow)) s = narrow;
-    }
-    // Narrow rows (17 to 64 vectors) whose pitch is not a multiple of 128 bytes: with 8 or 16 threads per row a
-    // wave's request is eight or four separate 128- or 256-byte pieces, each across two or three lines; with 16 to 32
-    // threads per row and one or two vectors each the pieces are longer and a wave touches about a third fewer lines.
-    // Forward: 2 vectors per thread in 256-thread workgroups, two per compute unit; backward: 1 vector per thread up
-    // to 32 vectors, 2 beyond, in 512-thread workgroups.  Kernels alone at 2^25 elements, before -> after: float32
-    // N = 72 forward 53.7 -> 49.1 us, backward 96.7 -> 71 us; N = 120 47.4 -> 45.5, 81.3 -> 69.7; N = 200 45.9 -> 45.5,
-    // 74.1 -> 70.3; bfloat16 N = 200 forward 24.0 -> 22.2, backward 41.1 -> 39.7; N = 248 23.6 -> 22.1, 40.5 -> 39.0.
-    // 16-bit rows of 17 to 32 vectors gain the same way at every pitch (N = 256: forward 22.3 -> 21.7, LayerNorm
-    // 23.6 -> 22.6); float32 rows on 128-byte lines do not (N = 128 forward 44.2 -> 44.8) and keep their shapes.
-    bool narrow_forward_pair = false;
-    if ((which == kNormFwd || which == kNormBwd) && aligned && n_vecs > 16 && n_vecs <= 64 &&
-        (pitch_bytes % 128 != 0 || (bytes == 2 && n_vecs <= 32))) {
-        const int k = (which == kNormFwd || n_vecs > 32) ? 2 : 1;
-        int tpr = 8;
         while (k * tpr < n_vecs) tpr *= 2;
-        const Shape narrow{k, tpr, which == kNormFwd ? 256 : 512};
+        const Shape narrow{k, tpr, 512};
         if (shape_compiled(which, aligned, ln16, narrow)) {
             s = narrow;
-            narrow_forward_pair = which == kNormFwd;
+            narrow_backward_pair = one_each;
+        }
+    }
+    // The norm forward over narrow rows (17 to 128 vectors) whose pitch is not a multiple of 128 bytes: 2 vectors per
+    // thread in 256-thread workgroups, two per compute unit, for the same reason (pieces of a wave's request that
+    // start and end inside a line).  Forward + backward of 2^26 elements with only the forward's shape changed,
+    // 4 x TPR / 256, one per compute unit -> 2 x TPR / 256, two: bfloat16 RMSNorm N = 200: 66.0 -> 68.0; 248:
+    // 70.0 -> 73.3; 456: 71.0 -> 72.1; float32 N = 72: 61.7 -> 63.3; 120: 77.7 -> 79.1; 136: 59.8 -> 61.3; rows on
+    // 128-byte lines that fill a 4-vector shape lose that way (float32 N = 256: 82.0 -> 80.4; bfloat16 N = 512:
+    // 79.1 -> 77.6) and keep theirs.
+    bool narrow_forward_pair = false;
+    if (which == kNormFwd && N >= vec_elems && n_vecs > 16 && n_vecs <= 128 && pitch_bytes % 128 != 0) {
+        int tpr = 8;
+        while (2 * tpr < n_vecs) tpr *= 2;
+        const Shape narrow{2, tpr, 256};
+        if (shape_compiled(which, aligned, ln16, narrow)) {
+            s = narrow;
+            narrow_forward_pair = true;
         }
     }
     // Rows that start off 128-byte lines: two-row workgroups of 256-thread rows cannot put their requests on line
@@ -578,7 +584,7 @@ int plan_launch(int which, int flavour, bool aligned, int64_t M, int64_t N, int 
             M <= 24 * static_cast<int64_t>(cus)) {
             cap = 2;
         }
-        if (narrow_forward_pair && cap < 2) cap = 2;
+        if ((narrow_forward_pair || narrow_backward_pair) && cap < 2) cap = 2;
     }
     if (cap < bpc) bpc = cap;
     const int rows_per_block = s.block / s.tpr;
@@ -712,9 +718,10 @@ int64_t bwd_workspace_bytes(int which, int flavour, int64_t M, int64_t N, int wa
     if (cus <= 0) return THN_E_DEVICE;
     int bpc = default_blocks_per_cu(which, flavour, 512);
     const int vec_elems = 16 / bytes;
-    const int narrow = narrow_row_blocks_per_cu(which, static_cast<int>((N + vec_elems - 1) / vec_elems),
-                                                bytes == 2 && N % vec_elems != 0);
+    const int n_vecs = static_cast<int>((N + vec_elems - 1) / vec_elems);
+    const int narrow = narrow_row_blocks_per_cu(which, n_vecs, bytes == 2 && N % vec_elems != 0);
     if (narrow > bpc) bpc = narrow;
+    if (bytes == 2 && n_vecs <= 96 && bpc < 2) bpc = 2;      // the LayerNorm backward over narrow 16-bit rows (plan_launch)
     const int forced = g_override[which].bpc.load();
     if (forced > bpc) bpc = forced;
     if (bpc > kMaxBlocksPerCu) bpc = kMaxBlocksPerCu;
