@@ -785,7 +785,7 @@ def ceiling_main(args, lib, dev):
 
     def norm_fwd(b_, m_, ln):
         rc = lib.thn_norm_fwd(p(b_["x"]), n, p(b_["y"]), n, p(w), p(b) if ln else 0, p(b_["mean"]) if ln else 0,
-                              p(b_["rstd"]), m_, n, 1e-6, code, code, stream)
+                              p(b_["rstd"]), m_, n, 1e-6, code | _native.X_STREAM, code, stream)     # a forward on its own: x streams
         assert rc == 0, rc
 
     def norm_bwd1(b_, m_, ln):
