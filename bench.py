@@ -428,6 +428,8 @@ def main():
                     help="instead of a workload: forward + backward of RMSNorm and LayerNorm over a grid of row widths "
                          "and row counts per storage type, % of HBM peak per cell (the table the launch heuristic is "
                          "fitted against)")
+    ap.add_argument("--scan-log2-elements", type=int, default=26,
+                    help="--scan: elements per tensor in the long class, as a power of two (26: 2^26)")
     ap.add_argument("--host", action="store_true",
                     help="instead of a workload: the host cost of the module path (per-call microseconds of the Python "
                          "layer) and where forward + backward through the modules turns host-bound")
@@ -584,13 +586,13 @@ def scan_main(args, lib, dev):
     from TritonHub.Normalization import _launch
     p = _native.ptr
     stream = torch.cuda.current_stream(dev).cuda_stream
-    total = 1 << 26                                       # elements per tensor in the long class
+    total = 1 << args.scan_log2_elements                   # elements per tensor in the long class
     steps = min(args.steps, 30)
     gen = torch.Generator(device=dev).manual_seed(0)
     props = torch.cuda.get_device_properties(dev)
     print(f"# bench.py --scan: forward + backward of one batch, % of {HBM_PEAK_GBPS:.0f} GB/s on the algorithmic bytes; "
           f"{props.name}, {props.multi_processor_count} compute units; {steps} timed steps per cell, four buffer sets")
-    print("# classes: long = 2^26 elements per tensor; short = 16 rows per compute unit (omitted where that is the long class "
+    print(f"# classes: long = 2^{args.scan_log2_elements} elements per tensor; short = 16 rows per compute unit (omitted where that is the long class "
           "or more)")
     print("# launch = forward KxTPR/BLOCK@grid | backward KxTPR/BLOCK@grid of the long class (LayerNorm)")
     print(f"{'dtype':5} {'N':>6} {'rows':>8} | {'RMS long':>8} {'LN long':>8} | {'rows':>6} {'RMS short':>9} {'LN short':>9} | launch")

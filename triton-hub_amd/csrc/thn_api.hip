@@ -8,6 +8,7 @@
 #include <unordered_map>
 
 #include "thn_dispatch.h"
+#include "thn_flat.h"
 #include "thn_fused_dispatch.h"
 #include "thn_reduce.h"
 #include "thn_act_dispatch.h"
@@ -648,6 +649,102 @@ int plan_launch(int which, int flavour, bool aligned, int64_t M, int64_t N, int 
     return THN_OK;
 }
 
+// ---- the flat mapping for narrow rows (thn_flat.h) ------------------------------------------------------------
+struct FlatPlan {
+    int rows_each;      // J: independent rows per lane and step
+    int log_steps;      // tree steps of the segmented row sums: ceil(log2(vectors per row)), at least 4
+    int grid;
+    int n_vecs;
+};
+
+int launch_flat_fwd(int dtype, bool ln, const FlatPlan& p, const FwdArgs& a, hipStream_t st, int* occ) {
+    switch (dtype) {
+        case THN_F32: return thn::launch_flat_fwd_f32(ln, p.rows_each, p.log_steps, a, p.grid, st, occ);
+        case THN_F16: return thn::launch_flat_fwd_f16(ln, p.rows_each, p.log_steps, a, p.grid, st, occ);
+        case THN_BF16: return thn::launch_flat_fwd_bf16(ln, p.rows_each, p.log_steps, a, p.grid, st, occ);
+        default: return 1;
+    }
+}
+
+int launch_flat_bwd(int dtype, bool ln, const FlatPlan& p, const BwdArgs& a, hipStream_t st, int* occ) {
+    switch (dtype) {
+        case THN_F32: return thn::launch_flat_bwd_f32(ln, p.rows_each, p.log_steps, a, p.grid, st, occ);
+        case THN_F16: return thn::launch_flat_bwd_f16(ln, p.rows_each, p.log_steps, a, p.grid, st, occ);
+        case THN_BF16: return thn::launch_flat_bwd_bf16(ln, p.rows_each, p.log_steps, a, p.grid, st, occ);
+        default: return 1;
+    }
+}
+
+// Upper limit of workgroups per compute unit of the flat kernels (the workspace bound of the backward counts on it).
+constexpr int kFlatBlocksPerCu = 4;
+
+// Whether a plain norm launch takes the flat mapping by itself.  Rows on the 128-bit path of 2 to 32 vectors in
+// float32 / float16 / bfloat16 storage whose vector count is not a power of two, where the segmented row sums (5 to 6
+// lane exchanges per value, against 3 to 5 DPP steps of the row kernels) cost less than the idle lanes and scattered
+// pieces of the row kernels do.  Forward + backward of 2^26 elements, % of 8 TB/s, row kernels -> flat (same box):
+//   RMSNorm (one value per row sum), forward and backward, up to 21 vectors: bfloat16 N = 24: 53.0 -> 73.3; 40: 67.9 ->
+//     74.7; 72: 69.7 -> 75.2; 88: 72.1 -> 74.3; 120: 73.8 -> 75.7; 136: 69.3 -> 72.3; 168: 71.5 -> 75.4; float32 N = 12:
+//     59.0 -> 75.0; 28: 73.2 -> 77.0; 36: 73.9 -> 76.4; 68: 73.2 -> 75.5; 84: 74.8 -> 77.6; from 22 vectors on the row
+//     kernels are as fast or faster (bfloat16 N = 200: 73.7 against 73.0);
+//   LayerNorm (three values per row in the forward and in the backward): the forward up to 7 vectors of 16-bit and 15
+//     of 32-bit storage (forward alone flat, bfloat16 N = 40: 64.9 -> 71.1; 56: 68.9 -> 71.8; float32 N = 20: 70.3 ->
+//     75.3; 28: 70.8 -> 76.3; 60: 73.5 -> 76.3; 16-bit rows of 9 and 10 vectors gain a point in one run and lose one
+//     in the next, wider ones lose 1-3), the backward only for rows of 3 vectors (bfloat16 N = 24: 48.7 -> 66.1; from
+//     5 vectors on it is 0-6 points slower than the row kernels' backward: three segmented sums per row).
+// The launch override selects the flat kernels explicitly with threads_per_row = the row's vector count (not a power
+// of two) and vecs_per_thread = rows per lane and step (1, 2 or 4), and keeps them off with any other threads_per_row.
+bool flat_by_default(int which, bool ln, int bytes, int n_vecs) {
+    if ((n_vecs & (n_vecs - 1)) == 0) return false;
+    if (which == kNormFwd) return ln ? n_vecs <= (bytes == 2 ? 7 : 15) : n_vecs <= 21;
+    return ln ? n_vecs == 3 : n_vecs <= 21;
+}
+
+bool plan_flat(int which, bool ln, bool aligned, int64_t M, int64_t N, int dtype, FlatPlan* out) {
+    const int bytes = elem_bytes(dtype);
+    if (!aligned || bytes == 0 || bytes == 8 || M <= 0) return false;
+    const int vec_elems = 16 / bytes;
+    if (N % vec_elems != 0) return false;
+    const int n_vecs = static_cast<int>(N / vec_elems);
+    if (n_vecs < 2 || n_vecs > thn::kFlatMaxVecs) return false;
+    const Override& ov = g_override[which];
+    // rows per lane and step, workgroups per compute unit: two and two measured best or within a point of it at every
+    // width (1, 2, 4 x 2, 4, 8); the 16-bit LayerNorm forward (the most registers per row) takes one and four
+    int rows_each = 2, bpc = 2;
+    if (which == kNormFwd && ln && bytes == 2) {
+        rows_each = 1;
+        bpc = 4;
+    }
+    if (ov.tpr.load() > 0 || ov.block.load() > 0 || ov.k.load() > 0) {
+        if (ov.tpr.load() != n_vecs || (n_vecs & (n_vecs - 1)) == 0) return false;     // a row-kernel shape is forced
+        if (ov.block.load() > 0 && ov.block.load() != thn::kFlatBlock) return false;
+        if (ov.k.load() > 0) rows_each = ov.k.load();
+        if (rows_each != 1 && rows_each != 2 && rows_each != 4) return false;
+    } else if (!flat_by_default(which, ln, bytes, n_vecs)) {
+        return false;
+    }
+    const int cus = current_cu_count();
+    if (cus <= 0) return false;
+    if (ov.bpc.load() > 0) bpc = ov.bpc.load();
+    if (bpc > kMaxBlocksPerCu) bpc = kMaxBlocksPerCu;
+    const int64_t rows_per_block = static_cast<int64_t>(thn::kFlatBlock / 64) * (64 / n_vecs) * rows_each;
+    const int64_t row_blocks = (M + rows_per_block - 1) / rows_per_block;
+    const int64_t grid_max = static_cast<int64_t>(cus) * bpc;
+    int64_t grid = row_blocks;
+    if (grid > grid_max) {
+        const int64_t iters = (row_blocks + grid_max - 1) / grid_max;
+        grid = (row_blocks + iters - 1) / iters;
+        if (grid > cus && grid % cus != 0) {
+            const int64_t up = (grid + cus - 1) / cus * cus;
+            if (up <= grid_max && up <= row_blocks) grid = up;
+        }
+    }
+    out->rows_each = rows_each;
+    out->log_steps = n_vecs <= 16 ? 4 : 5;
+    out->grid = static_cast<int>(grid);
+    out->n_vecs = n_vecs;
+    return true;
+}
+
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 // The bytes a (rows, row_bytes) operand with the given row pitch spans, as a half-open address range, with the
@@ -722,6 +819,7 @@ int64_t bwd_workspace_bytes(int which, int flavour, int64_t M, int64_t N, int wa
     const int narrow = narrow_row_blocks_per_cu(which, n_vecs, bytes == 2 && N % vec_elems != 0);
     if (narrow > bpc) bpc = narrow;
     if (bytes == 2 && n_vecs <= 96 && bpc < 2) bpc = 2;      // the LayerNorm backward over narrow 16-bit rows (plan_launch)
+    if (which == kNormBwd && n_vecs <= thn::kFlatMaxVecs && bpc < kFlatBlocksPerCu) bpc = kFlatBlocksPerCu;   // the flat mapping
     const int forced = g_override[which].bpc.load();
     if (forced > bpc) bpc = forced;
     if (bpc > kMaxBlocksPerCu) bpc = kMaxBlocksPerCu;
@@ -758,10 +856,18 @@ int norm_forward(const void* x, int64_t x_row_stride, void* y, int64_t y_row_str
     const bool aligned = (N % vec_elems) == 0 && aligned16(x) && aligned16(y) && aligned16(w) && aligned16(b) &&
                          (x_row_stride * bytes) % 16 == 0 && (y_row_stride * bytes) % 16 == 0;
     Plan p;
+    FlatPlan fp;
     const bool fused = act != thn::kNoAct;
-    const int rc = plan_launch(fused ? kFusedFwd : kNormFwd, fused ? ((ln ? 1 : 0) | (act << 1)) : (ln ? 1 : 0), aligned, M, N,
-                               x_dtype, &p, x_row_stride * bytes);
-    if (rc != THN_OK) return rc;
+    const bool flat = !fused && plan_flat(kNormFwd, ln, aligned, M, N, x_dtype, &fp);
+    if (flat) {
+        p.n_vecs = fp.n_vecs;
+        p.grid = fp.grid;
+        p.s = Shape{fp.rows_each, fp.n_vecs, thn::kFlatBlock};
+    } else {
+        const int rc = plan_launch(fused ? kFusedFwd : kNormFwd, fused ? ((ln ? 1 : 0) | (act << 1)) : (ln ? 1 : 0), aligned, M,
+                                   N, x_dtype, &p, x_row_stride * bytes);
+        if (rc != THN_OK) return rc;
+    }
 
     FwdArgs a{};
     a.x = static_cast<const char*>(x);
@@ -782,7 +888,9 @@ int norm_forward(const void* x, int64_t x_row_stride, void* y, int64_t y_row_str
     a.line_shift = line_shift_ok(aligned, p.s, p.grid, p.n_vecs, streams, 2) ? 1 : 0;
     a.keep_x = keep_x ? 1 : 0;
     hipStream_t st = static_cast<hipStream_t>(stream);
-    const int lrc = fused ? launch_fused_fwd(x_dtype, (ln ? 1 : 0) | (act << 1), aligned, p.s, a, p.grid, st, nullptr)
+    if (flat) a.line_shift = 0;
+    const int lrc = flat ? launch_flat_fwd(x_dtype, ln, fp, a, st, nullptr)
+                  : fused ? launch_fused_fwd(x_dtype, (ln ? 1 : 0) | (act << 1), aligned, p.s, a, p.grid, st, nullptr)
                           : launch_fwd(x_dtype, ln, aligned, p.s, a, p.grid, st, nullptr);
     if (lrc > 0) return THN_E_SHAPE;
     return lrc == 0 ? THN_OK : THN_E_LAUNCH;
@@ -818,9 +926,17 @@ int norm_backward_stage1(const void* x, int64_t x_row_stride, const void* dy, in
                          (x_row_stride * bytes) % 16 == 0 && (dy_row_stride * bytes) % 16 == 0 &&
                          (dx_row_stride * bytes) % 16 == 0;
     Plan p;
+    FlatPlan fp;
     const int variant = fused ? ((ln ? 1 : 0) | (act << 1)) : (ln ? 1 : 0);
-    const int rc = plan_launch(fused ? kFusedBwd : kNormBwd, variant, aligned, M, N, x_dtype, &p, x_row_stride * bytes);
-    if (rc != THN_OK) return rc;
+    const bool flat = !fused && plan_flat(kNormBwd, ln, aligned, M, N, x_dtype, &fp);
+    if (flat) {
+        p.n_vecs = fp.n_vecs;
+        p.grid = fp.grid;
+        p.s = Shape{fp.rows_each, fp.n_vecs, thn::kFlatBlock};
+    } else {
+        const int rc = plan_launch(fused ? kFusedBwd : kNormBwd, variant, aligned, M, N, x_dtype, &p, x_row_stride * bytes);
+        if (rc != THN_OK) return rc;
+    }
     const int64_t pitch = partial_pitch(N);
     const int64_t need = n_grads * static_cast<int64_t>(p.grid) * pitch * static_cast<int64_t>(sizeof(float));
     if (workspace_bytes < need) return THN_E_WORKSPACE;
@@ -848,7 +964,9 @@ int norm_backward_stage1(const void* x, int64_t x_row_stride, const void* dy, in
     const RowStream streams[3] = {{x, a.x_stride_bytes}, {dy, a.dy_stride_bytes}, {dx, a.dx_stride_bytes}};
     a.line_shift = line_shift_ok(aligned, p.s, p.grid, p.n_vecs, streams, 3) ? 1 : 0;
     hipStream_t st = static_cast<hipStream_t>(stream);
-    const int lrc = fused ? launch_fused_bwd(x_dtype, variant, aligned, p.s, a, p.grid, st, nullptr)
+    if (flat) a.line_shift = 0;
+    const int lrc = flat ? launch_flat_bwd(x_dtype, ln, fp, a, st, nullptr)
+                  : fused ? launch_fused_bwd(x_dtype, variant, aligned, p.s, a, p.grid, st, nullptr)
                           : launch_bwd(x_dtype, ln, aligned, p.s, a, p.grid, st, nullptr);
     if (lrc > 0) return THN_E_SHAPE;
     if (lrc < 0) return THN_E_LAUNCH;
@@ -1137,6 +1255,15 @@ int thn_norm_query_launch(int which, int is_layernorm, int64_t M, int64_t N, int
         shape[2] = block;
         shape[3] = grid;
         shape[4] = 0;
+        return THN_OK;
+    }
+    FlatPlan fp;
+    if ((which == kNormFwd || which == kNormBwd) && plan_flat(which, is_layernorm != 0, aligned, M, N, x_dtype, &fp)) {
+        shape[0] = fp.rows_each;       // the flat mapping: rows per lane and step, lanes per row = vectors per row
+        shape[1] = fp.n_vecs;
+        shape[2] = thn::kFlatBlock;
+        shape[3] = fp.grid;
+        shape[4] = 1;
         return THN_OK;
     }
     const int rc = plan_launch(which, flavour, aligned, M, N, x_dtype, &p, N * elem_bytes(x_dtype));   // contiguous rows
