@@ -49,6 +49,10 @@ WORKLOADS = {
     "layernorm_f32_4096x16384_wide": ("ln", 4096, 16384, "f32"),
     "layernorm_f32_12279x4099_ragged": ("ln", 12279, 4099, "f32"),
     "rmsnorm_bf16_24564x4098_ragged": ("rms", 24564, 4098, "bf16"),
+    # narrow rows, 2^26 elements: 9 vectors per row (the flat lane-to-vector mapping for RMSNorm) and 7 (for both)
+    "rmsnorm_bf16_932067x72_narrow": ("rms", 932067, 72, "bf16"),
+    "layernorm_bf16_932067x72_narrow": ("ln", 932067, 72, "bf16"),
+    "layernorm_f32_2396745x28_narrow": ("ln", 2396745, 28, "f32"),
     # norm with an activation epilogue (thn_norm_act_fwd + thn_norm_act_bwd): same bytes as the plain norm step
     "layernorm_gelu_bf16_16384x4096": ("ln+gelu", 16384, 4096, "bf16"),
     "layernorm_gelu_tanh_bf16_16384x4096": ("ln+gelu_tanh", 16384, 4096, "bf16"),
@@ -576,20 +580,91 @@ SCAN_WIDTHS = [64, 72, 96, 120, 128, 192, 200, 248, 256, 320, 384, 512, 640, 768
                9216, 10240, 12288, 14336, 16384, 20480, 24576, 28672, 32768]
 
 
+SCAN_TABLE = "norm_step_width_scan_bf16_f16_f32.txt"
+
+
+def scan_reference():
+    """{(storage type name, N): (RMSNorm %, LayerNorm %)} of the long class of the committed width scan (the first table
+    of profiles/norm_step_width_scan_bf16_f16_f32.txt, 2^26 elements per tensor): what `--scan` printed on the GPU and
+    the build the launch heuristic was last fitted on."""
+    table = {}
+    path = os.path.join(ROOT, "profiles", SCAN_TABLE)
+    if not os.path.exists(path):
+        return table
+    with open(path) as fh:
+        for line in fh:
+            if line.startswith("----"):
+                break                                       # the tables of other sizes follow
+            parts = line.split()
+            if len(parts) > 6 and parts[0] in ("bf16", "f16", "f32") and parts[3] == "|":
+                try:
+                    table[(parts[0], int(parts[1]))] = (float(parts[4]), float(parts[5]))
+                except ValueError:
+                    pass
+    return table
+
+
+def scan_pool(dev, dtype, total, gen):
+    import torch
+    return [{k: (torch.randn(total, device=dev, generator=gen).to(dtype) if k in ("x", "dy")
+                 else torch.empty(total, device=dev, dtype=dtype)) for k in ("x", "dy", "y", "dx")}
+            for _ in range(N_BUFFER_SETS)]
+
+
+def scan_cell(lib, dev, pool, m, n, dtype, ln, steps, gen):
+    """Forward + backward of one batch of m rows of n columns through the C ABI (same batch, 'keep' policy), the
+    buffers taken from `pool` in rotation: % of the HBM peak on the algorithmic bytes, best of two runs of `steps`."""
+    import torch
+    from TritonHub import _native
+    p = _native.ptr
+    stream = torch.cuda.current_stream(dev).cuda_stream
+    code = _native.dtype_code(dtype)
+    s = torch.empty(0, dtype=dtype).element_size()
+    w = (1.0 + 0.1 * torch.randn(n, device=dev, generator=gen)).to(dtype)
+    b = (0.1 * torch.randn(n, device=dev, generator=gen)).to(dtype)
+    dw, db = torch.empty_like(w), torch.empty_like(w)
+    mean = torch.empty(m, device=dev)
+    rstd = torch.empty(m, device=dev)
+    ws_bytes = lib.thn_norm_bwd_workspace_bytes(m, n, 1, 1, code)
+    ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=dev)
+
+    def step(i):
+        b_ = pool[i % N_BUFFER_SETS]
+        rc = lib.thn_norm_fwd(p(b_["x"]), n, p(b_["y"]), n, p(w), p(b) if ln else 0, p(mean) if ln else 0,
+                              p(rstd), m, n, 1e-6, code | _native.X_KEEP, code, stream)
+        assert rc == 0, _native.strerror(rc)
+        rc = lib.thn_norm_bwd(p(b_["x"]), n, p(b_["dy"]), n, p(b_["dx"]), n, p(w), p(mean) if ln else 0,
+                              p(rstd), p(dw), p(db) if ln else 0, p(ws), ws_bytes, m, n, code, code, stream)
+        assert rc == 0, _native.strerror(rc)
+    for i in range(8):
+        step(i)
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    best = float("inf")
+    for _ in range(2):
+        start.record()
+        for i in range(steps):
+            step(i)
+        stop.record()
+        torch.cuda.synchronize()
+        best = min(best, start.elapsed_time(stop) / steps)
+    f_, b__ = algorithmic_bytes("ln" if ln else "rms", m, n, s, s)
+    return 100.0 * (f_ + b__) / (best * 1e-3) / 1e9 / HBM_PEAK_GBPS
+
+
 def scan_main(args, lib, dev):
     """Forward + backward of one batch (same batch, 'keep' policy) for RMSNorm and LayerNorm over a grid of row widths
     and two row-count classes per storage type, in % of the HBM peak on the algorithmic bytes: the table the launch
     heuristic (plan_launch in thn_api.hip) was fitted against, regenerated for the build and the GPU at hand.
-    Prints a text table, one line per (storage type, width)."""
+    Prints a text table, one line per (storage type, width); at the size of the committed table (2^26 elements) a last
+    column gives the ratio to that table's figures, and the run ends with the cells that fell below 0.9 of them."""
     import torch
-    from TritonHub import _native
     from TritonHub.Normalization import _launch
-    p = _native.ptr
-    stream = torch.cuda.current_stream(dev).cuda_stream
     total = 1 << args.scan_log2_elements                   # elements per tensor in the long class
     steps = min(args.steps, 30)
     gen = torch.Generator(device=dev).manual_seed(0)
     props = torch.cuda.get_device_properties(dev)
+    reference = scan_reference() if args.scan_log2_elements == 26 else {}
+    behind = []
     print(f"# bench.py --scan: forward + backward of one batch, % of {HBM_PEAK_GBPS:.0f} GB/s on the algorithmic bytes; "
           f"{props.name}, {props.multi_processor_count} compute units; {steps} timed steps per cell, four buffer sets")
     print(f"# classes: long = 2^{args.scan_log2_elements} elements per tensor; short = 16 rows per compute unit (omitted where that is the long class "
@@ -599,57 +674,39 @@ def scan_main(args, lib, dev):
     for dname in ("bf16", "f32", "f16"):
         dtype = {"bf16": torch.bfloat16, "f16": torch.float16, "f32": torch.float32}[dname]
         s = torch.empty(0, dtype=dtype).element_size()
-        code = _native.dtype_code(dtype)
-        pool = [{k: (torch.randn(total, device=dev, generator=gen).to(dtype) if k in ("x", "dy")
-                     else torch.empty(total, device=dev, dtype=dtype)) for k in ("x", "dy", "y", "dx")}
-                for _ in range(N_BUFFER_SETS)]
+        pool = scan_pool(dev, dtype, total, gen)
         for n in SCAN_WIDTHS:
             if n * s > 65536:
                 continue
-            w = (1.0 + 0.1 * torch.randn(n, device=dev, generator=gen)).to(dtype)
-            b = (0.1 * torch.randn(n, device=dev, generator=gen)).to(dtype)
-            dw, db = torch.empty_like(w), torch.empty_like(w)
             cells = {}
             m_long = total // n
             m_short = 16 * props.multi_processor_count
             for cls, m in (("long", m_long), ("short", m_short)):
                 if cls == "short" and m_short >= m_long:
                     continue
-                mean = torch.empty(m, device=dev)
-                rstd = torch.empty(m, device=dev)
-                ws_bytes = lib.thn_norm_bwd_workspace_bytes(m, n, 1, 1, code)
-                ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=dev)
                 for ln in (False, True):
-                    def step(i):
-                        b_ = pool[i % N_BUFFER_SETS]
-                        rc = lib.thn_norm_fwd(p(b_["x"]), n, p(b_["y"]), n, p(w), p(b) if ln else 0, p(mean) if ln else 0,
-                                              p(rstd), m, n, 1e-6, code | _native.X_KEEP, code, stream)
-                        assert rc == 0, _native.strerror(rc)
-                        rc = lib.thn_norm_bwd(p(b_["x"]), n, p(b_["dy"]), n, p(b_["dx"]), n, p(w), p(mean) if ln else 0,
-                                              p(rstd), p(dw), p(db) if ln else 0, p(ws), ws_bytes, m, n, code, code, stream)
-                        assert rc == 0, _native.strerror(rc)
-                    for i in range(8):
-                        step(i)
-                    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-                    best = float("inf")
-                    for _ in range(2):
-                        start.record()
-                        for i in range(steps):
-                            step(i)
-                        stop.record()
-                        torch.cuda.synchronize()
-                        best = min(best, start.elapsed_time(stop) / steps)
-                    f_, b__ = algorithmic_bytes("ln" if ln else "rms", m, n, s, s)
-                    cells[(cls, ln)] = 100.0 * (f_ + b__) / (best * 1e-3) / 1e9 / HBM_PEAK_GBPS
+                    cells[(cls, ln)] = scan_cell(lib, dev, pool, m, n, dtype, ln, steps, gen)
             f = _launch.query_launch(0, True, m_long, n, dtype)
             g = _launch.query_launch(1, True, m_long, n, dtype)
             launch = f"{f[0]}x{f[1]}/{f[2]}@{f[3]} | {g[0]}x{g[1]}/{g[2]}@{g[3]}" + ("" if f[4] else "  (off the 128-bit path)")
             short = (f"{m_short:6d} {cells[('short', False)]:9.1f} {cells[('short', True)]:9.1f}" if ("short", False) in cells
                      else f"{'':6} {'':9} {'':9}")
-            print(f"{dname:5} {n:6d} {m_long:8d} | {cells[('long', False)]:8.1f} {cells[('long', True)]:8.1f} | {short} | {launch}",
+            against = ""
+            if (dname, n) in reference:
+                ratios = [cells[("long", ln)] / max(reference[(dname, n)][int(ln)], 1e-9) for ln in (False, True)]
+                against = f" | x{ratios[0]:.2f} x{ratios[1]:.2f} of the committed table"
+                for ln, r in zip((False, True), ratios):
+                    if r < 0.9:
+                        behind.append(f"{dname} N={n} {'LayerNorm' if ln else 'RMSNorm'}: {cells[('long', ln)]:.1f} % against "
+                                      f"{reference[(dname, n)][int(ln)]:.1f} %")
+            print(f"{dname:5} {n:6d} {m_long:8d} | {cells[('long', False)]:8.1f} {cells[('long', True)]:8.1f} | {short} | {launch}{against}",
                   flush=True)
         del pool
         torch.cuda.empty_cache()
+    if reference:
+        print(f"# cells below 0.9 of profiles/{SCAN_TABLE}: {len(behind)}")
+        for line in behind:
+            print("#   " + line)
 
 
 def host_main(args, lib, dev):

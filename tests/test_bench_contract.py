@@ -53,3 +53,13 @@ def test_traffic_comes_from_the_profile_summaries():
     assert t is not None and t["source"].startswith("profiles/") and b <= t["bytes"] < 1.1 * b
     assert bench.traffic_from_profiles("layernorm_f32_200x128_quickstart") is None
     assert bench.traffic_fields("no_such_workload") == {"traffic": None}
+
+
+def test_committed_width_scan_is_readable():
+    """`bench.py --scan` compares itself with the committed table, and the GPU throughput guard reads it: every storage
+    type and the guarded widths must parse."""
+    import bench
+    table = bench.scan_reference()
+    assert len(table) >= 140
+    for key in (("bf16", 72), ("bf16", 4096), ("bf16", 4098), ("f32", 256), ("f16", 6000)):
+        assert key in table and all(20.0 < v < 100.0 for v in table[key]), key
