@@ -49,7 +49,7 @@ WORKLOADS = {
     "layernorm_f32_4096x16384_wide": ("ln", 4096, 16384, "f32"),
     "layernorm_f32_12279x4099_ragged": ("ln", 12279, 4099, "f32"),
     "rmsnorm_bf16_24564x4098_ragged": ("rms", 24564, 4098, "bf16"),
-    # narrow rows, 2^26 elements: 9 vectors per row (the flat lane-to-vector mapping for RMSNorm) and 7 (for both)
+    # narrow rows, 2^26 elements: 9 vectors per 16-bit row (RMSNorm: the flat kernels) and 7 per float32 row (the staged kernels)
     "rmsnorm_bf16_932067x72_narrow": ("rms", 932067, 72, "bf16"),
     "layernorm_bf16_932067x72_narrow": ("ln", 932067, 72, "bf16"),
     "layernorm_f32_2396745x28_narrow": ("ln", 2396745, 28, "f32"),

@@ -358,11 +358,14 @@ int thn_dropout(const void* x, void* out, int64_t n, int64_t first_offset, float
  * activation epilogue forward / backward.
  * vecs_per_thread / threads_per_row / block_threads select a compiled kernel shape, blocks_per_cu caps the
  * persistent grid; 0 for any field keeps the heuristic's choice.
- * For the norm forward / backward (0, 1) a threads_per_row that is not a power of two selects the flat kernels for
- * rows of exactly that many 16-byte vectors (2 to 32, float32 / float16 / bfloat16 rows on the 128-bit path: lanes are
- * dealt to vectors without gaps, a wave holds 64 / threads_per_row whole rows); vecs_per_thread is then the number of
- * rows a lane carries per step (1, 2 or 4) and block_threads 0 or 256.  Problems of another width, and any other
- * override, run the row kernels.
+ * For the norm forward / backward (0, 1) two more kernel families for rows of at most 32 16-byte vectors (float32 /
+ * float16 / bfloat16 rows on the 128-bit path) are selected here as well: a threads_per_row that is not a power of two,
+ * with block_threads 0 or 256, selects the flat kernels for rows of exactly that many vectors (lanes are dealt to
+ * vectors without gaps, a wave holds 64 / threads_per_row whole rows; vecs_per_thread = rows a lane carries per step:
+ * 1, 2 or 4); block_threads = 64 selects the staged kernels (a wave copies a batch of rows into LDS and one lane sums a
+ * row; threads_per_row = the row's vector count or 0, vecs_per_thread = the batch in passes of the wave over its rows:
+ * 1 to 4, or 0 for the default).  Problems such an override does not fit are refused (THN_E_SHAPE); any other
+ * override runs the row kernels.
  * Process-wide; meant for benchmarks, not for concurrent production use.  Returns THN_E_SHAPE when no
  * compiled kernel has that shape.
  */
@@ -375,8 +378,9 @@ int thn_norm_set_launch_override(int which, int vecs_per_thread, int threads_per
  * For the epilogue families (9, 10) `is_layernorm` carries the activation too: bit 0 = LayerNorm, bits 1.. = the
  * thn_act code.  Rows wider than 64 KiB of the softmax and p-norm families report their looping kernels:
  * {vectors per thread and step, block_threads, block_threads, grid_blocks, 0}.  Norm problems that take the flat
- * kernels (narrow rows whose vector count is not a power of two) report {rows per lane and step, vectors per row, 256,
- * grid_blocks, 1}: a threads_per_row that is not a power of two identifies them.
+ * kernels (narrow 16-bit rows whose vector count is not a power of two) report {rows per lane and step, vectors per
+ * row, 256, grid_blocks, 1}: a threads_per_row that is not a power of two identifies them; those that take the staged
+ * kernels (rows of 1 to 8 vectors, narrow float32 rows) report {passes per batch, vectors per row, 64, grid_blocks, 1}.
  */
 int thn_norm_query_launch(int which, int is_layernorm, int64_t M, int64_t N, int x_dtype, int32_t shape[5]);
 

@@ -9,6 +9,7 @@
 
 #include "thn_dispatch.h"
 #include "thn_flat.h"
+#include "thn_staged.h"
 #include "thn_fused_dispatch.h"
 #include "thn_reduce.h"
 #include "thn_act_dispatch.h"
@@ -678,24 +679,24 @@ int launch_flat_bwd(int dtype, bool ln, const FlatPlan& p, const BwdArgs& a, hip
 // Upper limit of workgroups per compute unit of the flat kernels (the workspace bound of the backward counts on it).
 constexpr int kFlatBlocksPerCu = 4;
 
-// Whether a plain norm launch takes the flat mapping by itself.  Rows on the 128-bit path of 2 to 32 vectors in
-// float32 / float16 / bfloat16 storage whose vector count is not a power of two, where the segmented row sums (5 to 6
-// lane exchanges per value, against 3 to 5 DPP steps of the row kernels) cost less than the idle lanes and scattered
-// pieces of the row kernels do.  Forward + backward of 2^26 elements, % of 8 TB/s, row kernels -> flat (same box):
+// Whether a plain norm launch takes the flat mapping by itself.  16-bit rows on the 128-bit path of 3 to 21 vectors
+// whose vector count is not a power of two, where the segmented row sums (5 to 6 lane exchanges per value, against 3 to
+// 5 DPP steps of the row kernels) cost less than the idle lanes and scattered pieces of the row kernels do -- and less
+// than the staged kernels' detour through LDS, which wins for float32 rows (half the elements per vector) and is
+// within a point for these (bfloat16 RMSNorm N = 72: flat 112.2 us per forward + backward, staged 116.2, row kernels
+// 121).  Forward + backward of 2^26 elements, % of 8 TB/s, row kernels -> flat (same box):
 //   RMSNorm (one value per row sum), forward and backward, up to 21 vectors: bfloat16 N = 24: 53.0 -> 73.3; 40: 67.9 ->
-//     74.7; 72: 69.7 -> 75.2; 88: 72.1 -> 74.3; 120: 73.8 -> 75.7; 136: 69.3 -> 72.3; 168: 71.5 -> 75.4; float32 N = 12:
-//     59.0 -> 75.0; 28: 73.2 -> 77.0; 36: 73.9 -> 76.4; 68: 73.2 -> 75.5; 84: 74.8 -> 77.6; from 22 vectors on the row
-//     kernels are as fast or faster (bfloat16 N = 200: 73.7 against 73.0);
-//   LayerNorm (three values per row in the forward and in the backward): the forward up to 7 vectors of 16-bit and 15
-//     of 32-bit storage (forward alone flat, bfloat16 N = 40: 64.9 -> 71.1; 56: 68.9 -> 71.8; float32 N = 20: 70.3 ->
-//     75.3; 28: 70.8 -> 76.3; 60: 73.5 -> 76.3; 16-bit rows of 9 and 10 vectors gain a point in one run and lose one
-//     in the next, wider ones lose 1-3), the backward only for rows of 3 vectors (bfloat16 N = 24: 48.7 -> 66.1; from
-//     5 vectors on it is 0-6 points slower than the row kernels' backward: three segmented sums per row).
+//     74.7; 72: 69.7 -> 75.2; 88: 72.1 -> 74.3; 120: 73.8 -> 75.7; 136: 69.3 -> 72.3; 168: 71.5 -> 75.4; from 22 vectors
+//     on the row kernels are as fast or faster (bfloat16 N = 200: 73.7 against 73.0);
+//   LayerNorm (three values per row in the forward and in the backward): the forward up to 7 vectors (forward alone
+//     flat, bfloat16 N = 40: 64.9 -> 71.1; 56: 68.9 -> 71.8; rows of 9 and 10 vectors gain a point in one run and lose
+//     one in the next, wider ones lose 1-3), the backward only for rows of 3 vectors (bfloat16 N = 24: 48.7 -> 66.1;
+//     from 5 vectors on it is 0-6 points slower than the row kernels' backward: three segmented sums per row).
 // The launch override selects the flat kernels explicitly with threads_per_row = the row's vector count (not a power
-// of two) and vecs_per_thread = rows per lane and step (1, 2 or 4), and keeps them off with any other threads_per_row.
+// of two), block_threads = 0 or 256 and vecs_per_thread = rows per lane and step (1, 2 or 4).
 bool flat_by_default(int which, bool ln, int bytes, int n_vecs) {
-    if ((n_vecs & (n_vecs - 1)) == 0) return false;
-    if (which == kNormFwd) return ln ? n_vecs <= (bytes == 2 ? 7 : 15) : n_vecs <= 21;
+    if (bytes != 2 || (n_vecs & (n_vecs - 1)) == 0) return false;
+    if (which == kNormFwd) return ln ? n_vecs <= 7 : n_vecs <= 21;
     return ln ? n_vecs == 3 : n_vecs <= 21;
 }
 
@@ -740,6 +741,101 @@ bool plan_flat(int which, bool ln, bool aligned, int64_t M, int64_t N, int dtype
     }
     out->rows_each = rows_each;
     out->log_steps = n_vecs <= 16 ? 4 : 5;
+    out->grid = static_cast<int>(grid);
+    out->n_vecs = n_vecs;
+    return true;
+}
+
+// ---- the LDS-staged kernels for narrow rows (thn_staged.h) ------------------------------------------------------
+struct StagedPlan {
+    int passes;         // J: flat passes (vectors per lane) per batch
+    int grid;
+    int n_vecs;
+};
+
+int launch_staged_fwd(int dtype, bool ln, const StagedPlan& p, const FwdArgs& a, hipStream_t st, int* occ) {
+    switch (dtype) {
+        case THN_F32: return thn::launch_staged_fwd_f32(ln, p.passes, a, p.grid, st, occ);
+        case THN_F16: return thn::launch_staged_fwd_f16(ln, p.passes, a, p.grid, st, occ);
+        case THN_BF16: return thn::launch_staged_fwd_bf16(ln, p.passes, a, p.grid, st, occ);
+        default: return 1;
+    }
+}
+
+int launch_staged_bwd(int dtype, bool ln, const StagedPlan& p, const BwdArgs& a, hipStream_t st, int* occ) {
+    switch (dtype) {
+        case THN_F32: return thn::launch_staged_bwd_f32(ln, p.passes, a, p.grid, st, occ);
+        case THN_F16: return thn::launch_staged_bwd_f16(ln, p.passes, a, p.grid, st, occ);
+        case THN_BF16: return thn::launch_staged_bwd_bf16(ln, p.passes, a, p.grid, st, occ);
+        default: return 1;
+    }
+}
+
+// Upper limit of workgroups per compute unit of the staged kernels (the workspace bound of the backward counts on it).
+constexpr int kStagedBlocksPerCu = 4;
+
+// Whether a plain norm launch over rows of `n_vecs` vectors takes the staged kernels by itself: where forward +
+// backward of 2^26 elements measured faster than with the row kernels (same box, % of 8 TB/s, row kernels -> staged):
+//   rows of 1, 2 and 4 vectors in every storage type, forward and backward: bfloat16 N = 16 RMSNorm / LayerNorm
+//     39.3 / 35.1 -> 72.5 / 65.4; N = 32 63.9 / 60.0 -> 75.7 / 72.4; float32 N = 8 44.2 / 39.2 -> 75.3 / 72.8; N = 16
+//     69.3 / 65.3 -> 78.0 / 75.8; rows of 8 vectors, the forward only: bfloat16 N = 64 71.7 / 69.4 -> 77.2 / 74.1;
+//     float32 N = 32 73.8 / 71.5 -> 79.9 / 77.7 (wider powers of two fill the row kernels' lane groups: N = 128
+//     bfloat16 78.1 against 77.4);
+//   float32 rows whose vector count is not a power of two, RMSNorm and LayerNorm, forward and backward: RMSNorm N = 36
+//     73.9 -> 79.8; 80 76.6 -> 80.6; 100 76.6 -> 80.6; LayerNorm N = 36 70.0 -> 76.1; 68 64.5 -> 74.5; 100 68.7 -> 76.3;
+//     124 71.6 -> 78.2.  (16-bit rows of such widths: the flat mapping above, or the row kernels.)
+// The launch override selects the staged kernels explicitly with block_threads = 64 (a batch belongs to one wave),
+// threads_per_row = the row's vector count or 0, and vecs_per_thread = flat passes per batch (1 to 4) or 0.
+bool staged_by_default(int which, int bytes, int n_vecs) {
+    if ((n_vecs & (n_vecs - 1)) == 0) return n_vecs <= 4 || (n_vecs == 8 && which == kNormFwd);
+    return bytes >= 4;
+}
+
+bool plan_staged(int which, bool ln, bool aligned, int64_t M, int64_t N, int dtype, StagedPlan* out) {
+    const int bytes = elem_bytes(dtype);
+    if (!aligned || bytes == 0 || bytes == 8 || M <= 0) return false;
+    const int vec_elems = 16 / bytes;
+    if (N % vec_elems != 0) return false;
+    const int n_vecs = static_cast<int>(N / vec_elems);
+    if (n_vecs > thn::kStagedMaxVecs) return false;
+    const Override& ov = g_override[which];
+    // flat passes per batch and workgroups per compute unit, from a sweep over 1 to 4 passes x 1 to 4 workgroups at 26
+    // widths: the forward 2 x 2 (the 16-bit LayerNorm 4 x 4), the backward 4 x 2 (the 16-bit RMSNorm 2 x 2)
+    int passes, bpc = 2;
+    if (which == kNormFwd) {
+        passes = (ln && bytes == 2) ? 4 : 2;
+        if (ln && bytes == 2) bpc = 4;
+    } else {
+        passes = (!ln && bytes == 2) ? 2 : 4;
+    }
+    if (ov.tpr.load() > 0 || ov.block.load() > 0 || ov.k.load() > 0) {
+        if (ov.block.load() != thn::kStagedGroup) return false;                  // a row-kernel shape is forced
+        if (ov.tpr.load() > 0 && ov.tpr.load() != n_vecs) return false;
+        if (ov.k.load() > 0) {
+            passes = ov.k.load();
+            if (!thn::staged_fits(n_vecs, passes)) return false;
+        }
+    } else if (!staged_by_default(which, bytes, n_vecs)) {
+        return false;
+    }
+    while (passes > 1 && !thn::staged_fits(n_vecs, passes)) --passes;         // (rows of 2 and 3 vectors: a batch is 64 rows at most)
+    const int cus = current_cu_count();
+    if (cus <= 0) return false;
+    if (ov.bpc.load() > 0) bpc = ov.bpc.load();
+    if (bpc > kStagedBlocksPerCu) bpc = kStagedBlocksPerCu;
+    const int64_t rows_per_block = static_cast<int64_t>(thn::staged_geom(n_vecs, passes).R) * (thn::kStagedBlock / thn::kStagedGroup);
+    const int64_t row_blocks = (M + rows_per_block - 1) / rows_per_block;
+    const int64_t grid_max = static_cast<int64_t>(cus) * bpc;
+    int64_t grid = row_blocks;
+    if (grid > grid_max) {
+        const int64_t iters = (row_blocks + grid_max - 1) / grid_max;
+        grid = (row_blocks + iters - 1) / iters;
+        if (grid > cus && grid % cus != 0) {
+            const int64_t up = (grid + cus - 1) / cus * cus;
+            if (up <= grid_max && up <= row_blocks) grid = up;
+        }
+    }
+    out->passes = passes;
     out->grid = static_cast<int>(grid);
     out->n_vecs = n_vecs;
     return true;
@@ -819,7 +915,7 @@ int64_t bwd_workspace_bytes(int which, int flavour, int64_t M, int64_t N, int wa
     const int narrow = narrow_row_blocks_per_cu(which, n_vecs, bytes == 2 && N % vec_elems != 0);
     if (narrow > bpc) bpc = narrow;
     if (bytes == 2 && n_vecs <= 96 && bpc < 2) bpc = 2;      // the LayerNorm backward over narrow 16-bit rows (plan_launch)
-    if (which == kNormBwd && n_vecs <= thn::kFlatMaxVecs && bpc < kFlatBlocksPerCu) bpc = kFlatBlocksPerCu;   // the flat mapping
+    if (which == kNormBwd && n_vecs <= thn::kStagedMaxVecs && bpc < kStagedBlocksPerCu) bpc = kStagedBlocksPerCu;   // the staged kernels
     const int forced = g_override[which].bpc.load();
     if (forced > bpc) bpc = forced;
     if (bpc > kMaxBlocksPerCu) bpc = kMaxBlocksPerCu;
@@ -856,10 +952,16 @@ int norm_forward(const void* x, int64_t x_row_stride, void* y, int64_t y_row_str
     const bool aligned = (N % vec_elems) == 0 && aligned16(x) && aligned16(y) && aligned16(w) && aligned16(b) &&
                          (x_row_stride * bytes) % 16 == 0 && (y_row_stride * bytes) % 16 == 0;
     Plan p;
-    FlatPlan fp;
     const bool fused = act != thn::kNoAct;
-    const bool flat = !fused && plan_flat(kNormFwd, ln, aligned, M, N, x_dtype, &fp);
-    if (flat) {
+    StagedPlan sp;
+    FlatPlan fp;
+    const bool staged = !fused && plan_staged(kNormFwd, ln, aligned, M, N, x_dtype, &sp);
+    const bool flat = !fused && !staged && plan_flat(kNormFwd, ln, aligned, M, N, x_dtype, &fp);
+    if (staged) {
+        p.n_vecs = sp.n_vecs;
+        p.grid = sp.grid;
+        p.s = Shape{sp.passes, sp.n_vecs, thn::kStagedBlock};
+    } else if (flat) {
         p.n_vecs = fp.n_vecs;
         p.grid = fp.grid;
         p.s = Shape{fp.rows_each, fp.n_vecs, thn::kFlatBlock};
@@ -888,8 +990,9 @@ int norm_forward(const void* x, int64_t x_row_stride, void* y, int64_t y_row_str
     a.line_shift = line_shift_ok(aligned, p.s, p.grid, p.n_vecs, streams, 2) ? 1 : 0;
     a.keep_x = keep_x ? 1 : 0;
     hipStream_t st = static_cast<hipStream_t>(stream);
-    if (flat) a.line_shift = 0;
-    const int lrc = flat ? launch_flat_fwd(x_dtype, ln, fp, a, st, nullptr)
+    if (flat || staged) a.line_shift = 0;
+    const int lrc = staged ? launch_staged_fwd(x_dtype, ln, sp, a, st, nullptr)
+                  : flat ? launch_flat_fwd(x_dtype, ln, fp, a, st, nullptr)
                   : fused ? launch_fused_fwd(x_dtype, (ln ? 1 : 0) | (act << 1), aligned, p.s, a, p.grid, st, nullptr)
                           : launch_fwd(x_dtype, ln, aligned, p.s, a, p.grid, st, nullptr);
     if (lrc > 0) return THN_E_SHAPE;
@@ -926,10 +1029,16 @@ int norm_backward_stage1(const void* x, int64_t x_row_stride, const void* dy, in
                          (x_row_stride * bytes) % 16 == 0 && (dy_row_stride * bytes) % 16 == 0 &&
                          (dx_row_stride * bytes) % 16 == 0;
     Plan p;
-    FlatPlan fp;
     const int variant = fused ? ((ln ? 1 : 0) | (act << 1)) : (ln ? 1 : 0);
-    const bool flat = !fused && plan_flat(kNormBwd, ln, aligned, M, N, x_dtype, &fp);
-    if (flat) {
+    StagedPlan sp;
+    FlatPlan fp;
+    const bool staged = !fused && plan_staged(kNormBwd, ln, aligned, M, N, x_dtype, &sp);
+    const bool flat = !fused && !staged && plan_flat(kNormBwd, ln, aligned, M, N, x_dtype, &fp);
+    if (staged) {
+        p.n_vecs = sp.n_vecs;
+        p.grid = sp.grid;
+        p.s = Shape{sp.passes, sp.n_vecs, thn::kStagedBlock};
+    } else if (flat) {
         p.n_vecs = fp.n_vecs;
         p.grid = fp.grid;
         p.s = Shape{fp.rows_each, fp.n_vecs, thn::kFlatBlock};
@@ -964,8 +1073,9 @@ int norm_backward_stage1(const void* x, int64_t x_row_stride, const void* dy, in
     const RowStream streams[3] = {{x, a.x_stride_bytes}, {dy, a.dy_stride_bytes}, {dx, a.dx_stride_bytes}};
     a.line_shift = line_shift_ok(aligned, p.s, p.grid, p.n_vecs, streams, 3) ? 1 : 0;
     hipStream_t st = static_cast<hipStream_t>(stream);
-    if (flat) a.line_shift = 0;
-    const int lrc = flat ? launch_flat_bwd(x_dtype, ln, fp, a, st, nullptr)
+    if (flat || staged) a.line_shift = 0;
+    const int lrc = staged ? launch_staged_bwd(x_dtype, ln, sp, a, st, nullptr)
+                  : flat ? launch_flat_bwd(x_dtype, ln, fp, a, st, nullptr)
                   : fused ? launch_fused_bwd(x_dtype, variant, aligned, p.s, a, p.grid, st, nullptr)
                           : launch_bwd(x_dtype, ln, aligned, p.s, a, p.grid, st, nullptr);
     if (lrc > 0) return THN_E_SHAPE;
@@ -1255,6 +1365,15 @@ int thn_norm_query_launch(int which, int is_layernorm, int64_t M, int64_t N, int
         shape[2] = block;
         shape[3] = grid;
         shape[4] = 0;
+        return THN_OK;
+    }
+    StagedPlan sp;
+    if ((which == kNormFwd || which == kNormBwd) && plan_staged(which, is_layernorm != 0, aligned, M, N, x_dtype, &sp)) {
+        shape[0] = sp.passes;          // the staged kernels: flat passes per batch, vectors per row, a batch per wave
+        shape[1] = sp.n_vecs;
+        shape[2] = thn::kStagedGroup;
+        shape[3] = sp.grid;
+        shape[4] = 1;
         return THN_OK;
     }
     FlatPlan fp;
