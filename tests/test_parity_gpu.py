@@ -589,10 +589,11 @@ def compiled_shapes():
         for k, t, b in re.findall(r"X\((\d+), (\d+), (\w+)\)", body):
             shapes.append((int(k), int(t), block if b == "B" else int(b)))
         return shapes
-    fwd = expand("THN_FWD_SHAPES") + expand("THN_FWD_SHAPES_TWO_ROWS")
+    fwd = expand("THN_FWD_SHAPES") + expand("THN_FWD_SHAPES_TWO_ROWS") + expand("THN_FWD_SHAPES_THREE")
     bwd = [s for blk in (256, 512) for s in expand("THN_BWD_SHAPES_B", blk)]
     tail = re.search(r"#define THN_BWD_SHAPES\(X\)(.*?)\n\n", text, re.S).group(1)
     bwd += [(int(k), int(t), int(b)) for k, t, b in re.findall(r"X\((\d+), (\d+), (\d+)\)", tail)]
+    bwd += expand("THN_BWD_SHAPES_THREE")
     return fwd, bwd, expand("THN_BWD_SHAPES_LN16")
 
 

@@ -85,8 +85,10 @@ bool shape_compiled(int which, bool aligned, bool ln16, Shape s) {
         THN_SCALAR_SHAPES(THN_MATCH)
     } else if (!aligned && which == kNormBwd) {
         THN_BWD_SHAPES(THN_MATCH)
+        THN_BWD_SHAPES_THREE(THN_MATCH)
     } else if (which == kNormBwd) {
         THN_BWD_SHAPES(THN_MATCH)
+        THN_BWD_SHAPES_THREE(THN_MATCH)
         if (ln16) {
             THN_BWD_SHAPES_LN16(THN_MATCH)
         }
@@ -103,6 +105,7 @@ bool shape_compiled(int which, bool aligned, bool ln16, Shape s) {
         THN_FWD_SHAPES(THN_MATCH)
         if (which == kNormFwd) {
             THN_FWD_SHAPES_TWO_ROWS(THN_MATCH)
+            THN_FWD_SHAPES_THREE(THN_MATCH)
         }
     }
 #undef THN_MATCH
@@ -505,6 +508,34 @@ int plan_launch(int which, int flavour, bool aligned, int64_t M, int64_t N, int 
         if (shape_compiled(which, aligned, ln16, narrow)) {
             s = narrow;
             narrow_forward_pair = true;
+        }
+    }
+    // Rows of 33 to 48 and of 65 to 96 vectors (5 * 2^k elements and their neighbours: hidden sizes 320, 640 in 16-bit
+    // storage, 160, 320 in float32) fill 5/8 to 3/4 of the 2- and 4-vector shapes above and 5/6 or more of a 3-vector
+    // shape with the same threads per row.  The forward takes 3 x 16 / 3 x 32 in 256 threads, two workgroups per
+    // compute unit, in every storage type; the backward 3 x 16 / 3 x 32 in 512 threads for the 16-bit LayerNorm (whose
+    // arithmetic the idle lanes cost most), and 3 x 64 for its rows of 129 to 160 vectors.  Forward + backward of 2^26
+    // elements with that one launch changed, % of 8 TB/s -- forward: bfloat16 RMSNorm N = 272 68.6 -> 73.8; 320 74.5 ->
+    // 76.7; 544 70.9 -> 75.7; 640 74.5 -> 76.8; float32 N = 136 75.5 -> 78.6; 272 75.9 -> 79.7 (LayerNorm 72.9 -> 77.0);
+    // 320 78.4 -> 80.9; rows that fill the 4-vector shape to 3/4 gain nothing and lose nothing (N = 384 bfloat16 76.6 ->
+    // 77.0, float32 79.9 -> 79.6).  Backward, LayerNorm: float16 N = 272 56.3 -> 64.7; 320 63.0 -> 70.6; 544 58.4 ->
+    // 66.4; 640 66.2 -> 71.3; 768 71.1 -> 73.5; 1152 67.6 -> 71.0; 1280 70.1 -> 71.6; bfloat16 N = 320 69.9 -> 71.7; 544
+    // 62.5 -> 69.1; 640 69.1 -> 72.1; 1152 71.7 -> 73.7 (rows of 161 to 192 vectors lose a point that way and keep 2 x 128;
+    // the RMSNorm backward gains in float16, +1 to +3.6, and loses in bfloat16, -0.5 to -1.5: left as it is; float32
+    // backwards lose 0.5 to 6 points).
+    const bool fills_three_16 = n_vecs > 32 && n_vecs <= 48, fills_three_32 = n_vecs > 64 && n_vecs <= 96;
+    if (which == kNormFwd && N >= vec_elems && (fills_three_16 || fills_three_32)) {
+        const Shape three{3, fills_three_16 ? 16 : 32, 256};
+        if (shape_compiled(which, aligned, ln16, three)) {
+            s = three;
+            narrow_forward_pair = true;
+        }
+    }
+    if (which == kNormBwd && ln16 && (fills_three_16 || fills_three_32 || (n_vecs > 128 && n_vecs <= 160))) {
+        const Shape three{3, fills_three_16 ? 16 : (fills_three_32 ? 32 : 64), 512};
+        if (shape_compiled(which, aligned, ln16, three)) {
+            s = three;
+            narrow_backward_pair = false;
         }
     }
     // Rows that start off 128-byte lines: two-row workgroups of 256-thread rows cannot put their requests on line

@@ -34,6 +34,13 @@ struct Shape {
 // threads, 1 x 512 and, for rows of 1024 vectors, 2 x 512 in 1024 threads measured 1-4 % slower).
 #define THN_FWD_SHAPES_TWO_ROWS(X) X(3, 256, 512) X(2, 256, 512)
 
+// Norm forward and backward only: 3 vectors per thread for rows of 33 to 48 and 65 to 96 vectors (widths of 5 * 2^k
+// elements and their neighbours), which fill 5/8 of the next power of two of slots and 5/6 of these.  (The same for
+// rows of 17 to 24 vectors, 3 x 8, measured 1-8 points slower than the shapes those rows have.)
+#define THN_FWD_SHAPES_THREE(X) X(3, 16, 256) X(3, 32, 256)
+
+#define THN_BWD_SHAPES_THREE(X) X(3, 16, 512) X(3, 32, 512)
+
 #define THN_BWD_SHAPES_B(X, B)                                                       \
     X(1, 8, B) X(2, 8, B) X(4, 8, B)                                                 \
     X(1, 16, B) X(2, 16, B) X(4, 16, B)                                              \
@@ -103,9 +110,11 @@ inline int run_kernel(void (*kern)(const Args), const Args& a, int grid, int blo
         if (aligned) {                                                                                     \
             THN_FWD_SHAPES(THN_FWD_AL)                                                                     \
             THN_FWD_SHAPES_TWO_ROWS(THN_FWD_AL)                                                            \
+            THN_FWD_SHAPES_THREE(THN_FWD_AL)                                                               \
         } else if (a.n_cols >= TYPE::VEC) {                                                                \
             THN_FWD_SHAPES(THN_FWD_SC)                                                                     \
             THN_FWD_SHAPES_TWO_ROWS(THN_FWD_SC)                                                            \
+            THN_FWD_SHAPES_THREE(THN_FWD_SC)                                                               \
         } else {                                                                                           \
             using T = ElemIo<TYPE>;                                                                        \
             THN_FWD_SC(4, 8, 256)                                                                          \
@@ -119,6 +128,7 @@ inline int run_kernel(void (*kern)(const Args), const Args& a, int grid, int blo
         using T = TYPE;                                                                                    \
         if (aligned) {                                                                                     \
             THN_BWD_SHAPES(THN_BWD_AL)                                                                     \
+            THN_BWD_SHAPES_THREE(THN_BWD_AL)                                                               \
             if constexpr (TYPE::kBytes == 2) {                                                             \
                 if (ln) {                                                                                  \
                     THN_BWD_SHAPES_LN16(THN_BWD_AL_LN)                                                     \
@@ -126,6 +136,7 @@ inline int run_kernel(void (*kern)(const Args), const Args& a, int grid, int blo
             }                                                                                              \
         } else if (a.n_cols >= TYPE::VEC) {                                                                \
             THN_BWD_SHAPES(THN_BWD_SC)                                                                     \
+            THN_BWD_SHAPES_THREE(THN_BWD_SC)                                                               \
         } else {                                                                                           \
             using T = ElemIo<TYPE>;                                                                        \
             THN_BWD_SC(4, 8, 256)                                                                          \
