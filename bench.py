@@ -879,6 +879,25 @@ def ceiling_main(args, lib, dev):
             "us_per_launch": {str(m_): round(t, 2) for m_, t in pts},
             "GBps_at_16384_rows": round(units * 16384 * n * s / dict(pts)[16384] / 1e3, 1),
             "fit_intercept_us": round(a0, 2), "fit_slope_GBps": round(units * n * s / slope / 1e3, 1)}
+    # forward + backward of the SAME batch, back to back (16384 rows): what the memory-side cache gives a 2-read-1-write
+    # stream that follows a 1-read-1-write stream over one of its inputs -- the plain streams (the ReLU forward keeps x
+    # with cache-allocating loads, like the norm forward under the keep policy) next to the norm kernels
+    def norm_fwd_keep(b_, m_, ln):
+        rc = lib.thn_norm_fwd(p(b_["x"]), n, p(b_["y"]), n, p(w), p(b) if ln else 0, p(b_["mean"]) if ln else 0,
+                              p(b_["rstd"]), m_, n, 1e-6, code | _native.X_KEEP, code, stream)
+        assert rc == 0, rc
+
+    def pair(f, g_):
+        def both(b_):
+            f(b_, 16384)
+            g_(b_, 16384)
+        return both
+    out["same_batch_pairs_us_at_16384_rows"] = {
+        "thn_act_fwd + thn_act_bwd ReLU": round(timed(pair(act_fwd, act_bwd), 40), 2),
+        "rmsnorm forward (keep_x) + backward dx + partials": round(timed(pair(lambda b_, m_: norm_fwd_keep(b_, m_, False),
+                                                                              lambda b_, m_: norm_bwd1(b_, m_, False)), 40), 2),
+        "layernorm forward (keep_x) + backward dx + partials": round(timed(pair(lambda b_, m_: norm_fwd_keep(b_, m_, True),
+                                                                                lambda b_, m_: norm_bwd1(b_, m_, True)), 40), 2)}
     # the second stage alone, and launches that move nothing
     norm_bwd1(sets[0], 16384, False)
     out["second_stage_us"] = round(timed(lambda b_: lib.thn_norm_bwd_reduce_partials(p(ws), parts.value, p(dw), 0, n, code,
