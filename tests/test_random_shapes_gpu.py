@@ -110,3 +110,55 @@ def test_random_large_norm_problem(seed):
     b = (0.1 * torch.randn(n, generator=g)).to(dtype) if kind == "ln" else None
     parity_util.run_and_compare(kind, x, dy, w, b, 1e-5, f"random large {seed}",
                                 sample_chunks=8 if m * n > 8_000_000 else None)
+
+
+def draw_narrow(seed):
+    """LayerNorm / RMSNorm over rows of 1 to 100 16-byte vectors (the staged kernels, the flat mapping, the 3-vector
+    shapes and the row kernels' narrow-row rules, each by the library's own choice), 1 to 300000 rows, a third of them
+    as column blocks of a wider buffer."""
+    rng = np.random.default_rng(9000 + seed)
+    dtype = [torch.bfloat16, torch.float16, torch.float32][int(rng.integers(3))]
+    vec = 16 // torch.empty(0, dtype=dtype).element_size()
+    n_vecs = int(rng.integers(1, 101)) if seed % 4 else int(rng.integers(1, 33))
+    n = n_vecs * vec
+    m = max(1, min(log_uniform(rng, 1, 300000), 12_000_000 // n))
+    kind = "ln" if rng.random() < 0.5 else "rms"
+    pad = vec * int(rng.integers(1, 5)) if rng.random() < 0.33 else 0
+    return kind, dtype, m, n, pad
+
+
+@pytest.mark.parametrize("seed", range(80))
+def test_random_narrow_norm_problem(seed):
+    from TritonHub.Normalization import _launch
+    kind, dtype, m, n, pad = draw_narrow(seed)
+    fwd = tuple(_launch.query_launch(0, kind == "ln", m, n, dtype))[:4]
+    bwd = tuple(_launch.query_launch(1, kind == "ln", m, n, dtype))[:4]
+    print(f"\n[case] random narrow seed={seed} {kind} {dtype} M={m} N={n} pad={pad} forward{fwd} backward{bwd}", flush=True)
+    g = torch.Generator().manual_seed(seed)
+    xb = (torch.randn(m, n + pad, generator=g) * 2 + 0.5).to(dtype)
+    gb = torch.randn(m, n + pad, generator=g).to(dtype)
+    x, dy = xb[:, :n].contiguous(), gb[:, :n].contiguous()
+    w = (1 + 0.1 * torch.randn(n, generator=g)).to(dtype)
+    b = (0.1 * torch.randn(n, generator=g)).to(dtype) if kind == "ln" else None
+    eps = 1e-5 if n >= 16 else 1e-2
+    sample = 8 if m * n > 8_000_000 else None
+    if not pad:
+        parity_util.run_and_compare(kind, x, dy, w, b, eps, f"random narrow {seed}", sample_chunks=sample)
+        return
+    # rows that are column blocks of a wider buffer: the same call on strided device views
+    from TritonHub.Normalization.layernorm import layernorm
+    from TritonHub.Normalization.rmsnorm import rmsnorm
+    xg = xb.cuda()[:, :n].detach().requires_grad_(True)
+    wg = w.cuda().requires_grad_(True)
+    bg = None if b is None else b.cuda().requires_grad_(True)
+    assert xg.stride(0) == n + pad
+    if kind == "ln":
+        y = layernorm.apply(xg, wg, bg, eps)
+        mean, rstd = y.grad_fn.saved_tensors[3], y.grad_fn.saved_tensors[4]
+    else:
+        y = rmsnorm.apply(xg, wg, eps)
+        mean, rstd = None, y.grad_fn.saved_tensors[2]
+    y.backward(gb.cuda()[:, :n])
+    torch.cuda.synchronize()
+    out = dict(y=y.detach(), dx=xg.grad, dw=wg.grad, db=None if bg is None else bg.grad, mean=mean, rstd=rstd)
+    parity_util.compare_with_oracle(kind, x, dy, w, b, eps, out, f"random narrow {seed} (strided)", sample_chunks=sample)
