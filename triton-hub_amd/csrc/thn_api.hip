@@ -681,6 +681,24 @@ int plan_launch(int which, int flavour, bool aligned, int64_t M, int64_t N, int 
     return THN_OK;
 }
 
+// Persistent grid of the flat and the staged kernels: one workgroup per block of rows up to bpc per compute unit, then
+// as many as give every workgroup the same number of steps, rounded up to a whole number per compute unit where that
+// stays within both limits.
+int64_t narrow_row_grid(int64_t M, int64_t rows_per_block, int cus, int bpc) {
+    const int64_t row_blocks = (M + rows_per_block - 1) / rows_per_block;
+    const int64_t grid_max = static_cast<int64_t>(cus) * bpc;
+    int64_t grid = row_blocks;
+    if (grid > grid_max) {
+        const int64_t iters = (row_blocks + grid_max - 1) / grid_max;
+        grid = (row_blocks + iters - 1) / iters;
+        if (grid > cus && grid % cus != 0) {
+            const int64_t up = (grid + cus - 1) / cus * cus;
+            if (up <= grid_max && up <= row_blocks) grid = up;
+        }
+    }
+    return grid;
+}
+
 // ---- the flat mapping for narrow rows (thn_flat.h) ------------------------------------------------------------
 struct FlatPlan {
     int rows_each;      // J: independent rows per lane and step
@@ -759,17 +777,7 @@ bool plan_flat(int which, bool ln, bool aligned, int64_t M, int64_t N, int dtype
     if (ov.bpc.load() > 0) bpc = ov.bpc.load();
     if (bpc > kMaxBlocksPerCu) bpc = kMaxBlocksPerCu;
     const int64_t rows_per_block = static_cast<int64_t>(thn::kFlatBlock / 64) * (64 / n_vecs) * rows_each;
-    const int64_t row_blocks = (M + rows_per_block - 1) / rows_per_block;
-    const int64_t grid_max = static_cast<int64_t>(cus) * bpc;
-    int64_t grid = row_blocks;
-    if (grid > grid_max) {
-        const int64_t iters = (row_blocks + grid_max - 1) / grid_max;
-        grid = (row_blocks + iters - 1) / iters;
-        if (grid > cus && grid % cus != 0) {
-            const int64_t up = (grid + cus - 1) / cus * cus;
-            if (up <= grid_max && up <= row_blocks) grid = up;
-        }
-    }
+    const int64_t grid = narrow_row_grid(M, rows_per_block, cus, bpc);
     out->rows_each = rows_each;
     out->log_steps = n_vecs <= 16 ? 4 : 5;
     out->grid = static_cast<int>(grid);
@@ -814,12 +822,17 @@ constexpr int kStagedBlocksPerCu = 4;
 //     bfloat16 78.1 against 77.4);
 //   float32 rows whose vector count is not a power of two, RMSNorm and LayerNorm, forward and backward: RMSNorm N = 36
 //     73.9 -> 79.8; 80 76.6 -> 80.6; 100 76.6 -> 80.6; LayerNorm N = 36 70.0 -> 76.1; 68 64.5 -> 74.5; 100 68.7 -> 76.3;
-//     124 71.6 -> 78.2.  (16-bit rows of such widths: the flat mapping above, or the row kernels.)
+//     124 71.6 -> 78.2;
+//   the 16-bit LayerNorm over rows of 9 and of 17 to 19 vectors, which fill less than 0.6 of the row kernels' 16 and 32
+//     lanes (bfloat16 N = 72: 58-67 from run to run -> 69.4; N = 136 64.8 -> 66.8; rows that fill more of their lane
+//     group stay: N = 96 73.2 against 68.9, N = 200 72.8 against 68.8).  (The other 16-bit rows whose vector count is
+//     not a power of two: the flat mapping above, or the row kernels.)
 // The launch override selects the staged kernels explicitly with block_threads = 64 (a batch belongs to one wave),
 // threads_per_row = the row's vector count or 0, and vecs_per_thread = flat passes per batch (1 to 4) or 0.
-bool staged_by_default(int which, int bytes, int n_vecs) {
+bool staged_by_default(int which, bool ln, int bytes, int n_vecs) {
     if ((n_vecs & (n_vecs - 1)) == 0) return n_vecs <= 4 || (n_vecs == 8 && which == kNormFwd);
-    return bytes >= 4;
+    if (bytes >= 4) return true;
+    return ln && (n_vecs == 9 || (n_vecs >= 17 && n_vecs <= 19));
 }
 
 bool plan_staged(int which, bool ln, bool aligned, int64_t M, int64_t N, int dtype, StagedPlan* out) {
@@ -831,14 +844,9 @@ bool plan_staged(int which, bool ln, bool aligned, int64_t M, int64_t N, int dty
     if (n_vecs > thn::kStagedMaxVecs) return false;
     const Override& ov = g_override[which];
     // flat passes per batch and workgroups per compute unit, from a sweep over 1 to 4 passes x 1 to 4 workgroups at 26
-    // widths: the forward 2 x 2 (the 16-bit LayerNorm 4 x 4), the backward 4 x 2 (the 16-bit RMSNorm 2 x 2)
-    int passes, bpc = 2;
-    if (which == kNormFwd) {
-        passes = (ln && bytes == 2) ? 4 : 2;
-        if (ln && bytes == 2) bpc = 4;
-    } else {
-        passes = (!ln && bytes == 2) ? 2 : 4;
-    }
+    // widths: the forward 2 x 2, the backward 4 x 2 (the 16-bit RMSNorm 2 x 2)
+    int passes = 2, bpc = 2;
+    if (which == kNormBwd && (ln || bytes >= 4)) passes = 4;
     if (ov.tpr.load() > 0 || ov.block.load() > 0 || ov.k.load() > 0) {
         if (ov.block.load() != thn::kStagedGroup) return false;                  // a row-kernel shape is forced
         if (ov.tpr.load() > 0 && ov.tpr.load() != n_vecs) return false;
@@ -846,7 +854,7 @@ bool plan_staged(int which, bool ln, bool aligned, int64_t M, int64_t N, int dty
             passes = ov.k.load();
             if (!thn::staged_fits(n_vecs, passes)) return false;
         }
-    } else if (!staged_by_default(which, bytes, n_vecs)) {
+    } else if (!staged_by_default(which, ln, bytes, n_vecs)) {
         return false;
     }
     while (passes > 1 && !thn::staged_fits(n_vecs, passes)) --passes;         // (rows of 2 and 3 vectors: a batch is 64 rows at most)
@@ -855,17 +863,7 @@ bool plan_staged(int which, bool ln, bool aligned, int64_t M, int64_t N, int dty
     if (ov.bpc.load() > 0) bpc = ov.bpc.load();
     if (bpc > kStagedBlocksPerCu) bpc = kStagedBlocksPerCu;
     const int64_t rows_per_block = static_cast<int64_t>(thn::staged_geom(n_vecs, passes).R) * (thn::kStagedBlock / thn::kStagedGroup);
-    const int64_t row_blocks = (M + rows_per_block - 1) / rows_per_block;
-    const int64_t grid_max = static_cast<int64_t>(cus) * bpc;
-    int64_t grid = row_blocks;
-    if (grid > grid_max) {
-        const int64_t iters = (row_blocks + grid_max - 1) / grid_max;
-        grid = (row_blocks + iters - 1) / iters;
-        if (grid > cus && grid % cus != 0) {
-            const int64_t up = (grid + cus - 1) / cus * cus;
-            if (up <= grid_max && up <= row_blocks) grid = up;
-        }
-    }
+    const int64_t grid = narrow_row_grid(M, rows_per_block, cus, bpc);
     out->passes = passes;
     out->grid = static_cast<int>(grid);
     out->n_vecs = n_vecs;

@@ -44,26 +44,26 @@ struct StagedGeom {
     int P;        // lanes per row in the statistics pass: 1, 2, 4 or 8, R * P <= 64
     int log_p;
 };
-__host__ __device__ inline StagedGeom staged_geom(int L, int J, int group = kStagedGroup) {
+__host__ __device__ inline StagedGeom staged_geom(int L, int J) {
     StagedGeom g;
     g.L = L;
-    g.rpp = group / L;
+    g.rpp = kStagedGroup / L;
     g.S = g.rpp * L;
     g.pitch = L | 1;
     g.R = J * g.rpp;
     g.P = 1;
     g.log_p = 0;
-    while (2 * g.P * g.R <= group && g.P < 8) {
+    while (2 * g.P * g.R <= kStagedGroup && g.P < 8) {
         g.P *= 2;
         ++g.log_p;
     }
     return g;
 }
 // Whether a batch of J flat passes over rows of L vectors fits the kernels' LDS arrays and statistics threads.
-__host__ __device__ inline bool staged_fits(int L, int J, int vec_capacity = kStagedVecs, int group = kStagedGroup) {
+__host__ __device__ inline bool staged_fits(int L, int J) {
     if (L < 1 || L > kStagedMaxVecs || J < 1 || J > kStagedMaxPasses) return false;
-    const StagedGeom g = staged_geom(L, J, group);
-    return g.R <= group && g.R * g.pitch <= vec_capacity / (kStagedBlock / group);
+    const StagedGeom g = staged_geom(L, J);
+    return g.R <= kStagedGroup && g.R * g.pitch <= kStagedVecs / (kStagedBlock / kStagedGroup);
 }
 
 // The lanes of a wave have written LDS that other lanes of the wave read next.  A wave executes its LDS instructions in
@@ -82,29 +82,86 @@ __device__ __forceinline__ float few_lanes_allreduce(float v, int P) {
     return v;
 }
 
+// The statistics pass's walk over a row in LDS: calls f(vector, counts) for the vectors sp, sp + P, ... of the row, four
+// requested at a time while four remain, then one by one.  A lane whose last index falls past the row (only when P > 1)
+// re-reads the row's last vector and is told not to count it.
+template <typename F>
+__device__ __forceinline__ void walk_row(const u32x4* rowp, int sp, int log_p, int L, int n_steps, F&& f) {
+    int i = 0;
+    for (; i + 4 <= n_steps; i += 4) {
+        u32x4 v4[4];
+        bool ok[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int v = sp + ((i + u) << log_p);
+            ok[u] = v < L;
+            v4[u] = rowp[ok[u] ? v : L - 1];
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) f(v4[u], ok[u]);
+    }
+    for (; i < n_steps; ++i) {
+        const int v = sp + (i << log_p);
+        const bool ok = v < L;
+        f(rowp[ok ? v : L - 1], ok);
+    }
+}
+
+// The same over two tensors' copies of the row and the float32 weights of its columns, two vectors at a time.
+template <int VEC, typename F>
+__device__ __forceinline__ void walk_row_pair(const u32x4* xrow, const u32x4* grow, const float* wl, int sp, int log_p, int L,
+                                              int n_steps, F&& f) {
+    int i = 0;
+    for (; i + 2 <= n_steps; i += 2) {
+        u32x4 vx[2], vg[2];
+        float wf[2][VEC];
+        bool ok[2];
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            const int v = sp + ((i + u) << log_p);
+            ok[u] = v < L;
+            const int vc = ok[u] ? v : L - 1;
+            vx[u] = xrow[vc];
+            vg[u] = grow[vc];
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) wf[u][e] = wl[vc * VEC + e];
+        }
+#pragma unroll
+        for (int u = 0; u < 2; ++u) f(vx[u], vg[u], wf[u], ok[u]);
+    }
+    for (; i < n_steps; ++i) {
+        const int v = sp + (i << log_p);
+        const bool ok = v < L;
+        const int vc = ok ? v : L - 1;
+        float wf[VEC];
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) wf[e] = wl[vc * VEC + e];
+        f(xrow[vc], grow[vc], wf, ok);
+    }
+}
+
 // Forward.  Arithmetic as norm_fwd_kernel (LayerNorm: mean0, then {sum d, sum d^2} with the delta correction).
 template <typename T, bool LN, int J, bool KEEPX>
 __global__ void __launch_bounds__(kStagedBlock) norm_staged_fwd_kernel(const FwdArgs a) {
     constexpr int VEC = T::VEC;
-    constexpr int GROUP = kStagedGroup;
-    constexpr int NG = kStagedBlock / GROUP;                  // waves per workgroup
+    constexpr int NG = kStagedBlock / kStagedGroup;           // waves per workgroup
     __shared__ u32x4 xs_all[kStagedVecs];
     __shared__ float st_all[2][kStagedBlock][4];              // per row of the batch: mean0, delta, rstd
 
-    const StagedGeom g = staged_geom(a.n_vecs, J, GROUP);
-    const int tid = threadIdx.x & (GROUP - 1), grp = threadIdx.x / GROUP;
-    u32x4* xs = xs_all + grp * (kStagedVecs / NG);
-    float (*st)[kStagedBlock][4] = reinterpret_cast<float (*)[kStagedBlock][4]>(&st_all[0][grp * GROUP][0]);
-    const int tf = tid < g.S ? tid : g.S - 1;                // a thread without work mirrors the last one that has some
+    const StagedGeom g = staged_geom(a.n_vecs, J);
+    const int lane = threadIdx.x & (kStagedGroup - 1), wave = threadIdx.x / kStagedGroup;
+    u32x4* xs = xs_all + wave * (kStagedVecs / NG);
+    float (*st)[kStagedBlock][4] = reinterpret_cast<float (*)[kStagedBlock][4]>(&st_all[0][wave * kStagedGroup][0]);
+    const int tf = lane < g.S ? lane : g.S - 1;                // a thread without work mirrors the last one that has some
     const int fr = tf / g.L, ft = tf - fr * g.L;             // flat passes: row within a pass, vector within the row
     const int voff = ft * 16;
-    const int sr_raw = tid >> g.log_p, sp = tid & (g.P - 1); // statistics pass: row within the batch, place among its P threads
+    const int sr_raw = lane >> g.log_p, sp = lane & (g.P - 1); // statistics pass: row within the batch, place among its P threads
     const int sr = sr_raw < g.R ? sr_raw : g.R - 1;
     const int n_steps = (g.L + g.P - 1) >> g.log_p;           // vectors of a row per statistics thread
 
     const int64_t rows_per_iter = static_cast<int64_t>(gridDim.x) * NG * g.R;
     const int64_t last_row = a.M - 1;
-    int64_t base = (static_cast<int64_t>(blockIdx.x) * NG + grp) * g.R;
+    int64_t base = (static_cast<int64_t>(blockIdx.x) * NG + wave) * g.R;
     u32x4 cur[J];
 #pragma unroll
     for (int j = 0; j < J; ++j) {
@@ -135,52 +192,30 @@ __global__ void __launch_bounds__(kStagedBlock) norm_staged_fwd_kernel(const Fwd
         float mean0 = 0.0f, delta = 0.0f, rstd;
         if constexpr (LN) {
             float s = 0.0f;
-            for (int i0 = 0; i0 < n_steps; i0 += 4) {
-                u32x4 v4[4];
-                bool ok[4];
+            walk_row(rowp, sp, g.log_p, g.L, n_steps, [&](u32x4 v, bool counts) {
+                float xf[VEC];
+                T::unpack(v, xf);
+                float sk = 0.0f;
 #pragma unroll
-                for (int u = 0; u < 4; ++u) {
-                    const int v = sp + ((i0 + u) << g.log_p);
-                    ok[u] = v < g.L;
-                    v4[u] = rowp[ok[u] ? v : g.L - 1];
-                }
-#pragma unroll
-                for (int u = 0; u < 4; ++u) {
-                    float xf[VEC];
-                    T::unpack(v4[u], xf);
-                    float sk = 0.0f;
-#pragma unroll
-                    for (int e = 0; e < VEC; ++e) sk += xf[e];
-                    s += ok[u] ? sk : 0.0f;
-                }
-            }
+                for (int e = 0; e < VEC; ++e) sk += xf[e];
+                s += counts ? sk : 0.0f;
+            });
             s = few_lanes_allreduce(s, g.P);
             mean0 = s * a.inv_n;
             float q0 = 0.0f, q1 = 0.0f;
-            for (int i0 = 0; i0 < n_steps; i0 += 4) {
-                u32x4 v4[4];
-                bool ok[4];
+            walk_row(rowp, sp, g.log_p, g.L, n_steps, [&](u32x4 v, bool counts) {
+                float xf[VEC];
+                T::unpack(v, xf);
+                float a0 = 0.0f, a1 = 0.0f;
 #pragma unroll
-                for (int u = 0; u < 4; ++u) {
-                    const int v = sp + ((i0 + u) << g.log_p);
-                    ok[u] = v < g.L;
-                    v4[u] = rowp[ok[u] ? v : g.L - 1];
+                for (int e = 0; e < VEC; ++e) {
+                    const float d = xf[e] - mean0;
+                    a0 += d;
+                    a1 = fmaf(d, d, a1);
                 }
-#pragma unroll
-                for (int u = 0; u < 4; ++u) {
-                    float xf[VEC];
-                    T::unpack(v4[u], xf);
-                    float a0 = 0.0f, a1 = 0.0f;
-#pragma unroll
-                    for (int e = 0; e < VEC; ++e) {
-                        const float d = xf[e] - mean0;
-                        a0 += d;
-                        a1 = fmaf(d, d, a1);
-                    }
-                    q0 += ok[u] ? a0 : 0.0f;
-                    q1 += ok[u] ? a1 : 0.0f;
-                }
-            }
+                q0 += counts ? a0 : 0.0f;
+                q1 += counts ? a1 : 0.0f;
+            });
             q0 = few_lanes_allreduce(q0, g.P);
             q1 = few_lanes_allreduce(q1, g.P);
             delta = q0 * a.inv_n;
@@ -188,25 +223,14 @@ __global__ void __launch_bounds__(kStagedBlock) norm_staged_fwd_kernel(const Fwd
             rstd = rsqrt_refined(var + a.eps);
         } else {
             float q = 0.0f;
-            for (int i0 = 0; i0 < n_steps; i0 += 4) {
-                u32x4 v4[4];
-                bool ok[4];
+            walk_row(rowp, sp, g.log_p, g.L, n_steps, [&](u32x4 v, bool counts) {
+                float xf[VEC];
+                T::unpack(v, xf);
+                float qk = 0.0f;
 #pragma unroll
-                for (int u = 0; u < 4; ++u) {
-                    const int v = sp + ((i0 + u) << g.log_p);
-                    ok[u] = v < g.L;
-                    v4[u] = rowp[ok[u] ? v : g.L - 1];
-                }
-#pragma unroll
-                for (int u = 0; u < 4; ++u) {
-                    float xf[VEC];
-                    T::unpack(v4[u], xf);
-                    float qk = 0.0f;
-#pragma unroll
-                    for (int e = 0; e < VEC; ++e) qk = fmaf(xf[e], xf[e], qk);
-                    q += ok[u] ? qk : 0.0f;
-                }
-            }
+                for (int e = 0; e < VEC; ++e) qk = fmaf(xf[e], xf[e], qk);
+                q += counts ? qk : 0.0f;
+            });
             q = few_lanes_allreduce(q, g.P);
             rstd = rsqrt_refined(fmaf(q, a.inv_n, a.eps));
         }
@@ -250,8 +274,7 @@ __global__ void __launch_bounds__(kStagedBlock) norm_staged_fwd_kernel(const Fwd
 template <typename T, bool LN, int J>
 __global__ void __launch_bounds__(kStagedBlock) norm_staged_bwd_kernel(const BwdArgs a) {
     constexpr int VEC = T::VEC;
-    constexpr int GROUP = kStagedGroup;
-    constexpr int NG = kStagedBlock / GROUP;
+    constexpr int NG = kStagedBlock / kStagedGroup;
     using Acc = typename AccType<(T::kBytes >= 4)>::type;
     __shared__ u32x4 xs_all[kStagedVecs];
     __shared__ u32x4 gs_all[kStagedVecs];
@@ -259,22 +282,22 @@ __global__ void __launch_bounds__(kStagedBlock) norm_staged_bwd_kernel(const Bwd
     __shared__ float st_all[2][kStagedBlock][6];              // per row of the batch: rstd, c1, mean, delta', c2
     static_assert(sizeof(Acc) * kStagedBlock * VEC <= sizeof(u32x4) * kStagedVecs, "the column sums reuse xs / gs");
 
-    const StagedGeom g = staged_geom(a.n_vecs, J, GROUP);
-    const int tid = threadIdx.x & (GROUP - 1), grp = threadIdx.x / GROUP;
-    u32x4* xs = xs_all + grp * (kStagedVecs / NG);
-    u32x4* gs = gs_all + grp * (kStagedVecs / NG);
-    float (*st)[kStagedBlock][6] = reinterpret_cast<float (*)[kStagedBlock][6]>(&st_all[0][grp * GROUP][0]);
-    const bool works = tid < g.S;
-    const int tf = works ? tid : g.S - 1;
+    const StagedGeom g = staged_geom(a.n_vecs, J);
+    const int lane = threadIdx.x & (kStagedGroup - 1), wave = threadIdx.x / kStagedGroup;
+    u32x4* xs = xs_all + wave * (kStagedVecs / NG);
+    u32x4* gs = gs_all + wave * (kStagedVecs / NG);
+    float (*st)[kStagedBlock][6] = reinterpret_cast<float (*)[kStagedBlock][6]>(&st_all[0][wave * kStagedGroup][0]);
+    const bool works = lane < g.S;
+    const int tf = works ? lane : g.S - 1;
     const int fr = tf / g.L, ft = tf - fr * g.L;
     const int voff = ft * 16;
-    const int sr_raw = tid >> g.log_p, sp = tid & (g.P - 1);
+    const int sr_raw = lane >> g.log_p, sp = lane & (g.P - 1);
     const int sr = sr_raw < g.R ? sr_raw : g.R - 1;
     const int n_steps = (g.L + g.P - 1) >> g.log_p;
 
     const int64_t rows_per_iter = static_cast<int64_t>(gridDim.x) * NG * g.R;
     const int64_t last_row = a.M - 1;
-    int64_t base = (static_cast<int64_t>(blockIdx.x) * NG + grp) * g.R;
+    int64_t base = (static_cast<int64_t>(blockIdx.x) * NG + wave) * g.R;
     u32x4 cx[J], cg[J];
 #pragma unroll
     for (int j = 0; j < J; ++j) {
@@ -332,43 +355,28 @@ __global__ void __launch_bounds__(kStagedBlock) norm_staged_bwd_kernel(const Bwd
         const u32x4* xrow = xs + sr * g.pitch;
         const u32x4* grow = gs + sr * g.pitch;
         float s0 = 0.0f, s1 = 0.0f, s2 = 0.0f;
-        for (int i0 = 0; i0 < n_steps; i0 += 2) {
-            u32x4 vx[2], vg[2];
-            float wf[2][VEC];
-            bool ok[2];
+        walk_row_pair<VEC>(xrow, grow, wl, sp, g.log_p, g.L, n_steps,
+                           [&](u32x4 vx, u32x4 vg, const float (&wf)[VEC], bool counts) {
+            float xf[VEC], gf[VEC];
+            T::unpack(vx, xf);
+            T::unpack(vg, gf);
+            float a0 = 0.0f, a1 = 0.0f, a2 = 0.0f;
 #pragma unroll
-            for (int u = 0; u < 2; ++u) {
-                const int v = sp + ((i0 + u) << g.log_p);
-                ok[u] = v < g.L;
-                const int vc = ok[u] ? v : g.L - 1;
-                vx[u] = xrow[vc];
-                vg[u] = grow[vc];
-#pragma unroll
-                for (int e = 0; e < VEC; ++e) wf[u][e] = wl[vc * VEC + e];
-            }
-#pragma unroll
-            for (int u = 0; u < 2; ++u) {
-                float xf[VEC], gf[VEC];
-                T::unpack(vx[u], xf);
-                T::unpack(vg[u], gf);
-                float a0 = 0.0f, a1 = 0.0f, a2 = 0.0f;
-#pragma unroll
-                for (int e = 0; e < VEC; ++e) {
-                    const float uu = LN ? (xf[e] - c_mean) * c_rstd : xf[e] * c_rstd;
-                    const float wdy = wf[u][e] * gf[e];
-                    a0 = fmaf(uu, wdy, a0);
-                    if constexpr (LN) {
-                        a1 += wdy;
-                        a2 += uu;
-                    }
-                }
-                s0 += ok[u] ? a0 : 0.0f;
+            for (int e = 0; e < VEC; ++e) {
+                const float uu = LN ? (xf[e] - c_mean) * c_rstd : xf[e] * c_rstd;
+                const float wdy = wf[e] * gf[e];
+                a0 = fmaf(uu, wdy, a0);
                 if constexpr (LN) {
-                    s1 += ok[u] ? a1 : 0.0f;
-                    s2 += ok[u] ? a2 : 0.0f;
+                    a1 += wdy;
+                    a2 += uu;
                 }
             }
-        }
+            s0 += counts ? a0 : 0.0f;
+            if constexpr (LN) {
+                s1 += counts ? a1 : 0.0f;
+                s2 += counts ? a2 : 0.0f;
+            }
+        });
         s0 = few_lanes_allreduce(s0, g.P);
         float c1, c2 = 0.0f, dlt = 0.0f;
         if constexpr (LN) {
@@ -445,7 +453,7 @@ __global__ void __launch_bounds__(kStagedBlock) norm_staged_bwd_kernel(const Bwd
         Acc sw = Acc(0), sb = Acc(0);
         for (int gi = 0; gi < NG; ++gi) {
             for (int r = 0; r < g.rpp; ++r) {
-                const int src = gi * GROUP + r * g.L + t;
+                const int src = gi * kStagedGroup + r * g.L + t;
                 sw += tw[src * VEC + e];
                 sb += tb[src * VEC + e];
             }
