@@ -824,9 +824,10 @@ constexpr int kStagedBlocksPerCu = 4;
 //     73.9 -> 79.8; 80 76.6 -> 80.6; 100 76.6 -> 80.6; LayerNorm N = 36 70.0 -> 76.1; 68 64.5 -> 74.5; 100 68.7 -> 76.3;
 //     124 71.6 -> 78.2;
 //   the 16-bit LayerNorm over rows of 9 and of 17 to 19 vectors, which fill less than 0.6 of the row kernels' 16 and 32
-//     lanes (bfloat16 N = 72: 58-67 from run to run -> 69.4; N = 136 64.8 -> 66.8; rows that fill more of their lane
-//     group stay: N = 96 73.2 against 68.9, N = 200 72.8 against 68.8).  (The other 16-bit rows whose vector count is
-//     not a power of two: the flat mapping above, or the row kernels.)
+//     lanes: 1 to 2 points (bfloat16 N = 72, one direction changed: backward 66.4 -> 67.2, forward 67.7 -> 68.4; N = 144
+//     backward 66.3 -> 67.9; rows that fill more of their lane group stay: N = 96 73.6 against 70.7, N = 200 72.8 against
+//     70.2).  (The other 16-bit rows whose vector count is not a power of two: the flat mapping above, or the row
+//     kernels.)
 // The launch override selects the staged kernels explicitly with block_threads = 64 (a batch belongs to one wave),
 // threads_per_row = the row's vector count or 0, and vecs_per_thread = flat passes per batch (1 to 4) or 0.
 bool staged_by_default(int which, bool ln, int bytes, int n_vecs) {
