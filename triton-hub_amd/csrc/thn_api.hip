@@ -16,6 +16,7 @@
 #include "thn_dropout.h"
 #include "thn_pnorm_dispatch.h"
 #include "thn_softmax_dispatch.h"
+#include "thn_softmax_flat.h"
 
 namespace {
 
@@ -105,6 +106,8 @@ bool shape_compiled(int which, bool aligned, bool ln16, Shape s) {
         THN_FWD_SHAPES(THN_MATCH)
         if (which == kNormFwd) {
             THN_FWD_SHAPES_TWO_ROWS(THN_MATCH)
+        }
+        if (which == kNormFwd || ((which == kSoftmaxFwd || which == kSoftmaxBwd) && aligned)) {
             THN_FWD_SHAPES_THREE(THN_MATCH)
         }
     }
@@ -531,6 +534,18 @@ int plan_launch(int which, int flavour, bool aligned, int64_t M, int64_t N, int 
             narrow_forward_pair = true;
         }
     }
+    // The softmax family at the same widths: the forward as the norm forward; the backward over 33 to 48 vectors 3 x 16
+    // in 256 threads, one workgroup per compute unit (forward + backward of 2^26 elements, % of 8 TB/s, one launch
+    // changed: bfloat16 N = 272 54.6 -> 70.0; 320 61.2 -> 77.2; 384 69.5 -> 79.9; float32 N = 160 64.2 -> 80.3; forward:
+    // bfloat16 N = 544 71.5 -> 77.5; 640 76.8 -> 80.8; float32 N = 272 73.2 -> 79.8; the backward over 65 to 96 vectors
+    // gains nothing).
+    if ((which == kSoftmaxFwd || which == kSoftmaxBwd) && aligned && (fills_three_16 || fills_three_32)) {
+        const Shape three{3, fills_three_16 ? 16 : 32, 256};
+        if ((which == kSoftmaxFwd || fills_three_16) && shape_compiled(which, aligned, ln16, three)) {
+            s = three;
+            narrow_forward_pair = which == kSoftmaxFwd;
+        }
+    }
     if (which == kNormBwd && ln16 && (fills_three_16 || fills_three_32 || (n_vecs > 128 && n_vecs <= 160))) {
         const Shape three{3, fills_three_16 ? 16 : (fills_three_32 ? 32 : 64), 512};
         if (shape_compiled(which, aligned, ln16, three)) {
@@ -867,6 +882,66 @@ bool plan_staged(int which, bool ln, bool aligned, int64_t M, int64_t N, int dty
     const int64_t grid = narrow_row_grid(M, rows_per_block, cus, bpc);
     out->passes = passes;
     out->grid = static_cast<int>(grid);
+    out->n_vecs = n_vecs;
+    return true;
+}
+
+// ---- the flat mapping for narrow softmax rows (thn_softmax_flat.h) -------------------------------------------------
+struct SoftmaxFlatPlan {
+    int rows_each, log_steps, grid, n_vecs;
+};
+
+int launch_softmax_flat_fwd(int dtype, bool is_log, const SoftmaxFlatPlan& p, const SoftmaxFwdArgs& a, hipStream_t st) {
+    switch (dtype) {
+        case THN_F32: return thn::launch_softmax_flat_fwd_f32(is_log, p.rows_each, p.log_steps, a, p.grid, st);
+        case THN_F16: return thn::launch_softmax_flat_fwd_f16(is_log, p.rows_each, p.log_steps, a, p.grid, st);
+        case THN_BF16: return thn::launch_softmax_flat_fwd_bf16(is_log, p.rows_each, p.log_steps, a, p.grid, st);
+        default: return 1;
+    }
+}
+
+int launch_softmax_flat_bwd(int dtype, bool is_log, const SoftmaxFlatPlan& p, const SoftmaxBwdArgs& a, hipStream_t st) {
+    switch (dtype) {
+        case THN_F32: return thn::launch_softmax_flat_bwd_f32(is_log, p.rows_each, p.log_steps, a, p.grid, st);
+        case THN_F16: return thn::launch_softmax_flat_bwd_f16(is_log, p.rows_each, p.log_steps, a, p.grid, st);
+        case THN_BF16: return thn::launch_softmax_flat_bwd_bf16(is_log, p.rows_each, p.log_steps, a, p.grid, st);
+        default: return 1;
+    }
+}
+
+// Rows of 1, 2 and 4 vectors and rows of up to 32 vectors whose vector count is not a power of two, in float32 /
+// float16 / bfloat16 storage on the 128-bit path: where the row kernels' lane groups (8 lanes at least, a power of two)
+// stand half empty or worse.  Forward + backward of 2^26 elements, % of 8 TB/s, row kernels -> flat: bfloat16 N = 8
+// 17.7 -> 82.4; 16 31.0 -> 80.4; 32 53.1 -> 80.5; 72 59.1 -> 78.1; 96 66.9 -> 79.5; 136 52.5 -> 74.5; 192 69.3 -> 76.7;
+// float32 N = 4 20.7 -> 82.9; 16 56.1 -> 84.4; 36 59.7 -> 78.9; 68 53.3 -> 77.4; 96 73.0 -> 82.2 (rows of 8, 16 and 32
+// vectors fill their lane groups: 79-86 % with the row kernels).  The launch override reaches the kernels with threads_per_row = the row's vector count
+// and vecs_per_thread = rows per lane and step (2 or 4), and keeps them off with any other shape.
+bool plan_softmax_flat(int which, bool aligned, int64_t M, int64_t N, int dtype, SoftmaxFlatPlan* out) {
+    const int bytes = elem_bytes(dtype);
+    if (!aligned || (bytes != 2 && bytes != 4) || M <= 0) return false;
+    const int vec_elems = 16 / bytes;
+    if (N % vec_elems != 0) return false;
+    const int n_vecs = static_cast<int>(N / vec_elems);
+    if (n_vecs > thn::kFlatMaxVecs || ((n_vecs & (n_vecs - 1)) == 0 && n_vecs > 4)) return false;
+    const Override& ov = g_override[which];
+    // two rows per lane and step, two workgroups per compute unit: best or within a point of it over 2, 4 x 1, 2, 4 at 17
+    // widths; the forward over rows of 17 vectors and more (three rows per wave or fewer) takes four workgroups
+    // (bfloat16 N = 192 72.1 -> 76.7; float32 N = 96 77.0 -> 82.2)
+    int rows_each = 2, bpc = (which == kSoftmaxFwd && n_vecs >= 17) ? 4 : 2;
+    if (ov.tpr.load() > 0 || ov.block.load() > 0 || ov.k.load() > 0) {
+        if (ov.tpr.load() != n_vecs) return false;                                // a row-kernel shape is forced
+        if (ov.block.load() > 0 && ov.block.load() != thn::kFlatBlock) return false;
+        if (ov.k.load() > 0) rows_each = ov.k.load();
+        if (rows_each != 2 && rows_each != 4) return false;
+    }
+    const int cus = current_cu_count();
+    if (cus <= 0) return false;
+    if (ov.bpc.load() > 0) bpc = ov.bpc.load();
+    if (bpc > kMaxBlocksPerCu) bpc = kMaxBlocksPerCu;
+    const int64_t rows_per_block = static_cast<int64_t>(thn::kFlatBlock / 64) * (64 / n_vecs) * rows_each;
+    out->rows_each = rows_each;
+    out->log_steps = n_vecs == 1 ? 0 : (n_vecs <= 4 ? 2 : (n_vecs <= 16 ? 4 : 5));
+    out->grid = static_cast<int>(narrow_row_grid(M, rows_per_block, cus, bpc));
     out->n_vecs = n_vecs;
     return true;
 }
@@ -1397,6 +1472,15 @@ int thn_norm_query_launch(int which, int is_layernorm, int64_t M, int64_t N, int
         shape[4] = 0;
         return THN_OK;
     }
+    SoftmaxFlatPlan sfp;
+    if ((which == kSoftmaxFwd || which == kSoftmaxBwd) && plan_softmax_flat(which, aligned, M, N, x_dtype, &sfp)) {
+        shape[0] = sfp.rows_each;      // the flat mapping: rows per lane and step, lanes per row = vectors per row
+        shape[1] = sfp.n_vecs;
+        shape[2] = thn::kFlatBlock;
+        shape[3] = sfp.grid;
+        shape[4] = 1;
+        return THN_OK;
+    }
     StagedPlan sp;
     if ((which == kNormFwd || which == kNormBwd) && plan_staged(which, is_layernorm != 0, aligned, M, N, x_dtype, &sp)) {
         shape[0] = sp.passes;          // the staged kernels: flat passes per batch, vectors per row, a batch per wave
@@ -1635,6 +1719,21 @@ int thn_softmax_fwd(const void* x, int64_t x_row_stride, void* y, int64_t y_row_
     const bool aligned = (N % vec_elems) == 0 && aligned16(x) && aligned16(y) && (x_row_stride * bytes) % 16 == 0 &&
                          (y_row_stride * bytes) % 16 == 0;
     const bool is_log = kind == THN_LOGSOFTMAX;
+    SoftmaxFlatPlan fp;
+    if (plan_softmax_flat(kSoftmaxFwd, aligned, M, N, dtype, &fp)) {
+        SoftmaxFwdArgs a{};
+        a.x = static_cast<const char*>(x);
+        a.y = static_cast<char*>(y);
+        a.x_stride_bytes = x_row_stride * bytes;
+        a.y_stride_bytes = y_row_stride * bytes;
+        a.M = M;
+        a.n_cols = static_cast<int>(N);
+        a.n_vecs = fp.n_vecs;
+        a.sign = kind == THN_SOFTMIN ? -1.0f : 1.0f;
+        const int lrc = launch_softmax_flat_fwd(dtype, is_log, fp, a, static_cast<hipStream_t>(stream));
+        if (lrc > 0) return THN_E_SHAPE;
+        return lrc == 0 ? THN_OK : THN_E_LAUNCH;
+    }
     Plan p;
     const int rc = plan_launch(kSoftmaxFwd, is_log, aligned, M, N, dtype, &p, x_row_stride * elem_bytes(dtype));
     if (rc != THN_OK) return rc;
@@ -1692,6 +1791,23 @@ int thn_softmax_bwd(const void* y, int64_t y_row_stride, const void* dy, int64_t
                          (y_row_stride * bytes) % 16 == 0 && (dy_row_stride * bytes) % 16 == 0 &&
                          (dx_row_stride * bytes) % 16 == 0;
     const bool is_log = kind == THN_LOGSOFTMAX;
+    SoftmaxFlatPlan fp;
+    if (plan_softmax_flat(kSoftmaxBwd, aligned, M, N, dtype, &fp)) {
+        SoftmaxBwdArgs a{};
+        a.y = static_cast<const char*>(y);
+        a.dy = static_cast<const char*>(dy);
+        a.dx = static_cast<char*>(dx);
+        a.y_stride_bytes = y_row_stride * bytes;
+        a.dy_stride_bytes = dy_row_stride * bytes;
+        a.dx_stride_bytes = dx_row_stride * bytes;
+        a.M = M;
+        a.n_cols = static_cast<int>(N);
+        a.n_vecs = fp.n_vecs;
+        a.sign = kind == THN_SOFTMIN ? -1.0f : 1.0f;
+        const int lrc = launch_softmax_flat_bwd(dtype, is_log, fp, a, static_cast<hipStream_t>(stream));
+        if (lrc > 0) return THN_E_SHAPE;
+        return lrc == 0 ? THN_OK : THN_E_LAUNCH;
+    }
     Plan p;
     const int rc = plan_launch(kSoftmaxBwd, is_log, aligned, M, N, dtype, &p);
     if (rc != THN_OK) return rc;

@@ -42,6 +42,7 @@ THN_DECLARE_SOFTMAX_LAUNCHERS(f64)
         using T = TYPE;                                                                                         \
         if (aligned) {                                                                                          \
             THN_FWD_SHAPES(THN_SMF_AL)                                                                          \
+            THN_FWD_SHAPES_THREE(THN_SMF_AL)                                                                    \
         } else if (a.n_cols >= TYPE::VEC) { \
             THN_SCALAR_SHAPES(THN_SMF_SC) \
         } else { \
@@ -55,6 +56,7 @@ THN_DECLARE_SOFTMAX_LAUNCHERS(f64)
         using T = TYPE;                                                                                         \
         if (aligned) {                                                                                          \
             THN_FWD_SHAPES(THN_SMB_AL)                                                                          \
+            THN_FWD_SHAPES_THREE(THN_SMB_AL)                                                                    \
         } else if (a.n_cols >= TYPE::VEC) { \
             THN_SCALAR_SHAPES(THN_SMB_SC) \
         } else { \
