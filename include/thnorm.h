@@ -366,6 +366,10 @@ int thn_dropout(const void* x, void* out, int64_t n, int64_t first_offset, float
  * row; threads_per_row = the row's vector count or 0, vecs_per_thread = the batch in passes of the wave over its rows:
  * 1 to 4, or 0 for the default).  Problems such an override does not fit are refused (THN_E_SHAPE); any other
  * override runs the row kernels.
+ * The softmax and p-norm families (2 to 6) have flat kernels of their own for rows of 1, 2 and 4 vectors and of up to
+ * 32 vectors whose count is not a power of two, taken by default: threads_per_row = the row's vector count (with
+ * block_threads 0 or 256 and vecs_per_thread 0, 2 or, softmax only, 4 rows per lane and step) keeps them, any other
+ * shape selects the row kernels for such rows too.
  * Process-wide; meant for benchmarks, not for concurrent production use.  Returns THN_E_SHAPE when no
  * compiled kernel has that shape.
  */
@@ -381,6 +385,8 @@ int thn_norm_set_launch_override(int which, int vecs_per_thread, int threads_per
  * kernels (narrow 16-bit rows whose vector count is not a power of two) report {rows per lane and step, vectors per
  * row, 256, grid_blocks, 1}: a threads_per_row that is not a power of two identifies them; those that take the staged
  * kernels (rows of 1 to 8 vectors, narrow float32 rows) report {passes per batch, vectors per row, 64, grid_blocks, 1}.
+ * Softmax and p-norm problems on their flat kernels report {2 or 4, vectors per row, 256, grid_blocks, 1} (a p-norm
+ * problem is taken to be a dense (M, N) tensor here; tensors whose batches do not fold run the row kernels).
  */
 int thn_norm_query_launch(int which, int is_layernorm, int64_t M, int64_t N, int x_dtype, int32_t shape[5]);
 

@@ -17,6 +17,7 @@
 #include "thn_pnorm_dispatch.h"
 #include "thn_softmax_dispatch.h"
 #include "thn_softmax_flat.h"
+#include "thn_pnorm_flat.h"
 
 namespace {
 
@@ -740,9 +741,6 @@ int launch_flat_bwd(int dtype, bool ln, const FlatPlan& p, const BwdArgs& a, hip
     }
 }
 
-// Upper limit of workgroups per compute unit of the flat kernels (the workspace bound of the backward counts on it).
-constexpr int kFlatBlocksPerCu = 4;
-
 // Whether a plain norm launch takes the flat mapping by itself.  16-bit rows on the 128-bit path of 3 to 21 vectors
 // whose vector count is not a power of two, where the segmented row sums (5 to 6 lane exchanges per value, against 3 to
 // 5 DPP steps of the row kernels) cost less than the idle lanes and scattered pieces of the row kernels do -- and less
@@ -927,12 +925,13 @@ bool plan_softmax_flat(int which, bool aligned, int64_t M, int64_t N, int dtype,
     // two rows per lane and step, two workgroups per compute unit: best or within a point of it over 2, 4 x 1, 2, 4 at 17
     // widths; the forward over rows of 17 vectors and more (three rows per wave or fewer) takes four workgroups
     // (bfloat16 N = 192 72.1 -> 76.7; float32 N = 96 77.0 -> 82.2)
-    int rows_each = 2, bpc = (which == kSoftmaxFwd && n_vecs >= 17) ? 4 : 2;
+    const bool one_stream = which == kSoftmaxFwd || which == kPnormFwd;
+    int rows_each = 2, bpc = (one_stream && n_vecs >= 17) ? 4 : 2;
     if (ov.tpr.load() > 0 || ov.block.load() > 0 || ov.k.load() > 0) {
         if (ov.tpr.load() != n_vecs) return false;                                // a row-kernel shape is forced
         if (ov.block.load() > 0 && ov.block.load() != thn::kFlatBlock) return false;
         if (ov.k.load() > 0) rows_each = ov.k.load();
-        if (rows_each != 2 && rows_each != 4) return false;
+        if (rows_each != 2 && (rows_each != 4 || which >= kPnormFwd)) return false;
     }
     const int cus = current_cu_count();
     if (cus <= 0) return false;
@@ -944,6 +943,33 @@ bool plan_softmax_flat(int which, bool aligned, int64_t M, int64_t N, int dtype,
     out->grid = static_cast<int>(narrow_row_grid(M, rows_per_block, cus, bpc));
     out->n_vecs = n_vecs;
     return true;
+}
+
+// The p-norm / normalize family over the same narrow rows (thn_pnorm_flat.h): the plan is plan_softmax_flat's (two rows
+// per lane and step only); for tensors whose rows are one folded batch and integer p from 1 to 6.
+int launch_pnorm_flat_fwd(int dtype, int mode, bool normalize, const SoftmaxFlatPlan& p, const thn::PnormFwdArgs& a, hipStream_t st) {
+    switch (dtype) {
+        case THN_F32: return thn::launch_pnorm_flat_fwd_f32(mode, normalize, p.log_steps, a, p.grid, st);
+        case THN_F16: return thn::launch_pnorm_flat_fwd_f16(mode, normalize, p.log_steps, a, p.grid, st);
+        case THN_BF16: return thn::launch_pnorm_flat_fwd_bf16(mode, normalize, p.log_steps, a, p.grid, st);
+        default: return 1;
+    }
+}
+int launch_pnorm_flat_bwd(int dtype, int mode, const SoftmaxFlatPlan& p, const thn::PnormBwdArgs& a, hipStream_t st) {
+    switch (dtype) {
+        case THN_F32: return thn::launch_pnorm_flat_bwd_f32(mode, a, p.grid, st);
+        case THN_F16: return thn::launch_pnorm_flat_bwd_f16(mode, a, p.grid, st);
+        case THN_BF16: return thn::launch_pnorm_flat_bwd_bf16(mode, a, p.grid, st);
+        default: return 1;
+    }
+}
+int launch_normalize_flat_bwd(int dtype, int mode, const SoftmaxFlatPlan& p, const thn::NormalizeBwdArgs& a, hipStream_t st) {
+    switch (dtype) {
+        case THN_F32: return thn::launch_normalize_flat_bwd_f32(mode, p.log_steps, a, p.grid, st);
+        case THN_F16: return thn::launch_normalize_flat_bwd_f16(mode, p.log_steps, a, p.grid, st);
+        case THN_BF16: return thn::launch_normalize_flat_bwd_bf16(mode, p.log_steps, a, p.grid, st);
+        default: return 1;
+    }
 }
 
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
@@ -1287,7 +1313,11 @@ int pnorm_forward(const void* x, int64_t x_batch_stride, int64_t x_row_stride, v
     a.eps = eps;
     hipStream_t st = static_cast<hipStream_t>(stream);
     int lrc;
-    if (rp.engine) {
+    SoftmaxFlatPlan fp;
+    if (rp.engine && uniform && plan_softmax_flat(kPnormFwd, aligned, rp.rows, K, dtype, &fp)) {
+        a.n_vecs = fp.n_vecs;
+        lrc = launch_pnorm_flat_fwd(dtype, mode_of(rp.p_int), normalize, fp, a, st);
+    } else if (rp.engine) {
         const int variant = mode_of(rp.p_int) | (normalize ? 4 : 0);
         Plan plan;
         const int rc = plan_launch(kPnormFwd, variant, aligned, rp.rows, K, dtype, &plan, uniform ? a.xmap.row_stride_bytes : 0);
@@ -1473,7 +1503,7 @@ int thn_norm_query_launch(int which, int is_layernorm, int64_t M, int64_t N, int
         return THN_OK;
     }
     SoftmaxFlatPlan sfp;
-    if ((which == kSoftmaxFwd || which == kSoftmaxBwd) && plan_softmax_flat(which, aligned, M, N, x_dtype, &sfp)) {
+    if (which >= kSoftmaxFwd && which <= kNormalizeBwd && plan_softmax_flat(which, aligned, M, N, x_dtype, &sfp)) {
         shape[0] = sfp.rows_each;      // the flat mapping: rows per lane and step, lanes per row = vectors per row
         shape[1] = sfp.n_vecs;
         shape[2] = thn::kFlatBlock;
@@ -1870,7 +1900,11 @@ int thn_pnorm_bwd(const void* x, int64_t x_batch_stride, int64_t x_row_stride, c
     a.p = p;
     hipStream_t st = static_cast<hipStream_t>(stream);
     int lrc;
-    if (rp.engine) {
+    SoftmaxFlatPlan fp;
+    if (rp.engine && uniform && plan_softmax_flat(kPnormBwd, aligned, rp.rows, K, dtype, &fp)) {
+        a.n_vecs = fp.n_vecs;
+        lrc = launch_pnorm_flat_bwd(dtype, mode_of(rp.p_int), fp, a, st);
+    } else if (rp.engine) {
         const int mode = mode_of(rp.p_int);
         Plan plan;
         const int rc = plan_launch(kPnormBwd, mode, aligned, rp.rows, K, dtype, &plan);
@@ -1934,7 +1968,11 @@ int thn_normalize_bwd(const void* x, int64_t x_batch_stride, int64_t x_row_strid
     a.p = p;
     hipStream_t st = static_cast<hipStream_t>(stream);
     int lrc;
-    if (rp.engine) {
+    SoftmaxFlatPlan fp;
+    if (rp.engine && uniform && plan_softmax_flat(kNormalizeBwd, aligned, rp.rows, K, dtype, &fp)) {
+        a.n_vecs = fp.n_vecs;
+        lrc = launch_normalize_flat_bwd(dtype, mode_of(rp.p_int), fp, a, st);
+    } else if (rp.engine) {
         const int mode = mode_of(rp.p_int);
         Plan plan;
         const int rc = plan_launch(kNormalizeBwd, mode, aligned, rp.rows, K, dtype, &plan);
