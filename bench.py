@@ -65,6 +65,9 @@ WORKLOADS = {
     "softmin_bf16_16384x4096": ("softmin", 16384, 4096, "bf16"),
     "logsoftmax_bf16_8192x32768": ("logsoftmax", 8192, 32768, "bf16"),
     "logsoftmax_f32_16384x4096": ("logsoftmax", 16384, 4096, "f32"),
+    # narrow rows, 2^26 elements: one and nine vectors per row (the flat softmax kernels)
+    "softmax_bf16_8388608x8_narrow": ("softmax", 8388608, 8, "bf16"),
+    "softmax_bf16_932067x72_narrow": ("softmax", 932067, 72, "bf16"),
     # vocabulary-sized rows, wider than 64 KiB: the looping kernels (two walks per row)
     "logsoftmax_f32_8192x32000_vocab": ("logsoftmax", 8192, 32000, "f32"),
     "logsoftmax_bf16_4096x128256_vocab": ("logsoftmax", 4096, 128256, "bf16"),
@@ -76,6 +79,9 @@ WORKLOADS = {
     "normalize_p3_bf16_16384x4096": ("normalize_p3", 16384, 4096, "bf16"),
     "pnorm_p2_bf16_16384x4096": ("pnorm_p2", 16384, 4096, "bf16"),
     "pnorm_p3_f32_16384x4096": ("pnorm_p3", 16384, 4096, "f32"),
+    # rows of one float32 vector (quaternions) and of nine bfloat16 vectors, 2^26 elements: the flat p-norm kernels
+    "normalize_p2_f32_16777216x4_narrow": ("normalize_p2", 16777216, 4, "f32"),
+    "normalize_p2_bf16_932067x72_narrow": ("normalize_p2", 932067, 72, "bf16"),
     # element-wise activations (thn_act_fwd + thn_act_bwd per step)
     "act_gelu_bf16_16384x4096": ("act_gelu", 16384, 4096, "bf16"),
     "act_gelu_tanh_bf16_16384x4096": ("act_gelu_tanh", 16384, 4096, "bf16"),
