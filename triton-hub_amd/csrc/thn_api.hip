@@ -884,12 +884,13 @@ bool plan_staged(int which, bool ln, bool aligned, int64_t M, int64_t N, int dty
     return true;
 }
 
-// ---- the flat mapping for narrow softmax rows (thn_softmax_flat.h) -------------------------------------------------
-struct SoftmaxFlatPlan {
+// ---- the flat mapping for narrow rows of the softmax and p-norm families (thn_softmax_flat.h, thn_pnorm_flat.h): kernels
+// that reduce ONE value per row and round ---------------------------------------------------------------------------
+struct OneSumFlatPlan {
     int rows_each, log_steps, grid, n_vecs;
 };
 
-int launch_softmax_flat_fwd(int dtype, bool is_log, const SoftmaxFlatPlan& p, const SoftmaxFwdArgs& a, hipStream_t st) {
+int launch_softmax_flat_fwd(int dtype, bool is_log, const OneSumFlatPlan& p, const SoftmaxFwdArgs& a, hipStream_t st) {
     switch (dtype) {
         case THN_F32: return thn::launch_softmax_flat_fwd_f32(is_log, p.rows_each, p.log_steps, a, p.grid, st);
         case THN_F16: return thn::launch_softmax_flat_fwd_f16(is_log, p.rows_each, p.log_steps, a, p.grid, st);
@@ -898,7 +899,7 @@ int launch_softmax_flat_fwd(int dtype, bool is_log, const SoftmaxFlatPlan& p, co
     }
 }
 
-int launch_softmax_flat_bwd(int dtype, bool is_log, const SoftmaxFlatPlan& p, const SoftmaxBwdArgs& a, hipStream_t st) {
+int launch_softmax_flat_bwd(int dtype, bool is_log, const OneSumFlatPlan& p, const SoftmaxBwdArgs& a, hipStream_t st) {
     switch (dtype) {
         case THN_F32: return thn::launch_softmax_flat_bwd_f32(is_log, p.rows_each, p.log_steps, a, p.grid, st);
         case THN_F16: return thn::launch_softmax_flat_bwd_f16(is_log, p.rows_each, p.log_steps, a, p.grid, st);
@@ -909,12 +910,13 @@ int launch_softmax_flat_bwd(int dtype, bool is_log, const SoftmaxFlatPlan& p, co
 
 // Rows of 1, 2 and 4 vectors and rows of up to 32 vectors whose vector count is not a power of two, in float32 /
 // float16 / bfloat16 storage on the 128-bit path: where the row kernels' lane groups (8 lanes at least, a power of two)
-// stand half empty or worse.  Forward + backward of 2^26 elements, % of 8 TB/s, row kernels -> flat: bfloat16 N = 8
-// 17.7 -> 82.4; 16 31.0 -> 80.4; 32 53.1 -> 80.5; 72 59.1 -> 78.1; 96 66.9 -> 79.5; 136 52.5 -> 74.5; 192 69.3 -> 76.7;
-// float32 N = 4 20.7 -> 82.9; 16 56.1 -> 84.4; 36 59.7 -> 78.9; 68 53.3 -> 77.4; 96 73.0 -> 82.2 (rows of 8, 16 and 32
-// vectors fill their lane groups: 79-86 % with the row kernels).  The launch override reaches the kernels with threads_per_row = the row's vector count
-// and vecs_per_thread = rows per lane and step (2 or 4), and keeps them off with any other shape.
-bool plan_softmax_flat(int which, bool aligned, int64_t M, int64_t N, int dtype, SoftmaxFlatPlan* out) {
+// stand half empty or worse.  Softmax forward + backward of 2^26 elements, % of 8 TB/s, row kernels -> flat: bfloat16
+// N = 8 17.7 -> 82.4; 16 31.0 -> 80.4; 32 53.1 -> 80.5; 72 59.1 -> 78.1; 96 66.9 -> 79.5; 136 52.5 -> 74.5; 192 69.3 ->
+// 76.7; float32 N = 4 20.7 -> 82.9; 16 56.1 -> 84.4; 36 59.7 -> 78.9; 68 53.3 -> 77.4; 96 73.0 -> 82.2 (rows of 8, 16
+// and 32 vectors fill their lane groups: 79-86 % with the row kernels); normalize p = 2 alike (bfloat16 K = 8 16 -> 80,
+// float32 K = 4 17 -> 76).  The launch override reaches the kernels with threads_per_row = the row's vector count and
+// vecs_per_thread = rows per lane and step (2; the softmax kernels 4 as well), and keeps them off with any other shape.
+bool plan_one_sum_flat(int which, bool aligned, int64_t M, int64_t N, int dtype, OneSumFlatPlan* out) {
     const int bytes = elem_bytes(dtype);
     if (!aligned || (bytes != 2 && bytes != 4) || M <= 0) return false;
     const int vec_elems = 16 / bytes;
@@ -945,9 +947,9 @@ bool plan_softmax_flat(int which, bool aligned, int64_t M, int64_t N, int dtype,
     return true;
 }
 
-// The p-norm / normalize family over the same narrow rows (thn_pnorm_flat.h): the plan is plan_softmax_flat's (two rows
+// The p-norm / normalize family over the same narrow rows (thn_pnorm_flat.h): the plan is plan_one_sum_flat's (two rows
 // per lane and step only); for tensors whose rows are one folded batch and integer p from 1 to 6.
-int launch_pnorm_flat_fwd(int dtype, int mode, bool normalize, const SoftmaxFlatPlan& p, const thn::PnormFwdArgs& a, hipStream_t st) {
+int launch_pnorm_flat_fwd(int dtype, int mode, bool normalize, const OneSumFlatPlan& p, const thn::PnormFwdArgs& a, hipStream_t st) {
     switch (dtype) {
         case THN_F32: return thn::launch_pnorm_flat_fwd_f32(mode, normalize, p.log_steps, a, p.grid, st);
         case THN_F16: return thn::launch_pnorm_flat_fwd_f16(mode, normalize, p.log_steps, a, p.grid, st);
@@ -955,7 +957,7 @@ int launch_pnorm_flat_fwd(int dtype, int mode, bool normalize, const SoftmaxFlat
         default: return 1;
     }
 }
-int launch_pnorm_flat_bwd(int dtype, int mode, const SoftmaxFlatPlan& p, const thn::PnormBwdArgs& a, hipStream_t st) {
+int launch_pnorm_flat_bwd(int dtype, int mode, const OneSumFlatPlan& p, const thn::PnormBwdArgs& a, hipStream_t st) {
     switch (dtype) {
         case THN_F32: return thn::launch_pnorm_flat_bwd_f32(mode, a, p.grid, st);
         case THN_F16: return thn::launch_pnorm_flat_bwd_f16(mode, a, p.grid, st);
@@ -963,7 +965,7 @@ int launch_pnorm_flat_bwd(int dtype, int mode, const SoftmaxFlatPlan& p, const t
         default: return 1;
     }
 }
-int launch_normalize_flat_bwd(int dtype, int mode, const SoftmaxFlatPlan& p, const thn::NormalizeBwdArgs& a, hipStream_t st) {
+int launch_normalize_flat_bwd(int dtype, int mode, const OneSumFlatPlan& p, const thn::NormalizeBwdArgs& a, hipStream_t st) {
     switch (dtype) {
         case THN_F32: return thn::launch_normalize_flat_bwd_f32(mode, p.log_steps, a, p.grid, st);
         case THN_F16: return thn::launch_normalize_flat_bwd_f16(mode, p.log_steps, a, p.grid, st);
@@ -1313,8 +1315,8 @@ int pnorm_forward(const void* x, int64_t x_batch_stride, int64_t x_row_stride, v
     a.eps = eps;
     hipStream_t st = static_cast<hipStream_t>(stream);
     int lrc;
-    SoftmaxFlatPlan fp;
-    if (rp.engine && uniform && plan_softmax_flat(kPnormFwd, aligned, rp.rows, K, dtype, &fp)) {
+    OneSumFlatPlan fp;
+    if (rp.engine && uniform && plan_one_sum_flat(kPnormFwd, aligned, rp.rows, K, dtype, &fp)) {
         a.n_vecs = fp.n_vecs;
         lrc = launch_pnorm_flat_fwd(dtype, mode_of(rp.p_int), normalize, fp, a, st);
     } else if (rp.engine) {
@@ -1502,8 +1504,8 @@ int thn_norm_query_launch(int which, int is_layernorm, int64_t M, int64_t N, int
         shape[4] = 0;
         return THN_OK;
     }
-    SoftmaxFlatPlan sfp;
-    if (which >= kSoftmaxFwd && which <= kNormalizeBwd && plan_softmax_flat(which, aligned, M, N, x_dtype, &sfp)) {
+    OneSumFlatPlan sfp;
+    if (which >= kSoftmaxFwd && which <= kNormalizeBwd && plan_one_sum_flat(which, aligned, M, N, x_dtype, &sfp)) {
         shape[0] = sfp.rows_each;      // the flat mapping: rows per lane and step, lanes per row = vectors per row
         shape[1] = sfp.n_vecs;
         shape[2] = thn::kFlatBlock;
@@ -1749,8 +1751,8 @@ int thn_softmax_fwd(const void* x, int64_t x_row_stride, void* y, int64_t y_row_
     const bool aligned = (N % vec_elems) == 0 && aligned16(x) && aligned16(y) && (x_row_stride * bytes) % 16 == 0 &&
                          (y_row_stride * bytes) % 16 == 0;
     const bool is_log = kind == THN_LOGSOFTMAX;
-    SoftmaxFlatPlan fp;
-    if (plan_softmax_flat(kSoftmaxFwd, aligned, M, N, dtype, &fp)) {
+    OneSumFlatPlan fp;
+    if (plan_one_sum_flat(kSoftmaxFwd, aligned, M, N, dtype, &fp)) {
         SoftmaxFwdArgs a{};
         a.x = static_cast<const char*>(x);
         a.y = static_cast<char*>(y);
@@ -1821,8 +1823,8 @@ int thn_softmax_bwd(const void* y, int64_t y_row_stride, const void* dy, int64_t
                          (y_row_stride * bytes) % 16 == 0 && (dy_row_stride * bytes) % 16 == 0 &&
                          (dx_row_stride * bytes) % 16 == 0;
     const bool is_log = kind == THN_LOGSOFTMAX;
-    SoftmaxFlatPlan fp;
-    if (plan_softmax_flat(kSoftmaxBwd, aligned, M, N, dtype, &fp)) {
+    OneSumFlatPlan fp;
+    if (plan_one_sum_flat(kSoftmaxBwd, aligned, M, N, dtype, &fp)) {
         SoftmaxBwdArgs a{};
         a.y = static_cast<const char*>(y);
         a.dy = static_cast<const char*>(dy);
@@ -1900,8 +1902,8 @@ int thn_pnorm_bwd(const void* x, int64_t x_batch_stride, int64_t x_row_stride, c
     a.p = p;
     hipStream_t st = static_cast<hipStream_t>(stream);
     int lrc;
-    SoftmaxFlatPlan fp;
-    if (rp.engine && uniform && plan_softmax_flat(kPnormBwd, aligned, rp.rows, K, dtype, &fp)) {
+    OneSumFlatPlan fp;
+    if (rp.engine && uniform && plan_one_sum_flat(kPnormBwd, aligned, rp.rows, K, dtype, &fp)) {
         a.n_vecs = fp.n_vecs;
         lrc = launch_pnorm_flat_bwd(dtype, mode_of(rp.p_int), fp, a, st);
     } else if (rp.engine) {
@@ -1968,8 +1970,8 @@ int thn_normalize_bwd(const void* x, int64_t x_batch_stride, int64_t x_row_strid
     a.p = p;
     hipStream_t st = static_cast<hipStream_t>(stream);
     int lrc;
-    SoftmaxFlatPlan fp;
-    if (rp.engine && uniform && plan_softmax_flat(kNormalizeBwd, aligned, rp.rows, K, dtype, &fp)) {
+    OneSumFlatPlan fp;
+    if (rp.engine && uniform && plan_one_sum_flat(kNormalizeBwd, aligned, rp.rows, K, dtype, &fp)) {
         a.n_vecs = fp.n_vecs;
         lrc = launch_normalize_flat_bwd(dtype, mode_of(rp.p_int), fp, a, st);
     } else if (rp.engine) {
