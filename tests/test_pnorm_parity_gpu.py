@@ -342,7 +342,8 @@ def row_shapes():
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 def test_every_compiled_launch_shape(dtype):
     """Forces each kernel instance of the three families (4 forward, 5 norm backward, 6 normalize backward) through
-    the launch override, for the three p modes."""
+    the launch override, for the three p modes: on the 128-bit path, and off it (one column short of a whole number of
+    vectors: the unaligned-window instances, the last window overlapping its neighbour)."""
     lib = _native.lib()
     shapes = row_shapes()
     assert len(shapes) >= 20
@@ -350,19 +351,21 @@ def test_every_compiled_launch_shape(dtype):
     try:
         for k, tpr, block in shapes:
             for n_vecs in sorted({k * tpr, max((k - 1) * tpr + 1, k * tpr - tpr // 2 - 1)}):
-                n = n_vecs * vec
-                if n * (16 // vec) > 65536:
-                    continue
-                rows_per_block = block // tpr
-                m = 2 * rows_per_block + max(1, rows_per_block // 2)
-                announce(f"pnorm shape K={k} TPR={tpr} block={block} cols={n} rows={m} {dtype}")
-                for which in (4, 5, 6):
-                    assert lib.thn_norm_set_launch_override(which, k, tpr, block, 0) == 0
-                    assert query_launch(which, False, m, n, dtype)[:3] == (k, tpr, block)
-                x, gn, gy = make((1, m, n), dtype, seed=k * 1000 + tpr)
-                for p in (1, 2, 3):
-                    compare_norm(x, gn, p, 1e-6, f"norm shape {k},{tpr},{block} p={p}")
-                    compare_normalize(x, gy, p, 1e-6, f"normalize shape {k},{tpr},{block} p={p}")
+                for n in (n_vecs * vec, n_vecs * vec - 1):
+                    if n_vecs * 16 > 65536 or n < vec:
+                        continue
+                    on_path = n % vec == 0
+                    rows_per_block = block // tpr
+                    m = 2 * rows_per_block + max(1, rows_per_block // 2)
+                    announce(f"pnorm shape K={k} TPR={tpr} block={block} cols={n} rows={m} {dtype}")
+                    for which in (4, 5, 6):
+                        assert lib.thn_norm_set_launch_override(which, k, tpr, block, 0) == 0
+                        q = query_launch(which, False, m, n, dtype)
+                        assert q[:3] == (k, tpr, block) and q[4] == (1 if on_path else 0), q
+                    x, gn, gy = make((1, m, n), dtype, seed=k * 1000 + tpr)
+                    for p in (1, 2, 3):
+                        compare_norm(x, gn, p, 1e-6, f"norm shape {k},{tpr},{block} p={p} cols={n}")
+                        compare_normalize(x, gy, p, 1e-6, f"normalize shape {k},{tpr},{block} p={p} cols={n}")
     finally:
         for which in (4, 5, 6):
             lib.thn_norm_set_launch_override(which, 0, 0, 0, 0)

@@ -338,7 +338,10 @@ def compiled_forward_shapes():
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32, torch.float64])
 def test_every_compiled_launch_shape(dtype):
-    """Forces each softmax kernel instance through the launch override (forward: family 2, backward: family 3)."""
+    """Forces each softmax kernel instance through the launch override (forward: family 2, backward: family 3): on the
+    128-bit path, and off it (one column short of a whole number of vectors: the unaligned-window instances, the last
+    window overlapping its neighbour)."""
+    from TritonHub.Normalization._launch import query_launch
     lib = _native.lib()
     shapes = compiled_forward_shapes()
     assert len(shapes) >= 20
@@ -347,20 +350,21 @@ def test_every_compiled_launch_shape(dtype):
     try:
         for k, tpr, block in shapes:
             for n_vecs in sorted({k * tpr, max((k - 1) * tpr + 1, k * tpr - tpr // 2 - 1)}):
-                n = n_vecs * vec
-                if n * (16 // vec) > 65536:
-                    continue
-                rows_per_block = block // tpr
-                m = 2 * rows_per_block + max(1, rows_per_block // 2)
-                announce(f"softmax shape K={k} TPR={tpr} block={block} N={n} M={m} {dtype}")
-                assert lib.thn_norm_set_launch_override(2, k, tpr, block, 0) == 0
-                assert lib.thn_norm_set_launch_override(3, k, tpr, block, 0) == 0
-                from TritonHub.Normalization._launch import query_launch
-                assert query_launch(2, False, m, n, dtype)[:3] == (k, tpr, block)
-                assert query_launch(3, False, m, n, dtype)[:3] == (k, tpr, block)
-                x = (torch.randn(m, n, generator=g) * 2).to(dtype); dy = torch.randn(m, n, generator=g).to(dtype)
-                for kind in ("softmax", "logsoftmax"):
-                    run_and_compare(kind, x, dy, f"{kind} K={k} TPR={tpr} block={block} N={n}")
+                for n in (n_vecs * vec, n_vecs * vec - 1):
+                    if n_vecs * 16 > 65536 or n < vec:
+                        continue
+                    on_path = n % vec == 0
+                    rows_per_block = block // tpr
+                    m = 2 * rows_per_block + max(1, rows_per_block // 2)
+                    announce(f"softmax shape K={k} TPR={tpr} block={block} N={n} M={m} {dtype}")
+                    assert lib.thn_norm_set_launch_override(2, k, tpr, block, 0) == 0
+                    assert lib.thn_norm_set_launch_override(3, k, tpr, block, 0) == 0
+                    for which in (2, 3):
+                        q = query_launch(which, False, m, n, dtype)
+                        assert q[:3] == (k, tpr, block) and q[4] == (1 if on_path else 0), q
+                    x = (torch.randn(m, n, generator=g) * 2).to(dtype); dy = torch.randn(m, n, generator=g).to(dtype)
+                    for kind in ("softmax", "logsoftmax"):
+                        run_and_compare(kind, x, dy, f"{kind} K={k} TPR={tpr} block={block} N={n}")
     finally:
         lib.thn_norm_set_launch_override(2, 0, 0, 0, 0)
         lib.thn_norm_set_launch_override(3, 0, 0, 0, 0)

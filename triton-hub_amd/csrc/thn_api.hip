@@ -83,7 +83,7 @@ constexpr int kPolicyFlags = THN_X_KEEP | THN_X_STREAM;
 // `ln16`: LayerNorm over 16-bit rows (the two norm backwards have instances of their own for that).
 bool shape_compiled(int which, bool aligned, bool ln16, Shape s) {
 #define THN_MATCH(K_, TPR_, BLOCK_) if (s.k == K_ && s.tpr == TPR_ && s.block == BLOCK_) return true;
-    if (!aligned && which != kNormFwd && which != kNormBwd) {
+    if (!aligned && (which == kFusedFwd || which == kFusedBwd)) {
         THN_SCALAR_SHAPES(THN_MATCH)
     } else if (!aligned && which == kNormBwd) {
         THN_BWD_SHAPES(THN_MATCH)
@@ -108,9 +108,7 @@ bool shape_compiled(int which, bool aligned, bool ln16, Shape s) {
         if (which == kNormFwd) {
             THN_FWD_SHAPES_TWO_ROWS(THN_MATCH)
         }
-        if (which == kNormFwd || ((which == kSoftmaxFwd || which == kSoftmaxBwd) && aligned)) {
-            THN_FWD_SHAPES_THREE(THN_MATCH)
-        }
+        THN_FWD_SHAPES_THREE(THN_MATCH)
     }
 #undef THN_MATCH
     return false;
@@ -339,13 +337,13 @@ Shape heuristic_shape(int which, bool aligned, bool ln16, int n_vecs) {
     if ((which == kNormBwd || which == kFusedBwd) && aligned && ln16 && n_vecs > 2048) {
         return Shape{ceil_div(n_vecs, 512), 512, 512};
     }
-    // (the plain norm kernels take the same shapes off the 128-bit path as on it)
-    const bool norm_plain = which == kNormFwd || which == kNormBwd;
-    int kmax = ((aligned || norm_plain) && which == kNormBwd && n_vecs > 128) ? 3 : 4;
+    // (every family but the norm kernels with an activation epilogue takes the same shapes off the 128-bit path as on it)
+    const bool same_shapes = which != kFusedFwd && which != kFusedBwd;
+    int kmax = (which == kNormBwd && n_vecs > 128) ? 3 : 4;
     // Softmax backward: two input streams and nothing to hold; 2 vectors per thread per stream measured best,
     // except for 2 KiB rows, where one full wave per row (2 x 64) is 8 % slower than half a wave (4 x 32).
-    if (aligned && which == kSoftmaxBwd && n_vecs <= 2048 && !(n_vecs > 64 && n_vecs <= 128)) kmax = 2;
-    if (aligned && which == kNormalizeBwd && n_vecs <= 2048) kmax = 2;    // two or three input streams
+    if (which == kSoftmaxBwd && n_vecs <= 2048 && !(n_vecs > 64 && n_vecs <= 128)) kmax = 2;
+    if (which == kNormalizeBwd && n_vecs <= 2048) kmax = 2;    // two or three input streams
     if (aligned && which == kFusedBwd && n_vecs <= 2048) kmax = n_vecs > 128 ? 3 : 2;   // bias and pre-activation are live too
     Shape s{4, 1024, 1024};
     for (int tpr : kTprList) {
@@ -354,7 +352,7 @@ Shape heuristic_shape(int which, bool aligned, bool ln16, int n_vecs) {
             break;
         }
     }
-    if (!aligned && !norm_plain) {
+    if (!aligned && !same_shapes) {
         s.k = 4;
         s.block = s.tpr > 256 ? s.tpr : 256;
         return s;
@@ -408,12 +406,16 @@ void softmax_loop_launch(int which, int* block, int* bpc) {
 // rows and 2 up to 256-byte rows; those with two streams 2 up to 128-byte rows (the norm backward up to 256-byte
 // rows, where it runs one vector per thread: bf16 N = 128 5.2 -> 6.1 TB/s).
 int narrow_row_blocks_per_cu(int which, int n_vecs, bool ragged16) {
-    // 16-bit rows whose width is not a whole number of vectors, in the families whose unaligned-window instances
-    // shift the ragged vector in registers: 2-3 times the instructions per byte (shifts, per-column masks), and a
-    // second workgroup hides their latency (bf16 N = 4098 softmax: 2.6 -> 3.6 TB/s; float32 rows do not gain).  The
-    // norm kernels' overlapped windows cost no more than aligned vectors and lose 5-7 % with a second workgroup
-    // (bf16 24564 x 4098 forward 69.1 us with one, 73.4 with two; fp16 8192 x 12289 81.6 / 85.0).
-    if (ragged16 && n_vecs > 16 && which != kNormFwd && which != kNormBwd) return 2;
+    // 16-bit rows whose width is not a whole number of vectors.  The norm kernels with an activation epilogue run four
+    // vectors per thread there whatever the width, and a second workgroup hides the latency of their arithmetic.  The
+    // plain norm kernels' overlapped windows cost no more than aligned vectors and lose 5-7 % with a second workgroup (bf16 24564 x 4098 forward 69.1 us with one, 73.4 with two; fp16 8192 x 12289
+    // 81.6 / 85.0).  The softmax family has the same windows, but its forward holds so little per row that rows of more
+    // than 128 vectors still gain from the second workgroup (forward + backward of 2^26 bfloat16 elements, % of 8 TB/s,
+    // one / two: N = 1025 60.1 / 67.8; 2050 66.4 / 71.2; 4098 66.0 / 70.8; 5001 61.2 / 64.0) and narrower ones lose
+    // (N = 197 63.1 / 60.7; 300 72.2 / 70.5; 577 67.6 / 65.4; 1023 77.5 / 73.0); the p-norm family takes two workgroups
+    // of 256 threads anyway.
+    const bool fused = which == kFusedFwd || which == kFusedBwd;
+    if (ragged16 && n_vecs > 16 && which != kNormFwd && which != kNormBwd && (fused || n_vecs > 128)) return 2;
     const bool one_stream = which == kNormFwd || which == kSoftmaxFwd || which == kPnormFwd || which == kFusedFwd;
     if (n_vecs <= 8) return one_stream ? 4 : 2;
     if (n_vecs <= 16) return (one_stream || which == kNormBwd) ? 2 : 1;   // norm backward: with one vector per thread
@@ -540,7 +542,7 @@ int plan_launch(int which, int flavour, bool aligned, int64_t M, int64_t N, int 
     // changed: bfloat16 N = 272 54.6 -> 70.0; 320 61.2 -> 77.2; 384 69.5 -> 79.9; float32 N = 160 64.2 -> 80.3; forward:
     // bfloat16 N = 544 71.5 -> 77.5; 640 76.8 -> 80.8; float32 N = 272 73.2 -> 79.8; the backward over 65 to 96 vectors
     // gains nothing).
-    if ((which == kSoftmaxFwd || which == kSoftmaxBwd) && aligned && (fills_three_16 || fills_three_32)) {
+    if ((which == kSoftmaxFwd || which == kSoftmaxBwd) && N >= vec_elems && (fills_three_16 || fills_three_32)) {
         const Shape three{3, fills_three_16 ? 16 : 32, 256};
         if ((which == kSoftmaxFwd || fills_three_16) && shape_compiled(which, aligned, ln16, three)) {
             s = three;

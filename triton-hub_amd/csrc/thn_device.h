@@ -402,52 +402,13 @@ __device__ __forceinline__ u32x4 ld128u_keep(const void* p) { return *reinterpre
 __device__ __forceinline__ void st128u(void* p, u32x4 v) {
     __builtin_nontemporal_store(v, reinterpret_cast<u32x4_unaligned*>(p));
 }
+// The same store without the hint: for an output that is read again shortly.
+__device__ __forceinline__ void st128u_keep(void* p, u32x4 v) { *reinterpret_cast<u32x4_unaligned*>(p) = v; }
 
-// The 128-bit value w shifted down by `bytes` (0..15, a multiple of 2), zeros shifted in at the top.
-__device__ __forceinline__ u32x4 shift_down_bytes(u32x4 w, int bytes) {
-    const bool by1 = (bytes & 4) != 0, by2 = (bytes & 8) != 0;
-    const uint32_t r = static_cast<uint32_t>(bytes & 3) * 8u;
-    uint32_t e0 = w[0], e1 = w[1], e2 = w[2], e3 = w[3];
-    e0 = by1 ? e1 : e0; e1 = by1 ? e2 : e1; e2 = by1 ? e3 : e2; e3 = by1 ? 0u : e3;
-    e0 = by2 ? e2 : e0; e1 = by2 ? e3 : e1; e2 = by2 ? 0u : e2; e3 = by2 ? 0u : e3;
-    u32x4 out;
-    out[0] = __builtin_amdgcn_alignbit(e1, e0, r);
-    out[1] = __builtin_amdgcn_alignbit(e2, e1, r);
-    out[2] = __builtin_amdgcn_alignbit(e3, e2, r);
-    out[3] = e3 >> r;
-    return out;
-}
-
-// Vector slot `vec` of a row of n_cols >= VEC elements at any element-aligned address, as the 16-byte register
-// image the 128-bit path would hold (columns past the row end read as 0): ONE 16-byte load of the window that
-// ends at the row end at the latest, shifted down when the slot is the ragged last one.  No branch.
-template <typename T, bool KEEP = false>
-__device__ __forceinline__ u32x4 load_vec_window(const char* row, int vec, int n_cols) {
-    const int c0 = vec * T::VEC;
-    const int last = n_cols - T::VEC;
-    const int cw = c0 < last ? c0 : last;
-    const u32x4 w = KEEP ? ld128u_keep(row + cw * T::kBytes) : ld128u(row + cw * T::kBytes);
-    return shift_down_bytes(w, (c0 - cw) * T::kBytes);
-}
-
-// Stores slot `vec`: one 16-byte store when the whole slot lies inside the row, element stores for the ragged
-// last slot (one thread per row takes that branch).
-template <typename T>
-__device__ __forceinline__ void store_vec_window(char* row, int vec, int n_cols, const float (&f)[T::VEC]) {
-    const int c0 = vec * T::VEC;
-    if (c0 + T::VEC <= n_cols) {
-        st128u(row + c0 * T::kBytes, T::pack(f));
-    } else {
-#pragma unroll
-        for (int e = 0; e < T::VEC; ++e) {
-            if (c0 + e < n_cols) T::store1(row, c0 + e, f[e]);
-        }
-    }
-}
-
+// Element accesses with a column bound: for rows shorter than one vector (ElemIo<T>).  Columns past the row end read
+// as 0 and are not stored.
 template <typename T, bool KEEP = false>
 __device__ __forceinline__ u32x4 load_vec_elems(const char* row, int vec, int n_cols) {
-    if constexpr (T::kWindowIo) return load_vec_window<T, KEEP>(row, vec, n_cols);
     float f[T::VEC];
 #pragma unroll
     for (int e = 0; e < T::VEC; ++e) {
@@ -460,10 +421,6 @@ __device__ __forceinline__ u32x4 load_vec_elems(const char* row, int vec, int n_
 
 template <typename T>
 __device__ __forceinline__ void store_vec_elems(char* row, int vec, int n_cols, const float (&f)[T::VEC]) {
-    if constexpr (T::kWindowIo) {
-        store_vec_window<T>(row, vec, n_cols, f);
-        return;
-    }
 #pragma unroll
     for (int e = 0; e < T::VEC; ++e) {
         const int c = vec * T::VEC + e;

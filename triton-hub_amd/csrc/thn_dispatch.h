@@ -61,8 +61,8 @@ struct Shape {
 
 // Rows off the 128-bit path (N not a whole number of 16-byte vectors, or a pointer or stride off 16 bytes) run the
 // plain norm kernels in the same shapes as rows on it (their slots are 16-byte windows at element-aligned
-// addresses, the ragged last one overlapping its neighbour).  The other families and the norm kernels with an
-// activation epilogue keep one shape per row width there: four vectors per thread.
+// addresses, the ragged last one overlapping its neighbour), and so do the softmax and p-norm families.  The norm
+// kernels with an activation epilogue keep one shape per row width there: four vectors per thread.
 #define THN_SCALAR_SHAPES(X)                                                         \
     X(4, 8, 256) X(4, 16, 256) X(4, 32, 256) X(4, 64, 256) X(4, 128, 256)            \
     X(4, 256, 256) X(4, 512, 512) X(4, 1024, 1024)

@@ -79,26 +79,6 @@ __device__ __forceinline__ int row_line_shift(int enabled, const char* base, int
     return static_cast<int>(((reinterpret_cast<uintptr_t>(base) + static_cast<uint64_t>(first_row * stride_bytes)) & 127u) >> 4);
 }
 
-// Loads the K vectors of one row (KEEP: with cache-allocating loads, see ld128_keep).  `row` is already clamped
-// to a valid row; voff[k] is the byte offset of
-// the (clamped) vector slot k on the aligned 128-bit path and the vector index on the unaligned path.
-template <typename T, int K, bool ALIGNED, bool KEEP = false>
-__device__ __forceinline__ void load_row(u32x4 (&dst)[K], const char* base, int64_t stride_bytes, int64_t row,
-                                         const int (&voff)[K], int n_cols) {
-    const char* p = base + row * stride_bytes;
-#pragma unroll
-    for (int k = 0; k < K; ++k) {
-        if constexpr (ALIGNED) dst[k] = KEEP ? ld128_keep(p + voff[k]) : ld128(p + voff[k]);
-        else dst[k] = load_vec_elems<T, KEEP>(p, voff[k], n_cols);
-    }
-}
-
-template <typename T, bool ALIGNED, bool KEEP = false>
-__device__ __forceinline__ u32x4 load_row_vec(const char* rowp, int voff, int n_cols) {
-    if constexpr (ALIGNED) return KEEP ? ld128_keep(rowp + voff) : ld128(rowp + voff);
-    else return load_vec_elems<T, KEEP>(rowp, voff, n_cols);
-}
-
 // Vector slots of the norm kernels.  Three I/O modes, fixed at compile time:
 //   ALIGNED                      the 128-bit path: slot v is bytes [16 v, 16 v + 16) of the row;
 //   !ALIGNED, T::kWindowIo       rows off that path that hold at least one vector: slot v is the 16-byte window of
@@ -127,10 +107,22 @@ __device__ __forceinline__ void slot_load_row(u32x4 (&dst)[K], const char* base,
     for (int k = 0; k < K; ++k) dst[k] = slot_load<T, ALIGNED, KEEP>(p, voff[k], n_cols);
 }
 
-template <typename T, bool ALIGNED>
+// The 16 bytes of a slot on the 128-bit path or as an unaligned window.  KEEP: with an ordinary (cache-allocating)
+// store instead of a streaming one, for an output that the operator's backward reads again (see ld128_keep).
+template <bool ALIGNED, bool KEEP = false>
+__device__ __forceinline__ void slot_store_bits(char* p, u32x4 bits) {
+    if constexpr (ALIGNED) {
+        if constexpr (KEEP) st128_keep(p, bits);
+        else st128(p, bits);
+    } else {
+        if constexpr (KEEP) st128u_keep(p, bits);
+        else st128u(p, bits);
+    }
+}
+
+template <typename T, bool ALIGNED, bool KEEP = false>
 __device__ __forceinline__ void slot_store(char* rowp, int voff, int n_cols, const float (&f)[T::VEC]) {
-    if constexpr (ALIGNED) st128(rowp + voff, T::pack(f));
-    else if constexpr (T::kWindowIo) st128u(rowp + voff, T::pack(f));
+    if constexpr (ALIGNED || T::kWindowIo) slot_store_bits<ALIGNED, KEEP>(rowp + voff, T::pack(f));
     else store_vec_elems<T>(rowp, voff, n_cols, f);
 }
 
@@ -213,15 +205,6 @@ template <int K>
 __device__ __forceinline__ void forget_derived(u32x4 (&v)[K]) {
 #pragma unroll
     for (int k = 0; k < K; ++k) asm volatile("" : "+v"(v[k]));
-}
-
-// KEEP: an ordinary (cache-allocating) store instead of a streaming one, for an output that the operator's backward
-// reads again (see ld128_keep); on the 128-bit path only.
-template <typename T, bool ALIGNED, bool KEEP = false>
-__device__ __forceinline__ void store_row_vec(char* rowp, int voff, int n_cols, const float (&f)[T::VEC]) {
-    if constexpr (ALIGNED && KEEP) st128_keep(rowp + voff, T::pack(f));
-    else if constexpr (ALIGNED) st128(rowp + voff, T::pack(f));
-    else store_vec_elems<T>(rowp, voff, n_cols, f);
 }
 
 // ---------------------------------------------------------------------------------------------------

@@ -217,15 +217,13 @@ __global__ void __launch_bounds__(BLOCK) pnorm_fwd_kernel(const PnormFwdArgs a) 
     // the host sets line_shift only when the rows are one folded batch (row r at r * row stride), every row this
     // workgroup visits and every stream start in the same phase of a 128-byte line, and the slots have room
     const int shift = (ALIGNED && G == 1) ? row_line_shift(a.line_shift, a.x, a.xmap.row_stride_bytes, blockIdx.x) : 0;
-    int voff[K];
+    // Rows off the 128-bit path: unaligned 16-byte windows, the ragged last one overlapping its neighbour (slot_place()).
+    int voff[K], lead[K];
     bool own[K];
 #pragma unroll
-    for (int k = 0; k < K; ++k) {
-        const int v = t + k * TPR - shift;
-        const int vc = v < 0 ? 0 : (v < a.n_vecs ? v : a.n_vecs - 1);
-        voff[k] = ALIGNED ? vc * 16 : vc;
-        own[k] = v >= 0 && v < a.n_vecs;
-    }
+    for (int k = 0; k < K; ++k) slot_place<T, ALIGNED>(t + k * TPR - shift, a.n_vecs, a.n_cols, voff[k], lead[k], own[k]);
+    // element e of slot k counts in the row sum (always true on the 128-bit path)
+    auto counts = [&](int k, int e) -> bool { return slot_counts<T, ALIGNED>(voff[k], lead[k], e, a.n_cols); };
 
     const int64_t rows_per_iter = static_cast<int64_t>(gridDim.x) * G;
     const int64_t last_row = a.rows - 1;
@@ -237,7 +235,7 @@ __global__ void __launch_bounds__(BLOCK) pnorm_fwd_kernel(const PnormFwdArgs a) 
     last.init(a.walk, last_row);
     int64_t y_off = NORMALIZE ? row_offset(a.ymap, cursor) : 0;
     u32x4 cur[K];
-    load_row<T, K, ALIGNED, kKeepX>(cur, a.x + row_offset(a.xmap, cursor), 0, 0, voff, a.n_cols);
+    slot_load_row<T, K, ALIGNED, kKeepX>(cur, a.x + row_offset(a.xmap, cursor), 0, 0, voff, a.n_cols);
 
     drain_vector_memory(cur);
     for (int64_t base = static_cast<int64_t>(blockIdx.x) * G; base < a.rows; base += rows_per_iter) {
@@ -247,7 +245,7 @@ __global__ void __launch_bounds__(BLOCK) pnorm_fwd_kernel(const PnormFwdArgs a) 
         cursor.advance(a.walk);
         const RowCursor ncur = clamp_cursor(cursor, last, more);
         u32x4 nxt[K];
-        load_row<T, K, ALIGNED, kKeepX>(nxt, a.x + row_offset(a.xmap, ncur), 0, 0, voff, a.n_cols);
+        slot_load_row<T, K, ALIGNED, kKeepX>(nxt, a.x + row_offset(a.xmap, ncur), 0, 0, voff, a.n_cols);
 
         float xf[K][VEC];
         float s[1] = {0.0f};
@@ -256,7 +254,10 @@ __global__ void __launch_bounds__(BLOCK) pnorm_fwd_kernel(const PnormFwdArgs a) 
             T::unpack(cur[k], xf[k]);
             float sk = 0.0f;
 #pragma unroll
-            for (int e = 0; e < VEC; ++e) sk += norm_term<MODE>(xf[k][e], a.p_int);   // absent columns load as 0
+            for (int e = 0; e < VEC; ++e) {          // rows shorter than a vector: absent columns load as 0
+                const float term = norm_term<MODE>(xf[k][e], a.p_int);
+                sk += counts(k, e) ? term : 0.0f;
+            }
             s[0] += own[k] ? sk : 0.0f;
         }
         row_allreduce<TPR, G, 1>(s, red, phase, g, t);
@@ -274,7 +275,7 @@ __global__ void __launch_bounds__(BLOCK) pnorm_fwd_kernel(const PnormFwdArgs a) 
                 float yf[VEC];
 #pragma unroll
                 for (int e = 0; e < VEC; ++e) yf[e] = div_by_row(xf[k][e], nd, rn);
-                store_row_vec<T, ALIGNED, kKeepY>(yrow, voff[k], a.n_cols, yf);
+                slot_store<T, ALIGNED, kKeepY>(yrow, voff[k], a.n_cols, yf);
             }
             y_off = row_offset(a.ymap, ncur);
         }
@@ -302,10 +303,10 @@ __global__ void __launch_bounds__(BLOCK) pnorm_bwd_kernel(const PnormBwdArgs a) 
     const int shift = (ALIGNED && G == 1) ? row_line_shift(a.line_shift, a.x, a.xmap.row_stride_bytes, blockIdx.x) : 0;
     int voff[K];
 #pragma unroll
-    for (int k = 0; k < K; ++k) {
-        const int v = t + k * TPR - shift;        // slots off either end repeat their neighbour's vector (same bits)
-        const int vc = v < 0 ? 0 : (v < a.n_vecs ? v : a.n_vecs - 1);
-        voff[k] = ALIGNED ? vc * 16 : vc;
+    for (int k = 0; k < K; ++k) {      // slots off either end repeat their neighbour's vector (same bits)
+        int lead;
+        bool own;
+        slot_place<T, ALIGNED>(t + k * TPR - shift, a.n_vecs, a.n_cols, voff[k], lead, own);
     }
 
     const int64_t rows_per_iter = static_cast<int64_t>(gridDim.x) * G;
@@ -318,7 +319,7 @@ __global__ void __launch_bounds__(BLOCK) pnorm_bwd_kernel(const PnormBwdArgs a) 
     last.init(a.walk, last_row);
     int64_t dx_off = row_offset(a.dxmap, cursor);
     u32x4 cur[K];
-    load_row<T, K, ALIGNED>(cur, a.x + row_offset(a.xmap, cursor), 0, 0, voff, a.n_cols);
+    slot_load_row<T, K, ALIGNED>(cur, a.x + row_offset(a.xmap, cursor), 0, 0, voff, a.n_cols);
     float c_n = MODE == kP1 ? 1.0f : T::load1(a.norms, row);
     float c_g = T::load1(a.g, row);
 
@@ -331,7 +332,7 @@ __global__ void __launch_bounds__(BLOCK) pnorm_bwd_kernel(const PnormBwdArgs a) 
         cursor.advance(a.walk);
         const RowCursor ncur = clamp_cursor(cursor, last, more);
         u32x4 nxt[K];
-        load_row<T, K, ALIGNED>(nxt, a.x + row_offset(a.xmap, ncur), 0, 0, voff, a.n_cols);
+        slot_load_row<T, K, ALIGNED>(nxt, a.x + row_offset(a.xmap, ncur), 0, 0, voff, a.n_cols);
         // The next row's two scalars are requested here as raw bits and widened at the end of the step (hold_loaded_here
         // there keeps the compiler from widening them earlier): loads return in issue order, so an earlier use would
         // wait for the row's vectors in the middle of the step -- or, requested before them, for the previous row's
@@ -356,7 +357,7 @@ __global__ void __launch_bounds__(BLOCK) pnorm_bwd_kernel(const PnormBwdArgs a) 
                 else if constexpr (MODE == kP2) df[e] = div_by_row(c_g * x, den, rden);
                 else df[e] = div_by_row(c_g * sign_of(x) * pow_small(__builtin_fabsf(x), a.p_int - 1), den, rden);
             }
-            store_row_vec<T, ALIGNED>(dxrow, voff[k], a.n_cols, df);
+            slot_store<T, ALIGNED>(dxrow, voff[k], a.n_cols, df);
         }
 
 #pragma unroll
@@ -393,15 +394,13 @@ __global__ void __launch_bounds__(BLOCK) normalize_bwd_kernel(const NormalizeBwd
     // the host sets line_shift only when the rows are one folded batch (row r at r * row stride), every row this
     // workgroup visits and every stream start in the same phase of a 128-byte line, and the slots have room
     const int shift = (ALIGNED && G == 1) ? row_line_shift(a.line_shift, a.g, a.gmap.row_stride_bytes, blockIdx.x) : 0;
-    int voff[K];
+    // Rows off the 128-bit path: unaligned 16-byte windows, the ragged last one overlapping its neighbour (slot_place()).
+    int voff[K], lead[K];
     bool own[K];
 #pragma unroll
-    for (int k = 0; k < K; ++k) {
-        const int v = t + k * TPR - shift;
-        const int vc = v < 0 ? 0 : (v < a.n_vecs ? v : a.n_vecs - 1);
-        voff[k] = ALIGNED ? vc * 16 : vc;
-        own[k] = v >= 0 && v < a.n_vecs;
-    }
+    for (int k = 0; k < K; ++k) slot_place<T, ALIGNED>(t + k * TPR - shift, a.n_vecs, a.n_cols, voff[k], lead[k], own[k]);
+    // element e of slot k counts in the row sum (always true on the 128-bit path)
+    auto counts = [&](int k, int e) -> bool { return slot_counts<T, ALIGNED>(voff[k], lead[k], e, a.n_cols); };
 
     const int64_t rows_per_iter = static_cast<int64_t>(gridDim.x) * G;
     const int64_t last_row = a.rows - 1;
@@ -413,9 +412,9 @@ __global__ void __launch_bounds__(BLOCK) normalize_bwd_kernel(const NormalizeBwd
     last.init(a.walk, last_row);
     int64_t dx_off = row_offset(a.dxmap, cursor);
     u32x4 cx[NEED_X ? K : 1], cy[NEED_Y ? K : 1], cg[K];
-    if constexpr (NEED_X) load_row<T, K, ALIGNED>(cx, a.x + row_offset(a.xmap, cursor), 0, 0, voff, a.n_cols);
-    if constexpr (NEED_Y) load_row<T, K, ALIGNED>(cy, a.y + row_offset(a.ymap, cursor), 0, 0, voff, a.n_cols);
-    load_row<T, K, ALIGNED>(cg, a.g + row_offset(a.gmap, cursor), 0, 0, voff, a.n_cols);
+    if constexpr (NEED_X) slot_load_row<T, K, ALIGNED>(cx, a.x + row_offset(a.xmap, cursor), 0, 0, voff, a.n_cols);
+    if constexpr (NEED_Y) slot_load_row<T, K, ALIGNED>(cy, a.y + row_offset(a.ymap, cursor), 0, 0, voff, a.n_cols);
+    slot_load_row<T, K, ALIGNED>(cg, a.g + row_offset(a.gmap, cursor), 0, 0, voff, a.n_cols);
     float c_n = T::load1(a.norms, row);
 
     if constexpr (NEED_X) pin_loaded(cx);
@@ -428,9 +427,9 @@ __global__ void __launch_bounds__(BLOCK) normalize_bwd_kernel(const NormalizeBwd
         cursor.advance(a.walk);
         const RowCursor ncur = clamp_cursor(cursor, last, more);
         u32x4 nx[NEED_X ? K : 1], ny[NEED_Y ? K : 1], ng[K];
-        if constexpr (NEED_X) load_row<T, K, ALIGNED>(nx, a.x + row_offset(a.xmap, ncur), 0, 0, voff, a.n_cols);
-        if constexpr (NEED_Y) load_row<T, K, ALIGNED>(ny, a.y + row_offset(a.ymap, ncur), 0, 0, voff, a.n_cols);
-        load_row<T, K, ALIGNED>(ng, a.g + row_offset(a.gmap, ncur), 0, 0, voff, a.n_cols);
+        if constexpr (NEED_X) slot_load_row<T, K, ALIGNED>(nx, a.x + row_offset(a.xmap, ncur), 0, 0, voff, a.n_cols);
+        if constexpr (NEED_Y) slot_load_row<T, K, ALIGNED>(ny, a.y + row_offset(a.ymap, ncur), 0, 0, voff, a.n_cols);
+        slot_load_row<T, K, ALIGNED>(ng, a.g + row_offset(a.gmap, ncur), 0, 0, voff, a.n_cols);
         typename RowScalar<T>::bits_t raw_n = RowScalar<T>::load(a.norms, nrow);      // widened at the end of the step, as in pnorm_bwd_kernel
 
         float xf[NEED_X ? K : 1][VEC], yf[NEED_Y ? K : 1][VEC], gf[K][VEC];
@@ -443,8 +442,9 @@ __global__ void __launch_bounds__(BLOCK) normalize_bwd_kernel(const NormalizeBwd
             float sk = 0.0f;
 #pragma unroll
             for (int e = 0; e < VEC; ++e) {
-                if constexpr (MODE == kP1) sk = __builtin_fmaf(xf[k][e], gf[k][e], sk);       // normalize.py:92
-                else sk = __builtin_fmaf(yf[k][e], gf[k][e], sk);                             // normalize.py:96
+                const float ge = counts(k, e) ? gf[k][e] : 0.0f;
+                if constexpr (MODE == kP1) sk = __builtin_fmaf(xf[k][e], ge, sk);             // normalize.py:92
+                else sk = __builtin_fmaf(yf[k][e], ge, sk);                                   // normalize.py:96
             }
             s[0] += own[k] ? sk : 0.0f;
         }
@@ -474,7 +474,7 @@ __global__ void __launch_bounds__(BLOCK) normalize_bwd_kernel(const NormalizeBwd
                     df[e] = div_by_row(gg, nd, rn) - sign_of(x) * pow_small(__builtin_fabsf(x), a.p_int - 1) * coef;
                 }
             }
-            store_row_vec<T, ALIGNED>(dxrow, voff[k], a.n_cols, df);
+            slot_store<T, ALIGNED>(dxrow, voff[k], a.n_cols, df);
         }
 
 #pragma unroll

@@ -66,7 +66,7 @@ THN_DECLARE_PNORM_LAUNCHERS(f64)
         if (aligned) {                                                                                          \
             THN_ROW_SHAPES(THN_PNF_AL)                                                                          \
         } else if (a.n_cols >= TYPE::VEC) { \
-            THN_SCALAR_SHAPES(THN_PNF_SC) \
+            THN_ROW_SHAPES(THN_PNF_SC) \
         } else { \
             using T = ElemIo<TYPE>; \
             THN_PNF_SC(4, 8, 256) \
@@ -85,7 +85,7 @@ THN_DECLARE_PNORM_LAUNCHERS(f64)
         if (aligned) {                                                                                          \
             THN_ROW_SHAPES(THN_PNB_AL)                                                                          \
         } else if (a.n_cols >= TYPE::VEC) { \
-            THN_SCALAR_SHAPES(THN_PNB_SC) \
+            THN_ROW_SHAPES(THN_PNB_SC) \
         } else { \
             using T = ElemIo<TYPE>; \
             THN_PNB_SC(4, 8, 256) \
@@ -98,7 +98,7 @@ THN_DECLARE_PNORM_LAUNCHERS(f64)
         if (aligned) {                                                                                          \
             THN_ROW_SHAPES(THN_NZB_AL)                                                                          \
         } else if (a.n_cols >= TYPE::VEC) { \
-            THN_SCALAR_SHAPES(THN_NZB_SC) \
+            THN_ROW_SHAPES(THN_NZB_SC) \
         } else { \
             using T = ElemIo<TYPE>; \
             THN_NZB_SC(4, 8, 256) \

@@ -43,13 +43,14 @@ template <typename T, bool LOG> struct SoftmaxCompute {
     using type = typename std::conditional<T::kBytes == 8 && !LOG, double, float>::type;
 };
 
-// load_row for arithmetic type C: the unaligned path of the float32 engine narrows float64 storage on load,
-// which the float64 path must not do.
-template <typename T, typename C, int K, bool ALIGNED>
-__device__ __forceinline__ void load_row_as(u32x4 (&dst)[K], const char* base, int64_t stride_bytes, int64_t row,
-                                            const int (&voff)[K], int n_cols) {
-    if constexpr (ALIGNED || std::is_same<C, float>::value) {
-        load_row<T, K, ALIGNED>(dst, base, stride_bytes, row, voff, n_cols);
+// The vector slots of one row (slot_place() / slot_load() of thn_kernels.h) for arithmetic type C.  Rows shorter than
+// one vector come through element loads, and those of the float32 engine narrow float64 storage on the way, which the
+// float64 path must not do.
+template <typename T, typename C, int K, bool ALIGNED, bool KEEP = false>
+__device__ __forceinline__ void load_slots_as(u32x4 (&dst)[K], const char* base, int64_t stride_bytes, int64_t row,
+                                              const int (&voff)[K], int n_cols) {
+    if constexpr (ALIGNED || T::kWindowIo || std::is_same<C, float>::value) {
+        slot_load_row<T, K, ALIGNED, KEEP>(dst, base, stride_bytes, row, voff, n_cols);
     } else {
         const double* p = reinterpret_cast<const double*>(base + row * stride_bytes);
 #pragma unroll
@@ -66,17 +67,17 @@ __device__ __forceinline__ void load_row_as(u32x4 (&dst)[K], const char* base, i
     }
 }
 
-// KEEP: as store_row_vec.  The softmax family's forward keeps its output: the backward works from the saved y.
+// Stores one slot.  KEEP: as slot_store() -- the softmax family's forward keeps its output, the backward works from
+// the saved y.
 template <typename T, bool ALIGNED, bool KEEP = false>
-__device__ __forceinline__ void store_row_as(char* rowp, int voff, int n_cols, const float (&f)[T::VEC]) {
-    store_row_vec<T, ALIGNED, KEEP>(rowp, voff, n_cols, f);
+__device__ __forceinline__ void store_slot_as(char* rowp, int voff, int n_cols, const float (&f)[T::VEC]) {
+    slot_store<T, ALIGNED, KEEP>(rowp, voff, n_cols, f);
 }
 template <typename T, bool ALIGNED, bool KEEP = false>
-__device__ __forceinline__ void store_row_as(char* rowp, int voff, int n_cols, const double (&f)[T::VEC]) {
+__device__ __forceinline__ void store_slot_as(char* rowp, int voff, int n_cols, const double (&f)[T::VEC]) {
     static_assert(T::kBytes == 8, "float64 arithmetic is for float64 storage only");
-    if constexpr (ALIGNED) {
-        if constexpr (KEEP) st128_keep(rowp + voff, pack_f64(f));
-        else st128(rowp + voff, pack_f64(f));
+    if constexpr (ALIGNED || T::kWindowIo) {
+        slot_store_bits<ALIGNED, KEEP>(rowp + voff, pack_f64(f));
     } else {
 #pragma unroll
         for (int e = 0; e < 2; ++e) {
@@ -102,15 +103,13 @@ __global__ void __launch_bounds__(BLOCK) softmax_fwd_kernel(const SoftmaxFwdArgs
     int phase = 0;
 
     const int shift = (ALIGNED && G == 1) ? row_line_shift(a.line_shift, a.x, a.x_stride_bytes, blockIdx.x) : 0;
-    int voff[K];
+    // Rows off the 128-bit path: unaligned 16-byte windows, the ragged last one overlapping its neighbour (slot_place()).
+    int voff[K], lead[K];
     bool own[K];
 #pragma unroll
-    for (int k = 0; k < K; ++k) {
-        const int v = t + k * TPR - shift;
-        const int vc = v < 0 ? 0 : (v < a.n_vecs ? v : a.n_vecs - 1);
-        voff[k] = ALIGNED ? vc * 16 : vc;
-        own[k] = v >= 0 && v < a.n_vecs;
-    }
+    for (int k = 0; k < K; ++k) slot_place<T, ALIGNED>(t + k * TPR - shift, a.n_vecs, a.n_cols, voff[k], lead[k], own[k]);
+    // element e of slot k counts in the row sums (always true on the 128-bit path)
+    auto counts = [&](int k, int e) -> bool { return slot_counts<T, ALIGNED>(voff[k], lead[k], e, a.n_cols); };
     const C sign = static_cast<C>(a.sign);
     const C neg_inf = OpMax::identity<C>();
 
@@ -119,14 +118,14 @@ __global__ void __launch_bounds__(BLOCK) softmax_fwd_kernel(const SoftmaxFwdArgs
     int64_t row_raw = static_cast<int64_t>(blockIdx.x) * G + g;
     int64_t row = row_raw < a.M ? row_raw : last_row;
     u32x4 cur[K];
-    load_row_as<T, C, K, ALIGNED>(cur, a.x, a.x_stride_bytes, row, voff, a.n_cols);
+    load_slots_as<T, C, K, ALIGNED>(cur, a.x, a.x_stride_bytes, row, voff, a.n_cols);
 
     drain_vector_memory(cur);
     for (int64_t base = static_cast<int64_t>(blockIdx.x) * G; base < a.M; base += rows_per_iter) {
         const int64_t nrow_raw = row_raw + rows_per_iter;
         const int64_t nrow = nrow_raw < a.M ? nrow_raw : last_row;
         u32x4 nxt[K];
-        load_row_as<T, C, K, ALIGNED>(nxt, a.x, a.x_stride_bytes, nrow, voff, a.n_cols);
+        load_slots_as<T, C, K, ALIGNED>(nxt, a.x, a.x_stride_bytes, nrow, voff, a.n_cols);
 
         C xf[K][VEC];
         C m[1] = {neg_inf};
@@ -136,9 +135,9 @@ __global__ void __launch_bounds__(BLOCK) softmax_fwd_kernel(const SoftmaxFwdArgs
 #pragma unroll
             for (int e = 0; e < VEC; ++e) {
                 C v = xf[k][e] * sign;
-                if constexpr (!ALIGNED) v = (voff[k] * VEC + e < a.n_cols) ? v : neg_inf;
+                if constexpr (!ALIGNED && !T::kWindowIo) v = counts(k, e) ? v : neg_inf;     // past the end of a short row
                 xf[k][e] = v;
-                m[0] = OpMax::apply(m[0], v);      // clamped slots repeat real columns: harmless for a maximum
+                m[0] = OpMax::apply(m[0], v);      // clamped and overlapping slots repeat real columns: harmless for a maximum
             }
         }
         row_allreduce<TPR, G, 1, OpMax, C>(m, red, phase, g, t);
@@ -152,7 +151,7 @@ __global__ void __launch_bounds__(BLOCK) softmax_fwd_kernel(const SoftmaxFwdArgs
                 const C z = xf[k][e] - m[0];
                 const C ez = exp_c(z);              // columns past the row end: exp(-inf) = 0
                 xf[k][e] = LOG ? z : ez;
-                sk += ez;
+                sk += counts(k, e) ? ez : C(0);
             }
             s[0] += own[k] ? sk : C(0);
         }
@@ -167,7 +166,7 @@ __global__ void __launch_bounds__(BLOCK) softmax_fwd_kernel(const SoftmaxFwdArgs
             C yf[VEC];
 #pragma unroll
             for (int e = 0; e < VEC; ++e) yf[e] = LOG ? xf[k][e] - scale : xf[k][e] * scale;
-            store_row_as<T, ALIGNED, true>(yrow, voff[k], a.n_cols, yf);
+            store_slot_as<T, ALIGNED, true>(yrow, voff[k], a.n_cols, yf);
         }
 
 #pragma unroll
@@ -194,15 +193,13 @@ __global__ void __launch_bounds__(BLOCK) softmax_bwd_kernel(const SoftmaxBwdArgs
     int phase = 0;
 
     const int shift = (ALIGNED && G == 1) ? row_line_shift(a.line_shift, a.y, a.y_stride_bytes, blockIdx.x) : 0;
-    int voff[K];
+    // Rows off the 128-bit path: unaligned 16-byte windows, the ragged last one overlapping its neighbour (slot_place()).
+    int voff[K], lead[K];
     bool own[K];
 #pragma unroll
-    for (int k = 0; k < K; ++k) {
-        const int v = t + k * TPR - shift;
-        const int vc = v < 0 ? 0 : (v < a.n_vecs ? v : a.n_vecs - 1);
-        voff[k] = ALIGNED ? vc * 16 : vc;
-        own[k] = v >= 0 && v < a.n_vecs;
-    }
+    for (int k = 0; k < K; ++k) slot_place<T, ALIGNED>(t + k * TPR - shift, a.n_vecs, a.n_cols, voff[k], lead[k], own[k]);
+    // element e of slot k counts in the row sums (always true on the 128-bit path)
+    auto counts = [&](int k, int e) -> bool { return slot_counts<T, ALIGNED>(voff[k], lead[k], e, a.n_cols); };
 
     const int64_t rows_per_iter = static_cast<int64_t>(gridDim.x) * G;
     const int64_t last_row = a.M - 1;
@@ -210,28 +207,29 @@ __global__ void __launch_bounds__(BLOCK) softmax_bwd_kernel(const SoftmaxBwdArgs
     int64_t row = row_raw < a.M ? row_raw : last_row;
     const C sign = static_cast<C>(a.sign);
     u32x4 cy[K], cg[K];
-    load_row_as<T, C, K, ALIGNED>(cy, a.y, a.y_stride_bytes, row, voff, a.n_cols);
-    load_row_as<T, C, K, ALIGNED>(cg, a.dy, a.dy_stride_bytes, row, voff, a.n_cols);
+    load_slots_as<T, C, K, ALIGNED>(cy, a.y, a.y_stride_bytes, row, voff, a.n_cols);
+    load_slots_as<T, C, K, ALIGNED>(cg, a.dy, a.dy_stride_bytes, row, voff, a.n_cols);
 
     drain_vector_memory(cy, cg);
     for (int64_t base = static_cast<int64_t>(blockIdx.x) * G; base < a.M; base += rows_per_iter) {
         const int64_t nrow_raw = row_raw + rows_per_iter;
         const int64_t nrow = nrow_raw < a.M ? nrow_raw : last_row;
         u32x4 ny[K], ng[K];
-        load_row_as<T, C, K, ALIGNED>(ny, a.y, a.y_stride_bytes, nrow, voff, a.n_cols);
-        load_row_as<T, C, K, ALIGNED>(ng, a.dy, a.dy_stride_bytes, nrow, voff, a.n_cols);
+        load_slots_as<T, C, K, ALIGNED>(ny, a.y, a.y_stride_bytes, nrow, voff, a.n_cols);
+        load_slots_as<T, C, K, ALIGNED>(ng, a.dy, a.dy_stride_bytes, nrow, voff, a.n_cols);
 
         C yf[K][VEC], gf[K][VEC];
         C s[1] = {C(0)};
 #pragma unroll
         for (int k = 0; k < K; ++k) {
             unpack_as<T>(cy[k], yf[k]);
-            unpack_as<T>(cg[k], gf[k]);      // unaligned path: columns past the row end load as 0
+            unpack_as<T>(cg[k], gf[k]);      // rows shorter than a vector: columns past the row end load as 0
             C sk = C(0);
 #pragma unroll
             for (int e = 0; e < VEC; ++e) {
-                if constexpr (LOG) sk += gf[k][e];
-                else sk = fma(yf[k][e], gf[k][e], sk);
+                const C ge = counts(k, e) ? gf[k][e] : C(0);
+                if constexpr (LOG) sk += ge;
+                else sk = fma(yf[k][e], ge, sk);
             }
             s[0] += own[k] ? sk : C(0);
         }
@@ -248,7 +246,7 @@ __global__ void __launch_bounds__(BLOCK) softmax_bwd_kernel(const SoftmaxBwdArgs
                 else d = yf[k][e] * (gf[k][e] - s[0]);
                 dxf[e] = d * sign;
             }
-            store_row_as<T, ALIGNED>(dxrow, voff[k], a.n_cols, dxf);
+            store_slot_as<T, ALIGNED>(dxrow, voff[k], a.n_cols, dxf);
         }
 
 #pragma unroll

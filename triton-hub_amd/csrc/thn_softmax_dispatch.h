@@ -35,7 +35,8 @@ THN_DECLARE_SOFTMAX_LAUNCHERS(f64)
                       : run_kernel<ARGS_T>(KERNEL<TYPE, false, B>, a, grid, B, st, nullptr);                    \
     }
 
-// Both directions use the forward shape list of the norm kernels (no per-column accumulators to hold).
+// Both directions use the forward shape list of the norm kernels (no per-column accumulators to hold), on and off the
+// 128-bit path (off it the slots are unaligned 16-byte windows; rows shorter than one vector have one instance).
 #define THN_DEFINE_SOFTMAX_LAUNCHERS(NAME, TYPE)                                                                \
     int launch_softmax_fwd_##NAME(bool is_log, bool aligned, Shape s, const SoftmaxFwdArgs& a, int grid,        \
                                   hipStream_t st, int* occupancy) {                                             \
@@ -44,7 +45,8 @@ THN_DECLARE_SOFTMAX_LAUNCHERS(f64)
             THN_FWD_SHAPES(THN_SMF_AL)                                                                          \
             THN_FWD_SHAPES_THREE(THN_SMF_AL)                                                                    \
         } else if (a.n_cols >= TYPE::VEC) { \
-            THN_SCALAR_SHAPES(THN_SMF_SC) \
+            THN_FWD_SHAPES(THN_SMF_SC) \
+            THN_FWD_SHAPES_THREE(THN_SMF_SC) \
         } else { \
             using T = ElemIo<TYPE>; \
             THN_SMF_SC(4, 8, 256) \
@@ -58,7 +60,8 @@ THN_DECLARE_SOFTMAX_LAUNCHERS(f64)
             THN_FWD_SHAPES(THN_SMB_AL)                                                                          \
             THN_FWD_SHAPES_THREE(THN_SMB_AL)                                                                    \
         } else if (a.n_cols >= TYPE::VEC) { \
-            THN_SCALAR_SHAPES(THN_SMB_SC) \
+            THN_FWD_SHAPES(THN_SMB_SC) \
+            THN_FWD_SHAPES_THREE(THN_SMB_SC) \
         } else { \
             using T = ElemIo<TYPE>; \
             THN_SMB_SC(4, 8, 256) \
