@@ -38,6 +38,27 @@ def test_every_row_width_and_p(dtype):
                 compare_normalize(x, gy, p, 1e-6, f"flat normalize L={n_vecs} M={m} p={p}")
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32, torch.float16])
+def test_row_widths_off_the_128_bit_path(dtype):
+    """Rows that are not a whole number of vectors: the flat kernels' unaligned-window instances (the last window
+    overlaps its neighbour; its leading columns count once in the row sum)."""
+    vec = 16 // torch.empty(0, dtype=dtype).element_size()
+    for n_vecs in FLAT_WIDTHS:
+        rows_per_block = 4 * (64 // n_vecs) * 2
+        for n in sorted({(n_vecs - 1) * vec + 1, n_vecs * vec - 1}):
+            if n < vec:
+                continue
+            for m in sorted({1, rows_per_block - 1, 3 * rows_per_block + 5}):
+                for which in (4, 5, 6):
+                    q = query_launch(which, False, m, n, dtype)
+                    assert q[:3] == (2, n_vecs, 256) and q[4] == 0, (which, q)
+                for p in (1, 2, 3):
+                    announce(f"{dtype} L={n_vecs} ragged K={n} rows={m} p={p}")
+                    x, gn, gy = make((1, m, n), dtype, seed=n_vecs * 100 + p + n)
+                    compare_norm(x, gn, p, 1e-6, f"flat ragged norm K={n} M={m} p={p}")
+                    compare_normalize(x, gy, p, 1e-6, f"flat ragged normalize K={n} M={m} p={p}")
+
+
 def test_override_keeps_the_row_kernels_reachable():
     lib = _native.lib()
     try:

@@ -53,6 +53,36 @@ def test_every_flat_width_against_the_oracle(kind, dtype):
                     sm.run_and_compare(kind, x, dy, f"flat L={n_vecs} J={rows_each} M={m}")
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32, torch.float16])
+@pytest.mark.parametrize("kind", ["softmax", "softmin", "logsoftmax"])
+def test_flat_widths_off_the_128_bit_path(kind, dtype):
+    """Rows that are not a whole number of vectors (one column more than n_vecs - 1 vectors, one less than n_vecs): the
+    flat kernels' unaligned-window instances, the last window overlapping its neighbour; and whole vectors behind a
+    base pointer that is one element off 16 bytes."""
+    from TritonHub.Normalization import _launch
+    vec = 16 // torch.empty(0, dtype=dtype).element_size()
+    for n_vecs in FLAT_WIDTHS:
+        rows_per_block = 4 * (64 // n_vecs) * 2
+        for n in sorted({(n_vecs - 1) * vec + 1, n_vecs * vec - 1}):
+            if n < vec:
+                continue
+            for m in sorted({1, rows_per_block - 1, 3 * rows_per_block + 5, 1000 + n_vecs}):
+                announce(f"{kind} {dtype} L={n_vecs} ragged N={n} M={m}")
+                for which in (2, 3):
+                    q = _launch.query_launch(which, False, m, n, dtype)
+                    assert q[:3] == (2, n_vecs, 256) and q[4] == 0, q
+                x, dy = sm.make((m, n), dtype, 100 * n_vecs + n, scale=3.0)
+                sm.run_and_compare(kind, x, dy, f"flat ragged L={n_vecs} N={n} M={m}")
+        n, m = n_vecs * vec, 3 * rows_per_block + 5
+        announce(f"{kind} {dtype} L={n_vecs} N={n} M={m} behind a misaligned pointer")
+        x, dy = sm.make((m, n), dtype, 7 * n_vecs, scale=3.0)
+        buf = torch.empty(m * n + 1, dtype=dtype, device="cuda")
+        xg = buf[1:].view(m, n)
+        xg.copy_(x)
+        assert xg.data_ptr() % 16 != 0
+        sm.run_and_compare(kind, x, dy, f"flat misaligned L={n_vecs} M={m}", x_gpu=xg)
+
+
 def test_default_choice_masked_logits_strided_rows_and_determinism():
     from TritonHub.Normalization import _launch
     g = torch.Generator().manual_seed(11)

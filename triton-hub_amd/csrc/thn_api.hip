@@ -892,20 +892,20 @@ struct OneSumFlatPlan {
     int rows_each, log_steps, grid, n_vecs;
 };
 
-int launch_softmax_flat_fwd(int dtype, bool is_log, const OneSumFlatPlan& p, const SoftmaxFwdArgs& a, hipStream_t st) {
+int launch_softmax_flat_fwd(int dtype, bool is_log, bool aligned, const OneSumFlatPlan& p, const SoftmaxFwdArgs& a, hipStream_t st) {
     switch (dtype) {
-        case THN_F32: return thn::launch_softmax_flat_fwd_f32(is_log, p.rows_each, p.log_steps, a, p.grid, st);
-        case THN_F16: return thn::launch_softmax_flat_fwd_f16(is_log, p.rows_each, p.log_steps, a, p.grid, st);
-        case THN_BF16: return thn::launch_softmax_flat_fwd_bf16(is_log, p.rows_each, p.log_steps, a, p.grid, st);
+        case THN_F32: return thn::launch_softmax_flat_fwd_f32(is_log, aligned, p.rows_each, p.log_steps, a, p.grid, st);
+        case THN_F16: return thn::launch_softmax_flat_fwd_f16(is_log, aligned, p.rows_each, p.log_steps, a, p.grid, st);
+        case THN_BF16: return thn::launch_softmax_flat_fwd_bf16(is_log, aligned, p.rows_each, p.log_steps, a, p.grid, st);
         default: return 1;
     }
 }
 
-int launch_softmax_flat_bwd(int dtype, bool is_log, const OneSumFlatPlan& p, const SoftmaxBwdArgs& a, hipStream_t st) {
+int launch_softmax_flat_bwd(int dtype, bool is_log, bool aligned, const OneSumFlatPlan& p, const SoftmaxBwdArgs& a, hipStream_t st) {
     switch (dtype) {
-        case THN_F32: return thn::launch_softmax_flat_bwd_f32(is_log, p.rows_each, p.log_steps, a, p.grid, st);
-        case THN_F16: return thn::launch_softmax_flat_bwd_f16(is_log, p.rows_each, p.log_steps, a, p.grid, st);
-        case THN_BF16: return thn::launch_softmax_flat_bwd_bf16(is_log, p.rows_each, p.log_steps, a, p.grid, st);
+        case THN_F32: return thn::launch_softmax_flat_bwd_f32(is_log, aligned, p.rows_each, p.log_steps, a, p.grid, st);
+        case THN_F16: return thn::launch_softmax_flat_bwd_f16(is_log, aligned, p.rows_each, p.log_steps, a, p.grid, st);
+        case THN_BF16: return thn::launch_softmax_flat_bwd_bf16(is_log, aligned, p.rows_each, p.log_steps, a, p.grid, st);
         default: return 1;
     }
 }
@@ -920,10 +920,11 @@ int launch_softmax_flat_bwd(int dtype, bool is_log, const OneSumFlatPlan& p, con
 // vecs_per_thread = rows per lane and step (2; the softmax kernels 4 as well), and keeps them off with any other shape.
 bool plan_one_sum_flat(int which, bool aligned, int64_t M, int64_t N, int dtype, OneSumFlatPlan* out) {
     const int bytes = elem_bytes(dtype);
-    if (!aligned || (bytes != 2 && bytes != 4) || M <= 0) return false;
+    if ((bytes != 2 && bytes != 4) || M <= 0) return false;
     const int vec_elems = 16 / bytes;
-    if (N % vec_elems != 0) return false;
-    const int n_vecs = static_cast<int>(N / vec_elems);
+    // off the 128-bit path: rows of at least one vector (unaligned 16-byte windows, the last one overlapping)
+    if (aligned ? N % vec_elems != 0 : N < vec_elems) return false;
+    const int n_vecs = static_cast<int>((N + vec_elems - 1) / vec_elems);
     if (n_vecs > thn::kFlatMaxVecs || ((n_vecs & (n_vecs - 1)) == 0 && n_vecs > 4)) return false;
     const Override& ov = g_override[which];
     // two rows per lane and step, two workgroups per compute unit: best or within a point of it over 2, 4 x 1, 2, 4 at 17
@@ -935,7 +936,7 @@ bool plan_one_sum_flat(int which, bool aligned, int64_t M, int64_t N, int dtype,
         if (ov.tpr.load() != n_vecs) return false;                                // a row-kernel shape is forced
         if (ov.block.load() > 0 && ov.block.load() != thn::kFlatBlock) return false;
         if (ov.k.load() > 0) rows_each = ov.k.load();
-        if (rows_each != 2 && (rows_each != 4 || which >= kPnormFwd)) return false;
+        if (rows_each != 2 && (rows_each != 4 || which >= kPnormFwd || !aligned)) return false;
     }
     const int cus = current_cu_count();
     if (cus <= 0) return false;
@@ -951,27 +952,27 @@ bool plan_one_sum_flat(int which, bool aligned, int64_t M, int64_t N, int dtype,
 
 // The p-norm / normalize family over the same narrow rows (thn_pnorm_flat.h): the plan is plan_one_sum_flat's (two rows
 // per lane and step only); for tensors whose rows are one folded batch and integer p from 1 to 6.
-int launch_pnorm_flat_fwd(int dtype, int mode, bool normalize, const OneSumFlatPlan& p, const thn::PnormFwdArgs& a, hipStream_t st) {
+int launch_pnorm_flat_fwd(int dtype, int mode, bool normalize, bool aligned, const OneSumFlatPlan& p, const thn::PnormFwdArgs& a, hipStream_t st) {
     switch (dtype) {
-        case THN_F32: return thn::launch_pnorm_flat_fwd_f32(mode, normalize, p.log_steps, a, p.grid, st);
-        case THN_F16: return thn::launch_pnorm_flat_fwd_f16(mode, normalize, p.log_steps, a, p.grid, st);
-        case THN_BF16: return thn::launch_pnorm_flat_fwd_bf16(mode, normalize, p.log_steps, a, p.grid, st);
+        case THN_F32: return thn::launch_pnorm_flat_fwd_f32(mode, normalize, aligned, p.log_steps, a, p.grid, st);
+        case THN_F16: return thn::launch_pnorm_flat_fwd_f16(mode, normalize, aligned, p.log_steps, a, p.grid, st);
+        case THN_BF16: return thn::launch_pnorm_flat_fwd_bf16(mode, normalize, aligned, p.log_steps, a, p.grid, st);
         default: return 1;
     }
 }
-int launch_pnorm_flat_bwd(int dtype, int mode, const OneSumFlatPlan& p, const thn::PnormBwdArgs& a, hipStream_t st) {
+int launch_pnorm_flat_bwd(int dtype, int mode, bool aligned, const OneSumFlatPlan& p, const thn::PnormBwdArgs& a, hipStream_t st) {
     switch (dtype) {
-        case THN_F32: return thn::launch_pnorm_flat_bwd_f32(mode, a, p.grid, st);
-        case THN_F16: return thn::launch_pnorm_flat_bwd_f16(mode, a, p.grid, st);
-        case THN_BF16: return thn::launch_pnorm_flat_bwd_bf16(mode, a, p.grid, st);
+        case THN_F32: return thn::launch_pnorm_flat_bwd_f32(mode, aligned, a, p.grid, st);
+        case THN_F16: return thn::launch_pnorm_flat_bwd_f16(mode, aligned, a, p.grid, st);
+        case THN_BF16: return thn::launch_pnorm_flat_bwd_bf16(mode, aligned, a, p.grid, st);
         default: return 1;
     }
 }
-int launch_normalize_flat_bwd(int dtype, int mode, const OneSumFlatPlan& p, const thn::NormalizeBwdArgs& a, hipStream_t st) {
+int launch_normalize_flat_bwd(int dtype, int mode, bool aligned, const OneSumFlatPlan& p, const thn::NormalizeBwdArgs& a, hipStream_t st) {
     switch (dtype) {
-        case THN_F32: return thn::launch_normalize_flat_bwd_f32(mode, p.log_steps, a, p.grid, st);
-        case THN_F16: return thn::launch_normalize_flat_bwd_f16(mode, p.log_steps, a, p.grid, st);
-        case THN_BF16: return thn::launch_normalize_flat_bwd_bf16(mode, p.log_steps, a, p.grid, st);
+        case THN_F32: return thn::launch_normalize_flat_bwd_f32(mode, aligned, p.log_steps, a, p.grid, st);
+        case THN_F16: return thn::launch_normalize_flat_bwd_f16(mode, aligned, p.log_steps, a, p.grid, st);
+        case THN_BF16: return thn::launch_normalize_flat_bwd_bf16(mode, aligned, p.log_steps, a, p.grid, st);
         default: return 1;
     }
 }
@@ -1320,7 +1321,7 @@ int pnorm_forward(const void* x, int64_t x_batch_stride, int64_t x_row_stride, v
     OneSumFlatPlan fp;
     if (rp.engine && uniform && plan_one_sum_flat(kPnormFwd, aligned, rp.rows, K, dtype, &fp)) {
         a.n_vecs = fp.n_vecs;
-        lrc = launch_pnorm_flat_fwd(dtype, mode_of(rp.p_int), normalize, fp, a, st);
+        lrc = launch_pnorm_flat_fwd(dtype, mode_of(rp.p_int), normalize, aligned, fp, a, st);
     } else if (rp.engine) {
         const int variant = mode_of(rp.p_int) | (normalize ? 4 : 0);
         Plan plan;
@@ -1512,7 +1513,7 @@ int thn_norm_query_launch(int which, int is_layernorm, int64_t M, int64_t N, int
         shape[1] = sfp.n_vecs;
         shape[2] = thn::kFlatBlock;
         shape[3] = sfp.grid;
-        shape[4] = 1;
+        shape[4] = aligned ? 1 : 0;
         return THN_OK;
     }
     StagedPlan sp;
@@ -1764,7 +1765,7 @@ int thn_softmax_fwd(const void* x, int64_t x_row_stride, void* y, int64_t y_row_
         a.n_cols = static_cast<int>(N);
         a.n_vecs = fp.n_vecs;
         a.sign = kind == THN_SOFTMIN ? -1.0f : 1.0f;
-        const int lrc = launch_softmax_flat_fwd(dtype, is_log, fp, a, static_cast<hipStream_t>(stream));
+        const int lrc = launch_softmax_flat_fwd(dtype, is_log, aligned, fp, a, static_cast<hipStream_t>(stream));
         if (lrc > 0) return THN_E_SHAPE;
         return lrc == 0 ? THN_OK : THN_E_LAUNCH;
     }
@@ -1838,7 +1839,7 @@ int thn_softmax_bwd(const void* y, int64_t y_row_stride, const void* dy, int64_t
         a.n_cols = static_cast<int>(N);
         a.n_vecs = fp.n_vecs;
         a.sign = kind == THN_SOFTMIN ? -1.0f : 1.0f;
-        const int lrc = launch_softmax_flat_bwd(dtype, is_log, fp, a, static_cast<hipStream_t>(stream));
+        const int lrc = launch_softmax_flat_bwd(dtype, is_log, aligned, fp, a, static_cast<hipStream_t>(stream));
         if (lrc > 0) return THN_E_SHAPE;
         return lrc == 0 ? THN_OK : THN_E_LAUNCH;
     }
@@ -1907,7 +1908,7 @@ int thn_pnorm_bwd(const void* x, int64_t x_batch_stride, int64_t x_row_stride, c
     OneSumFlatPlan fp;
     if (rp.engine && uniform && plan_one_sum_flat(kPnormBwd, aligned, rp.rows, K, dtype, &fp)) {
         a.n_vecs = fp.n_vecs;
-        lrc = launch_pnorm_flat_bwd(dtype, mode_of(rp.p_int), fp, a, st);
+        lrc = launch_pnorm_flat_bwd(dtype, mode_of(rp.p_int), aligned, fp, a, st);
     } else if (rp.engine) {
         const int mode = mode_of(rp.p_int);
         Plan plan;
@@ -1975,7 +1976,7 @@ int thn_normalize_bwd(const void* x, int64_t x_batch_stride, int64_t x_row_strid
     OneSumFlatPlan fp;
     if (rp.engine && uniform && plan_one_sum_flat(kNormalizeBwd, aligned, rp.rows, K, dtype, &fp)) {
         a.n_vecs = fp.n_vecs;
-        lrc = launch_normalize_flat_bwd(dtype, mode_of(rp.p_int), fp, a, st);
+        lrc = launch_normalize_flat_bwd(dtype, mode_of(rp.p_int), aligned, fp, a, st);
     } else if (rp.engine) {
         const int mode = mode_of(rp.p_int);
         Plan plan;

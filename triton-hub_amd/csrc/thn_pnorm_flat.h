@@ -4,8 +4,8 @@
 // sum, or the projection of the gradient).  The row kernels of thn_pnorm.h give a row 8, 16 or 32 lanes: rows of 1, 2
 // and 4 vectors -- normalising 4-, 8- or 16-component float32 vectors -- leave 7/8, 3/4 and half of their lanes idle.
 // Arithmetic as pnorm_fwd_kernel / pnorm_bwd_kernel / normalize_bwd_kernel.  For tensors whose rows are one folded
-// batch (row r at r * row stride), float32 / float16 / bfloat16 on the 128-bit path, integer p from 1 to 6; two rows
-// per lane and step.
+// batch (row r at r * row stride), float32 / float16 / bfloat16, integer p from 1 to 6; two rows per lane and step.
+// ALIGNED = false: rows of at least one vector off the 128-bit path (unaligned 16-byte windows, see thn_softmax_flat.h).
 #pragma once
 
 #include "thn_pnorm.h"
@@ -15,7 +15,7 @@ namespace thn {
 
 constexpr int kRowsFlatJ = 2;     // rows per lane and step of these kernels
 
-template <typename T, int MODE, bool NORMALIZE, int LOG>
+template <typename T, int MODE, bool NORMALIZE, int LOG, bool ALIGNED>
 __global__ void __launch_bounds__(kFlatBlock) pnorm_flat_fwd_kernel(const PnormFwdArgs a) {
     constexpr int VEC = T::VEC;
     constexpr int W = kFlatBlock / 64;
@@ -26,7 +26,8 @@ __global__ void __launch_bounds__(kFlatBlock) pnorm_flat_fwd_kernel(const PnormF
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int rpw = 64 / L;
     const FlatLane f = flat_lane(lane, L);
-    const int voff = f.t * 16;
+    int voff, lead;
+    flat_slot<T, ALIGNED>(f.t, L, a.n_cols, voff, lead);
 
     const int64_t rows_per_block = static_cast<int64_t>(W) * rpw * J;
     const int64_t rows_per_iter = static_cast<int64_t>(gridDim.x) * rows_per_block;
@@ -37,8 +38,7 @@ __global__ void __launch_bounds__(kFlatBlock) pnorm_flat_fwd_kernel(const PnormF
     for (int j = 0; j < J; ++j) {
         row_raw[j] = static_cast<int64_t>(blockIdx.x) * rows_per_block + static_cast<int64_t>(j * W + wave) * rpw + f.r;
         row[j] = row_raw[j] < a.rows ? row_raw[j] : last_row;
-        const char* p = a.x + row[j] * a.xmap.row_stride_bytes + voff;
-        cur[j] = kKeepX ? ld128_keep(p) : ld128(p);
+        cur[j] = slot_load<T, ALIGNED, kKeepX>(a.x + row[j] * a.xmap.row_stride_bytes, voff, a.n_cols);
     }
     drain_vector_memory(cur);
 
@@ -49,8 +49,7 @@ __global__ void __launch_bounds__(kFlatBlock) pnorm_flat_fwd_kernel(const PnormF
         for (int j = 0; j < J; ++j) {
             nrow_raw[j] = row_raw[j] + rows_per_iter;
             nrow[j] = nrow_raw[j] < a.rows ? nrow_raw[j] : last_row;
-            const char* p = a.x + nrow[j] * a.xmap.row_stride_bytes + voff;
-            nxt[j] = kKeepX ? ld128_keep(p) : ld128(p);
+            nxt[j] = slot_load<T, ALIGNED, kKeepX>(a.x + nrow[j] * a.xmap.row_stride_bytes, voff, a.n_cols);
         }
         float xf[J][VEC];
         float s[J];
@@ -59,7 +58,10 @@ __global__ void __launch_bounds__(kFlatBlock) pnorm_flat_fwd_kernel(const PnormF
             T::unpack(cur[j], xf[j]);
             float sk = 0.0f;
 #pragma unroll
-            for (int e = 0; e < VEC; ++e) sk += norm_term<MODE>(xf[j][e], a.p_int);
+            for (int e = 0; e < VEC; ++e) {      // an overlapping window's leading columns count in the slot before
+                const float term = norm_term<MODE>(xf[j][e], a.p_int);
+                sk += e >= lead ? term : 0.0f;
+            }
             s[j] = f.own ? sk : 0.0f;
         }
         segment_allreduce_op<LOG, J, OpSum>(s, lane, f.pos, L, f.first);
@@ -74,9 +76,7 @@ __global__ void __launch_bounds__(kFlatBlock) pnorm_flat_fwd_kernel(const PnormF
                 float yf[VEC];
 #pragma unroll
                 for (int e = 0; e < VEC; ++e) yf[e] = div_by_row(xf[j][e], nd, rn);
-                char* p = a.y + row[j] * a.ymap.row_stride_bytes + voff;
-                if constexpr (kKeepY) st128_keep(p, T::pack(yf));
-                else st128(p, T::pack(yf));
+                slot_store<T, ALIGNED, kKeepY>(a.y + row[j] * a.ymap.row_stride_bytes, voff, a.n_cols, yf);
             }
         }
 #pragma unroll
@@ -89,7 +89,7 @@ __global__ void __launch_bounds__(kFlatBlock) pnorm_flat_fwd_kernel(const PnormF
 }
 
 // Norm backward: element-wise with two per-row scalars, no row sum.
-template <typename T, int MODE>
+template <typename T, int MODE, bool ALIGNED>
 __global__ void __launch_bounds__(kFlatBlock) pnorm_flat_bwd_kernel(const PnormBwdArgs a) {
     constexpr int VEC = T::VEC;
     constexpr int W = kFlatBlock / 64;
@@ -98,7 +98,8 @@ __global__ void __launch_bounds__(kFlatBlock) pnorm_flat_bwd_kernel(const PnormB
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int rpw = 64 / L;
     const FlatLane f = flat_lane(lane, L);
-    const int voff = f.t * 16;
+    int voff, lead;
+    flat_slot<T, ALIGNED>(f.t, L, a.n_cols, voff, lead);
 
     const int64_t rows_per_block = static_cast<int64_t>(W) * rpw * J;
     const int64_t rows_per_iter = static_cast<int64_t>(gridDim.x) * rows_per_block;
@@ -110,7 +111,7 @@ __global__ void __launch_bounds__(kFlatBlock) pnorm_flat_bwd_kernel(const PnormB
     for (int j = 0; j < J; ++j) {
         row_raw[j] = static_cast<int64_t>(blockIdx.x) * rows_per_block + static_cast<int64_t>(j * W + wave) * rpw + f.r;
         row[j] = row_raw[j] < a.rows ? row_raw[j] : last_row;
-        cur[j] = ld128(a.x + row[j] * a.xmap.row_stride_bytes + voff);
+        cur[j] = slot_load<T, ALIGNED>(a.x + row[j] * a.xmap.row_stride_bytes, voff, a.n_cols);
         c_n[j] = MODE == kP1 ? 1.0f : T::load1(a.norms, row[j]);
         c_g[j] = T::load1(a.g, row[j]);
     }
@@ -129,7 +130,7 @@ __global__ void __launch_bounds__(kFlatBlock) pnorm_flat_bwd_kernel(const PnormB
         for (int j = 0; j < J; ++j) {
             nrow_raw[j] = row_raw[j] + rows_per_iter;
             nrow[j] = nrow_raw[j] < a.rows ? nrow_raw[j] : last_row;
-            nxt[j] = ld128(a.x + nrow[j] * a.xmap.row_stride_bytes + voff);
+            nxt[j] = slot_load<T, ALIGNED>(a.x + nrow[j] * a.xmap.row_stride_bytes, voff, a.n_cols);
             raw_n[j] = MODE == kP1 ? 0 : RowScalar<T>::load(a.norms, nrow[j]);
             raw_g[j] = RowScalar<T>::load(a.g, nrow[j]);
         }
@@ -148,7 +149,7 @@ __global__ void __launch_bounds__(kFlatBlock) pnorm_flat_bwd_kernel(const PnormB
                 else if constexpr (MODE == kP2) df[e] = div_by_row(c_g[j] * x, den, rden);
                 else df[e] = div_by_row(c_g[j] * sign_of(x) * pow_small(__builtin_fabsf(x), a.p_int - 1), den, rden);
             }
-            st128(a.dx + row[j] * a.dxmap.row_stride_bytes + voff, T::pack(df));
+            slot_store<T, ALIGNED>(a.dx + row[j] * a.dxmap.row_stride_bytes, voff, a.n_cols, df);
         }
 #pragma unroll
         for (int j = 0; j < J; ++j) {
@@ -166,7 +167,7 @@ __global__ void __launch_bounds__(kFlatBlock) pnorm_flat_bwd_kernel(const PnormB
 }
 
 // Normalize backward: one segmented row sum (the projection of the gradient on x or y).
-template <typename T, int MODE, int LOG>
+template <typename T, int MODE, int LOG, bool ALIGNED>
 __global__ void __launch_bounds__(kFlatBlock) normalize_flat_bwd_kernel(const NormalizeBwdArgs a) {
     constexpr int VEC = T::VEC;
     constexpr int W = kFlatBlock / 64;
@@ -177,7 +178,8 @@ __global__ void __launch_bounds__(kFlatBlock) normalize_flat_bwd_kernel(const No
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int rpw = 64 / L;
     const FlatLane f = flat_lane(lane, L);
-    const int voff = f.t * 16;
+    int voff, lead;
+    flat_slot<T, ALIGNED>(f.t, L, a.n_cols, voff, lead);
 
     const int64_t rows_per_block = static_cast<int64_t>(W) * rpw * J;
     const int64_t rows_per_iter = static_cast<int64_t>(gridDim.x) * rows_per_block;
@@ -189,9 +191,9 @@ __global__ void __launch_bounds__(kFlatBlock) normalize_flat_bwd_kernel(const No
     for (int j = 0; j < J; ++j) {
         row_raw[j] = static_cast<int64_t>(blockIdx.x) * rows_per_block + static_cast<int64_t>(j * W + wave) * rpw + f.r;
         row[j] = row_raw[j] < a.rows ? row_raw[j] : last_row;
-        if constexpr (NEED_X) cx[j] = ld128(a.x + row[j] * a.xmap.row_stride_bytes + voff);
-        if constexpr (NEED_Y) cy[j] = ld128(a.y + row[j] * a.ymap.row_stride_bytes + voff);
-        cg[j] = ld128(a.g + row[j] * a.gmap.row_stride_bytes + voff);
+        if constexpr (NEED_X) cx[j] = slot_load<T, ALIGNED>(a.x + row[j] * a.xmap.row_stride_bytes, voff, a.n_cols);
+        if constexpr (NEED_Y) cy[j] = slot_load<T, ALIGNED>(a.y + row[j] * a.ymap.row_stride_bytes, voff, a.n_cols);
+        cg[j] = slot_load<T, ALIGNED>(a.g + row[j] * a.gmap.row_stride_bytes, voff, a.n_cols);
         c_n[j] = T::load1(a.norms, row[j]);
     }
 #pragma unroll
@@ -208,9 +210,9 @@ __global__ void __launch_bounds__(kFlatBlock) normalize_flat_bwd_kernel(const No
         for (int j = 0; j < J; ++j) {
             nrow_raw[j] = row_raw[j] + rows_per_iter;
             nrow[j] = nrow_raw[j] < a.rows ? nrow_raw[j] : last_row;
-            if constexpr (NEED_X) nx[j] = ld128(a.x + nrow[j] * a.xmap.row_stride_bytes + voff);
-            if constexpr (NEED_Y) ny[j] = ld128(a.y + nrow[j] * a.ymap.row_stride_bytes + voff);
-            ng[j] = ld128(a.g + nrow[j] * a.gmap.row_stride_bytes + voff);
+            if constexpr (NEED_X) nx[j] = slot_load<T, ALIGNED>(a.x + nrow[j] * a.xmap.row_stride_bytes, voff, a.n_cols);
+            if constexpr (NEED_Y) ny[j] = slot_load<T, ALIGNED>(a.y + nrow[j] * a.ymap.row_stride_bytes, voff, a.n_cols);
+            ng[j] = slot_load<T, ALIGNED>(a.g + nrow[j] * a.gmap.row_stride_bytes, voff, a.n_cols);
             raw_n[j] = RowScalar<T>::load(a.norms, nrow[j]);
         }
         float xf[NEED_X ? J : 1][VEC], yf[NEED_Y ? J : 1][VEC], gf[J][VEC];
@@ -223,8 +225,9 @@ __global__ void __launch_bounds__(kFlatBlock) normalize_flat_bwd_kernel(const No
             float sk = 0.0f;
 #pragma unroll
             for (int e = 0; e < VEC; ++e) {
-                if constexpr (MODE == kP1) sk = __builtin_fmaf(xf[j][e], gf[j][e], sk);
-                else sk = __builtin_fmaf(yf[j][e], gf[j][e], sk);
+                const float ge = e >= lead ? gf[j][e] : 0.0f;
+                if constexpr (MODE == kP1) sk = __builtin_fmaf(xf[j][e], ge, sk);
+                else sk = __builtin_fmaf(yf[j][e], ge, sk);
             }
             s[j] = f.own ? sk : 0.0f;
         }
@@ -251,7 +254,7 @@ __global__ void __launch_bounds__(kFlatBlock) normalize_flat_bwd_kernel(const No
                     df[e] = div_by_row(gg, nd, rn) - sign_of(x) * pow_small(__builtin_fabsf(x), a.p_int - 1) * coef;
                 }
             }
-            st128(a.dx + row[j] * a.dxmap.row_stride_bytes + voff, T::pack(df));
+            slot_store<T, ALIGNED>(a.dx + row[j] * a.dxmap.row_stride_bytes, voff, a.n_cols, df);
         }
 #pragma unroll
         for (int j = 0; j < J; ++j) {
@@ -269,46 +272,64 @@ __global__ void __launch_bounds__(kFlatBlock) normalize_flat_bwd_kernel(const No
 // Launchers: 0 launched, 1 no such instance, <0 HIP error.  `mode`: kP1 / kP2 / kPInt; `log_steps` as in
 // thn_softmax_flat.h.
 #define THN_DECLARE_PNORM_FLAT_LAUNCHERS(NAME)                                                                  \
-    int launch_pnorm_flat_fwd_##NAME(int mode, bool normalize, int log_steps, const PnormFwdArgs& a, int grid,  \
-                                     hipStream_t st);                                                           \
-    int launch_pnorm_flat_bwd_##NAME(int mode, const PnormBwdArgs& a, int grid, hipStream_t st);                \
-    int launch_normalize_flat_bwd_##NAME(int mode, int log_steps, const NormalizeBwdArgs& a, int grid, hipStream_t st);
+    int launch_pnorm_flat_fwd_##NAME(int mode, bool normalize, bool aligned, int log_steps, const PnormFwdArgs& a, \
+                                     int grid, hipStream_t st);                                                 \
+    int launch_pnorm_flat_bwd_##NAME(int mode, bool aligned, const PnormBwdArgs& a, int grid, hipStream_t st);  \
+    int launch_normalize_flat_bwd_##NAME(int mode, bool aligned, int log_steps, const NormalizeBwdArgs& a, int grid, \
+                                         hipStream_t st);
 
 THN_DECLARE_PNORM_FLAT_LAUNCHERS(f32)
 THN_DECLARE_PNORM_FLAT_LAUNCHERS(f16)
 THN_DECLARE_PNORM_FLAT_LAUNCHERS(bf16)
 
-#define THN_PNORM_FLAT_FWD_CASE(MODE_, LOG_)                                                                    \
+#define THN_PNORM_FLAT_FWD_CASE(AL, MODE_, LOG_)                                                                \
     if (mode == MODE_ && log_steps == LOG_) {                                                                   \
-        return normalize ? run_kernel<PnormFwdArgs>(pnorm_flat_fwd_kernel<T, MODE_, true, LOG_>, a, grid, kFlatBlock, st, nullptr)  \
-                         : run_kernel<PnormFwdArgs>(pnorm_flat_fwd_kernel<T, MODE_, false, LOG_>, a, grid, kFlatBlock, st, nullptr); \
+        return normalize ? run_kernel<PnormFwdArgs>(pnorm_flat_fwd_kernel<T, MODE_, true, LOG_, AL>, a, grid, kFlatBlock, st, nullptr)  \
+                         : run_kernel<PnormFwdArgs>(pnorm_flat_fwd_kernel<T, MODE_, false, LOG_, AL>, a, grid, kFlatBlock, st, nullptr); \
     }
-#define THN_NORMALIZE_FLAT_BWD_CASE(MODE_, LOG_)                                                                \
+#define THN_NORMALIZE_FLAT_BWD_CASE(AL, MODE_, LOG_)                                                            \
     if (mode == MODE_ && log_steps == LOG_) {                                                                   \
-        return run_kernel<NormalizeBwdArgs>(normalize_flat_bwd_kernel<T, MODE_, LOG_>, a, grid, kFlatBlock, st, nullptr); \
+        return run_kernel<NormalizeBwdArgs>(normalize_flat_bwd_kernel<T, MODE_, LOG_, AL>, a, grid, kFlatBlock, st, nullptr); \
     }
-#define THN_PNORM_FLAT_BWD_CASE(MODE_)                                                                          \
-    if (mode == MODE_) return run_kernel<PnormBwdArgs>(pnorm_flat_bwd_kernel<T, MODE_>, a, grid, kFlatBlock, st, nullptr);
+#define THN_PNORM_FLAT_BWD_CASE(AL, MODE_)                                                                      \
+    if (mode == MODE_) return run_kernel<PnormBwdArgs>(pnorm_flat_bwd_kernel<T, MODE_, AL>, a, grid, kFlatBlock, st, nullptr);
+#define THN_PNF_FLAT_AL(MODE_, LOG_) THN_PNORM_FLAT_FWD_CASE(true, MODE_, LOG_)
+#define THN_PNF_FLAT_SC(MODE_, LOG_) THN_PNORM_FLAT_FWD_CASE(false, MODE_, LOG_)
+#define THN_NZB_FLAT_AL(MODE_, LOG_) THN_NORMALIZE_FLAT_BWD_CASE(true, MODE_, LOG_)
+#define THN_NZB_FLAT_SC(MODE_, LOG_) THN_NORMALIZE_FLAT_BWD_CASE(false, MODE_, LOG_)
 // X(MODE, LOG)
 #define THN_PNORM_FLAT_SHAPES(X)                                                                                \
     X(kP1, 0) X(kP1, 2) X(kP1, 4) X(kP1, 5) X(kP2, 0) X(kP2, 2) X(kP2, 4) X(kP2, 5)                             \
     X(kPInt, 0) X(kPInt, 2) X(kPInt, 4) X(kPInt, 5)
 
 #define THN_DEFINE_PNORM_FLAT_LAUNCHERS(NAME, TYPE)                                                             \
-    int launch_pnorm_flat_fwd_##NAME(int mode, bool normalize, int log_steps, const PnormFwdArgs& a, int grid,  \
-                                     hipStream_t st) {                                                          \
+    int launch_pnorm_flat_fwd_##NAME(int mode, bool normalize, bool aligned, int log_steps, const PnormFwdArgs& a, \
+                                     int grid, hipStream_t st) {                                                \
         using T = TYPE;                                                                                         \
-        THN_PNORM_FLAT_SHAPES(THN_PNORM_FLAT_FWD_CASE)                                                          \
+        if (aligned) {                                                                                          \
+            THN_PNORM_FLAT_SHAPES(THN_PNF_FLAT_AL)                                                              \
+        } else {                                                                                                \
+            THN_PNORM_FLAT_SHAPES(THN_PNF_FLAT_SC)                                                              \
+        }                                                                                                       \
         return 1;                                                                                               \
     }                                                                                                           \
-    int launch_pnorm_flat_bwd_##NAME(int mode, const PnormBwdArgs& a, int grid, hipStream_t st) {               \
+    int launch_pnorm_flat_bwd_##NAME(int mode, bool aligned, const PnormBwdArgs& a, int grid, hipStream_t st) { \
         using T = TYPE;                                                                                         \
-        THN_PNORM_FLAT_BWD_CASE(kP1) THN_PNORM_FLAT_BWD_CASE(kP2) THN_PNORM_FLAT_BWD_CASE(kPInt)                \
+        if (aligned) {                                                                                          \
+            THN_PNORM_FLAT_BWD_CASE(true, kP1) THN_PNORM_FLAT_BWD_CASE(true, kP2) THN_PNORM_FLAT_BWD_CASE(true, kPInt) \
+        } else {                                                                                                \
+            THN_PNORM_FLAT_BWD_CASE(false, kP1) THN_PNORM_FLAT_BWD_CASE(false, kP2) THN_PNORM_FLAT_BWD_CASE(false, kPInt) \
+        }                                                                                                       \
         return 1;                                                                                               \
     }                                                                                                           \
-    int launch_normalize_flat_bwd_##NAME(int mode, int log_steps, const NormalizeBwdArgs& a, int grid, hipStream_t st) { \
+    int launch_normalize_flat_bwd_##NAME(int mode, bool aligned, int log_steps, const NormalizeBwdArgs& a, int grid, \
+                                         hipStream_t st) {                                                      \
         using T = TYPE;                                                                                         \
-        THN_PNORM_FLAT_SHAPES(THN_NORMALIZE_FLAT_BWD_CASE)                                                      \
+        if (aligned) {                                                                                          \
+            THN_PNORM_FLAT_SHAPES(THN_NZB_FLAT_AL)                                                              \
+        } else {                                                                                                \
+            THN_PNORM_FLAT_SHAPES(THN_NZB_FLAT_SC)                                                              \
+        }                                                                                                       \
         return 1;                                                                                               \
     }
 

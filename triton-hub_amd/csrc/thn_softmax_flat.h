@@ -4,7 +4,8 @@
 // lanes, so rows of 1, 2 and 4 vectors leave 7/8, 3/4 and half of their lanes idle, and 9 vectors 7 of 16.  A softmax
 // needs ONE value per reduction round (the row maximum, the row sum; the backward one sum), which is what the
 // segmented ds_bpermute reductions are cheapest at.  Arithmetic as softmax_fwd_kernel / softmax_bwd_kernel, in float32;
-// float32 / float16 / bfloat16 rows on the 128-bit path only.
+// float32 / float16 / bfloat16 rows; ALIGNED = false: rows of at least one vector off the 128-bit path, whose slots are
+// unaligned 16-byte windows, the ragged last one overlapping its neighbour (slot_place() in thn_kernels.h).
 #pragma once
 
 #include "thn_flat.h"
@@ -30,7 +31,15 @@ __device__ __forceinline__ void segment_allreduce_op(float (&v)[NV], int lane, i
     for (int i = 0; i < NV; ++i) v[i] = lane_read(v[i], first);
 }
 
-template <typename T, bool LOGSM, int J, int LOG>
+// Byte offset of vector t of a row of L vectors and the number of its leading columns that the slot before it owns
+// (0 on the 128-bit path).
+template <typename T, bool ALIGNED>
+__device__ __forceinline__ void flat_slot(int t, int L, int n_cols, int& voff, int& lead) {
+    bool own;
+    slot_place<T, ALIGNED>(t, L, n_cols, voff, lead, own);
+}
+
+template <typename T, bool LOGSM, int J, int LOG, bool ALIGNED>
 __global__ void __launch_bounds__(kFlatBlock) softmax_flat_fwd_kernel(const SoftmaxFwdArgs a) {
     constexpr int VEC = T::VEC;
     constexpr int W = kFlatBlock / 64;
@@ -38,7 +47,8 @@ __global__ void __launch_bounds__(kFlatBlock) softmax_flat_fwd_kernel(const Soft
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int rpw = 64 / L;
     const FlatLane f = flat_lane(lane, L);
-    const int voff = f.t * 16;
+    int voff, lead;
+    flat_slot<T, ALIGNED>(f.t, L, a.n_cols, voff, lead);
     const float neg_inf = OpMax::identity<float>();
 
     const int64_t rows_per_block = static_cast<int64_t>(W) * rpw * J;
@@ -50,7 +60,7 @@ __global__ void __launch_bounds__(kFlatBlock) softmax_flat_fwd_kernel(const Soft
     for (int j = 0; j < J; ++j) {
         row_raw[j] = static_cast<int64_t>(blockIdx.x) * rows_per_block + static_cast<int64_t>(j * W + wave) * rpw + f.r;
         row[j] = row_raw[j] < a.M ? row_raw[j] : last_row;
-        cur[j] = ld128(a.x + row[j] * a.x_stride_bytes + voff);
+        cur[j] = slot_load<T, ALIGNED>(a.x + row[j] * a.x_stride_bytes, voff, a.n_cols);
     }
     drain_vector_memory(cur);
 
@@ -61,7 +71,7 @@ __global__ void __launch_bounds__(kFlatBlock) softmax_flat_fwd_kernel(const Soft
         for (int j = 0; j < J; ++j) {
             nrow_raw[j] = row_raw[j] + rows_per_iter;
             nrow[j] = nrow_raw[j] < a.M ? nrow_raw[j] : last_row;
-            nxt[j] = ld128(a.x + nrow[j] * a.x_stride_bytes + voff);
+            nxt[j] = slot_load<T, ALIGNED>(a.x + nrow[j] * a.x_stride_bytes, voff, a.n_cols);
         }
         float xf[J][VEC];
         float m[J];
@@ -72,7 +82,7 @@ __global__ void __launch_bounds__(kFlatBlock) softmax_flat_fwd_kernel(const Soft
 #pragma unroll
             for (int e = 0; e < VEC; ++e) {
                 xf[j][e] *= a.sign;
-                mj = fmaxf(mj, xf[j][e]);          // a mirror lane repeats real columns: harmless for a maximum
+                mj = fmaxf(mj, xf[j][e]);          // mirror lanes and overlapping windows repeat real columns: harmless for a maximum
             }
             m[j] = mj;
         }
@@ -86,7 +96,7 @@ __global__ void __launch_bounds__(kFlatBlock) softmax_flat_fwd_kernel(const Soft
                 const float z = xf[j][e] - m[j];
                 const float ez = exp_c(z);
                 xf[j][e] = LOGSM ? z : ez;
-                sk += ez;
+                sk += e >= lead ? ez : 0.0f;          // an overlapping window's leading columns count in the slot before
             }
             s[j] = f.own ? sk : 0.0f;
         }
@@ -97,7 +107,7 @@ __global__ void __launch_bounds__(kFlatBlock) softmax_flat_fwd_kernel(const Soft
             float yf[VEC];
 #pragma unroll
             for (int e = 0; e < VEC; ++e) yf[e] = LOGSM ? xf[j][e] - scale : xf[j][e] * scale;
-            st128_keep(a.y + row[j] * a.y_stride_bytes + voff, T::pack(yf));     // the backward works from the saved y
+            slot_store<T, ALIGNED, true>(a.y + row[j] * a.y_stride_bytes, voff, a.n_cols, yf);   // the backward works from the saved y
         }
 #pragma unroll
         for (int j = 0; j < J; ++j) {
@@ -108,7 +118,7 @@ __global__ void __launch_bounds__(kFlatBlock) softmax_flat_fwd_kernel(const Soft
     }
 }
 
-template <typename T, bool LOGSM, int J, int LOG>
+template <typename T, bool LOGSM, int J, int LOG, bool ALIGNED>
 __global__ void __launch_bounds__(kFlatBlock) softmax_flat_bwd_kernel(const SoftmaxBwdArgs a) {
     constexpr int VEC = T::VEC;
     constexpr int W = kFlatBlock / 64;
@@ -116,7 +126,8 @@ __global__ void __launch_bounds__(kFlatBlock) softmax_flat_bwd_kernel(const Soft
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int rpw = 64 / L;
     const FlatLane f = flat_lane(lane, L);
-    const int voff = f.t * 16;
+    int voff, lead;
+    flat_slot<T, ALIGNED>(f.t, L, a.n_cols, voff, lead);
 
     const int64_t rows_per_block = static_cast<int64_t>(W) * rpw * J;
     const int64_t rows_per_iter = static_cast<int64_t>(gridDim.x) * rows_per_block;
@@ -127,8 +138,8 @@ __global__ void __launch_bounds__(kFlatBlock) softmax_flat_bwd_kernel(const Soft
     for (int j = 0; j < J; ++j) {
         row_raw[j] = static_cast<int64_t>(blockIdx.x) * rows_per_block + static_cast<int64_t>(j * W + wave) * rpw + f.r;
         row[j] = row_raw[j] < a.M ? row_raw[j] : last_row;
-        cy[j] = ld128(a.y + row[j] * a.y_stride_bytes + voff);
-        cg[j] = ld128(a.dy + row[j] * a.dy_stride_bytes + voff);
+        cy[j] = slot_load<T, ALIGNED>(a.y + row[j] * a.y_stride_bytes, voff, a.n_cols);
+        cg[j] = slot_load<T, ALIGNED>(a.dy + row[j] * a.dy_stride_bytes, voff, a.n_cols);
     }
     drain_vector_memory(cy, cg);
 
@@ -139,8 +150,8 @@ __global__ void __launch_bounds__(kFlatBlock) softmax_flat_bwd_kernel(const Soft
         for (int j = 0; j < J; ++j) {
             nrow_raw[j] = row_raw[j] + rows_per_iter;
             nrow[j] = nrow_raw[j] < a.M ? nrow_raw[j] : last_row;
-            ny[j] = ld128(a.y + nrow[j] * a.y_stride_bytes + voff);
-            ng[j] = ld128(a.dy + nrow[j] * a.dy_stride_bytes + voff);
+            ny[j] = slot_load<T, ALIGNED>(a.y + nrow[j] * a.y_stride_bytes, voff, a.n_cols);
+            ng[j] = slot_load<T, ALIGNED>(a.dy + nrow[j] * a.dy_stride_bytes, voff, a.n_cols);
         }
         float yf[J][VEC], gf[J][VEC];
         float s[J];
@@ -151,8 +162,9 @@ __global__ void __launch_bounds__(kFlatBlock) softmax_flat_bwd_kernel(const Soft
             float sk = 0.0f;
 #pragma unroll
             for (int e = 0; e < VEC; ++e) {
-                if constexpr (LOGSM) sk += gf[j][e];
-                else sk = fmaf(yf[j][e], gf[j][e], sk);
+                const float ge = e >= lead ? gf[j][e] : 0.0f;
+                if constexpr (LOGSM) sk += ge;
+                else sk = fmaf(yf[j][e], ge, sk);
             }
             s[j] = f.own ? sk : 0.0f;
         }
@@ -167,7 +179,7 @@ __global__ void __launch_bounds__(kFlatBlock) softmax_flat_bwd_kernel(const Soft
                 else d = yf[j][e] * (gf[j][e] - s[j]);
                 dxf[e] = d * a.sign;
             }
-            st128(a.dx + row[j] * a.dx_stride_bytes + voff, T::pack(dxf));
+            slot_store<T, ALIGNED>(a.dx + row[j] * a.dx_stride_bytes, voff, a.n_cols, dxf);
         }
 #pragma unroll
         for (int j = 0; j < J; ++j) {
@@ -182,36 +194,48 @@ __global__ void __launch_bounds__(kFlatBlock) softmax_flat_bwd_kernel(const Soft
 // Launchers: 0 launched, 1 no such instance, <0 HIP error.  `log_steps`: tree steps of the segmented reductions (0 for
 // rows of one vector, 2 up to 4 vectors, 4 up to 16, 5 up to 32); `rows_each` = J.
 #define THN_DECLARE_SOFTMAX_FLAT_LAUNCHERS(NAME)                                                                \
-    int launch_softmax_flat_fwd_##NAME(bool is_log, int rows_each, int log_steps, const SoftmaxFwdArgs& a, int grid, \
-                                       hipStream_t st);                                                         \
-    int launch_softmax_flat_bwd_##NAME(bool is_log, int rows_each, int log_steps, const SoftmaxBwdArgs& a, int grid, \
-                                       hipStream_t st);
+    int launch_softmax_flat_fwd_##NAME(bool is_log, bool aligned, int rows_each, int log_steps, const SoftmaxFwdArgs& a, \
+                                       int grid, hipStream_t st);                                               \
+    int launch_softmax_flat_bwd_##NAME(bool is_log, bool aligned, int rows_each, int log_steps, const SoftmaxBwdArgs& a, \
+                                       int grid, hipStream_t st);
 
 THN_DECLARE_SOFTMAX_FLAT_LAUNCHERS(f32)
 THN_DECLARE_SOFTMAX_FLAT_LAUNCHERS(f16)
 THN_DECLARE_SOFTMAX_FLAT_LAUNCHERS(bf16)
 
-#define THN_SOFTMAX_FLAT_CASE(KERNEL, ARGS_T, J_, LOG_)                                                         \
+#define THN_SOFTMAX_FLAT_CASE(KERNEL, ARGS_T, AL, J_, LOG_)                                                     \
     if (rows_each == J_ && log_steps == LOG_) {                                                                 \
-        return is_log ? run_kernel<ARGS_T>(KERNEL<T, true, J_, LOG_>, a, grid, kFlatBlock, st, nullptr)          \
-                      : run_kernel<ARGS_T>(KERNEL<T, false, J_, LOG_>, a, grid, kFlatBlock, st, nullptr);        \
+        return is_log ? run_kernel<ARGS_T>(KERNEL<T, true, J_, LOG_, AL>, a, grid, kFlatBlock, st, nullptr)      \
+                      : run_kernel<ARGS_T>(KERNEL<T, false, J_, LOG_, AL>, a, grid, kFlatBlock, st, nullptr);    \
     }
-#define THN_SOFTMAX_FLAT_FWD_CASE(J_, LOG_) THN_SOFTMAX_FLAT_CASE(softmax_flat_fwd_kernel, SoftmaxFwdArgs, J_, LOG_)
-#define THN_SOFTMAX_FLAT_BWD_CASE(J_, LOG_) THN_SOFTMAX_FLAT_CASE(softmax_flat_bwd_kernel, SoftmaxBwdArgs, J_, LOG_)
+#define THN_SOFTMAX_FLAT_FWD_AL(J_, LOG_) THN_SOFTMAX_FLAT_CASE(softmax_flat_fwd_kernel, SoftmaxFwdArgs, true, J_, LOG_)
+#define THN_SOFTMAX_FLAT_BWD_AL(J_, LOG_) THN_SOFTMAX_FLAT_CASE(softmax_flat_bwd_kernel, SoftmaxBwdArgs, true, J_, LOG_)
+#define THN_SOFTMAX_FLAT_FWD_SC(J_, LOG_) THN_SOFTMAX_FLAT_CASE(softmax_flat_fwd_kernel, SoftmaxFwdArgs, false, J_, LOG_)
+#define THN_SOFTMAX_FLAT_BWD_SC(J_, LOG_) THN_SOFTMAX_FLAT_CASE(softmax_flat_bwd_kernel, SoftmaxBwdArgs, false, J_, LOG_)
 // X(J, LOG): rows per lane and step x tree steps
 #define THN_SOFTMAX_FLAT_SHAPES(X) X(2, 0) X(4, 0) X(2, 2) X(4, 2) X(2, 4) X(4, 4) X(2, 5) X(4, 5)
+// off the 128-bit path: two rows per lane only
+#define THN_SOFTMAX_FLAT_SHAPES_UNALIGNED(X) X(2, 0) X(2, 2) X(2, 4) X(2, 5)
 
 #define THN_DEFINE_SOFTMAX_FLAT_LAUNCHERS(NAME, TYPE)                                                           \
-    int launch_softmax_flat_fwd_##NAME(bool is_log, int rows_each, int log_steps, const SoftmaxFwdArgs& a, int grid, \
-                                       hipStream_t st) {                                                        \
+    int launch_softmax_flat_fwd_##NAME(bool is_log, bool aligned, int rows_each, int log_steps, const SoftmaxFwdArgs& a, \
+                                       int grid, hipStream_t st) {                                              \
         using T = TYPE;                                                                                         \
-        THN_SOFTMAX_FLAT_SHAPES(THN_SOFTMAX_FLAT_FWD_CASE)                                                      \
+        if (aligned) {                                                                                          \
+            THN_SOFTMAX_FLAT_SHAPES(THN_SOFTMAX_FLAT_FWD_AL)                                                    \
+        } else {                                                                                                \
+            THN_SOFTMAX_FLAT_SHAPES_UNALIGNED(THN_SOFTMAX_FLAT_FWD_SC)                                          \
+        }                                                                                                       \
         return 1;                                                                                               \
     }                                                                                                           \
-    int launch_softmax_flat_bwd_##NAME(bool is_log, int rows_each, int log_steps, const SoftmaxBwdArgs& a, int grid, \
-                                       hipStream_t st) {                                                        \
+    int launch_softmax_flat_bwd_##NAME(bool is_log, bool aligned, int rows_each, int log_steps, const SoftmaxBwdArgs& a, \
+                                       int grid, hipStream_t st) {                                              \
         using T = TYPE;                                                                                         \
-        THN_SOFTMAX_FLAT_SHAPES(THN_SOFTMAX_FLAT_BWD_CASE)                                                      \
+        if (aligned) {                                                                                          \
+            THN_SOFTMAX_FLAT_SHAPES(THN_SOFTMAX_FLAT_BWD_AL)                                                    \
+        } else {                                                                                                \
+            THN_SOFTMAX_FLAT_SHAPES_UNALIGNED(THN_SOFTMAX_FLAT_BWD_SC)                                          \
+        }                                                                                                       \
         return 1;                                                                                               \
     }
 
