@@ -362,14 +362,16 @@ int thn_dropout(const void* x, void* out, int64_t n, int64_t first_offset, float
  * float16 / bfloat16 rows on the 128-bit path) are selected here as well: a threads_per_row that is not a power of two,
  * with block_threads 0 or 256, selects the flat kernels for rows of exactly that many vectors (lanes are dealt to
  * vectors without gaps, a wave holds 64 / threads_per_row whole rows; vecs_per_thread = rows a lane carries per step:
- * 1, 2 or 4); block_threads = 64 selects the staged kernels (a wave copies a batch of rows into LDS and one lane sums a
+ * 1, 2 or 4; rows off the 128-bit path -- a width that is not a whole number of vectors, a pointer or pitch off 16
+ * bytes -- of 2 to 32 vectors, powers of two included, with 1 or 2); block_threads = 64 selects the staged kernels (a wave copies a batch of rows into LDS and one lane sums a
  * row; threads_per_row = the row's vector count or 0, vecs_per_thread = the batch in passes of the wave over its rows:
  * 1 to 4, or 0 for the default).  Problems such an override does not fit are refused (THN_E_SHAPE); any other
  * override runs the row kernels.
  * The softmax and p-norm families (2 to 6) have flat kernels of their own for rows of 1, 2 and 4 vectors and of up to
  * 32 vectors whose count is not a power of two, taken by default: threads_per_row = the row's vector count (with
  * block_threads 0 or 256 and vecs_per_thread 0, 2 or, softmax only, 4 rows per lane and step) keeps them, any other
- * shape selects the row kernels for such rows too.
+ * shape selects the row kernels for such rows too.  Off the 128-bit path (rows of at least one vector) they take 2 rows
+ * per lane only.
  * Process-wide; meant for benchmarks, not for concurrent production use.  Returns THN_E_SHAPE when no
  * compiled kernel has that shape.
  */
@@ -379,11 +381,14 @@ int thn_norm_set_launch_override(int which, int vecs_per_thread, int threads_per
 /*
  * What the heuristic (or the override) would launch for this problem: fills shape[0..4] with
  * {vecs_per_thread, threads_per_row, block_threads, grid_blocks, aligned 128-bit path (1) or unaligned-row path (0)}.
+ * (the last field is 0 for every kind of kernel when the rows are off the 128-bit path).
  * For the epilogue families (9, 10) `is_layernorm` carries the activation too: bit 0 = LayerNorm, bits 1.. = the
  * thn_act code.  Rows wider than 64 KiB of the softmax and p-norm families report their looping kernels:
  * {vectors per thread and step, block_threads, block_threads, grid_blocks, 0}.  Norm problems that take the flat
- * kernels (narrow 16-bit rows whose vector count is not a power of two) report {rows per lane and step, vectors per
- * row, 256, grid_blocks, 1}: a threads_per_row that is not a power of two identifies them; those that take the staged
+ * kernels (narrow 16-bit rows whose vector count is not a power of two; off the 128-bit path narrow rows of any
+ * vector count and type) report {rows per lane and step, vectors per row, 256, grid_blocks, 1}: a threads_per_row that
+ * is not a power of two identifies them (off the path a flat launch over 8, 16 or 32 vectors with one row per lane
+ * reads like the row kernels' 1 x 8, 1 x 16 and 1 x 32 shapes in 256 threads); those that take the staged
  * kernels (rows of 1 to 8 vectors, narrow float32 rows) report {passes per batch, vectors per row, 64, grid_blocks, 1}.
  * Softmax and p-norm problems on their flat kernels report {2 or 4, vectors per row, 256, grid_blocks, 1} (a p-norm
  * problem is taken to be a dense (M, N) tensor here; tensors whose batches do not fold run the row kernels).

@@ -60,6 +60,32 @@ def test_every_row_width_against_the_oracle(kind, dtype):
                     run_and_compare(kind, x, dy, w, b, 1e-5, f"flat L={n_vecs} J={rows_each} M={m}")
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32, torch.float16])
+@pytest.mark.parametrize("kind", ["ln", "rms"])
+def test_row_widths_off_the_128_bit_path(kind, dtype):
+    """Rows that are not a whole number of vectors (one column more than n_vecs - 1 vectors, one less than n_vecs), every
+    vector count from 2 to 32 -- powers of two included: off the 128-bit path the flat kernels take those too -- with 1
+    and 2 rows per lane: the unaligned-window instances, whose last window overlaps its neighbour (its leading columns
+    are stored twice and counted once in the row sums and in dW / dB)."""
+    vec = 16 // torch.empty(0, dtype=dtype).element_size()
+    g = torch.Generator().manual_seed(77)
+    for n_vecs in range(2, 33):
+        for n in sorted({(n_vecs - 1) * vec + 1, n_vecs * vec - 1}):
+            for rows_each in (1, 2):
+                rows_per_block = 4 * (64 // n_vecs) * rows_each
+                for m in sorted({1, rows_per_block - 1, 3 * rows_per_block + 5}):
+                    announce(f"{kind} {dtype} L={n_vecs} ragged N={n} J={rows_each} M={m}")
+                    with forced_flat(n_vecs, rows_each):
+                        for which in (0, 1):
+                            q = _launch.query_launch(which, kind == "ln", m, n, dtype)
+                            assert q[:3] == (rows_each, n_vecs, 256) and q[4] == 0, q
+                        x = (torch.randn(m, n, generator=g) * 2 + 0.5).to(dtype)
+                        dy = torch.randn(m, n, generator=g).to(dtype)
+                        w = (1 + 0.1 * torch.randn(n, generator=g)).to(dtype)
+                        b = (0.1 * torch.randn(n, generator=g)).to(dtype) if kind == "ln" else None
+                        run_and_compare(kind, x, dy, w, b, 1e-5, f"flat ragged L={n_vecs} N={n} J={rows_each} M={m}")
+
+
 def test_many_rows_hostile_mean_and_strided_views():
     """2^20 rows of 72 bf16 columns (every workgroup takes many steps), the hostile mean in float32, and rows that
     are not dense (column blocks of a wider buffer: the flat kernels address every lane's row by itself)."""

@@ -194,8 +194,8 @@ def test_ragged_hidden_sizes(kind, n, dtype):
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_odd_widths_of_16_bit_rows_reach_every_two_vector_shape(dtype):
-    """Rows off the 128-bit path run in the same slot shapes as rows on it: one odd width for each threads-per-row
-    value, LayerNorm (16-bit and float32 parameters) and RMSNorm."""
+    """Rows off the 128-bit path run in the same slot shapes as rows on it (or, up to 32 vectors, on the flat kernels):
+    one odd width for each threads-per-row value, LayerNorm (16-bit and float32 parameters) and RMSNorm."""
     g = torch.Generator().manual_seed(77)
     for n in (9, 121, 201, 499, 1001, 1501, 3001, 4099, 12289, 20001):
         announce(f"odd width {n} {dtype}")
@@ -203,7 +203,10 @@ def test_odd_widths_of_16_bit_rows_reach_every_two_vector_shape(dtype):
         for which, ln in ((0, True), (0, False), (1, True), (1, False)):
             kk, tt, _, _, vector_path = _launch.query_launch(which, ln, m, n, dtype)
             n_vecs = (n + 7) // 8
-            assert vector_path == 0 and kk * tt >= n_vecs and (kk - 1) * tt < n_vecs    # no emptier than it has to be
+            assert vector_path == 0
+            if n_vecs <= 32 and tt == n_vecs:
+                continue                      # the flat kernels: a lane per vector, kk rows per lane
+            assert kk * tt >= n_vecs and (kk - 1) * tt < n_vecs    # no emptier than it has to be
         x = (0.5 + torch.randn(m, n, generator=g)).to(dtype); dy = torch.randn(m, n, generator=g).to(dtype)
         w = (1 + 0.1 * torch.randn(n, generator=g)); b = 0.1 * torch.randn(n, generator=g)
         run_and_compare("ln", x, dy, w.to(dtype), b.to(dtype), 1e-5, f"odd LN N={n}")

@@ -725,20 +725,20 @@ struct FlatPlan {
     int n_vecs;
 };
 
-int launch_flat_fwd(int dtype, bool ln, const FlatPlan& p, const FwdArgs& a, hipStream_t st, int* occ) {
+int launch_flat_fwd(int dtype, bool ln, bool aligned, const FlatPlan& p, const FwdArgs& a, hipStream_t st, int* occ) {
     switch (dtype) {
-        case THN_F32: return thn::launch_flat_fwd_f32(ln, p.rows_each, p.log_steps, a, p.grid, st, occ);
-        case THN_F16: return thn::launch_flat_fwd_f16(ln, p.rows_each, p.log_steps, a, p.grid, st, occ);
-        case THN_BF16: return thn::launch_flat_fwd_bf16(ln, p.rows_each, p.log_steps, a, p.grid, st, occ);
+        case THN_F32: return thn::launch_flat_fwd_f32(ln, aligned, p.rows_each, p.log_steps, a, p.grid, st, occ);
+        case THN_F16: return thn::launch_flat_fwd_f16(ln, aligned, p.rows_each, p.log_steps, a, p.grid, st, occ);
+        case THN_BF16: return thn::launch_flat_fwd_bf16(ln, aligned, p.rows_each, p.log_steps, a, p.grid, st, occ);
         default: return 1;
     }
 }
 
-int launch_flat_bwd(int dtype, bool ln, const FlatPlan& p, const BwdArgs& a, hipStream_t st, int* occ) {
+int launch_flat_bwd(int dtype, bool ln, bool aligned, const FlatPlan& p, const BwdArgs& a, hipStream_t st, int* occ) {
     switch (dtype) {
-        case THN_F32: return thn::launch_flat_bwd_f32(ln, p.rows_each, p.log_steps, a, p.grid, st, occ);
-        case THN_F16: return thn::launch_flat_bwd_f16(ln, p.rows_each, p.log_steps, a, p.grid, st, occ);
-        case THN_BF16: return thn::launch_flat_bwd_bf16(ln, p.rows_each, p.log_steps, a, p.grid, st, occ);
+        case THN_F32: return thn::launch_flat_bwd_f32(ln, aligned, p.rows_each, p.log_steps, a, p.grid, st, occ);
+        case THN_F16: return thn::launch_flat_bwd_f16(ln, aligned, p.rows_each, p.log_steps, a, p.grid, st, occ);
+        case THN_BF16: return thn::launch_flat_bwd_bf16(ln, aligned, p.rows_each, p.log_steps, a, p.grid, st, occ);
         default: return 1;
     }
 }
@@ -764,12 +764,41 @@ bool flat_by_default(int which, bool ln, int bytes, int n_vecs) {
     return ln ? n_vecs == 3 : n_vecs <= 21;
 }
 
+// Rows off the 128-bit path (a width that is not a whole number of vectors, a pointer or pitch off 16 bytes): the row
+// kernels' lane groups are no fuller there than on the path, and the staged kernels do not take such rows, so the flat
+// kernels serve more widths than on the path, powers of two included.  Forward + backward of 2^26 elements with ONE of
+// the two launches changed from the row kernels to the flat ones, % of 8 TB/s (bfloat16 widths N = 8 (L - 1) + 1 or + 5,
+// float32 N = 4 (L - 1) + 1 or + 3):
+//   RMSNorm forward: bfloat16 L = 2 17.7 -> 23.8; 4 41.6 -> 47.2; 8 67.6 -> 71.3; 15 70.0 -> 72.5; 21 66.7 -> 67.9; from
+//     22 vectors on the same or lower; float32 L = 3 41.9 -> 48.4; 8 71.1 -> 77.2; 16 74.4 -> 76.9; 21 72.4 -> 73.1;
+//   RMSNorm backward: every width up to 32 vectors (bfloat16 L = 2 17.7 -> 27.2; 5 53.5 -> 60.1; 9 56.3 -> 66.4; 17
+//     58.9 -> 65.5; 24 68.1 -> 70.9; float32 L = 2 22.5 -> 41.1; 4 48.0 -> 64.1; 9 59.7 -> 71.7; 32 67.4 -> 76.7);
+//   LayerNorm forward: 16-bit rows up to 12 vectors (L = 2 15.6 -> 20.7; 4 36.9 -> 42.1; 8 62.5 -> 64.9; from 13 on 0-4
+//     points lower), float32 rows up to 16 (L = 3 38.1 -> 43.1; 8 67.0 -> 72.6; 16 70.4 -> 73.1);
+//   LayerNorm backward: 16-bit rows of up to 6, of 9 to 12 and of 17 to 20 vectors (L = 2 15.6 -> 24.9; 5 46.8 -> 51.2;
+//     9 50.6 -> 59.1; 17 53.2 -> 56.3; rows of 7, 8 and 13 to 16 vectors fill the row kernels' lane groups and are 1-5
+//     points faster there), float32 rows up to 12 (L = 2 19.9 -> 36.7; 4 43.6 -> 58.4; 9 54.2 -> 67.2; 12 64.1 -> 68.1).
+// Both launches changed: bfloat16 RMSNorm N = 9 17.7 -> 44.9; 21 36.1 -> 60.3; 69 56.3 -> 70.6; 129 58.9 -> 69.6; LayerNorm
+// N = 9 15.6 -> 38.4; 69 50.6 -> 60.1; float32 RMSNorm N = 5 22.5 -> 71.4; 11 41.9 -> 74.2; 35 59.7 -> 75.0; 125 67.4 ->
+// 76.9; LayerNorm N = 5 19.9 -> 53.4; 11 38.1 -> 67.4; 35 54.2 -> 70.7 (the statistics of such rows -- 4 or 8 bytes per
+// row and pass next to 18 to 40 bytes of row -- are not in the algorithmic bytes).
+bool flat_off_path_by_default(int which, bool ln, int bytes, int n_vecs) {
+    if (which == kNormFwd) {
+        if (!ln) return n_vecs <= 21;
+        return bytes == 2 ? n_vecs <= 12 : n_vecs <= 16;
+    }
+    if (!ln) return true;
+    if (bytes == 2) return n_vecs <= 6 || (n_vecs >= 9 && n_vecs <= 12) || (n_vecs >= 17 && n_vecs <= 20);
+    return n_vecs <= 12;
+}
+
 bool plan_flat(int which, bool ln, bool aligned, int64_t M, int64_t N, int dtype, FlatPlan* out) {
     const int bytes = elem_bytes(dtype);
-    if (!aligned || bytes == 0 || bytes == 8 || M <= 0) return false;
+    if (bytes == 0 || bytes == 8 || M <= 0) return false;
     const int vec_elems = 16 / bytes;
-    if (N % vec_elems != 0) return false;
-    const int n_vecs = static_cast<int>(N / vec_elems);
+    // off the 128-bit path: rows of at least one vector (unaligned 16-byte windows, the last one overlapping)
+    if (aligned ? N % vec_elems != 0 : N < vec_elems) return false;
+    const int n_vecs = static_cast<int>((N + vec_elems - 1) / vec_elems);
     if (n_vecs < 2 || n_vecs > thn::kFlatMaxVecs) return false;
     const Override& ov = g_override[which];
     // rows per lane and step, workgroups per compute unit: two and two measured best or within a point of it at every
@@ -779,12 +808,15 @@ bool plan_flat(int which, bool ln, bool aligned, int64_t M, int64_t N, int dtype
         rows_each = 1;
         bpc = 4;
     }
+    // the 16-bit LayerNorm backward off the 128-bit path: four workgroups (2-5 points over two at 9 to 20 vectors)
+    if (which == kNormBwd && ln && bytes == 2 && !aligned) bpc = 4;
     if (ov.tpr.load() > 0 || ov.block.load() > 0 || ov.k.load() > 0) {
-        if (ov.tpr.load() != n_vecs || (n_vecs & (n_vecs - 1)) == 0) return false;     // a row-kernel shape is forced
+        // (a row-kernel shape is forced; on the 128-bit path a power of two is one: there the staged kernels take over)
+        if (ov.tpr.load() != n_vecs || (aligned && (n_vecs & (n_vecs - 1)) == 0)) return false;
         if (ov.block.load() > 0 && ov.block.load() != thn::kFlatBlock) return false;
         if (ov.k.load() > 0) rows_each = ov.k.load();
-        if (rows_each != 1 && rows_each != 2 && rows_each != 4) return false;
-    } else if (!flat_by_default(which, ln, bytes, n_vecs)) {
+        if (rows_each != 1 && rows_each != 2 && (rows_each != 4 || !aligned)) return false;
+    } else if (!(aligned ? flat_by_default(which, ln, bytes, n_vecs) : flat_off_path_by_default(which, ln, bytes, n_vecs))) {
         return false;
     }
     const int cus = current_cu_count();
@@ -1128,7 +1160,7 @@ int norm_forward(const void* x, int64_t x_row_stride, void* y, int64_t y_row_str
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (flat || staged) a.line_shift = 0;
     const int lrc = staged ? launch_staged_fwd(x_dtype, ln, sp, a, st, nullptr)
-                  : flat ? launch_flat_fwd(x_dtype, ln, fp, a, st, nullptr)
+                  : flat ? launch_flat_fwd(x_dtype, ln, aligned, fp, a, st, nullptr)
                   : fused ? launch_fused_fwd(x_dtype, (ln ? 1 : 0) | (act << 1), aligned, p.s, a, p.grid, st, nullptr)
                           : launch_fwd(x_dtype, ln, aligned, p.s, a, p.grid, st, nullptr);
     if (lrc > 0) return THN_E_SHAPE;
@@ -1211,7 +1243,7 @@ int norm_backward_stage1(const void* x, int64_t x_row_stride, const void* dy, in
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (flat || staged) a.line_shift = 0;
     const int lrc = staged ? launch_staged_bwd(x_dtype, ln, sp, a, st, nullptr)
-                  : flat ? launch_flat_bwd(x_dtype, ln, fp, a, st, nullptr)
+                  : flat ? launch_flat_bwd(x_dtype, ln, aligned, fp, a, st, nullptr)
                   : fused ? launch_fused_bwd(x_dtype, variant, aligned, p.s, a, p.grid, st, nullptr)
                           : launch_bwd(x_dtype, ln, aligned, p.s, a, p.grid, st, nullptr);
     if (lrc > 0) return THN_E_SHAPE;
@@ -1531,7 +1563,7 @@ int thn_norm_query_launch(int which, int is_layernorm, int64_t M, int64_t N, int
         shape[1] = fp.n_vecs;
         shape[2] = thn::kFlatBlock;
         shape[3] = fp.grid;
-        shape[4] = 1;
+        shape[4] = aligned ? 1 : 0;
         return THN_OK;
     }
     const int rc = plan_launch(which, flavour, aligned, M, N, x_dtype, &p, N * elem_bytes(x_dtype));   // contiguous rows

@@ -18,8 +18,9 @@
 // Everything else follows the row kernels: a persistent grid, J independent rows per lane and step with the next J
 // requested before the current ones are reduced, no branch around a load or store (rows past the end are clamped
 // onto the last row and masked out of dW / dB), float32 arithmetic, the statistics stored by every lane of a row,
-// one float32 partial row of dW / dB per workgroup summed in a fixed order.  128-bit path only (N a whole number of
-// vectors, 16-byte aligned rows).
+// one float32 partial row of dW / dB per workgroup summed in a fixed order.  ALIGNED = false: rows of at least two
+// vectors off the 128-bit path, whose slots are unaligned 16-byte windows, the ragged last one overlapping its neighbour
+// (slot_place() in thn_kernels.h: the overlapped columns are computed and stored twice, and counted once in every sum).
 #pragma once
 
 #include "thn_dispatch.h"
@@ -73,7 +74,7 @@ __device__ __forceinline__ FlatLane flat_lane(int lane, int L) {
 }
 
 // Forward.  Arithmetic as norm_fwd_kernel (LayerNorm: mean0, then {sum d, sum d^2} with the delta correction).
-template <typename T, bool LN, int J, int LOG, bool KEEPX>
+template <typename T, bool LN, int J, int LOG, bool KEEPX, bool ALIGNED>
 __global__ void __launch_bounds__(kFlatBlock) norm_flat_fwd_kernel(const FwdArgs a) {
     constexpr int VEC = T::VEC;
     constexpr int W = kFlatBlock / 64;
@@ -81,7 +82,11 @@ __global__ void __launch_bounds__(kFlatBlock) norm_flat_fwd_kernel(const FwdArgs
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int rpw = 64 / L;
     const FlatLane f = flat_lane(lane, L);
-    const int voff = f.t * 16;
+    int voff, lead;
+    {
+        bool in_row;
+        slot_place<T, ALIGNED>(f.t, L, a.n_cols, voff, lead, in_row);
+    }
 
     const int64_t rows_per_block = static_cast<int64_t>(W) * rpw * J;
     const int64_t rows_per_iter = static_cast<int64_t>(gridDim.x) * rows_per_block;
@@ -92,12 +97,12 @@ __global__ void __launch_bounds__(kFlatBlock) norm_flat_fwd_kernel(const FwdArgs
     for (int j = 0; j < J; ++j) {
         row_raw[j] = static_cast<int64_t>(blockIdx.x) * rows_per_block + static_cast<int64_t>(j * W + wave) * rpw + f.r;
         row[j] = row_raw[j] < a.M ? row_raw[j] : last_row;
-        cur[j] = slot_load<T, true, KEEPX>(a.x + row[j] * a.x_stride_bytes, voff, a.n_cols);
+        cur[j] = slot_load<T, ALIGNED, KEEPX>(a.x + row[j] * a.x_stride_bytes, voff, a.n_cols);
     }
     float wr[1][VEC], br[1][VEC];
     const int pv[1] = {voff};
-    load_params_clamped<1, VEC, true>(wr, a.w, a.w_dtype, pv, a.n_cols, 1.0f);
-    if constexpr (LN) load_params_clamped<1, VEC, true>(br, a.b, a.w_dtype, pv, a.n_cols, 0.0f);
+    slot_params<T, 1, ALIGNED>(wr, a.w, a.w_dtype, pv, a.n_cols, 1.0f);
+    if constexpr (LN) slot_params<T, 1, ALIGNED>(br, a.b, a.w_dtype, pv, a.n_cols, 0.0f);
     drain_vector_memory(cur);
 
     for (int64_t base = static_cast<int64_t>(blockIdx.x) * rows_per_block; base < a.M; base += rows_per_iter) {
@@ -107,7 +112,7 @@ __global__ void __launch_bounds__(kFlatBlock) norm_flat_fwd_kernel(const FwdArgs
         for (int j = 0; j < J; ++j) {
             nrow_raw[j] = row_raw[j] + rows_per_iter;
             nrow[j] = nrow_raw[j] < a.M ? nrow_raw[j] : last_row;
-            nxt[j] = slot_load<T, true, KEEPX>(a.x + nrow[j] * a.x_stride_bytes, voff, a.n_cols);
+            nxt[j] = slot_load<T, ALIGNED, KEEPX>(a.x + nrow[j] * a.x_stride_bytes, voff, a.n_cols);
         }
         float xf[J][VEC];
 #pragma unroll
@@ -119,7 +124,7 @@ __global__ void __launch_bounds__(kFlatBlock) norm_flat_fwd_kernel(const FwdArgs
             for (int j = 0; j < J; ++j) {
                 float sk = 0.0f;
 #pragma unroll
-                for (int e = 0; e < VEC; ++e) sk += xf[j][e];
+                for (int e = 0; e < VEC; ++e) sk += e >= lead ? xf[j][e] : 0.0f;     // overlapped columns count once
                 s[j] = f.own ? sk : 0.0f;
             }
             segment_allreduce<LOG, J>(s, lane, f.pos, L, f.first);
@@ -132,8 +137,9 @@ __global__ void __launch_bounds__(kFlatBlock) norm_flat_fwd_kernel(const FwdArgs
                 for (int e = 0; e < VEC; ++e) {
                     const float d = xf[j][e] - mean0;
                     xf[j][e] = d;
-                    q0 += d;
-                    q1 = fmaf(d, d, q1);
+                    const float dm = e >= lead ? d : 0.0f;
+                    q0 += dm;
+                    q1 = fmaf(dm, dm, q1);
                 }
                 q[2 * j] = f.own ? q0 : 0.0f;
                 q[2 * j + 1] = f.own ? q1 : 0.0f;
@@ -153,7 +159,10 @@ __global__ void __launch_bounds__(kFlatBlock) norm_flat_fwd_kernel(const FwdArgs
             for (int j = 0; j < J; ++j) {
                 float qk = 0.0f;
 #pragma unroll
-                for (int e = 0; e < VEC; ++e) qk = fmaf(xf[j][e], xf[j][e], qk);
+                for (int e = 0; e < VEC; ++e) {
+                    const float xm = e >= lead ? xf[j][e] : 0.0f;
+                    qk = fmaf(xm, xm, qk);
+                }
                 q[j] = f.own ? qk : 0.0f;
             }
             segment_allreduce<LOG, J>(q, lane, f.pos, L, f.first);
@@ -172,7 +181,7 @@ __global__ void __launch_bounds__(kFlatBlock) norm_flat_fwd_kernel(const FwdArgs
                 if constexpr (LN) yf[e] = fmaf((xf[j][e] - delta[j]) * rstd[j], wr[0][e], br[0][e]);
                 else yf[e] = xf[j][e] * rstd[j] * wr[0][e];
             }
-            slot_store<T, true>(a.y + row[j] * a.y_stride_bytes, voff, a.n_cols, yf);
+            slot_store<T, ALIGNED>(a.y + row[j] * a.y_stride_bytes, voff, a.n_cols, yf);
             if constexpr (LN) a.mean[row[j]] = mean[j];
             a.rstd[row[j]] = rstd[j];
         }
@@ -187,7 +196,7 @@ __global__ void __launch_bounds__(kFlatBlock) norm_flat_fwd_kernel(const FwdArgs
 
 // Backward.  Arithmetic as norm_bwd_kernel: one round of {sum u*wdy, sum wdy, sum u}; per-lane column sums of dW / dB
 // (float64 for float32 rows), which the workgroup adds up at the end, in a fixed order, into ONE float32 partial row.
-template <typename T, bool LN, int J, int LOG>
+template <typename T, bool LN, int J, int LOG, bool ALIGNED>
 __global__ void __launch_bounds__(kFlatBlock) norm_flat_bwd_kernel(const BwdArgs a) {
     constexpr int VEC = T::VEC;
     constexpr int W = kFlatBlock / 64;
@@ -199,7 +208,11 @@ __global__ void __launch_bounds__(kFlatBlock) norm_flat_bwd_kernel(const BwdArgs
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int rpw = 64 / L;
     const FlatLane f = flat_lane(lane, L);
-    const int voff = f.t * 16;
+    int voff, lead;
+    {
+        bool in_row;
+        slot_place<T, ALIGNED>(f.t, L, a.n_cols, voff, lead, in_row);
+    }
 
     const int64_t rows_per_block = static_cast<int64_t>(W) * rpw * J;
     const int64_t rows_per_iter = static_cast<int64_t>(gridDim.x) * rows_per_block;
@@ -211,14 +224,14 @@ __global__ void __launch_bounds__(kFlatBlock) norm_flat_bwd_kernel(const BwdArgs
     for (int j = 0; j < J; ++j) {
         row_raw[j] = static_cast<int64_t>(blockIdx.x) * rows_per_block + static_cast<int64_t>(j * W + wave) * rpw + f.r;
         row[j] = row_raw[j] < a.M ? row_raw[j] : last_row;
-        cx[j] = slot_load<T, true>(a.x + row[j] * a.x_stride_bytes, voff, a.n_cols);
-        cg[j] = slot_load<T, true>(a.dy + row[j] * a.dy_stride_bytes, voff, a.n_cols);
+        cx[j] = slot_load<T, ALIGNED>(a.x + row[j] * a.x_stride_bytes, voff, a.n_cols);
+        cg[j] = slot_load<T, ALIGNED>(a.dy + row[j] * a.dy_stride_bytes, voff, a.n_cols);
         c_mean[j] = LN ? a.mean[row[j]] : 0.0f;
         c_rstd[j] = a.rstd[row[j]];
     }
     float wr[1][VEC];
     const int pv[1] = {voff};
-    load_params_clamped<1, VEC, true>(wr, a.w, a.w_dtype, pv, a.n_cols, 1.0f);
+    slot_params<T, 1, ALIGNED>(wr, a.w, a.w_dtype, pv, a.n_cols, 1.0f);
     Acc dw[VEC], db[VEC];
 #pragma unroll
     for (int e = 0; e < VEC; ++e) { dw[e] = Acc(0); db[e] = Acc(0); }
@@ -237,8 +250,8 @@ __global__ void __launch_bounds__(kFlatBlock) norm_flat_bwd_kernel(const BwdArgs
         for (int j = 0; j < J; ++j) {
             nrow_raw[j] = row_raw[j] + rows_per_iter;
             nrow[j] = nrow_raw[j] < a.M ? nrow_raw[j] : last_row;
-            nx[j] = slot_load<T, true>(a.x + nrow[j] * a.x_stride_bytes, voff, a.n_cols);
-            ng[j] = slot_load<T, true>(a.dy + nrow[j] * a.dy_stride_bytes, voff, a.n_cols);
+            nx[j] = slot_load<T, ALIGNED>(a.x + nrow[j] * a.x_stride_bytes, voff, a.n_cols);
+            ng[j] = slot_load<T, ALIGNED>(a.dy + nrow[j] * a.dy_stride_bytes, voff, a.n_cols);
             n_mean[j] = LN ? a.mean[nrow[j]] : 0.0f;
             n_rstd[j] = a.rstd[nrow[j]];
         }
@@ -254,10 +267,12 @@ __global__ void __launch_bounds__(kFlatBlock) norm_flat_bwd_kernel(const BwdArgs
                 if constexpr (LN) u[j][e] = (u[j][e] - c_mean[j]) * c_rstd[j];
                 else u[j][e] *= c_rstd[j];
                 wdy[j][e] = wr[0][e] * gf[j][e];
-                s0 = fmaf(u[j][e], wdy[j][e], s0);
+                const bool counts = e >= lead;               // overlapped columns count once
+                const float wm = counts ? wdy[j][e] : 0.0f;
+                s0 = fmaf(u[j][e], wm, s0);
                 if constexpr (LN) {
-                    s1 += wdy[j][e];
-                    s2 += u[j][e];
+                    s1 += wm;
+                    s2 += counts ? u[j][e] : 0.0f;
                 }
             }
             s[NV * j] = f.own ? s0 : 0.0f;
@@ -284,11 +299,11 @@ __global__ void __launch_bounds__(kFlatBlock) norm_flat_bwd_kernel(const BwdArgs
                 float xhat = u[j][e];
                 if constexpr (LN) xhat -= dlt;
                 dxf[e] = (wdy[j][e] - fmaf(xhat, c1, c2)) * c_rstd[j];
-                const float gl = adds ? gf[j][e] : 0.0f;
+                const float gl = (adds && e >= lead) ? gf[j][e] : 0.0f;
                 dw[e] = fma(static_cast<Acc>(gl), static_cast<Acc>(xhat), dw[e]);
                 if constexpr (LN) db[e] += static_cast<Acc>(gl);
             }
-            slot_store<T, true>(a.dx + row[j] * a.dx_stride_bytes, voff, a.n_cols, dxf);
+            slot_store<T, ALIGNED>(a.dx + row[j] * a.dx_stride_bytes, voff, a.n_cols, dxf);
         }
 #pragma unroll
         for (int j = 0; j < J; ++j) {
@@ -312,7 +327,9 @@ __global__ void __launch_bounds__(kFlatBlock) norm_flat_bwd_kernel(const BwdArgs
     }
     __syncthreads();
     for (int c = threadIdx.x; c < a.n_cols; c += kFlatBlock) {
-        const int t = c / VEC, e = c - t * VEC;
+        const int t = c / VEC;                                 // the slot that owns column c, and c's place in its window
+        const int start = (!ALIGNED && t * VEC > a.n_cols - VEC) ? a.n_cols - VEC : t * VEC;
+        const int e = c - start;
         Acc sw = Acc(0), sb = Acc(0);
         for (int w = 0; w < W; ++w) {
             for (int r = 0; r < rpw; ++r) {
@@ -330,43 +347,57 @@ __global__ void __launch_bounds__(kFlatBlock) norm_flat_bwd_kernel(const BwdArgs
 // Launchers: 0 launched (or occupancy written), 1 no such instance, <0 HIP error.  `log_steps` = ceil(log2(L)): 4 or 5
 // (rows of up to 16 vectors use the 4-step instances as well); `rows_each` = J.
 #define THN_DECLARE_FLAT_LAUNCHERS(NAME)                                                                        \
-    int launch_flat_fwd_##NAME(bool ln, int rows_each, int log_steps, const FwdArgs& a, int grid, hipStream_t st, \
-                               int* occupancy);                                                                 \
-    int launch_flat_bwd_##NAME(bool ln, int rows_each, int log_steps, const BwdArgs& a, int grid, hipStream_t st, \
-                               int* occupancy);
+    int launch_flat_fwd_##NAME(bool ln, bool aligned, int rows_each, int log_steps, const FwdArgs& a, int grid, \
+                               hipStream_t st, int* occupancy);                                                 \
+    int launch_flat_bwd_##NAME(bool ln, bool aligned, int rows_each, int log_steps, const BwdArgs& a, int grid, \
+                               hipStream_t st, int* occupancy);
 
 THN_DECLARE_FLAT_LAUNCHERS(f32)
 THN_DECLARE_FLAT_LAUNCHERS(f16)
 THN_DECLARE_FLAT_LAUNCHERS(bf16)
 
-#define THN_FLAT_FWD_CASE(J_, LOG_)                                                                             \
+#define THN_FLAT_FWD_CASE(AL, J_, LOG_)                                                                         \
     if (rows_each == J_ && log_steps == LOG_) {                                                                 \
         if (a.keep_x) {                                                                                         \
-            return ln ? run_kernel<FwdArgs>(norm_flat_fwd_kernel<T, true, J_, LOG_, true>, a, grid, kFlatBlock, st, occupancy)  \
-                      : run_kernel<FwdArgs>(norm_flat_fwd_kernel<T, false, J_, LOG_, true>, a, grid, kFlatBlock, st, occupancy); \
+            return ln ? run_kernel<FwdArgs>(norm_flat_fwd_kernel<T, true, J_, LOG_, true, AL>, a, grid, kFlatBlock, st, occupancy)  \
+                      : run_kernel<FwdArgs>(norm_flat_fwd_kernel<T, false, J_, LOG_, true, AL>, a, grid, kFlatBlock, st, occupancy); \
         }                                                                                                       \
-        return ln ? run_kernel<FwdArgs>(norm_flat_fwd_kernel<T, true, J_, LOG_, false>, a, grid, kFlatBlock, st, occupancy)     \
-                  : run_kernel<FwdArgs>(norm_flat_fwd_kernel<T, false, J_, LOG_, false>, a, grid, kFlatBlock, st, occupancy);   \
+        return ln ? run_kernel<FwdArgs>(norm_flat_fwd_kernel<T, true, J_, LOG_, false, AL>, a, grid, kFlatBlock, st, occupancy)     \
+                  : run_kernel<FwdArgs>(norm_flat_fwd_kernel<T, false, J_, LOG_, false, AL>, a, grid, kFlatBlock, st, occupancy);   \
     }
-#define THN_FLAT_BWD_CASE(J_, LOG_)                                                                             \
+#define THN_FLAT_BWD_CASE(AL, J_, LOG_)                                                                         \
     if (rows_each == J_ && log_steps == LOG_) {                                                                 \
-        return ln ? run_kernel<BwdArgs>(norm_flat_bwd_kernel<T, true, J_, LOG_>, a, grid, kFlatBlock, st, occupancy)   \
-                  : run_kernel<BwdArgs>(norm_flat_bwd_kernel<T, false, J_, LOG_>, a, grid, kFlatBlock, st, occupancy);  \
+        return ln ? run_kernel<BwdArgs>(norm_flat_bwd_kernel<T, true, J_, LOG_, AL>, a, grid, kFlatBlock, st, occupancy)   \
+                  : run_kernel<BwdArgs>(norm_flat_bwd_kernel<T, false, J_, LOG_, AL>, a, grid, kFlatBlock, st, occupancy);  \
     }
+#define THN_FLAT_FWD_AL(J_, LOG_) THN_FLAT_FWD_CASE(true, J_, LOG_)
+#define THN_FLAT_FWD_SC(J_, LOG_) THN_FLAT_FWD_CASE(false, J_, LOG_)
+#define THN_FLAT_BWD_AL(J_, LOG_) THN_FLAT_BWD_CASE(true, J_, LOG_)
+#define THN_FLAT_BWD_SC(J_, LOG_) THN_FLAT_BWD_CASE(false, J_, LOG_)
 // X(J, LOG): rows per lane and step x tree steps
 #define THN_FLAT_SHAPES(X) X(1, 4) X(2, 4) X(4, 4) X(1, 5) X(2, 5) X(4, 5)
+// off the 128-bit path: one or two rows per lane
+#define THN_FLAT_SHAPES_UNALIGNED(X) X(1, 4) X(2, 4) X(1, 5) X(2, 5)
 
 #define THN_DEFINE_FLAT_LAUNCHERS(NAME, TYPE)                                                                   \
-    int launch_flat_fwd_##NAME(bool ln, int rows_each, int log_steps, const FwdArgs& a, int grid, hipStream_t st, \
-                               int* occupancy) {                                                                \
+    int launch_flat_fwd_##NAME(bool ln, bool aligned, int rows_each, int log_steps, const FwdArgs& a, int grid, \
+                               hipStream_t st, int* occupancy) {                                                \
         using T = TYPE;                                                                                         \
-        THN_FLAT_SHAPES(THN_FLAT_FWD_CASE)                                                                      \
+        if (aligned) {                                                                                          \
+            THN_FLAT_SHAPES(THN_FLAT_FWD_AL)                                                                    \
+        } else {                                                                                                \
+            THN_FLAT_SHAPES_UNALIGNED(THN_FLAT_FWD_SC)                                                          \
+        }                                                                                                       \
         return 1;                                                                                               \
     }                                                                                                           \
-    int launch_flat_bwd_##NAME(bool ln, int rows_each, int log_steps, const BwdArgs& a, int grid, hipStream_t st, \
-                               int* occupancy) {                                                                \
+    int launch_flat_bwd_##NAME(bool ln, bool aligned, int rows_each, int log_steps, const BwdArgs& a, int grid, \
+                               hipStream_t st, int* occupancy) {                                                \
         using T = TYPE;                                                                                         \
-        THN_FLAT_SHAPES(THN_FLAT_BWD_CASE)                                                                      \
+        if (aligned) {                                                                                          \
+            THN_FLAT_SHAPES(THN_FLAT_BWD_AL)                                                                    \
+        } else {                                                                                                \
+            THN_FLAT_SHAPES_UNALIGNED(THN_FLAT_BWD_SC)                                                          \
+        }                                                                                                       \
         return 1;                                                                                               \
     }
 
