@@ -581,7 +581,7 @@ def main():
     print(json.dumps(out), flush=True)
 
 
-SCAN_WIDTHS = [64, 72, 96, 120, 128, 192, 200, 248, 256, 320, 384, 512, 640, 768, 896, 1024, 1152, 1280, 1408, 1536, 1600, 1792,
+SCAN_WIDTHS = [20, 50, 64, 72, 96, 100, 120, 128, 192, 197, 200, 248, 256, 320, 384, 512, 640, 768, 896, 1000, 1024, 1152, 1280, 1408, 1536, 1600, 1792,
                2048, 2304, 2560, 2816, 3072, 3584, 4000, 4096, 4098, 4104, 4608, 5120, 5632, 6000, 6144, 6656, 7168, 8192,
                9216, 10240, 12288, 14336, 16384, 20480, 24576, 28672, 32768]
 
