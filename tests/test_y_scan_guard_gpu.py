@@ -2,7 +2,7 @@
 of row widths must stay within reach of the committed width scan (profiles/norm_step_width_scan_bf16_f16_f32.txt,
 the output of `bench.py --scan`).  The bound is loose on purpose -- 0.75 of the committed figure: boxes differ by a
 few per cent, a launch rule that picks a wrong shape costs 20 to 50 -- and the widths are the ones a rule boundary sits
-next to: narrow rows on and off powers of two, the staged kernels, rows off the 128-bit path, the widest one-row shapes.
+next to: narrow rows on and off powers of two, the flat and staged kernels, rows off the 128-bit path (narrow and wide), the widest one-row shapes.
 Collected late (the file name sorts behind the parity tests): it says nothing about correctness."""
 import os
 import sys
@@ -16,8 +16,8 @@ sys.path.insert(0, ROOT)
 pytestmark = pytest.mark.gpu
 
 GUARDED = {
-    "bf16": [72, 128, 200, 640, 1024, 2048, 4096, 4098, 6000, 8192, 16384],
-    "f32": [72, 256, 1536, 4096],
+    "bf16": [50, 72, 128, 197, 200, 640, 1024, 2048, 4096, 4098, 6000, 8192, 16384],
+    "f32": [50, 72, 256, 1536, 4096],
 }
 FLOOR = 0.75
 
