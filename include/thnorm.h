@@ -390,6 +390,9 @@ int thn_norm_set_launch_override(int which, int vecs_per_thread, int threads_per
  * is not a power of two identifies them (off the path a flat launch over 8, 16 or 32 vectors with one row per lane
  * reads like the row kernels' 1 x 8, 1 x 16 and 1 x 32 shapes in 256 threads); those that take the staged
  * kernels (rows of 1 to 8 vectors, narrow float32 rows) report {passes per batch, vectors per row, 64, grid_blocks, 1}.
+ * Softmax and p-norm problems over rows shorter than one vector report {4, 1, 256, grid_blocks, 0}: four rows per
+ * lane and step, ONE lane per row (any launch override with a shape field set selects the row kernels' element-wise
+ * instance, 4 x 8 in 256 threads, instead).
  * Softmax and p-norm problems on their flat kernels report {2 or 4, vectors per row, 256, grid_blocks, 1} (a p-norm
  * problem is taken to be a dense (M, N) tensor here; tensors whose batches do not fold run the row kernels).
  */

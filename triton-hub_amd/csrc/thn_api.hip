@@ -18,6 +18,7 @@
 #include "thn_softmax_dispatch.h"
 #include "thn_softmax_flat.h"
 #include "thn_pnorm_flat.h"
+#include "thn_tiny.h"
 
 namespace {
 
@@ -1009,6 +1010,54 @@ int launch_normalize_flat_bwd(int dtype, int mode, bool aligned, const OneSumFla
     }
 }
 
+// ---- rows shorter than one vector: a lane per row (thn_tiny.h) -------------------------------------------------------
+// Softmax and p-norm families, float32 / float16 / bfloat16.  Forward + backward of 2^25 elements, % of 8 TB/s, the row
+// kernels' element-wise instance -> a lane per row, softmax / normalize p = 2: float32 N = 1 2.4 / 2.5 -> 66.8 / 44.7;
+// 2 4.5 / 4.6 -> 61.1 / 52.5; 3 6.4 / 6.4 -> 50.7 / 46.5; bfloat16 N = 2 1.0 / 1.0 -> 24.0 / 22.9; 4 1.8 / 1.8 -> 26.6 /
+// 25.9; 7 3.0 / 2.9 -> 23.5 / 22.5 (two-byte accesses: a wave's store instruction is seven partial lines; torch's own
+// softmax forward moves its bytes at 44-61 % of the peak in float32 and 17-28 % in bfloat16 at these widths).
+// A launch override with any shape field set keeps the row kernels' element-wise instance (4 x 8 in 256 threads).
+bool tiny_rows(int which, int64_t N, int dtype) {
+    const int bytes = elem_bytes(dtype);
+    const Override& ov = g_override[which];
+    if (ov.k.load() > 0 || ov.tpr.load() > 0 || ov.block.load() > 0) return false;
+    return (bytes == 2 || bytes == 4) && N < 16 / bytes;
+}
+int tiny_grid(int64_t rows, int cus) {
+    const int64_t per_block = static_cast<int64_t>(thn::kTinyBlock) * thn::kTinyRows;
+    const int64_t blocks = (rows + per_block - 1) / per_block;
+    const int64_t cap = static_cast<int64_t>(cus) * 8;
+    return static_cast<int>(blocks < cap ? blocks : cap);
+}
+#define THN_TINY_SWITCH(CALL_F32, CALL_F16, CALL_BF16)  \
+    switch (dtype) {                                    \
+        case THN_F32: return CALL_F32;                  \
+        case THN_F16: return CALL_F16;                  \
+        case THN_BF16: return CALL_BF16;                \
+        default: return 1;                              \
+    }
+int launch_softmax_tiny_fwd(int dtype, bool is_log, const SoftmaxFwdArgs& a, int grid, hipStream_t st) {
+    THN_TINY_SWITCH(thn::launch_softmax_tiny_fwd_f32(is_log, a, grid, st), thn::launch_softmax_tiny_fwd_f16(is_log, a, grid, st),
+                    thn::launch_softmax_tiny_fwd_bf16(is_log, a, grid, st))
+}
+int launch_softmax_tiny_bwd(int dtype, bool is_log, const SoftmaxBwdArgs& a, int grid, hipStream_t st) {
+    THN_TINY_SWITCH(thn::launch_softmax_tiny_bwd_f32(is_log, a, grid, st), thn::launch_softmax_tiny_bwd_f16(is_log, a, grid, st),
+                    thn::launch_softmax_tiny_bwd_bf16(is_log, a, grid, st))
+}
+int launch_pnorm_tiny_fwd(int dtype, int mode, bool normalize, const thn::PnormFwdArgs& a, int grid, hipStream_t st) {
+    THN_TINY_SWITCH(thn::launch_pnorm_tiny_fwd_f32(mode, normalize, a, grid, st), thn::launch_pnorm_tiny_fwd_f16(mode, normalize, a, grid, st),
+                    thn::launch_pnorm_tiny_fwd_bf16(mode, normalize, a, grid, st))
+}
+int launch_pnorm_tiny_bwd(int dtype, int mode, const thn::PnormBwdArgs& a, int grid, hipStream_t st) {
+    THN_TINY_SWITCH(thn::launch_pnorm_tiny_bwd_f32(mode, a, grid, st), thn::launch_pnorm_tiny_bwd_f16(mode, a, grid, st),
+                    thn::launch_pnorm_tiny_bwd_bf16(mode, a, grid, st))
+}
+int launch_normalize_tiny_bwd(int dtype, int mode, const thn::NormalizeBwdArgs& a, int grid, hipStream_t st) {
+    THN_TINY_SWITCH(thn::launch_normalize_tiny_bwd_f32(mode, a, grid, st), thn::launch_normalize_tiny_bwd_f16(mode, a, grid, st),
+                    thn::launch_normalize_tiny_bwd_bf16(mode, a, grid, st))
+}
+#undef THN_TINY_SWITCH
+
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 // The bytes a (rows, row_bytes) operand with the given row pitch spans, as a half-open address range, with the
@@ -1351,7 +1400,9 @@ int pnorm_forward(const void* x, int64_t x_batch_stride, int64_t x_row_stride, v
     hipStream_t st = static_cast<hipStream_t>(stream);
     int lrc;
     OneSumFlatPlan fp;
-    if (rp.engine && uniform && plan_one_sum_flat(kPnormFwd, aligned, rp.rows, K, dtype, &fp)) {
+    if (rp.engine && uniform && tiny_rows(kPnormFwd, K, dtype)) {
+        lrc = launch_pnorm_tiny_fwd(dtype, mode_of(rp.p_int), normalize, a, tiny_grid(rp.rows, current_cu_count()), st);
+    } else if (rp.engine && uniform && plan_one_sum_flat(kPnormFwd, aligned, rp.rows, K, dtype, &fp)) {
         a.n_vecs = fp.n_vecs;
         lrc = launch_pnorm_flat_fwd(dtype, mode_of(rp.p_int), normalize, aligned, fp, a, st);
     } else if (rp.engine) {
@@ -1536,6 +1587,16 @@ int thn_norm_query_launch(int which, int is_layernorm, int64_t M, int64_t N, int
         shape[1] = block;
         shape[2] = block;
         shape[3] = grid;
+        shape[4] = 0;
+        return THN_OK;
+    }
+    if (which >= kSoftmaxFwd && which <= kNormalizeBwd && tiny_rows(which, N, x_dtype)) {
+        const int tiny_cus = current_cu_count();
+        if (tiny_cus <= 0) return THN_E_DEVICE;
+        shape[0] = thn::kTinyRows;     // a lane per row: rows per lane and step, ONE lane per row
+        shape[1] = 1;
+        shape[2] = thn::kTinyBlock;
+        shape[3] = tiny_grid(M, tiny_cus);
         shape[4] = 0;
         return THN_OK;
     }
@@ -1786,6 +1847,21 @@ int thn_softmax_fwd(const void* x, int64_t x_row_stride, void* y, int64_t y_row_
     const bool aligned = (N % vec_elems) == 0 && aligned16(x) && aligned16(y) && (x_row_stride * bytes) % 16 == 0 &&
                          (y_row_stride * bytes) % 16 == 0;
     const bool is_log = kind == THN_LOGSOFTMAX;
+    if (tiny_rows(kSoftmaxFwd, N, dtype)) {
+        const int cus = current_cu_count();
+        if (cus <= 0) return THN_E_DEVICE;
+        SoftmaxFwdArgs a{};
+        a.x = static_cast<const char*>(x);
+        a.y = static_cast<char*>(y);
+        a.x_stride_bytes = x_row_stride * bytes;
+        a.y_stride_bytes = y_row_stride * bytes;
+        a.M = M;
+        a.n_cols = static_cast<int>(N);
+        a.sign = kind == THN_SOFTMIN ? -1.0f : 1.0f;
+        const int lrc = launch_softmax_tiny_fwd(dtype, is_log, a, tiny_grid(M, cus), static_cast<hipStream_t>(stream));
+        if (lrc > 0) return THN_E_SHAPE;
+        return lrc == 0 ? THN_OK : THN_E_LAUNCH;
+    }
     OneSumFlatPlan fp;
     if (plan_one_sum_flat(kSoftmaxFwd, aligned, M, N, dtype, &fp)) {
         SoftmaxFwdArgs a{};
@@ -1858,6 +1934,23 @@ int thn_softmax_bwd(const void* y, int64_t y_row_stride, const void* dy, int64_t
                          (y_row_stride * bytes) % 16 == 0 && (dy_row_stride * bytes) % 16 == 0 &&
                          (dx_row_stride * bytes) % 16 == 0;
     const bool is_log = kind == THN_LOGSOFTMAX;
+    if (tiny_rows(kSoftmaxBwd, N, dtype)) {
+        const int cus = current_cu_count();
+        if (cus <= 0) return THN_E_DEVICE;
+        SoftmaxBwdArgs a{};
+        a.y = static_cast<const char*>(y);
+        a.dy = static_cast<const char*>(dy);
+        a.dx = static_cast<char*>(dx);
+        a.y_stride_bytes = y_row_stride * bytes;
+        a.dy_stride_bytes = dy_row_stride * bytes;
+        a.dx_stride_bytes = dx_row_stride * bytes;
+        a.M = M;
+        a.n_cols = static_cast<int>(N);
+        a.sign = kind == THN_SOFTMIN ? -1.0f : 1.0f;
+        const int lrc = launch_softmax_tiny_bwd(dtype, is_log, a, tiny_grid(M, cus), static_cast<hipStream_t>(stream));
+        if (lrc > 0) return THN_E_SHAPE;
+        return lrc == 0 ? THN_OK : THN_E_LAUNCH;
+    }
     OneSumFlatPlan fp;
     if (plan_one_sum_flat(kSoftmaxBwd, aligned, M, N, dtype, &fp)) {
         SoftmaxBwdArgs a{};
@@ -1938,7 +2031,9 @@ int thn_pnorm_bwd(const void* x, int64_t x_batch_stride, int64_t x_row_stride, c
     hipStream_t st = static_cast<hipStream_t>(stream);
     int lrc;
     OneSumFlatPlan fp;
-    if (rp.engine && uniform && plan_one_sum_flat(kPnormBwd, aligned, rp.rows, K, dtype, &fp)) {
+    if (rp.engine && uniform && tiny_rows(kPnormBwd, K, dtype)) {
+        lrc = launch_pnorm_tiny_bwd(dtype, mode_of(rp.p_int), a, tiny_grid(rp.rows, current_cu_count()), st);
+    } else if (rp.engine && uniform && plan_one_sum_flat(kPnormBwd, aligned, rp.rows, K, dtype, &fp)) {
         a.n_vecs = fp.n_vecs;
         lrc = launch_pnorm_flat_bwd(dtype, mode_of(rp.p_int), aligned, fp, a, st);
     } else if (rp.engine) {
@@ -2006,7 +2101,9 @@ int thn_normalize_bwd(const void* x, int64_t x_batch_stride, int64_t x_row_strid
     hipStream_t st = static_cast<hipStream_t>(stream);
     int lrc;
     OneSumFlatPlan fp;
-    if (rp.engine && uniform && plan_one_sum_flat(kNormalizeBwd, aligned, rp.rows, K, dtype, &fp)) {
+    if (rp.engine && uniform && tiny_rows(kNormalizeBwd, K, dtype)) {
+        lrc = launch_normalize_tiny_bwd(dtype, mode_of(rp.p_int), a, tiny_grid(rp.rows, current_cu_count()), st);
+    } else if (rp.engine && uniform && plan_one_sum_flat(kNormalizeBwd, aligned, rp.rows, K, dtype, &fp)) {
         a.n_vecs = fp.n_vecs;
         lrc = launch_normalize_flat_bwd(dtype, mode_of(rp.p_int), aligned, fp, a, st);
     } else if (rp.engine) {
