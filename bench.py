@@ -68,6 +68,8 @@ WORKLOADS = {
     # narrow rows, 2^26 elements: one and nine vectors per row (the flat softmax kernels)
     "softmax_bf16_8388608x8_narrow": ("softmax", 8388608, 8, "bf16"),
     "softmax_bf16_932067x72_narrow": ("softmax", 932067, 72, "bf16"),
+    # off the 128-bit path: a ViT's attention row (197 columns, 25 unaligned windows: the flat kernels' other instances)
+    "softmax_bf16_340654x197_ragged": ("softmax", 340654, 197, "bf16"),
     # vocabulary-sized rows, wider than 64 KiB: the looping kernels (two walks per row)
     "logsoftmax_f32_8192x32000_vocab": ("logsoftmax", 8192, 32000, "f32"),
     "logsoftmax_bf16_4096x128256_vocab": ("logsoftmax", 4096, 128256, "bf16"),
@@ -82,6 +84,8 @@ WORKLOADS = {
     # rows of one float32 vector (quaternions) and of nine bfloat16 vectors, 2^26 elements: the flat p-norm kernels
     "normalize_p2_f32_16777216x4_narrow": ("normalize_p2", 16777216, 4, "f32"),
     "normalize_p2_bf16_932067x72_narrow": ("normalize_p2", 932067, 72, "bf16"),
+    # rows shorter than one vector: 3-component float32 vectors, a lane per row
+    "normalize_p2_f32_11184810x3_short": ("normalize_p2", 11184810, 3, "f32"),
     # element-wise activations (thn_act_fwd + thn_act_bwd per step)
     "act_gelu_bf16_16384x4096": ("act_gelu", 16384, 4096, "bf16"),
     "act_gelu_tanh_bf16_16384x4096": ("act_gelu_tanh", 16384, 4096, "bf16"),

@@ -958,13 +958,16 @@ bool plan_one_sum_flat(int which, bool aligned, int64_t M, int64_t N, int dtype,
     // off the 128-bit path: rows of at least one vector (unaligned 16-byte windows, the last one overlapping)
     if (aligned ? N % vec_elems != 0 : N < vec_elems) return false;
     const int n_vecs = static_cast<int>((N + vec_elems - 1) / vec_elems);
-    if (n_vecs > thn::kFlatMaxVecs || ((n_vecs & (n_vecs - 1)) == 0 && n_vecs > 4)) return false;
+    // On the 128-bit path rows of 8, 16 and 32 vectors fill the row kernels' lane groups; off it they are taken here too
+    // (softmax / normalize p = 2, row kernels -> flat: bfloat16 N = 127 62.4 / 50.0 -> 74.3 / 74.8; 255 70.1 / 59.4 -> 71.3 /
+    // 73.7; float32 N = 31 77.8 / 73.3 -> 80.1 / 80.9; 63 66.4 / 59.3 -> 78.6 / 79.0; bfloat16 N = 63 76.9 / 73.1 -> 73.3 / 73.9).
+    if (n_vecs > thn::kFlatMaxVecs || ((n_vecs & (n_vecs - 1)) == 0 && n_vecs > 4 && aligned)) return false;
     const Override& ov = g_override[which];
     // two rows per lane and step, two workgroups per compute unit: best or within a point of it over 2, 4 x 1, 2, 4 at 17
-    // widths; the forward over rows of 17 vectors and more (three rows per wave or fewer) takes four workgroups
-    // (bfloat16 N = 192 72.1 -> 76.7; float32 N = 96 77.0 -> 82.2)
-    const bool one_stream = which == kSoftmaxFwd || which == kPnormFwd;
-    int rows_each = 2, bpc = (one_stream && n_vecs >= 17) ? 4 : 2;
+    // widths; the softmax forward over rows of 17 vectors and more (three rows per wave or fewer) takes four workgroups
+    // (bfloat16 N = 192 72.1 -> 76.7; float32 N = 96 77.0 -> 82.2; the normalize forward is 1-3 points faster with two:
+    // float32 N = 68 / 80 / 96 / 116 75.6 / 79.6 / 79.3 / 78.0 with four, 78.5 / 82.1 / 81.7 / 80.7 with two)
+    int rows_each = 2, bpc = (which == kSoftmaxFwd && n_vecs >= 17) ? 4 : 2;
     if (ov.tpr.load() > 0 || ov.block.load() > 0 || ov.k.load() > 0) {
         if (ov.tpr.load() != n_vecs) return false;                                // a row-kernel shape is forced
         if (ov.block.load() > 0 && ov.block.load() != thn::kFlatBlock) return false;
