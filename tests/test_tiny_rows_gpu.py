@@ -1,7 +1,8 @@
 """GPU parity of the lane-per-row kernels for rows shorter than one 16-byte vector (csrc/thn_tiny.h): softmax / softmin /
 log-softmax and row p-norm / normalize over 1 to 3 float32 columns and 1 to 7 columns of a 16-bit type, against the CPU
-oracle with the tolerances of the families' parity tests; row counts around a wave, a workgroup and a grid step; rows
-that are columns of a wider buffer; masked logits; tensors whose batches do not fold (the row kernels' element-wise
+oracle with the tolerances of the families' parity tests; row counts around a wave, a workgroup and a grid step (dense
+rows behind aligned pointers go through LDS in whole vectors, the last incomplete batch of 64 rows by element accesses);
+rows that are columns of a wider buffer and rows behind a misaligned pointer (element accesses); masked logits; tensors whose batches do not fold (the row kernels' element-wise
 instance takes those, as it does under a launch override); run-to-run identical results."""
 import pytest
 import torch
@@ -119,6 +120,16 @@ def test_views_batches_masks_override_and_determinism():
     keep = ~torch.isnan(ref).any(-1)
     assert bool(torch.isnan(y[11]).all()) and bool((y[keep][xm[keep] == float("-inf")] == 0).all())
     assert torch.allclose(y[keep].double(), ref[keep], atol=4e-3)
+    # dense rows behind a pointer one element off 16 bytes: the element accesses instead of the staged vectors
+    announce("misaligned base")
+    for dtype, n in ((torch.bfloat16, 5), (torch.float32, 3)):
+        m = 5000
+        x, dy = sm.make((m, n), dtype, 17, scale=2.0)
+        store = torch.empty(m * n + 1, dtype=dtype, device="cuda")
+        xg = store[1:].view(m, n)
+        xg.copy_(x)
+        assert xg.data_ptr() % 16 != 0
+        sm.run_and_compare("softmax", x, dy, f"tiny softmax misaligned {dtype}", x_gpu=xg)
     # a launch override keeps the row kernels' element-wise instance reachable; both give the oracle's results
     announce("override")
     lib = _native.lib()

@@ -1015,10 +1015,10 @@ int launch_normalize_flat_bwd(int dtype, int mode, bool aligned, const OneSumFla
 
 // ---- rows shorter than one vector: a lane per row (thn_tiny.h) -------------------------------------------------------
 // Softmax and p-norm families, float32 / float16 / bfloat16.  Forward + backward of 2^25 elements, % of 8 TB/s, the row
-// kernels' element-wise instance -> a lane per row, softmax / normalize p = 2: float32 N = 1 2.4 / 2.5 -> 66.8 / 44.7;
-// 2 4.5 / 4.6 -> 61.1 / 52.5; 3 6.4 / 6.4 -> 50.7 / 46.5; bfloat16 N = 2 1.0 / 1.0 -> 24.0 / 22.9; 4 1.8 / 1.8 -> 26.6 /
-// 25.9; 7 3.0 / 2.9 -> 23.5 / 22.5 (two-byte accesses: a wave's store instruction is seven partial lines; torch's own
-// softmax forward moves its bytes at 44-61 % of the peak in float32 and 17-28 % in bfloat16 at these widths).
+// kernels' element-wise instance -> a lane per row (element accesses), softmax / normalize p = 2: float32 N = 1 2.4 / 2.5
+// -> 66.8 / 44.7; 2 4.5 / 4.6 -> 61.1 / 52.5; 3 6.4 / 6.4 -> 50.7 / 46.5; bfloat16 N = 2 1.0 / 1.0 -> 24.0 / 22.9; 4 1.8 /
+// 1.8 -> 26.6 / 25.9; 7 3.0 / 2.9 -> 23.5 / 22.5 (torch's own softmax forward moves its bytes at 44-61 % of the peak in
+// float32 and 17-28 % in bfloat16 at these widths).
 // A launch override with any shape field set keeps the row kernels' element-wise instance (4 x 8 in 256 threads).
 bool tiny_rows(int which, int64_t N, int dtype) {
     const int bytes = elem_bytes(dtype);
@@ -1026,6 +1026,11 @@ bool tiny_rows(int which, int64_t N, int dtype) {
     if (ov.k.load() > 0 || ov.tpr.load() > 0 || ov.block.load() > 0) return false;
     return (bytes == 2 || bytes == 4) && N < 16 / bytes;
 }
+// Dense rows behind aligned pointers go through LDS in whole vectors (TinyStage in thn_tiny.h) from two columns on:
+// forward + backward of 2^25 elements, % of 8 TB/s, element accesses -> staged, softmax / normalize p = 2: bfloat16
+// N = 2 24.0 / 22.9 -> 34.6 / 35.2; 4 26.6 / 25.9 -> 49.6 / 49.1; 7 23.5 / 22.5 -> 48.8 / 47.3; float32 N = 3 50.7 / 46.5 ->
+// 64.5 / 57.0; a single float32 column is one dword per lane already and loses that way (66.8 / 44.7 -> 45.8 / 39.3).
+bool tiny_staged(int64_t N) { return N >= 2; }
 int tiny_grid(int64_t rows, int cus) {
     const int64_t per_block = static_cast<int64_t>(thn::kTinyBlock) * thn::kTinyRows;
     const int64_t blocks = (rows + per_block - 1) / per_block;
@@ -1039,25 +1044,25 @@ int tiny_grid(int64_t rows, int cus) {
         case THN_BF16: return CALL_BF16;                \
         default: return 1;                              \
     }
-int launch_softmax_tiny_fwd(int dtype, bool is_log, const SoftmaxFwdArgs& a, int grid, hipStream_t st) {
-    THN_TINY_SWITCH(thn::launch_softmax_tiny_fwd_f32(is_log, a, grid, st), thn::launch_softmax_tiny_fwd_f16(is_log, a, grid, st),
-                    thn::launch_softmax_tiny_fwd_bf16(is_log, a, grid, st))
+int launch_softmax_tiny_fwd(int dtype, bool is_log, bool staged, const SoftmaxFwdArgs& a, int grid, hipStream_t st) {
+    THN_TINY_SWITCH(thn::launch_softmax_tiny_fwd_f32(is_log, staged, a, grid, st), thn::launch_softmax_tiny_fwd_f16(is_log, staged, a, grid, st),
+                    thn::launch_softmax_tiny_fwd_bf16(is_log, staged, a, grid, st))
 }
-int launch_softmax_tiny_bwd(int dtype, bool is_log, const SoftmaxBwdArgs& a, int grid, hipStream_t st) {
-    THN_TINY_SWITCH(thn::launch_softmax_tiny_bwd_f32(is_log, a, grid, st), thn::launch_softmax_tiny_bwd_f16(is_log, a, grid, st),
-                    thn::launch_softmax_tiny_bwd_bf16(is_log, a, grid, st))
+int launch_softmax_tiny_bwd(int dtype, bool is_log, bool staged, const SoftmaxBwdArgs& a, int grid, hipStream_t st) {
+    THN_TINY_SWITCH(thn::launch_softmax_tiny_bwd_f32(is_log, staged, a, grid, st), thn::launch_softmax_tiny_bwd_f16(is_log, staged, a, grid, st),
+                    thn::launch_softmax_tiny_bwd_bf16(is_log, staged, a, grid, st))
 }
-int launch_pnorm_tiny_fwd(int dtype, int mode, bool normalize, const thn::PnormFwdArgs& a, int grid, hipStream_t st) {
-    THN_TINY_SWITCH(thn::launch_pnorm_tiny_fwd_f32(mode, normalize, a, grid, st), thn::launch_pnorm_tiny_fwd_f16(mode, normalize, a, grid, st),
-                    thn::launch_pnorm_tiny_fwd_bf16(mode, normalize, a, grid, st))
+int launch_pnorm_tiny_fwd(int dtype, int mode, bool normalize, bool staged, const thn::PnormFwdArgs& a, int grid, hipStream_t st) {
+    THN_TINY_SWITCH(thn::launch_pnorm_tiny_fwd_f32(mode, normalize, staged, a, grid, st), thn::launch_pnorm_tiny_fwd_f16(mode, normalize, staged, a, grid, st),
+                    thn::launch_pnorm_tiny_fwd_bf16(mode, normalize, staged, a, grid, st))
 }
-int launch_pnorm_tiny_bwd(int dtype, int mode, const thn::PnormBwdArgs& a, int grid, hipStream_t st) {
-    THN_TINY_SWITCH(thn::launch_pnorm_tiny_bwd_f32(mode, a, grid, st), thn::launch_pnorm_tiny_bwd_f16(mode, a, grid, st),
-                    thn::launch_pnorm_tiny_bwd_bf16(mode, a, grid, st))
+int launch_pnorm_tiny_bwd(int dtype, int mode, bool staged, const thn::PnormBwdArgs& a, int grid, hipStream_t st) {
+    THN_TINY_SWITCH(thn::launch_pnorm_tiny_bwd_f32(mode, staged, a, grid, st), thn::launch_pnorm_tiny_bwd_f16(mode, staged, a, grid, st),
+                    thn::launch_pnorm_tiny_bwd_bf16(mode, staged, a, grid, st))
 }
-int launch_normalize_tiny_bwd(int dtype, int mode, const thn::NormalizeBwdArgs& a, int grid, hipStream_t st) {
-    THN_TINY_SWITCH(thn::launch_normalize_tiny_bwd_f32(mode, a, grid, st), thn::launch_normalize_tiny_bwd_f16(mode, a, grid, st),
-                    thn::launch_normalize_tiny_bwd_bf16(mode, a, grid, st))
+int launch_normalize_tiny_bwd(int dtype, int mode, bool staged, const thn::NormalizeBwdArgs& a, int grid, hipStream_t st) {
+    THN_TINY_SWITCH(thn::launch_normalize_tiny_bwd_f32(mode, staged, a, grid, st), thn::launch_normalize_tiny_bwd_f16(mode, staged, a, grid, st),
+                    thn::launch_normalize_tiny_bwd_bf16(mode, staged, a, grid, st))
 }
 #undef THN_TINY_SWITCH
 
@@ -1404,7 +1409,10 @@ int pnorm_forward(const void* x, int64_t x_batch_stride, int64_t x_row_stride, v
     int lrc;
     OneSumFlatPlan fp;
     if (rp.engine && uniform && tiny_rows(kPnormFwd, K, dtype)) {
-        lrc = launch_pnorm_tiny_fwd(dtype, mode_of(rp.p_int), normalize, a, tiny_grid(rp.rows, current_cu_count()), st);
+        const int64_t row_bytes = K * rp.bytes;
+        const bool dense = tiny_staged(K) && aligned16(x) && a.xmap.row_stride_bytes == row_bytes &&
+                           (!normalize || (aligned16(y) && a.ymap.row_stride_bytes == row_bytes));
+        lrc = launch_pnorm_tiny_fwd(dtype, mode_of(rp.p_int), normalize, dense, a, tiny_grid(rp.rows, current_cu_count()), st);
     } else if (rp.engine && uniform && plan_one_sum_flat(kPnormFwd, aligned, rp.rows, K, dtype, &fp)) {
         a.n_vecs = fp.n_vecs;
         lrc = launch_pnorm_flat_fwd(dtype, mode_of(rp.p_int), normalize, aligned, fp, a, st);
@@ -1861,7 +1869,8 @@ int thn_softmax_fwd(const void* x, int64_t x_row_stride, void* y, int64_t y_row_
         a.M = M;
         a.n_cols = static_cast<int>(N);
         a.sign = kind == THN_SOFTMIN ? -1.0f : 1.0f;
-        const int lrc = launch_softmax_tiny_fwd(dtype, is_log, a, tiny_grid(M, cus), static_cast<hipStream_t>(stream));
+        const bool dense = tiny_staged(N) && aligned16(x) && aligned16(y) && x_row_stride == N && y_row_stride == N;
+        const int lrc = launch_softmax_tiny_fwd(dtype, is_log, dense, a, tiny_grid(M, cus), static_cast<hipStream_t>(stream));
         if (lrc > 0) return THN_E_SHAPE;
         return lrc == 0 ? THN_OK : THN_E_LAUNCH;
     }
@@ -1950,7 +1959,9 @@ int thn_softmax_bwd(const void* y, int64_t y_row_stride, const void* dy, int64_t
         a.M = M;
         a.n_cols = static_cast<int>(N);
         a.sign = kind == THN_SOFTMIN ? -1.0f : 1.0f;
-        const int lrc = launch_softmax_tiny_bwd(dtype, is_log, a, tiny_grid(M, cus), static_cast<hipStream_t>(stream));
+        const bool dense = tiny_staged(N) && aligned16(y) && aligned16(dy) && aligned16(dx) && y_row_stride == N && dy_row_stride == N &&
+                           dx_row_stride == N;
+        const int lrc = launch_softmax_tiny_bwd(dtype, is_log, dense, a, tiny_grid(M, cus), static_cast<hipStream_t>(stream));
         if (lrc > 0) return THN_E_SHAPE;
         return lrc == 0 ? THN_OK : THN_E_LAUNCH;
     }
@@ -2035,7 +2046,10 @@ int thn_pnorm_bwd(const void* x, int64_t x_batch_stride, int64_t x_row_stride, c
     int lrc;
     OneSumFlatPlan fp;
     if (rp.engine && uniform && tiny_rows(kPnormBwd, K, dtype)) {
-        lrc = launch_pnorm_tiny_bwd(dtype, mode_of(rp.p_int), a, tiny_grid(rp.rows, current_cu_count()), st);
+        const int64_t row_bytes = K * rp.bytes;
+        const bool dense = tiny_staged(K) && aligned16(x) && aligned16(dx) && a.xmap.row_stride_bytes == row_bytes &&
+                           a.dxmap.row_stride_bytes == row_bytes;
+        lrc = launch_pnorm_tiny_bwd(dtype, mode_of(rp.p_int), dense, a, tiny_grid(rp.rows, current_cu_count()), st);
     } else if (rp.engine && uniform && plan_one_sum_flat(kPnormBwd, aligned, rp.rows, K, dtype, &fp)) {
         a.n_vecs = fp.n_vecs;
         lrc = launch_pnorm_flat_bwd(dtype, mode_of(rp.p_int), aligned, fp, a, st);
@@ -2105,7 +2119,11 @@ int thn_normalize_bwd(const void* x, int64_t x_batch_stride, int64_t x_row_strid
     int lrc;
     OneSumFlatPlan fp;
     if (rp.engine && uniform && tiny_rows(kNormalizeBwd, K, dtype)) {
-        lrc = launch_normalize_tiny_bwd(dtype, mode_of(rp.p_int), a, tiny_grid(rp.rows, current_cu_count()), st);
+        const int64_t row_bytes = K * rp.bytes;
+        const bool dense = tiny_staged(K) && (!need_x || (aligned16(x) && a.xmap.row_stride_bytes == row_bytes)) &&
+                           (!need_y || (aligned16(y) && a.ymap.row_stride_bytes == row_bytes)) && aligned16(dy) &&
+                           a.gmap.row_stride_bytes == row_bytes && aligned16(dx) && a.dxmap.row_stride_bytes == row_bytes;
+        lrc = launch_normalize_tiny_bwd(dtype, mode_of(rp.p_int), dense, a, tiny_grid(rp.rows, current_cu_count()), st);
     } else if (rp.engine && uniform && plan_one_sum_flat(kNormalizeBwd, aligned, rp.rows, K, dtype, &fp)) {
         a.n_vecs = fp.n_vecs;
         lrc = launch_normalize_flat_bwd(dtype, mode_of(rp.p_int), aligned, fp, a, st);

@@ -5,7 +5,8 @@
 // wave cover one contiguous stretch of memory between them, so every cache line is fetched once), does the row's
 // arithmetic in its own registers -- no exchange between lanes at all -- and stores the columns the same way.  J rows
 // per lane and step are requested before the first is used; the grid is persistent.  The column count is uniform over
-// the launch: the `c < n` tests below are scalar branches, not lane masks.
+// the launch: the `c < n` tests below are scalar branches, not lane masks.  Dense rows behind aligned pointers go through
+// LDS in whole vectors instead (TinyStage below).
 // Arithmetic as the row kernels (softmax_fwd_kernel / softmax_bwd_kernel, pnorm_fwd_kernel / pnorm_bwd_kernel /
 // normalize_bwd_kernel), in float32, with the one rounding on store; float32 / float16 / bfloat16 storage.
 #pragma once
@@ -13,12 +14,14 @@
 #include "thn_dispatch.h"
 #include "thn_pnorm.h"
 #include "thn_softmax.h"
+#include "thn_staged.h"
 
 namespace thn {
 
 constexpr int kTinyBlock = 256;
 constexpr int kTinyRows = 4;        // J: rows per lane and step
 constexpr int kTinyMaxCols = 7;     // one short of a 16-bit vector: the registers a lane spends on a row and stream
+constexpr int kTinyStageBytes = 1024;   // LDS per wave, stream and batch of 64 rows: 64 x 16 bytes
 
 // Row j of this lane in the step that starts at row `base`: consecutive lanes take consecutive rows.
 __device__ __forceinline__ int64_t tiny_row(int64_t base, int j, int64_t threads, int64_t last_row) {
@@ -44,102 +47,206 @@ __device__ __forceinline__ void tiny_store(char* rowp, int n, const float (&f)[C
     }
 }
 
-template <typename T, bool LOGSM>
+// STAGED: dense rows (row r at r * n elements) behind 16-byte aligned pointers.  The 64 rows of a wave and step are then
+// one aligned stretch of 64 * n elements = 4 * n * (bytes per element) vectors: the wave fetches it with one 16-byte load
+// per lane, spreads it through LDS, from where every lane picks up the columns of its row, and sends the results back
+// the same way -- the memory system sees whole vectors instead of 64 two- or four-byte pieces per instruction (a wave's
+// two-byte store is seven partial lines).  The last, incomplete batch of 64 rows of a tensor takes the element accesses.
+template <typename T, int C>
+struct TinyStage {
+    // The wave's stretch of stream `base`, one vector per lane (lanes past its end repeat the last vector).
+    __device__ static __forceinline__ u32x4 fetch(const char* base, int64_t row0, int n, int lane, bool keep) {
+        const int vecs = 4 * n * T::kBytes;
+        const char* p = base + row0 * n * T::kBytes + 16 * (lane < vecs ? lane : vecs - 1);
+        return keep ? ld128_keep(p) : ld128(p);
+    }
+    __device__ static __forceinline__ void spread(u32x4 v, char* lds, int n, int lane, float (&f)[C]) {
+        *reinterpret_cast<u32x4*>(lds + 16 * lane) = v;
+        wave_sync();
+#pragma unroll
+        for (int c = 0; c < C; ++c) {
+            f[c] = 0.0f;
+            if (c < n) f[c] = T::load1(lds, lane * n + c);
+        }
+    }
+    // The lanes' results back through the same LDS (every lane has read its inputs from it: spread() of this batch came
+    // before in program order, and a wave executes its LDS instructions in order).
+    __device__ static __forceinline__ void collect_store(char* base, int64_t row0, char* lds, int n, int lane,
+                                                         const float (&f)[C], bool keep) {
+        wave_sync();
+#pragma unroll
+        for (int c = 0; c < C; ++c) {
+            if (c < n) T::store1(lds, lane * n + c, f[c]);
+        }
+        wave_sync();
+        const int vecs = 4 * n * T::kBytes;
+        const int l = lane < vecs ? lane : vecs - 1;
+        const u32x4 v = *reinterpret_cast<const u32x4*>(lds + 16 * l);
+        char* p = base + row0 * n * T::kBytes + 16 * l;
+        if (keep) st128_keep(p, v);
+        else st128(p, v);
+    }
+};
+
+// First row of the wave's batch j in the step that starts at `base` for this lane, and whether all 64 rows exist.
+__device__ __forceinline__ int64_t tiny_row0(int64_t base, int j, int64_t threads, int lane) {
+    return base - lane + static_cast<int64_t>(j) * threads;
+}
+
+// One stream of a step: J batches of rows, fetched first (staged: one vector per lane and batch; otherwise the elements
+// themselves), handed out batch by batch.
+template <typename T, int C, bool STAGED>
+struct TinyIn {
+    u32x4 v[STAGED ? kTinyRows : 1];
+    float f[STAGED ? 1 : kTinyRows][C];
+    __device__ __forceinline__ void request(const char* base, int64_t stride_bytes, const int64_t (&row)[kTinyRows],
+                                            const int64_t (&row0)[kTinyRows], const bool (&whole)[kTinyRows], int n,
+                                            int lane, bool keep = false) {
+#pragma unroll
+        for (int j = 0; j < kTinyRows; ++j) {
+            if constexpr (STAGED) {
+                if (whole[j]) v[j] = TinyStage<T, C>::fetch(base, row0[j], n, lane, keep);
+            } else {
+                tiny_load<T, C>(base + row[j] * stride_bytes, n, f[j]);
+            }
+        }
+    }
+    // The columns of this lane's row of batch j (staged: through `lds`; an incomplete batch by element loads).
+    __device__ __forceinline__ void take(int j, const char* base, int64_t stride_bytes, int64_t row, bool whole, int n,
+                                         int lane, char* lds, float (&out)[C]) {
+        if constexpr (STAGED) {
+            if (whole) TinyStage<T, C>::spread(v[j], lds, n, lane, out);
+            else tiny_load<T, C>(base + row * stride_bytes, n, out);
+        } else {
+#pragma unroll
+            for (int c = 0; c < C; ++c) out[c] = f[j][c];
+        }
+    }
+};
+
+template <typename T, int C, bool STAGED>
+__device__ __forceinline__ void tiny_out(char* base, int64_t stride_bytes, int64_t row, int64_t row0, bool whole, int n,
+                                         int lane, char* lds, const float (&f)[C], bool keep = false) {
+    if constexpr (STAGED) {
+        if (whole) {
+            TinyStage<T, C>::collect_store(base, row0, lds, n, lane, f, keep);
+            return;
+        }
+    }
+    tiny_store<T, C>(base + row * stride_bytes, n, f);
+}
+
+// The rows of this lane in one step, the first row of each of its wave's batches, and whether a batch is complete.
+#define THN_TINY_STEP_ROWS(M_)                                                                                  \
+    int64_t row[J], row0[J];                                                                                    \
+    bool whole[J];                                                                                              \
+    _Pragma("unroll") for (int j = 0; j < J; ++j) {                                                             \
+        row[j] = tiny_row(base, j, threads, last_row);                                                          \
+        row0[j] = tiny_row0(base, j, threads, lane);                                                            \
+        whole[j] = row0[j] + 64 <= (M_);                                                                        \
+    }
+
+template <typename T, bool LOGSM, bool STAGED>
 __global__ void __launch_bounds__(kTinyBlock) softmax_tiny_fwd_kernel(const SoftmaxFwdArgs a) {
     constexpr int C = T::VEC - 1, J = kTinyRows;
+    __shared__ __align__(16) char stage[STAGED ? (kTinyBlock / 64) * kTinyStageBytes : 16];
     const int n = a.n_cols;
+    const int lane = threadIdx.x & 63;
+    char* lds = stage + (STAGED ? (threadIdx.x >> 6) * kTinyStageBytes : 0);
     const int64_t threads = static_cast<int64_t>(gridDim.x) * kTinyBlock;
     const int64_t last_row = a.M - 1;
     const float neg_inf = OpMax::identity<float>();
-    for (int64_t base = static_cast<int64_t>(blockIdx.x) * kTinyBlock + threadIdx.x; base < a.M; base += J * threads) {
-        int64_t row[J];
-        float x[J][C];
+    for (int64_t base = static_cast<int64_t>(blockIdx.x) * kTinyBlock + threadIdx.x; base - lane < a.M; base += J * threads) {
+        THN_TINY_STEP_ROWS(a.M)
+        TinyIn<T, C, STAGED> in;
+        in.request(a.x, a.x_stride_bytes, row, row0, whole, n, lane);
 #pragma unroll
         for (int j = 0; j < J; ++j) {
-            row[j] = tiny_row(base, j, threads, last_row);
-            tiny_load<T, C>(a.x + row[j] * a.x_stride_bytes, n, x[j]);
-        }
-#pragma unroll
-        for (int j = 0; j < J; ++j) {
+            float x[C];
+            in.take(j, a.x, a.x_stride_bytes, row[j], whole[j], n, lane, lds, x);
             float m = neg_inf;
 #pragma unroll
             for (int c = 0; c < C; ++c) {
-                x[j][c] = c < n ? x[j][c] * a.sign : neg_inf;
-                m = fmaxf(m, x[j][c]);
+                x[c] = c < n ? x[c] * a.sign : neg_inf;
+                m = fmaxf(m, x[c]);
             }
             float s = 0.0f;
 #pragma unroll
             for (int c = 0; c < C; ++c) {
-                const float z = x[j][c] - m;
+                const float z = x[c] - m;
                 const float ez = exp_c(z);              // columns past the row end: exp(-inf) = 0
-                x[j][c] = LOGSM ? z : ez;
+                x[c] = LOGSM ? z : ez;
                 s += ez;
             }
             const float scale = LOGSM ? logf(s) : 1.0f / s;
             float y[C];
 #pragma unroll
-            for (int c = 0; c < C; ++c) y[c] = LOGSM ? x[j][c] - scale : x[j][c] * scale;
-            tiny_store<T, C>(a.y + row[j] * a.y_stride_bytes, n, y);
+            for (int c = 0; c < C; ++c) y[c] = LOGSM ? x[c] - scale : x[c] * scale;
+            tiny_out<T, C, STAGED>(a.y, a.y_stride_bytes, row[j], row0[j], whole[j], n, lane, lds, y, true);
         }
     }
 }
 
-template <typename T, bool LOGSM>
+template <typename T, bool LOGSM, bool STAGED>
 __global__ void __launch_bounds__(kTinyBlock) softmax_tiny_bwd_kernel(const SoftmaxBwdArgs a) {
     constexpr int C = T::VEC - 1, J = kTinyRows;
+    __shared__ __align__(16) char stage[STAGED ? 2 * (kTinyBlock / 64) * kTinyStageBytes : 16];
     const int n = a.n_cols;
+    const int lane = threadIdx.x & 63;
+    char* lds = stage + (STAGED ? (threadIdx.x >> 6) * 2 * kTinyStageBytes : 0);
     const int64_t threads = static_cast<int64_t>(gridDim.x) * kTinyBlock;
     const int64_t last_row = a.M - 1;
-    for (int64_t base = static_cast<int64_t>(blockIdx.x) * kTinyBlock + threadIdx.x; base < a.M; base += J * threads) {
-        int64_t row[J];
-        float y[J][C], g[J][C];
+    for (int64_t base = static_cast<int64_t>(blockIdx.x) * kTinyBlock + threadIdx.x; base - lane < a.M; base += J * threads) {
+        THN_TINY_STEP_ROWS(a.M)
+        TinyIn<T, C, STAGED> iy, ig;
+        iy.request(a.y, a.y_stride_bytes, row, row0, whole, n, lane);
+        ig.request(a.dy, a.dy_stride_bytes, row, row0, whole, n, lane);
 #pragma unroll
         for (int j = 0; j < J; ++j) {
-            row[j] = tiny_row(base, j, threads, last_row);
-            tiny_load<T, C>(a.y + row[j] * a.y_stride_bytes, n, y[j]);
-            tiny_load<T, C>(a.dy + row[j] * a.dy_stride_bytes, n, g[j]);       // columns past the row end read as 0
-        }
-#pragma unroll
-        for (int j = 0; j < J; ++j) {
-            float s = 0.0f;
+            float y[C], g[C];
+            iy.take(j, a.y, a.y_stride_bytes, row[j], whole[j], n, lane, lds, y);
+            ig.take(j, a.dy, a.dy_stride_bytes, row[j], whole[j], n, lane, lds + (STAGED ? kTinyStageBytes : 0), g);
+            float s = 0.0f;                              // columns past the row end read as 0
 #pragma unroll
             for (int c = 0; c < C; ++c) {
-                if constexpr (LOGSM) s += g[j][c];
-                else s = fmaf(y[j][c], g[j][c], s);
+                if constexpr (LOGSM) s += g[c];
+                else s = fmaf(y[c], g[c], s);
             }
             float dx[C];
 #pragma unroll
             for (int c = 0; c < C; ++c) {
                 float d;
-                if constexpr (LOGSM) d = fmaf(-exp_c(y[j][c]), s, g[j][c]);
-                else d = y[j][c] * (g[j][c] - s);
+                if constexpr (LOGSM) d = fmaf(-exp_c(y[c]), s, g[c]);
+                else d = y[c] * (g[c] - s);
                 dx[c] = d * a.sign;
             }
-            tiny_store<T, C>(a.dx + row[j] * a.dx_stride_bytes, n, dx);
+            tiny_out<T, C, STAGED>(a.dx, a.dx_stride_bytes, row[j], row0[j], whole[j], n, lane, lds, dx);
         }
     }
 }
 
 // p-norm family: for tensors whose rows are one folded batch (row r at r * row stride), integer p from 1 to 6.
-template <typename T, int MODE, bool NORMALIZE>
+template <typename T, int MODE, bool NORMALIZE, bool STAGED>
 __global__ void __launch_bounds__(kTinyBlock) pnorm_tiny_fwd_kernel(const PnormFwdArgs a) {
     constexpr int C = T::VEC - 1, J = kTinyRows;
+    constexpr bool kKeepY = NORMALIZE && MODE == kP2;      // what the backward reads again stays in the caches
+    __shared__ __align__(16) char stage[STAGED ? (kTinyBlock / 64) * kTinyStageBytes : 16];
     const int n = a.n_cols;
+    const int lane = threadIdx.x & 63;
+    char* lds = stage + (STAGED ? (threadIdx.x >> 6) * kTinyStageBytes : 0);
     const int64_t threads = static_cast<int64_t>(gridDim.x) * kTinyBlock;
     const int64_t last_row = a.rows - 1;
-    for (int64_t base = static_cast<int64_t>(blockIdx.x) * kTinyBlock + threadIdx.x; base < a.rows; base += J * threads) {
-        int64_t row[J];
-        float x[J][C];
+    for (int64_t base = static_cast<int64_t>(blockIdx.x) * kTinyBlock + threadIdx.x; base - lane < a.rows; base += J * threads) {
+        THN_TINY_STEP_ROWS(a.rows)
+        TinyIn<T, C, STAGED> in;
+        in.request(a.x, a.xmap.row_stride_bytes, row, row0, whole, n, lane, !kKeepY);
 #pragma unroll
         for (int j = 0; j < J; ++j) {
-            row[j] = tiny_row(base, j, threads, last_row);
-            tiny_load<T, C>(a.x + row[j] * a.xmap.row_stride_bytes, n, x[j]);   // columns past the row end read as 0
-        }
+            float x[C];
+            in.take(j, a.x, a.xmap.row_stride_bytes, row[j], whole[j], n, lane, lds, x);
+            float s = 0.0f;                              // columns past the row end read as 0
 #pragma unroll
-        for (int j = 0; j < J; ++j) {
-            float s = 0.0f;
-#pragma unroll
-            for (int c = 0; c < C; ++c) s += norm_term<MODE>(x[j][c], a.p_int);
+            for (int c = 0; c < C; ++c) s += norm_term<MODE>(x[c], a.p_int);
             const float nrm = fmaxf(norm_root<MODE>(s, a.p_int, a.p), a.eps);
             T::store1(a.norms, row[j], nrm);
             if constexpr (NORMALIZE) {
@@ -148,31 +255,36 @@ __global__ void __launch_bounds__(kTinyBlock) pnorm_tiny_fwd_kernel(const PnormF
                 const float nd = residual_divisor(nr);
                 float y[C];
 #pragma unroll
-                for (int c = 0; c < C; ++c) y[c] = div_by_row(x[j][c], nd, rn);
-                tiny_store<T, C>(a.y + row[j] * a.ymap.row_stride_bytes, n, y);
+                for (int c = 0; c < C; ++c) y[c] = div_by_row(x[c], nd, rn);
+                tiny_out<T, C, STAGED>(a.y, a.ymap.row_stride_bytes, row[j], row0[j], whole[j], n, lane, lds, y, kKeepY);
             }
         }
     }
 }
 
-template <typename T, int MODE>
+template <typename T, int MODE, bool STAGED>
 __global__ void __launch_bounds__(kTinyBlock) pnorm_tiny_bwd_kernel(const PnormBwdArgs a) {
     constexpr int C = T::VEC - 1, J = kTinyRows;
+    __shared__ __align__(16) char stage[STAGED ? (kTinyBlock / 64) * kTinyStageBytes : 16];
     const int n = a.n_cols;
+    const int lane = threadIdx.x & 63;
+    char* lds = stage + (STAGED ? (threadIdx.x >> 6) * kTinyStageBytes : 0);
     const int64_t threads = static_cast<int64_t>(gridDim.x) * kTinyBlock;
     const int64_t last_row = a.rows - 1;
-    for (int64_t base = static_cast<int64_t>(blockIdx.x) * kTinyBlock + threadIdx.x; base < a.rows; base += J * threads) {
-        int64_t row[J];
-        float x[J][C], c_n[J], c_g[J];
+    for (int64_t base = static_cast<int64_t>(blockIdx.x) * kTinyBlock + threadIdx.x; base - lane < a.rows; base += J * threads) {
+        THN_TINY_STEP_ROWS(a.rows)
+        TinyIn<T, C, STAGED> in;
+        in.request(a.x, a.xmap.row_stride_bytes, row, row0, whole, n, lane);
+        float c_n[J], c_g[J];
 #pragma unroll
         for (int j = 0; j < J; ++j) {
-            row[j] = tiny_row(base, j, threads, last_row);
-            tiny_load<T, C>(a.x + row[j] * a.xmap.row_stride_bytes, n, x[j]);
             c_n[j] = MODE == kP1 ? 1.0f : T::load1(a.norms, row[j]);
             c_g[j] = T::load1(a.g, row[j]);
         }
 #pragma unroll
         for (int j = 0; j < J; ++j) {
+            float x[C];
+            in.take(j, a.x, a.xmap.row_stride_bytes, row[j], whole[j], n, lane, lds, x);
             float den = c_n[j];
             if constexpr (MODE == kPInt) den = pow_small(c_n[j], a.p_int - 1);
             const float rden = 1.0f / den;
@@ -180,42 +292,47 @@ __global__ void __launch_bounds__(kTinyBlock) pnorm_tiny_bwd_kernel(const PnormB
             float d[C];
 #pragma unroll
             for (int c = 0; c < C; ++c) {
-                const float xv = x[j][c];
+                const float xv = x[c];
                 if constexpr (MODE == kP1) d[c] = c_g[j] * sign_of(xv);
                 else if constexpr (MODE == kP2) d[c] = div_by_row(c_g[j] * xv, den, rden);
                 else d[c] = div_by_row(c_g[j] * sign_of(xv) * pow_small(__builtin_fabsf(xv), a.p_int - 1), den, rden);
             }
-            tiny_store<T, C>(a.dx + row[j] * a.dxmap.row_stride_bytes, n, d);
+            tiny_out<T, C, STAGED>(a.dx, a.dxmap.row_stride_bytes, row[j], row0[j], whole[j], n, lane, lds, d);
         }
     }
 }
 
-template <typename T, int MODE>
+template <typename T, int MODE, bool STAGED>
 __global__ void __launch_bounds__(kTinyBlock) normalize_tiny_bwd_kernel(const NormalizeBwdArgs a) {
     constexpr int C = T::VEC - 1, J = kTinyRows;
     constexpr bool NEED_X = MODE != kP2;
     constexpr bool NEED_Y = MODE != kP1;
+    __shared__ __align__(16) char stage[STAGED ? 3 * (kTinyBlock / 64) * kTinyStageBytes : 16];
     const int n = a.n_cols;
+    const int lane = threadIdx.x & 63;
+    char* lds = stage + (STAGED ? (threadIdx.x >> 6) * 3 * kTinyStageBytes : 0);
     const int64_t threads = static_cast<int64_t>(gridDim.x) * kTinyBlock;
     const int64_t last_row = a.rows - 1;
-    for (int64_t base = static_cast<int64_t>(blockIdx.x) * kTinyBlock + threadIdx.x; base < a.rows; base += J * threads) {
-        int64_t row[J];
-        float x[NEED_X ? J : 1][C], y[NEED_Y ? J : 1][C], g[J][C], c_n[J];
+    for (int64_t base = static_cast<int64_t>(blockIdx.x) * kTinyBlock + threadIdx.x; base - lane < a.rows; base += J * threads) {
+        THN_TINY_STEP_ROWS(a.rows)
+        TinyIn<T, C, STAGED> ix, iy, ig;
+        if constexpr (NEED_X) ix.request(a.x, a.xmap.row_stride_bytes, row, row0, whole, n, lane);
+        if constexpr (NEED_Y) iy.request(a.y, a.ymap.row_stride_bytes, row, row0, whole, n, lane);
+        ig.request(a.g, a.gmap.row_stride_bytes, row, row0, whole, n, lane);
+        float c_n[J];
+#pragma unroll
+        for (int j = 0; j < J; ++j) c_n[j] = T::load1(a.norms, row[j]);
 #pragma unroll
         for (int j = 0; j < J; ++j) {
-            row[j] = tiny_row(base, j, threads, last_row);
-            if constexpr (NEED_X) tiny_load<T, C>(a.x + row[j] * a.xmap.row_stride_bytes, n, x[j]);
-            if constexpr (NEED_Y) tiny_load<T, C>(a.y + row[j] * a.ymap.row_stride_bytes, n, y[j]);
-            tiny_load<T, C>(a.g + row[j] * a.gmap.row_stride_bytes, n, g[j]);  // columns past the row end read as 0
-            c_n[j] = T::load1(a.norms, row[j]);
-        }
-#pragma unroll
-        for (int j = 0; j < J; ++j) {
-            float proj = 0.0f;
+            float x[C], y[C], g[C];
+            if constexpr (NEED_X) ix.take(j, a.x, a.xmap.row_stride_bytes, row[j], whole[j], n, lane, lds, x);
+            if constexpr (NEED_Y) iy.take(j, a.y, a.ymap.row_stride_bytes, row[j], whole[j], n, lane, lds + (STAGED ? kTinyStageBytes : 0), y);
+            ig.take(j, a.g, a.gmap.row_stride_bytes, row[j], whole[j], n, lane, lds + (STAGED ? 2 * kTinyStageBytes : 0), g);
+            float proj = 0.0f;                           // columns past the row end read as 0
 #pragma unroll
             for (int c = 0; c < C; ++c) {
-                if constexpr (MODE == kP1) proj = __builtin_fmaf(x[j][c], g[j][c], proj);
-                else proj = __builtin_fmaf(y[j][c], g[j][c], proj);
+                if constexpr (MODE == kP1) proj = __builtin_fmaf(x[c], g[c], proj);
+                else proj = __builtin_fmaf(y[c], g[c], proj);
             }
             const float nrm = c_n[j];
             const float rn = 1.0f / nrm;
@@ -226,65 +343,70 @@ __global__ void __launch_bounds__(kTinyBlock) normalize_tiny_bwd_kernel(const No
             float d[C];
 #pragma unroll
             for (int c = 0; c < C; ++c) {
-                const float gg = g[j][c];
+                const float gg = g[c];
                 if constexpr (MODE == kP2) {
-                    d[c] = div_by_row(gg - y[j][c] * proj, nd, rn);
+                    d[c] = div_by_row(gg - y[c] * proj, nd, rn);
                 } else if constexpr (MODE == kP1) {
-                    d[c] = div_by_row(gg, nd, rn) - sign_of(x[j][c]) * coef;
+                    d[c] = div_by_row(gg, nd, rn) - sign_of(x[c]) * coef;
                 } else {
-                    const float xv = x[j][c];
+                    const float xv = x[c];
                     d[c] = div_by_row(gg, nd, rn) - sign_of(xv) * pow_small(__builtin_fabsf(xv), a.p_int - 1) * coef;
                 }
             }
-            tiny_store<T, C>(a.dx + row[j] * a.dxmap.row_stride_bytes, n, d);
+            tiny_out<T, C, STAGED>(a.dx, a.dxmap.row_stride_bytes, row[j], row0[j], whole[j], n, lane, lds + (STAGED ? 2 * kTinyStageBytes : 0), d);
         }
     }
 }
 
-// Launchers: 0 launched, 1 no such instance, <0 HIP error.  `mode`: kP1 / kP2 / kPInt.
+// Launchers: 0 launched, 1 no such instance, <0 HIP error.  `mode`: kP1 / kP2 / kPInt; `staged`: every stream is dense
+// (row r at r * n elements) behind a 16-byte aligned pointer.
 #define THN_DECLARE_TINY_LAUNCHERS(NAME)                                                                        \
-    int launch_softmax_tiny_fwd_##NAME(bool is_log, const SoftmaxFwdArgs& a, int grid, hipStream_t st);         \
-    int launch_softmax_tiny_bwd_##NAME(bool is_log, const SoftmaxBwdArgs& a, int grid, hipStream_t st);         \
-    int launch_pnorm_tiny_fwd_##NAME(int mode, bool normalize, const PnormFwdArgs& a, int grid, hipStream_t st); \
-    int launch_pnorm_tiny_bwd_##NAME(int mode, const PnormBwdArgs& a, int grid, hipStream_t st);                \
-    int launch_normalize_tiny_bwd_##NAME(int mode, const NormalizeBwdArgs& a, int grid, hipStream_t st);
+    int launch_softmax_tiny_fwd_##NAME(bool is_log, bool staged, const SoftmaxFwdArgs& a, int grid, hipStream_t st); \
+    int launch_softmax_tiny_bwd_##NAME(bool is_log, bool staged, const SoftmaxBwdArgs& a, int grid, hipStream_t st); \
+    int launch_pnorm_tiny_fwd_##NAME(int mode, bool normalize, bool staged, const PnormFwdArgs& a, int grid, hipStream_t st); \
+    int launch_pnorm_tiny_bwd_##NAME(int mode, bool staged, const PnormBwdArgs& a, int grid, hipStream_t st);   \
+    int launch_normalize_tiny_bwd_##NAME(int mode, bool staged, const NormalizeBwdArgs& a, int grid, hipStream_t st);
 
 THN_DECLARE_TINY_LAUNCHERS(f32)
 THN_DECLARE_TINY_LAUNCHERS(f16)
 THN_DECLARE_TINY_LAUNCHERS(bf16)
 
+#define THN_TINY_RUN(ARGS_T, KERNEL, ...)                                                                       \
+    (staged ? run_kernel<ARGS_T>(KERNEL<T, __VA_ARGS__, true>, a, grid, kTinyBlock, st, nullptr)                \
+            : run_kernel<ARGS_T>(KERNEL<T, __VA_ARGS__, false>, a, grid, kTinyBlock, st, nullptr))
 #define THN_TINY_MODE_CASE(KERNEL, ARGS_T, MODE_)                                                               \
-    if (mode == MODE_) return run_kernel<ARGS_T>(KERNEL<T, MODE_>, a, grid, kTinyBlock, st, nullptr);
+    if (mode == MODE_) return THN_TINY_RUN(ARGS_T, KERNEL, MODE_);
 #define THN_TINY_FWD_MODE_CASE(MODE_)                                                                           \
     if (mode == MODE_) {                                                                                        \
-        return normalize ? run_kernel<PnormFwdArgs>(pnorm_tiny_fwd_kernel<T, MODE_, true>, a, grid, kTinyBlock, st, nullptr)  \
-                         : run_kernel<PnormFwdArgs>(pnorm_tiny_fwd_kernel<T, MODE_, false>, a, grid, kTinyBlock, st, nullptr); \
+        return normalize ? THN_TINY_RUN(PnormFwdArgs, pnorm_tiny_fwd_kernel, MODE_, true)                       \
+                         : THN_TINY_RUN(PnormFwdArgs, pnorm_tiny_fwd_kernel, MODE_, false);                     \
     }
 
 #define THN_DEFINE_TINY_LAUNCHERS(NAME, TYPE)                                                                   \
-    int launch_softmax_tiny_fwd_##NAME(bool is_log, const SoftmaxFwdArgs& a, int grid, hipStream_t st) {        \
+    int launch_softmax_tiny_fwd_##NAME(bool is_log, bool staged, const SoftmaxFwdArgs& a, int grid, hipStream_t st) { \
         using T = TYPE;                                                                                         \
-        return is_log ? run_kernel<SoftmaxFwdArgs>(softmax_tiny_fwd_kernel<T, true>, a, grid, kTinyBlock, st, nullptr)   \
-                      : run_kernel<SoftmaxFwdArgs>(softmax_tiny_fwd_kernel<T, false>, a, grid, kTinyBlock, st, nullptr); \
+        return is_log ? THN_TINY_RUN(SoftmaxFwdArgs, softmax_tiny_fwd_kernel, true)                             \
+                      : THN_TINY_RUN(SoftmaxFwdArgs, softmax_tiny_fwd_kernel, false);                           \
     }                                                                                                           \
-    int launch_softmax_tiny_bwd_##NAME(bool is_log, const SoftmaxBwdArgs& a, int grid, hipStream_t st) {        \
+    int launch_softmax_tiny_bwd_##NAME(bool is_log, bool staged, const SoftmaxBwdArgs& a, int grid, hipStream_t st) { \
         using T = TYPE;                                                                                         \
-        return is_log ? run_kernel<SoftmaxBwdArgs>(softmax_tiny_bwd_kernel<T, true>, a, grid, kTinyBlock, st, nullptr)   \
-                      : run_kernel<SoftmaxBwdArgs>(softmax_tiny_bwd_kernel<T, false>, a, grid, kTinyBlock, st, nullptr); \
+        return is_log ? THN_TINY_RUN(SoftmaxBwdArgs, softmax_tiny_bwd_kernel, true)                             \
+                      : THN_TINY_RUN(SoftmaxBwdArgs, softmax_tiny_bwd_kernel, false);                           \
     }                                                                                                           \
-    int launch_pnorm_tiny_fwd_##NAME(int mode, bool normalize, const PnormFwdArgs& a, int grid, hipStream_t st) { \
+    int launch_pnorm_tiny_fwd_##NAME(int mode, bool normalize, bool staged, const PnormFwdArgs& a, int grid,    \
+                                     hipStream_t st) {                                                          \
         using T = TYPE;                                                                                         \
         THN_TINY_FWD_MODE_CASE(kP1) THN_TINY_FWD_MODE_CASE(kP2) THN_TINY_FWD_MODE_CASE(kPInt)                   \
         return 1;                                                                                               \
     }                                                                                                           \
-    int launch_pnorm_tiny_bwd_##NAME(int mode, const PnormBwdArgs& a, int grid, hipStream_t st) {               \
+    int launch_pnorm_tiny_bwd_##NAME(int mode, bool staged, const PnormBwdArgs& a, int grid, hipStream_t st) {  \
         using T = TYPE;                                                                                         \
         THN_TINY_MODE_CASE(pnorm_tiny_bwd_kernel, PnormBwdArgs, kP1)                                            \
         THN_TINY_MODE_CASE(pnorm_tiny_bwd_kernel, PnormBwdArgs, kP2)                                            \
         THN_TINY_MODE_CASE(pnorm_tiny_bwd_kernel, PnormBwdArgs, kPInt)                                          \
         return 1;                                                                                               \
     }                                                                                                           \
-    int launch_normalize_tiny_bwd_##NAME(int mode, const NormalizeBwdArgs& a, int grid, hipStream_t st) {       \
+    int launch_normalize_tiny_bwd_##NAME(int mode, bool staged, const NormalizeBwdArgs& a, int grid, hipStream_t st) { \
         using T = TYPE;                                                                                         \
         THN_TINY_MODE_CASE(normalize_tiny_bwd_kernel, NormalizeBwdArgs, kP1)                                    \
         THN_TINY_MODE_CASE(normalize_tiny_bwd_kernel, NormalizeBwdArgs, kP2)                                    \
