@@ -162,3 +162,71 @@ def test_random_narrow_norm_problem(seed):
     torch.cuda.synchronize()
     out = dict(y=y.detach(), dx=xg.grad, dw=wg.grad, db=None if bg is None else bg.grad, mean=mean, rstd=rstd)
     parity_util.compare_with_oracle(kind, x, dy, w, b, eps, out, f"random narrow {seed} (strided)", sample_chunks=sample)
+
+
+SHORT_FAMILIES = ["ln", "rms", "softmax", "softmin", "logsoftmax", "norm", "normalize"]
+
+
+def draw_short(seed):
+    """Every row family over rows of 1 to 280 columns, any width -- shorter than a vector (a lane per row), not a whole
+    number of vectors (unaligned windows: the flat kernels' other instances, the row kernels' narrow shapes), whole
+    vectors (the flat and staged kernels) -- 1 to 200000 rows, a third of them as column blocks of a wider buffer that
+    start 0 to 3 columns in (rows behind pointers and pitches off 16 bytes)."""
+    rng = np.random.default_rng(31000 + seed)
+    family = SHORT_FAMILIES[seed % len(SHORT_FAMILIES)]
+    dtype = [torch.bfloat16, torch.float16, torch.float32][int(rng.integers(3))]
+    n = int(rng.integers(1, 281)) if seed % 3 else int(rng.integers(1, 40))
+    m = max(1, min(log_uniform(rng, 1, 200000), 6_000_000 // n))
+    if family in ("norm", "normalize") and n < 8:
+        m = min(m, 2000)        # nearly one-dimensional rows among many thousand: see test_tiny_rows_gpu.py
+    offset = int(rng.integers(0, 4)) if rng.random() < 0.33 else -1
+    return family, dtype, m, n, offset, rng
+
+
+@pytest.mark.parametrize("seed", range(140))
+def test_random_short_row_problem(seed):
+    family, dtype, m, n, offset, rng = draw_short(seed)
+    print(f"\n[case] random short seed={seed} {family} {dtype} M={m} N={n} offset={offset}", flush=True)
+    g = torch.Generator().manual_seed(seed)
+    pad = 0 if offset < 0 else offset + int(rng.integers(1, 6))
+    off = max(offset, 0)
+    xb = (torch.randn(m, n + pad, generator=g) * 2 + 0.25).to(dtype)
+    gb = torch.randn(m, n + pad, generator=g).to(dtype)
+    x, dy = xb[:, off:off + n].contiguous(), gb[:, off:off + n].contiguous()
+    what = f"random short {seed} {family} {m}x{n}"
+    eps = 1e-5 if n >= 16 else 1e-2
+    sample = 8 if m * n > 4_000_000 else None
+    if family in ("ln", "rms"):
+        w = (1 + 0.1 * torch.randn(n, generator=g)).to(dtype)
+        b = (0.1 * torch.randn(n, generator=g)).to(dtype) if family == "ln" else None
+        if not pad:
+            parity_util.run_and_compare(family, x, dy, w, b, eps, what, sample_chunks=sample)
+            return
+        from TritonHub.Normalization.layernorm import layernorm
+        from TritonHub.Normalization.rmsnorm import rmsnorm
+        xg = xb.cuda()[:, off:off + n].detach().requires_grad_(True)
+        wg = w.cuda().requires_grad_(True)
+        bg = None if b is None else b.cuda().requires_grad_(True)
+        if family == "ln":
+            y = layernorm.apply(xg, wg, bg, eps)
+            mean, rstd = y.grad_fn.saved_tensors[3], y.grad_fn.saved_tensors[4]
+        else:
+            y = rmsnorm.apply(xg, wg, eps)
+            mean, rstd = None, y.grad_fn.saved_tensors[2]
+        y.backward(gb.cuda()[:, off:off + n])
+        torch.cuda.synchronize()
+        out = dict(y=y.detach(), dx=xg.grad, dw=wg.grad, db=None if bg is None else bg.grad, mean=mean, rstd=rstd)
+        parity_util.compare_with_oracle(family, x, dy, w, b, eps, out, what + " (strided)", sample_chunks=sample)
+    elif family in ("softmax", "softmin", "logsoftmax"):
+        x_gpu = xb.cuda()[:, off:off + n].detach() if pad else None
+        dy_gpu = gb.cuda()[:, off:off + n] if pad else None
+        softmax_t.run_and_compare(family, x, dy, what, x_gpu=x_gpu, dy_gpu=dy_gpu)
+    else:
+        p = [1, 2, 3, 2, 4, 2][int(rng.integers(6))]
+        x_gpu = xb.cuda()[:, off:off + n].unsqueeze(0).detach() if pad else None
+        if family == "norm":
+            gn = torch.rand(1, m, generator=g).to(dtype)
+            pnorm_t.compare_norm(x.view(1, m, n), gn, p, 1e-6, f"{what} p={p}", x_gpu=x_gpu)
+        else:
+            gy_gpu = gb.cuda()[:, off:off + n].unsqueeze(0) if pad else None
+            pnorm_t.compare_normalize(x.view(1, m, n), dy.view(1, m, n), p, 1e-6, f"{what} p={p}", x_gpu=x_gpu, gy_gpu=gy_gpu)
