@@ -1,5 +1,5 @@
-"""GPU parity of the lane-per-row kernels for rows shorter than one 16-byte vector (csrc/thn_tiny.h): softmax / softmin /
-log-softmax and row p-norm / normalize over 1 to 3 float32 columns and 1 to 7 columns of a 16-bit type, against the CPU
+"""GPU parity of the lane-per-row kernels for rows shorter than one 16-byte vector (csrc/thn_tiny.h): LayerNorm / RMSNorm,
+softmax / softmin / log-softmax and row p-norm / normalize over 1 to 3 float32 columns and 1 to 7 columns of a 16-bit type, against the CPU
 oracle with the tolerances of the families' parity tests; row counts around a wave, a workgroup and a grid step (dense
 rows behind aligned pointers go through LDS in whole vectors, the last incomplete batch of 64 rows by element accesses);
 rows that are columns of a wider buffer and rows behind a misaligned pointer (element accesses); masked logits; tensors whose batches do not fold (the row kernels' element-wise
@@ -63,6 +63,77 @@ def test_pnorm_family_over_every_short_width(dtype):
                 dx = ops_launch.normalize_bwd(xg, y, nrm, gy.cuda(), p)
                 bound = 16 * 2.0 ** -24 * gy.float().abs() / x.float().abs().clamp_min(1e-6)
                 assert bool((dx.float().cpu().abs() <= bound + 1e-30).all()), f"tiny normalize K=1 p={p}"
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("kind", ["ln", "rms"])
+def test_norm_kernels_over_every_short_width(kind, dtype):
+    """LayerNorm / RMSNorm over fewer columns than a vector holds: y, the saved statistics, dx, dW and dB against the
+    oracle (eps = 1e-2: rows of a few elements are often nearly constant, and with a tiny eps rstd multiplies the float32
+    rounding of x - mean beyond any fixed bound); 16-bit and float32 parameters; rows as columns of a wider buffer."""
+    from parity_util import compare_with_oracle, run_and_compare
+    from TritonHub.Normalization.layernorm import layernorm
+    from TritonHub.Normalization.rmsnorm import rmsnorm
+    g = torch.Generator().manual_seed(41)
+    for n in widths(dtype):
+        for m in (1, 63, 4 * 256 + 3, 70001):
+            announce(f"{kind} {dtype} N={n} M={m}")
+            for which in (0, 1):
+                q = query_launch(which, kind == "ln", m, n, dtype)
+                assert q[:3] == (4, 1, 256) and q[4] == 0, q
+            x = (torch.randn(m, n, generator=g) * 2 + 0.5).to(dtype)
+            dy = torch.randn(m, n, generator=g).to(dtype)
+            w = 1 + 0.1 * torch.randn(n, generator=g)
+            b = 0.1 * torch.randn(n, generator=g) if kind == "ln" else None
+            run_and_compare(kind, x, dy, w.to(dtype), None if b is None else b.to(dtype), 1e-2, f"tiny {kind} N={n} M={m}")
+            if m == 63 and dtype != torch.float32:
+                run_and_compare(kind, x, dy, w, b, 1e-2, f"tiny {kind} N={n} M={m}, float32 parameters")
+        # columns 2 .. 2 + n of a buffer of n + 5 columns
+        m = 3001
+        xb = (torch.randn(m, n + 5, generator=g) * 2 + 0.5).to(dtype)
+        gb = torch.randn(m, n + 5, generator=g).to(dtype)
+        x, dy = xb[:, 2:2 + n].contiguous(), gb[:, 2:2 + n].contiguous()
+        w = (1 + 0.1 * torch.randn(n, generator=g)).to(dtype)
+        b = (0.1 * torch.randn(n, generator=g)).to(dtype) if kind == "ln" else None
+        xg = xb.cuda()[:, 2:2 + n].detach().requires_grad_(True)
+        wg = w.cuda().requires_grad_(True)
+        bg = None if b is None else b.cuda().requires_grad_(True)
+        if kind == "ln":
+            y = layernorm.apply(xg, wg, bg, 1e-2)
+            mean, rstd = y.grad_fn.saved_tensors[3], y.grad_fn.saved_tensors[4]
+        else:
+            y = rmsnorm.apply(xg, wg, 1e-2)
+            mean, rstd = None, y.grad_fn.saved_tensors[2]
+        y.backward(gb.cuda()[:, 2:2 + n])
+        torch.cuda.synchronize()
+        out = dict(y=y.detach(), dx=xg.grad, dw=wg.grad, db=None if bg is None else bg.grad, mean=mean, rstd=rstd)
+        compare_with_oracle(kind, x, dy, w, b, 1e-2, out, f"tiny {kind} N={n} column block")
+
+
+def test_norm_kernels_short_rows_bits():
+    """Run-to-run identical (dW / dB are summed in a fixed order); dense rows (through LDS in whole vectors) and the same
+    rows behind a misaligned pointer (element accesses) agree to float32 rounding."""
+    from TritonHub.Normalization import _launch as nl
+    g = torch.Generator().manual_seed(8)
+    m, n = 300001, 3
+    x = torch.randn(m, n, generator=g).cuda(); dy = torch.randn(m, n, generator=g).cuda()
+    w = (1 + 0.1 * torch.randn(n, generator=g)).cuda(); b = (0.1 * torch.randn(n, generator=g)).cuda()
+
+    def run(xx, gg):
+        y, mean, rstd = nl.norm_fwd(xx, w, b, 1e-5, True)
+        dx, dw, db = nl.norm_bwd(xx, gg, w, b, mean, rstd, True)
+        torch.cuda.synchronize()
+        return y, mean, rstd, dx, dw, db
+
+    first = run(x, dy)
+    for u, v in zip(first, run(x, dy)):
+        assert torch.equal(u, v)
+    store = torch.empty(m * n + 1, device="cuda"); gstore = torch.empty(m * n + 1, device="cuda")
+    xm = store[1:].view(m, n); gm = gstore[1:].view(m, n)
+    xm.copy_(x); gm.copy_(dy)
+    assert xm.data_ptr() % 16 != 0
+    for u, v in zip(first, run(xm, gm)):
+        assert torch.allclose(u, v, rtol=2e-5, atol=2e-5)      # two compiled forms of one formula: float32 roundings apart
 
 
 @pytest.mark.parametrize("dtype", DTYPES)

@@ -1064,6 +1064,22 @@ int launch_normalize_tiny_bwd(int dtype, int mode, bool staged, const thn::Norma
     THN_TINY_SWITCH(thn::launch_normalize_tiny_bwd_f32(mode, staged, a, grid, st), thn::launch_normalize_tiny_bwd_f16(mode, staged, a, grid, st),
                     thn::launch_normalize_tiny_bwd_bf16(mode, staged, a, grid, st))
 }
+int launch_norm_tiny_fwd(int dtype, bool ln, bool staged, const FwdArgs& a, int grid, hipStream_t st) {
+    THN_TINY_SWITCH(thn::launch_norm_tiny_fwd_f32(ln, staged, a, grid, st), thn::launch_norm_tiny_fwd_f16(ln, staged, a, grid, st),
+                    thn::launch_norm_tiny_fwd_bf16(ln, staged, a, grid, st))
+}
+int launch_norm_tiny_bwd(int dtype, bool ln, bool staged, const BwdArgs& a, int grid, hipStream_t st) {
+    THN_TINY_SWITCH(thn::launch_norm_tiny_bwd_f32(ln, staged, a, grid, st), thn::launch_norm_tiny_bwd_f16(ln, staged, a, grid, st),
+                    thn::launch_norm_tiny_bwd_bf16(ln, staged, a, grid, st))
+}
+// The norm backward writes one partial row per workgroup: its grid stays within what thn_norm_bwd_workspace_bytes()
+// promises for narrow rows (kStagedBlocksPerCu workgroups per compute unit, at most one per row).
+int tiny_bwd_grid(int64_t rows, int cus) {
+    const int64_t per_block = static_cast<int64_t>(thn::kTinyBlock) * thn::kTinyRows;
+    const int64_t blocks = (rows + per_block - 1) / per_block;
+    const int64_t cap = static_cast<int64_t>(cus) * kStagedBlocksPerCu;
+    return static_cast<int>(blocks < cap ? blocks : cap);
+}
 #undef THN_TINY_SWITCH
 
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
@@ -1178,6 +1194,29 @@ int norm_forward(const void* x, int64_t x_row_stride, void* y, int64_t y_row_str
                          (x_row_stride * bytes) % 16 == 0 && (y_row_stride * bytes) % 16 == 0;
     Plan p;
     const bool fused = act != thn::kNoAct;
+    if (!fused && tiny_rows(kNormFwd, N, x_dtype)) {        // rows shorter than one vector: a lane per row
+        const int cus = current_cu_count();
+        if (cus <= 0) return THN_E_DEVICE;
+        FwdArgs t{};
+        t.x = static_cast<const char*>(x);
+        t.y = static_cast<char*>(y);
+        t.w = w;
+        t.b = b;
+        t.mean = mean;
+        t.rstd = rstd;
+        t.x_stride_bytes = x_row_stride * bytes;
+        t.y_stride_bytes = y_row_stride * bytes;
+        t.M = M;
+        t.n_cols = static_cast<int>(N);
+        t.w_dtype = w_dtype;
+        t.eps = eps;
+        t.inv_n = 1.0f / static_cast<float>(N);
+        t.keep_x = keep_x ? 1 : 0;
+        const bool dense = tiny_staged(N) && aligned16(x) && aligned16(y) && x_row_stride == N && y_row_stride == N;
+        const int lrc = launch_norm_tiny_fwd(x_dtype, ln, dense, t, tiny_grid(M, cus), static_cast<hipStream_t>(stream));
+        if (lrc > 0) return THN_E_SHAPE;
+        return lrc == 0 ? THN_OK : THN_E_LAUNCH;
+    }
     StagedPlan sp;
     FlatPlan fp;
     const bool staged = !fused && plan_staged(kNormFwd, ln, aligned, M, N, x_dtype, &sp);
@@ -1257,9 +1296,16 @@ int norm_backward_stage1(const void* x, int64_t x_row_stride, const void* dy, in
     const int variant = fused ? ((ln ? 1 : 0) | (act << 1)) : (ln ? 1 : 0);
     StagedPlan sp;
     FlatPlan fp;
-    const bool staged = !fused && plan_staged(kNormBwd, ln, aligned, M, N, x_dtype, &sp);
-    const bool flat = !fused && !staged && plan_flat(kNormBwd, ln, aligned, M, N, x_dtype, &fp);
-    if (staged) {
+    const bool tiny = !fused && tiny_rows(kNormBwd, N, x_dtype);      // rows shorter than one vector: a lane per row
+    const bool staged = !fused && !tiny && plan_staged(kNormBwd, ln, aligned, M, N, x_dtype, &sp);
+    const bool flat = !fused && !tiny && !staged && plan_flat(kNormBwd, ln, aligned, M, N, x_dtype, &fp);
+    if (tiny) {
+        const int cus = current_cu_count();
+        if (cus <= 0) return THN_E_DEVICE;
+        p.n_vecs = 1;
+        p.grid = tiny_bwd_grid(M, cus);
+        p.s = Shape{thn::kTinyRows, 1, thn::kTinyBlock};
+    } else if (staged) {
         p.n_vecs = sp.n_vecs;
         p.grid = sp.grid;
         p.s = Shape{sp.passes, sp.n_vecs, thn::kStagedBlock};
@@ -1298,8 +1344,11 @@ int norm_backward_stage1(const void* x, int64_t x_row_stride, const void* dy, in
     const RowStream streams[3] = {{x, a.x_stride_bytes}, {dy, a.dy_stride_bytes}, {dx, a.dx_stride_bytes}};
     a.line_shift = line_shift_ok(aligned, p.s, p.grid, p.n_vecs, streams, 3) ? 1 : 0;
     hipStream_t st = static_cast<hipStream_t>(stream);
-    if (flat || staged) a.line_shift = 0;
-    const int lrc = staged ? launch_staged_bwd(x_dtype, ln, sp, a, st, nullptr)
+    if (flat || staged || tiny) a.line_shift = 0;
+    const bool dense = tiny && tiny_staged(N) && aligned16(x) && aligned16(dy) && aligned16(dx) && x_row_stride == N &&
+                       dy_row_stride == N && dx_row_stride == N;
+    const int lrc = tiny ? launch_norm_tiny_bwd(x_dtype, ln, dense, a, p.grid, st)
+                  : staged ? launch_staged_bwd(x_dtype, ln, sp, a, st, nullptr)
                   : flat ? launch_flat_bwd(x_dtype, ln, aligned, fp, a, st, nullptr)
                   : fused ? launch_fused_bwd(x_dtype, variant, aligned, p.s, a, p.grid, st, nullptr)
                           : launch_bwd(x_dtype, ln, aligned, p.s, a, p.grid, st, nullptr);
@@ -1601,13 +1650,13 @@ int thn_norm_query_launch(int which, int is_layernorm, int64_t M, int64_t N, int
         shape[4] = 0;
         return THN_OK;
     }
-    if (which >= kSoftmaxFwd && which <= kNormalizeBwd && tiny_rows(which, N, x_dtype)) {
+    if (which <= kNormalizeBwd && tiny_rows(which, N, x_dtype)) {
         const int tiny_cus = current_cu_count();
         if (tiny_cus <= 0) return THN_E_DEVICE;
         shape[0] = thn::kTinyRows;     // a lane per row: rows per lane and step, ONE lane per row
         shape[1] = 1;
         shape[2] = thn::kTinyBlock;
-        shape[3] = tiny_grid(M, tiny_cus);
+        shape[3] = which == kNormBwd ? tiny_bwd_grid(M, tiny_cus) : tiny_grid(M, tiny_cus);
         shape[4] = 0;
         return THN_OK;
     }

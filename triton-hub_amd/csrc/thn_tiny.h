@@ -1,5 +1,5 @@
-// Rows SHORTER than one 16-byte vector (1 to 3 float32 columns, 1 to 7 of a 16-bit type) for the softmax and the p-norm /
-// normalize families: class scores over a handful of classes, 2- and 3-component vectors.  No vector slot fits such a
+// Rows SHORTER than one 16-byte vector (1 to 3 float32 columns, 1 to 7 of a 16-bit type) for the norm kernels, the softmax
+// and the p-norm / normalize families: class scores over a handful of classes, 2- and 3-component vectors.  No vector slot fits such a
 // row, and the row kernels' element-wise instances (ElemIo<T>) spend 32 slots of 8 lanes on it.  Here ONE LANE OWNS A
 // WHOLE ROW: it loads the row's columns one element at a time (the rows being dense or evenly pitched, the 64 lanes of a
 // wave cover one contiguous stretch of memory between them, so every cache line is fetched once), does the row's
@@ -7,8 +7,9 @@
 // per lane and step are requested before the first is used; the grid is persistent.  The column count is uniform over
 // the launch: the `c < n` tests below are scalar branches, not lane masks.  Dense rows behind aligned pointers go through
 // LDS in whole vectors instead (TinyStage below).
-// Arithmetic as the row kernels (softmax_fwd_kernel / softmax_bwd_kernel, pnorm_fwd_kernel / pnorm_bwd_kernel /
-// normalize_bwd_kernel), in float32, with the one rounding on store; float32 / float16 / bfloat16 storage.
+// Arithmetic as the row kernels (norm_fwd_kernel / norm_bwd_kernel, softmax_fwd_kernel / softmax_bwd_kernel,
+// pnorm_fwd_kernel / pnorm_bwd_kernel / normalize_bwd_kernel), in float32, with the one rounding on store; float32 /
+// float16 / bfloat16 storage.
 #pragma once
 
 #include "thn_dispatch.h"
@@ -358,6 +359,158 @@ __global__ void __launch_bounds__(kTinyBlock) normalize_tiny_bwd_kernel(const No
     }
 }
 
+// LayerNorm / RMSNorm over rows shorter than one vector.  Arithmetic as norm_fwd_kernel / norm_bwd_kernel (LayerNorm:
+// mean0, then {sum d, sum d^2} with the delta correction; the backward's {sum u*wdy, sum wdy, sum u}); the weights and
+// the bias are launch-uniform values every lane loads once.  dW / dB: per-lane column sums (float64 for float32 rows),
+// added up by the workgroup at the end, in a fixed order, into ONE float32 partial row (the second stage is the row
+// kernels').
+template <typename T, bool LN, bool STAGED>
+__global__ void __launch_bounds__(kTinyBlock) norm_tiny_fwd_kernel(const FwdArgs a) {
+    constexpr int C = T::VEC - 1, J = kTinyRows;
+    __shared__ __align__(16) char stage[STAGED ? (kTinyBlock / 64) * kTinyStageBytes : 16];
+    const int n = a.n_cols;
+    const int lane = threadIdx.x & 63;
+    char* lds = stage + (STAGED ? (threadIdx.x >> 6) * kTinyStageBytes : 0);
+    const int64_t threads = static_cast<int64_t>(gridDim.x) * kTinyBlock;
+    const int64_t last_row = a.M - 1;
+    float wr[1][T::VEC], br[1][T::VEC];
+    const int first[1] = {0};
+    load_params_clamped<1, T::VEC, false>(wr, a.w, a.w_dtype, first, n, 1.0f);
+    load_params_clamped<1, T::VEC, false>(br, LN ? a.b : nullptr, a.w_dtype, first, n, 0.0f);
+    for (int64_t base = static_cast<int64_t>(blockIdx.x) * kTinyBlock + threadIdx.x; base - lane < a.M; base += J * threads) {
+        THN_TINY_STEP_ROWS(a.M)
+        TinyIn<T, C, STAGED> in;
+        in.request(a.x, a.x_stride_bytes, row, row0, whole, n, lane, a.keep_x != 0);
+#pragma unroll
+        for (int j = 0; j < J; ++j) {
+            float x[C];
+            in.take(j, a.x, a.x_stride_bytes, row[j], whole[j], n, lane, lds, x);   // columns past the row end read as 0
+            float mean = 0.0f, delta = 0.0f, rstd;
+            if constexpr (LN) {
+                float s = 0.0f;
+#pragma unroll
+                for (int c = 0; c < C; ++c) s += x[c];
+                const float mean0 = s * a.inv_n;
+                float q0 = 0.0f, q1 = 0.0f;
+#pragma unroll
+                for (int c = 0; c < C; ++c) {
+                    const float d = x[c] - mean0;
+                    x[c] = d;
+                    const float dm = c < n ? d : 0.0f;
+                    q0 += dm;
+                    q1 = fmaf(dm, dm, q1);
+                }
+                delta = q0 * a.inv_n;
+                const float var = fmaxf(fmaf(-delta, delta, q1 * a.inv_n), 0.0f);
+                rstd = rsqrt_refined(var + a.eps);
+                mean = mean0 + delta;
+            } else {
+                float q = 0.0f;
+#pragma unroll
+                for (int c = 0; c < C; ++c) q = fmaf(x[c], x[c], q);
+                rstd = rsqrt_refined(fmaf(q, a.inv_n, a.eps));
+            }
+            float y[C];
+#pragma unroll
+            for (int c = 0; c < C; ++c) {
+                if constexpr (LN) y[c] = fmaf((x[c] - delta) * rstd, wr[0][c], br[0][c]);
+                else y[c] = x[c] * rstd * wr[0][c];
+            }
+            tiny_out<T, C, STAGED>(a.y, a.y_stride_bytes, row[j], row0[j], whole[j], n, lane, lds, y);
+            if constexpr (LN) a.mean[row[j]] = mean;
+            a.rstd[row[j]] = rstd;
+        }
+    }
+}
+
+template <typename T, bool LN, bool STAGED>
+__global__ void __launch_bounds__(kTinyBlock) norm_tiny_bwd_kernel(const BwdArgs a) {
+    constexpr int C = T::VEC - 1, J = kTinyRows;
+    using Acc = typename AccType<(T::kBytes >= 4)>::type;
+    __shared__ __align__(16) char stage[STAGED ? 2 * (kTinyBlock / 64) * kTinyStageBytes : 16];
+    __shared__ Acc totals[2][kTinyBlock][C];             // [dW | dB][thread][column]
+    const int n = a.n_cols;
+    const int lane = threadIdx.x & 63;
+    char* lds = stage + (STAGED ? (threadIdx.x >> 6) * 2 * kTinyStageBytes : 0);
+    const int64_t threads = static_cast<int64_t>(gridDim.x) * kTinyBlock;
+    const int64_t last_row = a.M - 1;
+    float wr[1][T::VEC];
+    const int first[1] = {0};
+    load_params_clamped<1, T::VEC, false>(wr, a.w, a.w_dtype, first, n, 1.0f);
+    Acc dw[C], db[C];
+#pragma unroll
+    for (int c = 0; c < C; ++c) { dw[c] = Acc(0); db[c] = Acc(0); }
+    for (int64_t base = static_cast<int64_t>(blockIdx.x) * kTinyBlock + threadIdx.x; base - lane < a.M; base += J * threads) {
+        THN_TINY_STEP_ROWS(a.M)
+        TinyIn<T, C, STAGED> ix, ig;
+        ix.request(a.x, a.x_stride_bytes, row, row0, whole, n, lane);
+        ig.request(a.dy, a.dy_stride_bytes, row, row0, whole, n, lane);
+        float c_mean[J], c_rstd[J];
+#pragma unroll
+        for (int j = 0; j < J; ++j) {
+            c_mean[j] = LN ? a.mean[row[j]] : 0.0f;
+            c_rstd[j] = a.rstd[row[j]];
+        }
+#pragma unroll
+        for (int j = 0; j < J; ++j) {
+            float u[C], g[C], wdy[C];
+            ix.take(j, a.x, a.x_stride_bytes, row[j], whole[j], n, lane, lds, u);
+            ig.take(j, a.dy, a.dy_stride_bytes, row[j], whole[j], n, lane, lds + (STAGED ? kTinyStageBytes : 0), g);
+            float s0 = 0.0f, s1 = 0.0f, s2 = 0.0f;
+#pragma unroll
+            for (int c = 0; c < C; ++c) {
+                if constexpr (LN) u[c] = c < n ? (u[c] - c_mean[j]) * c_rstd[j] : 0.0f;
+                else u[c] *= c_rstd[j];
+                wdy[c] = wr[0][c] * g[c];                 // columns past the row end: g reads as 0
+                s0 = fmaf(u[c], wdy[c], s0);
+                if constexpr (LN) {
+                    s1 += wdy[c];
+                    s2 += u[c];
+                }
+            }
+            float c1, c2 = 0.0f, dlt = 0.0f;
+            if constexpr (LN) {
+                dlt = s2 * a.inv_n;
+                c2 = s1 * a.inv_n;
+                c1 = fmaf(-dlt, c2, s0 * a.inv_n);
+            } else {
+                c1 = s0 * a.inv_n;
+            }
+            const bool adds = base + static_cast<int64_t>(j) * threads < a.M;      // a row past the end adds nothing to dW / dB
+            float dx[C];
+#pragma unroll
+            for (int c = 0; c < C; ++c) {
+                float xhat = u[c];
+                if constexpr (LN) xhat -= dlt;
+                dx[c] = (wdy[c] - fmaf(xhat, c1, c2)) * c_rstd[j];
+                const float gl = adds ? g[c] : 0.0f;
+                dw[c] = fma(static_cast<Acc>(gl), static_cast<Acc>(xhat), dw[c]);
+                if constexpr (LN) db[c] += static_cast<Acc>(gl);
+            }
+            tiny_out<T, C, STAGED>(a.dx, a.dx_stride_bytes, row[j], row0[j], whole[j], n, lane, lds, dx);
+        }
+    }
+    // The workgroup's partial row: one thread per column adds the threads' sums in thread order.
+    const bool want_dw = a.dw_part != nullptr;
+    const bool want_db = LN && a.db_part != nullptr;
+#pragma unroll
+    for (int c = 0; c < C; ++c) {
+        totals[0][threadIdx.x][c] = dw[c];
+        totals[1][threadIdx.x][c] = LN ? db[c] : Acc(0);
+    }
+    __syncthreads();
+    if (threadIdx.x < n) {
+        Acc sw = Acc(0), sb = Acc(0);
+        for (int t = 0; t < kTinyBlock; ++t) {
+            sw += totals[0][t][threadIdx.x];
+            sb += totals[1][t][threadIdx.x];
+        }
+        const int64_t off = static_cast<int64_t>(blockIdx.x) * a.part_pitch + threadIdx.x;
+        if (want_dw) a.dw_part[off] = static_cast<float>(sw);
+        if (want_db) a.db_part[off] = static_cast<float>(sb);
+    }
+}
+
 // Launchers: 0 launched, 1 no such instance, <0 HIP error.  `mode`: kP1 / kP2 / kPInt; `staged`: every stream is dense
 // (row r at r * n elements) behind a 16-byte aligned pointer.
 #define THN_DECLARE_TINY_LAUNCHERS(NAME)                                                                        \
@@ -365,7 +518,9 @@ __global__ void __launch_bounds__(kTinyBlock) normalize_tiny_bwd_kernel(const No
     int launch_softmax_tiny_bwd_##NAME(bool is_log, bool staged, const SoftmaxBwdArgs& a, int grid, hipStream_t st); \
     int launch_pnorm_tiny_fwd_##NAME(int mode, bool normalize, bool staged, const PnormFwdArgs& a, int grid, hipStream_t st); \
     int launch_pnorm_tiny_bwd_##NAME(int mode, bool staged, const PnormBwdArgs& a, int grid, hipStream_t st);   \
-    int launch_normalize_tiny_bwd_##NAME(int mode, bool staged, const NormalizeBwdArgs& a, int grid, hipStream_t st);
+    int launch_normalize_tiny_bwd_##NAME(int mode, bool staged, const NormalizeBwdArgs& a, int grid, hipStream_t st); \
+    int launch_norm_tiny_fwd_##NAME(bool ln, bool staged, const FwdArgs& a, int grid, hipStream_t st);          \
+    int launch_norm_tiny_bwd_##NAME(bool ln, bool staged, const BwdArgs& a, int grid, hipStream_t st);
 
 THN_DECLARE_TINY_LAUNCHERS(f32)
 THN_DECLARE_TINY_LAUNCHERS(f16)
@@ -412,6 +567,14 @@ THN_DECLARE_TINY_LAUNCHERS(bf16)
         THN_TINY_MODE_CASE(normalize_tiny_bwd_kernel, NormalizeBwdArgs, kP2)                                    \
         THN_TINY_MODE_CASE(normalize_tiny_bwd_kernel, NormalizeBwdArgs, kPInt)                                  \
         return 1;                                                                                               \
+    }                                                                                                           \
+    int launch_norm_tiny_fwd_##NAME(bool ln, bool staged, const FwdArgs& a, int grid, hipStream_t st) {         \
+        using T = TYPE;                                                                                         \
+        return ln ? THN_TINY_RUN(FwdArgs, norm_tiny_fwd_kernel, true) : THN_TINY_RUN(FwdArgs, norm_tiny_fwd_kernel, false); \
+    }                                                                                                           \
+    int launch_norm_tiny_bwd_##NAME(bool ln, bool staged, const BwdArgs& a, int grid, hipStream_t st) {         \
+        using T = TYPE;                                                                                         \
+        return ln ? THN_TINY_RUN(BwdArgs, norm_tiny_bwd_kernel, true) : THN_TINY_RUN(BwdArgs, norm_tiny_bwd_kernel, false); \
     }
 
 }  // namespace thn
