@@ -53,6 +53,11 @@ WORKLOADS = {
     "rmsnorm_bf16_932067x72_narrow": ("rms", 932067, 72, "bf16"),
     "layernorm_bf16_932067x72_narrow": ("ln", 932067, 72, "bf16"),
     "layernorm_f32_2396745x28_narrow": ("ln", 2396745, 28, "f32"),
+    # off the 128-bit path (50 columns: 7 unaligned windows of bfloat16, 13 of float32: the flat kernels' other instances)
+    # and shorter than one vector (3 float32 columns: a lane per row)
+    "rmsnorm_bf16_1342177x50_ragged": ("rms", 1342177, 50, "bf16"),
+    "layernorm_f32_1342177x50_ragged": ("ln", 1342177, 50, "f32"),
+    "layernorm_f32_11184810x3_short": ("ln", 11184810, 3, "f32"),
     # norm with an activation epilogue (thn_norm_act_fwd + thn_norm_act_bwd): same bytes as the plain norm step
     "layernorm_gelu_bf16_16384x4096": ("ln+gelu", 16384, 4096, "bf16"),
     "layernorm_gelu_tanh_bf16_16384x4096": ("ln+gelu_tanh", 16384, 4096, "bf16"),
