@@ -609,7 +609,10 @@ int plan_launch(int which, int flavour, bool aligned, int64_t M, int64_t N, int 
         // with two; softmax and normalize the same way).
         const bool one_stream = which == kNormFwd || which == kSoftmaxFwd || which == kPnormFwd || which == kFusedFwd;
         const bool shifted_one_row = pitch_bytes % 128 != 0 && s.block == s.tpr;
-        if (one_stream && aligned && s.block * s.k < 1024 && n_vecs > 16 && cap < 2 &&
+        // (rows off the 128-bit path alike, except under an activation epilogue, whose one shape there has four vectors
+        // per thread: bfloat16 N = 1025 RMSNorm / LayerNorm forward 56.2 / 59.5 -> 49.9 / 53.5 us per 2^26 elements, 2049:
+        // 56.8 / 69.2 -> 50.8 / 55.0; float32 N = 513 106.1 / 109.4 -> 96.8 / 97.3)
+        if (one_stream && (aligned || which != kFusedFwd) && s.block * s.k < 1024 && n_vecs > 16 && cap < 2 &&
             (!shifted_one_row || M <= 32 * static_cast<int64_t>(cus))) {
             cap = 2;
         }
@@ -634,6 +637,14 @@ int plan_launch(int which, int flavour, bool aligned, int64_t M, int64_t N, int 
         // rows 8.9 / 14.6 -> 8.3 / 14.0 us with two per compute unit; the same from 8192 rows on.
         if (which == kNormFwd && aligned && s.k == 3 && s.tpr == 256 && s.block == 512 && cap < 2 &&
             M <= 24 * static_cast<int64_t>(cus)) {
+            cap = 2;
+        }
+        // The 16-bit LayerNorm forward off the 128-bit path in 4-vector 256-thread workgroups: the masks that keep a row's
+        // overlapped columns out of its three sums make it the most arithmetic of the forwards, and a second workgroup
+        // covers it (bfloat16 N = 1593: 62.9 -> 51.2 us per 2^26 elements; 3193: 56.6 -> 52.5; RMSNorm and float32 rows
+        // are as fast or faster with one).
+        if (which == kNormFwd && !aligned && bytes == 2 && (flavour & 1) != 0 && s.k == 4 && s.block == 256 && n_vecs > 16 &&
+            cap < 2) {
             cap = 2;
         }
         if ((narrow_forward_pair || narrow_backward_pair) && cap < 2) cap = 2;
