@@ -441,7 +441,9 @@ int plan_launch(int which, int flavour, bool aligned, int64_t M, int64_t N, int 
     // The norm forward over rows of 385 to 512 vectors: 2 x 256 vectors, two rows at a time in 512 threads
     // (THN_FWD_SHAPES_TWO_ROWS), unless the kernel is so short that the 256-thread shape takes two workgroups per
     // compute unit (below).
-    if (which == kNormFwd && aligned && s.k == 4 && s.tpr == 128 && s.block == 256 && n_vecs > 384 &&
+    // (off the 128-bit path as well: bfloat16 N = 3357 / 3997 LayerNorm forward 53.0 / 50.7 -> 49.9 / 47.3 us per 2^26
+    // elements, RMSNorm 47.6 / 47.3 -> 46.8 / 46.7)
+    if (which == kNormFwd && N >= vec_elems && s.k == 4 && s.tpr == 128 && s.block == 256 && n_vecs > 384 &&
         M > 16 * static_cast<int64_t>(cus)) {
         s = Shape{2, 256, 512};
     }
@@ -470,8 +472,10 @@ int plan_launch(int which, int flavour, bool aligned, int64_t M, int64_t N, int 
     // 32768 x 7168 158.0 / 157.7 -> 156.9 / 156.1, 4608 x 8192 22.8 / 25.4 -> 22.8 / 23.8; from 16384 rows on the
     // rows of more than 896 vectors are 1-5 % faster as 4 x 256: 16384 x 8192 87.8 / 87.7 against 89.0 / 90.8).
     // Up to 8 rows per compute unit the 256-thread shape takes two workgroups per compute unit (below) and stays.
-    if (which == kNormFwd && aligned && bytes == 2 && s.k == 4 && s.tpr == 256 && s.block == 256 &&
-        M > 8 * static_cast<int64_t>(cus) && (n_vecs <= 896 || M <= 32 * static_cast<int64_t>(cus))) {
+    // Off the 128-bit path at every row count (bfloat16 N = 7197 / 7997 LayerNorm forward 59.0 / 60.5 -> 56.4 / 50.8 us
+    // per 2^26 elements, RMSNorm 53.5 / 48.2 -> 52.3 / 47.6).
+    if (which == kNormFwd && N >= vec_elems && bytes == 2 && s.k == 4 && s.tpr == 256 && s.block == 256 &&
+        M > 8 * static_cast<int64_t>(cus) && (n_vecs <= 896 || !aligned || M <= 32 * static_cast<int64_t>(cus))) {
         s = Shape{2, 512, 512};
     }
     // The norm backward over narrow rows (17 to 192 vectors, every storage type, on and off the 128-bit path): 2
