@@ -64,7 +64,8 @@ def test_two_vector_rows_stay_two_to_a_workgroup():
     assert shape(1, True, 16384, 2204, f32) == (3, 256, 256)
     assert shape(0, True, 16384, 3072, bf16) == (3, 128, 256)                # the 16-bit LayerNorm forward keeps 3 x 128
     assert shape(1, True, 16384, 3072, bf16) == (2, 256, 512)
-    assert shape(0, False, 16384, 2688, bf16) == (3, 128, 256)               # 336 vectors: too empty for 2 x 256
+    assert shape(0, False, 16384, 2688, bf16) == (3, 128, 512)               # 336 vectors: too empty for 2 x 256;
+    assert shape(1, False, 16384, 2688, bf16) == (3, 128, 512)               # four rows per workgroup in both directions
     # 16-bit forward rows of 769-1024 vectors: 2 x 512 in 512 threads up to 896 vectors, and beyond up to 32 rows per
     # compute unit; short kernels (two 256-thread workgroups per compute unit) and float32 rows keep 4 x 256
     cus = torch.cuda.get_device_properties(0).multi_processor_count

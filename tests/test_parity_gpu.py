@@ -593,6 +593,7 @@ def compiled_shapes():
             shapes.append((int(k), int(t), block if b == "B" else int(b)))
         return shapes
     fwd = expand("THN_FWD_SHAPES") + expand("THN_FWD_SHAPES_TWO_ROWS") + expand("THN_FWD_SHAPES_THREE")
+    fwd += expand("THN_FWD_SHAPES_AS_BACKWARD")
     bwd = [s for blk in (256, 512) for s in expand("THN_BWD_SHAPES_B", blk)]
     tail = re.search(r"#define THN_BWD_SHAPES\(X\)(.*?)\n\n", text, re.S).group(1)
     bwd += [(int(k), int(t), int(b)) for k, t, b in re.findall(r"X\((\d+), (\d+), (\d+)\)", tail)]
@@ -645,3 +646,27 @@ def test_every_compiled_launch_shape(kind, dtype):
     finally:
         lib.thn_norm_set_launch_override(0, 0, 0, 0, 0)
         lib.thn_norm_set_launch_override(1, 0, 0, 0, 0)
+
+
+@pytest.mark.parametrize("dtype,n", [(torch.bfloat16, 2560), (torch.bfloat16, 2800), (torch.bfloat16, 2501),
+                                     (torch.float16, 2304), (torch.float32, 1280), (torch.float32, 1301),
+                                     (torch.bfloat16, 1280), (torch.float16, 1100)])
+def test_forward_takes_the_row_groups_of_the_backward(dtype, n):
+    """Rows of 257 to 351 vectors (16-bit LayerNorm: also 129 to 160): the forward runs as many rows per workgroup as
+    the backward, so that a row meets the same XCD -- and its L2 -- in both directions; checked against the oracle."""
+    vec = 16 // torch.empty(0, dtype=dtype).element_size()
+    n_vecs = -(-n // vec)
+    g = torch.Generator().manual_seed(n)
+    for kind in ("rms", "ln"):
+        if n_vecs <= 160 and kind == "rms":
+            continue
+        for m in (37, 4096):
+            f = _launch.query_launch(0, kind == "ln", m, n, dtype)
+            b = _launch.query_launch(1, kind == "ln", m, n, dtype)
+            announce(f"row groups N={n} M={m} {kind} {dtype} fwd={f} bwd={b}")
+            assert f[:3] == (3, 128 if n_vecs > 256 else 64, 512), f
+            assert f[2] // f[1] == b[2] // b[1], (f, b)
+        x = torch.randn(37, n, generator=g).to(dtype); dy = torch.randn(37, n, generator=g).to(dtype)
+        w = (1 + 0.1 * torch.randn(n, generator=g)).to(dtype)
+        b = (0.1 * torch.randn(n, generator=g)).to(dtype) if kind == "ln" else None
+        run_and_compare(kind, x, dy, w, b, 1e-5, f"row groups N={n} {kind}")

@@ -108,6 +108,7 @@ bool shape_compiled(int which, bool aligned, bool ln16, Shape s) {
         THN_FWD_SHAPES(THN_MATCH)
         if (which == kNormFwd) {
             THN_FWD_SHAPES_TWO_ROWS(THN_MATCH)
+            THN_FWD_SHAPES_AS_BACKWARD(THN_MATCH)
         }
         THN_FWD_SHAPES_THREE(THN_MATCH)
     }
@@ -560,6 +561,14 @@ int plan_launch(int which, int flavour, bool aligned, int64_t M, int64_t N, int 
             s = three;
             narrow_backward_pair = false;
         }
+    }
+    // The forward over rows of 257 to 351 vectors, and the 16-bit LayerNorm forward over 129 to 160: 3 x 128 / 3 x 64
+    // vectors in 512 threads instead of 256, the backward's rows per workgroup (THN_FWD_SHAPES_AS_BACKWARD; the 16-bit
+    // LayerNorm forward over 352 to 384 vectors keeps 3 x 128 in 256 threads, two rows at a time like its backward).
+    if (which == kNormFwd && N >= vec_elems && s.k == 3 && s.block == 256 &&
+        ((s.tpr == 128 && n_vecs <= 351) || (s.tpr == 64 && bytes == 2 && (flavour & 1) != 0 && n_vecs <= 160))) {
+        const Shape grouped{3, s.tpr, 512};
+        if (shape_compiled(which, aligned, ln16, grouped)) s = grouped;
     }
     // Rows that start off 128-byte lines: two-row workgroups of 256-thread rows cannot put their requests on line
     // boundaries (the two rows differ in phase, line_shift_ok() below), one-row workgroups can.  Backward: as fast
