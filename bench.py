@@ -445,7 +445,7 @@ def main():
                          "launches) and the launch intercept / slope of the norm kernels over 8192 ... 32768 rows")
     ap.add_argument("--scan", action="store_true",
                     help="instead of a workload: forward + backward of RMSNorm and LayerNorm over a grid of row widths "
-                         "and row counts per storage type, % of HBM peak per cell (the table the launch heuristic is "
+                         "and row counts per storage type, %% of HBM peak per cell (the table the launch heuristic is "
                          "fitted against)")
     ap.add_argument("--scan-log2-elements", type=int, default=26,
                     help="--scan: elements per tensor in the long class, as a power of two (26: 2^26)")

@@ -23,6 +23,11 @@ def test_more_than_one_gpu_is_refused_with_a_message():
     assert r.returncode != 0 and "ONE GPU" in (r.stderr + r.stdout)
 
 
+def test_help_prints():
+    r = run("--help")
+    assert r.returncode == 0 and "--workload" in r.stdout and "--scan" in r.stdout, r.stderr[-400:]
+
+
 def test_workload_table():
     assert "rmsnorm_bf16_16384x4096" in bench.WORKLOADS           # the configuration the headline metric is quoted on
     for name, (kind, m, n, dname) in bench.WORKLOADS.items():

@@ -342,9 +342,12 @@ Shape heuristic_shape(int which, bool aligned, bool ln16, int n_vecs) {
     // (every family but the norm kernels with an activation epilogue takes the same shapes off the 128-bit path as on it)
     const bool same_shapes = which != kFusedFwd && which != kFusedBwd;
     int kmax = (which == kNormBwd && n_vecs > 128) ? 3 : 4;
-    // Softmax backward: two input streams and nothing to hold; 2 vectors per thread per stream measured best,
-    // except for 2 KiB rows, where one full wave per row (2 x 64) is 8 % slower than half a wave (4 x 32).
-    if (which == kSoftmaxBwd && n_vecs <= 2048 && !(n_vecs > 64 && n_vecs <= 128)) kmax = 2;
+    // Softmax backward: the forward's shape up to 8 KiB rows -- as many rows per workgroup in both directions, so a row
+    // meets the same XCD and its L2 (forward + backward of 2^26 elements: bfloat16 N = 512 / 2048 / 4096 101.2 / 102.7 /
+    // 103.3 -> 98.9 / 99.1 / 98.9 us, N = 1792 / 3584 110.2 / 111.0 -> 102.0 / 102.2, N = 4095 122.8 -> 110.6; float32
+    // N = 224 / 896 / 1792 216.2 / 216.9 / 217.1 -> 195.8 / 195.5 / 197.4; the backward by itself gains 1-6 % as well);
+    // wider rows 2 vectors per thread per stream (bfloat16 N = 8192 98.5 us against 98.9, float32 N = 8192 198.7 / 200.8).
+    if (which == kSoftmaxBwd && n_vecs > 512 && n_vecs <= 2048) kmax = 2;
     if (which == kNormalizeBwd && n_vecs <= 2048) kmax = 2;    // two or three input streams
     if (aligned && which == kFusedBwd && n_vecs <= 2048) kmax = n_vecs > 128 ? 3 : 2;   // bias and pre-activation are live too
     Shape s{4, 1024, 1024};
@@ -561,6 +564,12 @@ int plan_launch(int which, int flavour, bool aligned, int64_t M, int64_t N, int 
             s = three;
             narrow_backward_pair = false;
         }
+    }
+    // The normalize backward over 16-bit rows of 385 to 512 vectors off the 128-bit path: 4 x 128 vectors two rows at a
+    // time instead of one row of 2 x 256 per workgroup (bfloat16, 2^26 elements, N = 3583 / 3999 / 4095: backward 81.7 /
+    // 81.5 / 83.5 -> 72.3 / 70.7 / 70.1 us; narrower and wider rows off the path, and every row on it, keep 2 vectors).
+    if (which == kNormalizeBwd && !aligned && bytes == 2 && N >= vec_elems && s.k == 2 && s.tpr == 256 && s.block == 256) {
+        s = Shape{4, 128, 256};
     }
     // The forward over rows of 257 to 351 vectors, and the 16-bit LayerNorm forward over 129 to 160: 3 x 128 / 3 x 64
     // vectors in 512 threads instead of 256, the backward's rows per workgroup (THN_FWD_SHAPES_AS_BACKWARD; the 16-bit
