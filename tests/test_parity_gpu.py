@@ -648,12 +648,16 @@ def test_every_compiled_launch_shape(kind, dtype):
         lib.thn_norm_set_launch_override(1, 0, 0, 0, 0)
 
 
-@pytest.mark.parametrize("dtype,n", [(torch.bfloat16, 2560), (torch.bfloat16, 2800), (torch.bfloat16, 2501),
-                                     (torch.float16, 2304), (torch.float32, 1280), (torch.float32, 1301),
-                                     (torch.bfloat16, 1280), (torch.float16, 1100)])
-def test_forward_takes_the_row_groups_of_the_backward(dtype, n):
-    """Rows of 257 to 351 vectors (16-bit LayerNorm: also 129 to 160): the forward runs as many rows per workgroup as
-    the backward, so that a row meets the same XCD -- and its L2 -- in both directions; checked against the oracle."""
+@pytest.mark.parametrize("dtype,n,want", [
+    (torch.bfloat16, 2560, (3, 128, 512)), (torch.bfloat16, 2800, (3, 128, 512)), (torch.bfloat16, 2501, (3, 128, 512)),
+    (torch.float16, 2304, (3, 128, 512)), (torch.float32, 1280, (3, 128, 512)), (torch.float32, 1301, (3, 128, 512)),
+    (torch.bfloat16, 1280, (3, 64, 512)), (torch.float16, 1100, (3, 64, 512)),
+    (torch.bfloat16, 256, (2, 16, 256)), (torch.float16, 512, (2, 32, 256)), (torch.bfloat16, 450, (2, 32, 256)),
+    (torch.bfloat16, 320, (3, 16, 512)), (torch.float16, 768, (3, 32, 512)), (torch.bfloat16, 701, (3, 32, 512))])
+def test_forward_takes_the_row_groups_of_the_backward(dtype, n, want):
+    """Rows of 257 to 351 vectors (16-bit LayerNorm: also 17 to 96 and 129 to 160): the forward runs as many rows per
+    workgroup as the backward, so that a row meets the same XCD -- and its L2 -- in both directions; the 3-vector
+    512-thread shapes of narrow rows only while x fits the L2s.  Checked against the oracle."""
     vec = 16 // torch.empty(0, dtype=dtype).element_size()
     n_vecs = -(-n // vec)
     g = torch.Generator().manual_seed(n)
@@ -664,8 +668,11 @@ def test_forward_takes_the_row_groups_of_the_backward(dtype, n):
             f = _launch.query_launch(0, kind == "ln", m, n, dtype)
             b = _launch.query_launch(1, kind == "ln", m, n, dtype)
             announce(f"row groups N={n} M={m} {kind} {dtype} fwd={f} bwd={b}")
-            assert f[:3] == (3, 128 if n_vecs > 256 else 64, 512), f
+            assert f[:3] == want, f
             assert f[2] // f[1] == b[2] // b[1], (f, b)
+        if want[0] == 3 and n_vecs <= 96:
+            big = (32 << 20) // (n * (16 // vec))
+            assert _launch.query_launch(0, kind == "ln", big, n, dtype)[:3] == (3, want[1], 256)
         x = torch.randn(37, n, generator=g).to(dtype); dy = torch.randn(37, n, generator=g).to(dtype)
         w = (1 + 0.1 * torch.randn(n, generator=g)).to(dtype)
         b = (0.1 * torch.randn(n, generator=g)).to(dtype) if kind == "ln" else None

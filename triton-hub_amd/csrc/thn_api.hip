@@ -565,6 +565,23 @@ int plan_launch(int which, int flavour, bool aligned, int64_t M, int64_t N, int 
             narrow_backward_pair = false;
         }
     }
+    // The 16-bit LayerNorm forward over rows of 17 to 96 vectors: the shape with the rows per workgroup of its backward
+    // (1 x 32, 3 x 16, 1 x 64, 3 x 32 in 512 threads: 16, 32, 8, 16 rows), two workgroups per compute unit, so that a row
+    // stays on its XCD.  2 x 16 / 2 x 32 in 256 threads for rows of 17 to 32 / 49 to 64 vectors at every row count
+    // (bfloat16, forward + backward, 16384 rows / 2^26 elements: N = 256 17.2 / 110.2 -> 16.3 / 109.1 us, 448 23.9 / 112.1
+    // -> 21.6 / 111.4, 512 24.8 / 110.7 -> 22.4 / 110.2); 3 x 16 / 3 x 32 in 512 threads for 33 to 48 / 65 to 96 vectors
+    // while x fits three quarters of the eight L2s (24 MiB): 16384 rows, N = 320 22.6 -> 21.5 us, 384 22.5 -> 21.2, 640
+    // 29.0 -> 26.3, 768 31.7 -> 28.9; from 32 MiB on they are 0-4 % slower than in 256 threads (2^24 elements: N = 320
+    // 39.3 -> 40.7 us, 640 38.0 -> 39.5; 2^26: 115.5 -> 117.9), so larger batches keep those.
+    if (which == kNormFwd && bytes == 2 && (flavour & 1) != 0 && n_vecs > 16 && n_vecs <= 96) {
+        const bool three = fills_three_16 || fills_three_32;
+        const Shape grouped = fills_three_16 ? Shape{3, 16, 512} : fills_three_32 ? Shape{3, 32, 512}
+                            : n_vecs <= 32 ? Shape{2, 16, 256} : Shape{2, 32, 256};
+        if ((!three || M * N * bytes <= (24ll << 20)) && shape_compiled(which, aligned, ln16, grouped)) {
+            s = grouped;
+            narrow_forward_pair = true;
+        }
+    }
     // The normalize backward over 16-bit rows of 385 to 512 vectors off the 128-bit path: 4 x 128 vectors two rows at a
     // time instead of one row of 2 x 256 per workgroup (bfloat16, 2^26 elements, N = 3583 / 3999 / 4095: backward 81.7 /
     // 81.5 / 83.5 -> 72.3 / 70.7 / 70.1 us; narrower and wider rows off the path, and every row on it, keep 2 vectors).

@@ -47,8 +47,10 @@ struct Shape {
 // that L2 whatever of x its forward left there (the 256-thread shapes put half as many rows in a workgroup and so a
 // different XCD under every second row).  bfloat16 LayerNorm, forward + backward of one batch, 4096 x 2560 28.4 ->
 // 25.5 us, 4096 x 2800 30.2 -> 27.5, 26214 x 2560 114.1 -> 111.8; float32 4096 x 1280 27.0 -> 24.1; the forward by
-// itself is as fast or faster (float32 48770 x 1376 92.2 -> 89.6 us, bfloat16 23967 x 2800 48.9 -> 46.7).
-#define THN_FWD_SHAPES_AS_BACKWARD(X) X(3, 64, 512) X(3, 128, 512)
+// itself is as fast or faster (float32 48770 x 1376 92.2 -> 89.6 us, bfloat16 23967 x 2800 48.9 -> 46.7).  3 x 16 and
+// 3 x 32 are the 16-bit LayerNorm backward's shapes for rows of 33 to 48 and 65 to 96 vectors; the forward takes them
+// while x fits the eight L2s (plan_launch()).
+#define THN_FWD_SHAPES_AS_BACKWARD(X) X(3, 16, 512) X(3, 32, 512) X(3, 64, 512) X(3, 128, 512)
 
 #define THN_BWD_SHAPES_B(X, B)                                                       \
     X(1, 8, B) X(2, 8, B) X(4, 8, B)                                                 \
