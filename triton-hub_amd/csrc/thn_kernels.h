@@ -528,20 +528,7 @@ __global__ void __launch_bounds__(BLOCK) norm_bwd_kernel(const BwdArgs a) {
 
     const int64_t rows_per_iter = static_cast<int64_t>(gridDim.x) * G;
     const int64_t last_row = a.M - 1;
-    // A workgroup visits its row blocks (blockIdx.x, blockIdx.x + gridDim.x, ...) from the last full one down to the
-    // first, then the one that may run past the end (the only masked step, as before): the forward walks the same
-    // blocks upwards, so the backward starts on the rows that the forward touched last and that its XCD's L2 still
-    // holds (forward + backward of one batch, bfloat16 16384 x 4096 104.4 -> 104.0 us, float16 65536 x 1024 109.5 ->
-    // 108.0, float32 16384 x 4096 201.5 -> 200.7; the same on a batch that no cache holds).  Which rows meet in a
-    // partial row of dW / dB does not change, only the order in which a workgroup adds them.
-    const int64_t wg_first = static_cast<int64_t>(blockIdx.x) * G;
-    const int64_t n_full = (a.M - G >= wg_first) ? (a.M - G - wg_first) / rows_per_iter + 1 : 0;
-    const int64_t first_raw = wg_first + g, tail_raw = first_raw + n_full * rows_per_iter;
-    auto next_raw = [&](int64_t r) -> int64_t {
-        if (r >= tail_raw) return r + rows_per_iter;
-        return r - rows_per_iter >= first_raw ? r - rows_per_iter : tail_raw;
-    };
-    int64_t row_raw = n_full > 0 ? tail_raw - rows_per_iter : first_raw;
+    int64_t row_raw = static_cast<int64_t>(blockIdx.x) * G + g;
     int64_t row = row_raw < a.M ? row_raw : last_row;
     u32x4 cx[K], cg[K];
     slot_load_row<T, K, ALIGNED>(cx, a.x, a.x_stride_bytes, row, voff, a.n_cols);    // first, so they overlap the params
@@ -579,7 +566,7 @@ __global__ void __launch_bounds__(BLOCK) norm_bwd_kernel(const BwdArgs a) {
     // groups may have run past the end and mirror the last row: they must add nothing to dW / dB.
     auto step = [&](auto masked_tag) {
         constexpr bool MASKED = decltype(masked_tag)::value;
-        const int64_t nrow_raw = next_raw(row_raw);
+        const int64_t nrow_raw = row_raw + rows_per_iter;
         const int64_t nrow = nrow_raw < a.M ? nrow_raw : last_row;
         u32x4 nx[K], ng[K];
         slot_load_row<T, K, ALIGNED>(nx, a.x, a.x_stride_bytes, nrow, voff, a.n_cols);
@@ -702,7 +689,7 @@ __global__ void __launch_bounds__(BLOCK) norm_bwd_kernel(const BwdArgs a) {
                 return voff[k];
             }
         };
-        const int64_t nrow_raw = next_raw(row_raw);
+        const int64_t nrow_raw = row_raw + rows_per_iter;
         const int64_t nrow = nrow_raw < a.M ? nrow_raw : last_row;
         const bool live = !MASKED || row_raw < a.M;
         const char* nxrow = a.x + nrow * a.x_stride_bytes;
