@@ -1584,7 +1584,7 @@ int act_launch(const void* x, int64_t x_row_stride, const void* g, int64_t g_row
         const int vec_elems = 16 / bytes;
         a.total_elems = M * N;
         a.total_vecs = a.total_elems / vec_elems;
-        const int per_block = thn::kActBlock * (bwd ? thn::kActBwdVecs : thn::kActFwdVecs);
+        const int per_block = thn::kActBlock * (bwd ? thn::act_bwd_vecs(act) : thn::kActFwdVecs);
         const int64_t blocks = (a.total_vecs + per_block - 1) / per_block;
         const int64_t cap = static_cast<int64_t>(cus) * (bpc_override > 0 ? bpc_override : act_blocks_per_cu(act, bwd, bytes));
         int64_t n = blocks < cap ? blocks : cap;
@@ -1600,7 +1600,7 @@ int act_launch(const void* x, int64_t x_row_stride, const void* g, int64_t g_row
         a.g_stride_bytes = g_row_stride * bytes;
         a.out_stride_bytes = out_row_stride * bytes;
         // Threads along a row: one per vector slot, at most the whole workgroup; a thread takes `vecs` rows per step.
-        const int vecs = bwd ? thn::kActBwdVecs : thn::kActFwdVecs;
+        const int vecs = bwd ? thn::kActRowsBwdVecs : thn::kActFwdVecs;
         const int64_t slots = (N + 16 / bytes - 1) / (16 / bytes);
         int lx = 0;
         while (lx < 8 && (int64_t{1} << lx) < slots) ++lx;
