@@ -414,13 +414,18 @@ int narrow_row_blocks_per_cu(int which, int n_vecs, bool ragged16) {
     // 16-bit rows whose width is not a whole number of vectors.  The norm kernels with an activation epilogue run four
     // vectors per thread there whatever the width, and a second workgroup hides the latency of their arithmetic.  The
     // plain norm kernels' overlapped windows cost no more than aligned vectors and lose 5-7 % with a second workgroup (bf16 24564 x 4098 forward 69.1 us with one, 73.4 with two; fp16 8192 x 12289
-    // 81.6 / 85.0).  The softmax family has the same windows, but its forward holds so little per row that rows of more
-    // than 128 vectors still gain from the second workgroup (forward + backward of 2^26 bfloat16 elements, % of 8 TB/s,
-    // one / two: N = 1025 60.1 / 67.8; 2050 66.4 / 71.2; 4098 66.0 / 70.8; 5001 61.2 / 64.0) and narrower ones lose
-    // (N = 197 63.1 / 60.7; 300 72.2 / 70.5; 577 67.6 / 65.4; 1023 77.5 / 73.0); the p-norm family takes two workgroups
-    // of 256 threads anyway.
+    // 81.6 / 85.0).  The softmax forward has the same windows, but holds so little per row that rows of more than 128
+    // vectors still gain from the second workgroup (bfloat16, 2^26 elements, one / two: N = 1025 74.7 / 57.4 us, 2050
+    // 63.9 / 57.4, 5001 63.8 / 60.1) and narrower ones lose (forward + backward, % of 8 TB/s: N = 197 63.1 / 60.7; 300
+    // 72.2 / 70.5; 577 67.6 / 65.4; 1023 77.5 / 73.0); the softmax backward is 3-10 % faster with one at every width
+    // (N = 1025 71.0 / 76.7 us, 1500 64.7 / 70.0, 2050 67.2 / 73.3, 4098 67.4 / 73.8, 6001 68.6 / 82.2, 8191 68.3 / 79.7);
+    // the p-norm family takes two workgroups of 256 threads anyway, and the normalize backward one of 512 threads
+    // (rows of more than 512 vectors: N = 4098 70.8 / 77.4 us, 6001 73.0 / 85.4, 8191 68.4 / 80.8).
     const bool fused = which == kFusedFwd || which == kFusedBwd;
-    if (ragged16 && n_vecs > 16 && which != kNormFwd && which != kNormBwd && (fused || n_vecs > 128)) return 2;
+    if (ragged16 && n_vecs > 16 && which != kNormFwd && which != kNormBwd && which != kSoftmaxBwd &&
+        which != kNormalizeBwd && (fused || n_vecs > 128)) {
+        return 2;
+    }
     const bool one_stream = which == kNormFwd || which == kSoftmaxFwd || which == kPnormFwd || which == kFusedFwd;
     if (n_vecs <= 8) return one_stream ? 4 : 2;
     if (n_vecs <= 16) return (one_stream || which == kNormBwd) ? 2 : 1;   // norm backward: with one vector per thread
@@ -581,6 +586,18 @@ int plan_launch(int which, int flavour, bool aligned, int64_t M, int64_t N, int 
             s = grouped;
             narrow_forward_pair = true;
         }
+    }
+    // The normalize backward over 16-bit rows of 129 to 191 and 257 to 383 vectors: 3 x 64 / 3 x 128 vectors, the shape
+    // (and the rows per workgroup) of its forward, instead of 2 x 128 / 2 x 256 -- by itself the kernel is as fast either
+    // way on the 128-bit path, but a row then stays on one XCD through forward and backward, and off the path the
+    // fuller shape is faster by itself as well.  bfloat16, forward + backward of 2^26 elements: N = 1032 117.3 -> 114.1
+    // us, 1152 107.6 -> 103.6, 1280 104.2 -> 103.8, 2304 106.5 -> 103.1, 2560 104.1 -> 103.9; off the path N = 1025
+    // 135.9 -> 123.5, 1281 120.1 -> 116.0, 2050 122.9 -> 117.2, 2900 112.7 -> 110.7 (float32 rows lose 1 % that way, and
+    // rows that fill the 3-vector shape exactly lose as much: N = 3072 102.1 -> 102.9).
+    if (which == kNormalizeBwd && bytes == 2 && N >= vec_elems && s.k == 2 && s.block == 256 &&
+        (s.tpr == 128 || s.tpr == 256) && 2 * n_vecs < 3 * s.tpr) {
+        const Shape three{3, s.tpr / 2, 256};
+        if (shape_compiled(which, aligned, ln16, three)) s = three;
     }
     // The normalize backward over 16-bit rows of 385 to 512 vectors off the 128-bit path: 4 x 128 vectors two rows at a
     // time instead of one row of 2 x 256 per workgroup (bfloat16, 2^26 elements, N = 3583 / 3999 / 4095: backward 81.7 /
