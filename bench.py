@@ -1019,10 +1019,11 @@ def softmax_main(args, lib, dev, kind, m, n, dname, dtype):
     achieved = bwd_bytes / (bwd_us * 1e-6) / 1e9
     fam = {None: (2, 3), "normalize": (4, 6), "pnorm": (4, 5), "act": None}[row_op]
     if fam is not None:
-        fs = _launch.query_launch(fam[0], kind == "logsoftmax", m, n, dtype)
+        # (for the p-norm forward the flag asks for the launch of the normalize entry point)
+        fs = _launch.query_launch(fam[0], kind == "logsoftmax" or row_op == "normalize", m, n, dtype)
         bs = _launch.query_launch(fam[1], kind == "logsoftmax", m, n, dtype)
-    else:                                   # flat element-wise kernels: 4 / 2 vectors per thread, no rows
-        fs, bs = (4, 0, 256, 0), (2, 0, 256, 0)
+    else:                                   # flat element-wise kernels: vectors per thread and step, no rows
+        fs, bs = (4, 0, 256, 0), (2 if act_name in ("gelu", "gelu_tanh", "mish") else 4, 0, 256, 0)
     bwd_kernel = {None: "softmax_bwd_kernel", "normalize": "normalize_bwd_kernel", "pnorm": "pnorm_bwd_kernel",
                   "act": "act_flat_kernel (backward)"}[row_op]
     entry = {None: "thn_softmax_fwd + thn_softmax_bwd", "normalize": "thn_normalize_fwd + thn_normalize_bwd",

@@ -383,7 +383,8 @@ int thn_norm_set_launch_override(int which, int vecs_per_thread, int threads_per
  * {vecs_per_thread, threads_per_row, block_threads, grid_blocks, aligned 128-bit path (1) or unaligned-row path (0)}.
  * (the last field is 0 for every kind of kernel when the rows are off the 128-bit path).
  * For the epilogue families (9, 10) `is_layernorm` carries the activation too: bit 0 = LayerNorm, bits 1.. = the
- * thn_act code.  Rows wider than 64 KiB of the softmax and p-norm families report their looping kernels:
+ * thn_act code.  For the p-norm / normalize forward (4) a non-zero `is_layernorm` asks for thn_normalize_fwd's launch
+ * (0: thn_pnorm_fwd's; they differ for 16-bit rows of 769 to 1024 vectors off the 128-bit path).  Rows wider than 64 KiB of the softmax and p-norm families report their looping kernels:
  * {vectors per thread and step, block_threads, block_threads, grid_blocks, 0}.  Norm problems that take the flat
  * kernels (narrow 16-bit rows whose vector count is not a power of two; off the 128-bit path narrow rows of any
  * vector count and type) report {rows per lane and step, vectors per row, 256, grid_blocks, 1}: a threads_per_row that

@@ -368,3 +368,26 @@ def test_every_compiled_launch_shape(dtype):
     finally:
         lib.thn_norm_set_launch_override(2, 0, 0, 0, 0)
         lib.thn_norm_set_launch_override(3, 0, 0, 0, 0)
+
+
+def test_launch_rules_of_rows_off_the_128_bit_path_and_of_the_backward():
+    """The backward takes the forward's launch shape for rows of up to 512 vectors (the same rows per workgroup in
+    both directions); off the 128-bit path in 16-bit storage the forward over 769 to 1024 vectors runs 2 x 512 in 512
+    threads and the backward one workgroup per compute unit.  Each shape against the oracle."""
+    from TritonHub.Normalization._launch import query_launch
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    bf16, f32 = torch.bfloat16, torch.float32
+    for n, dt in ((512, bf16), (1792, bf16), (2048, bf16), (4096, bf16), (4095, bf16), (224, f32), (1024, f32), (2048, f32)):
+        f = query_launch(2, False, 1 << 16, n, dt); b = query_launch(3, False, 1 << 16, n, dt)
+        assert f[:3] == b[:3], (n, dt, f, b)
+    assert query_launch(3, False, 8192, 8192, bf16)[:3] == (2, 512, 512)            # wider rows: 2 vectors per thread
+    assert query_launch(2, False, 8192, 8191, bf16)[:4] == (2, 512, 512, cus)
+    assert query_launch(2, False, 8192, 8191, f32)[:3] != (2, 512, 512)
+    for n in (1025, 2050, 4098, 6001, 8191):
+        assert query_launch(3, False, 1 << 16, n, bf16)[3] <= cus, n
+        assert query_launch(2, False, 1 << 16, n, bf16)[3] == (cus if n == 8191 else 2 * cus), n
+    for kind in KINDS:
+        for n, dt in ((8191, bf16), (7001, torch.float16), (1792, bf16), (4095, bf16), (896, f32)):
+            announce(f"launch rules {kind} N={n} {dt}")
+            x, dy = make((21, n), dt, seed=n, scale=3.0)
+            run_and_compare(kind, x, dy, f"{kind} N={n} {dt}")

@@ -587,6 +587,20 @@ int plan_launch(int which, int flavour, bool aligned, int64_t M, int64_t N, int 
             narrow_forward_pair = true;
         }
     }
+    // The softmax and the normalize forward over 16-bit rows of 769 to 1024 vectors off the 128-bit path: 2 x 512 vectors
+    // in 512 threads, one workgroup per compute unit, as the norm forward takes them, instead of 4 x 256 in 256 threads,
+    // two per compute unit (bfloat16 N = 8191, forward / forward + backward: softmax 58.8 / 115.2 -> 52.8 / 113.0 us,
+    // normalize 58.1 / 115.4 -> 51.0 / 110.3; N = 7001 normalize 57.4 / 122.7 -> 52.6 / 119.8; the p-norm by itself, which
+    // writes one value per row, keeps 4 x 256: N = 8191 27.5 us against 30.9).
+    bool wide_ragged_forward = false;
+    if ((which == kSoftmaxFwd || (which == kPnormFwd && (flavour & 4) != 0)) && !aligned && bytes == 2 && s.k == 4 &&
+        s.tpr == 256 && s.block == 256) {
+        const Shape wide{2, 512, 512};
+        if (shape_compiled(which, aligned, ln16, wide)) {
+            s = wide;
+            wide_ragged_forward = true;
+        }
+    }
     // The normalize backward over 16-bit rows of 129 to 191 and 257 to 383 vectors: 3 x 64 / 3 x 128 vectors, the shape
     // (and the rows per workgroup) of its forward, instead of 2 x 128 / 2 x 256 -- by itself the kernel is as fast either
     // way on the 128-bit path, but a row then stays on one XCD through forward and backward, and off the path the
@@ -652,7 +666,7 @@ int plan_launch(int which, int flavour, bool aligned, int64_t M, int64_t N, int 
     int cap = ov.bpc.load();
     if (cap <= 0) {
         cap = default_blocks_per_cu(which, flavour, s.block);
-        const int narrow = narrow_row_blocks_per_cu(which, n_vecs, bytes == 2 && N % vec_elems != 0);
+        const int narrow = narrow_row_blocks_per_cu(which, n_vecs, bytes == 2 && N % vec_elems != 0 && !wide_ragged_forward);
         if (narrow > cap) cap = narrow;
         // One input stream and fewer than 1024 vectors per workgroup step (3 vectors per thread in 256-thread
         // workgroups: row widths of 5 * 2^k elements and their neighbours): a second workgroup brings the bytes in
@@ -1693,7 +1707,9 @@ int thn_norm_query_launch(int which, int is_layernorm, int64_t M, int64_t N, int
     Plan p;
     const bool aligned = N > 0 && (N % (16 / bytes)) == 0;
     int flavour = is_layernorm != 0 ? 1 : 0;
-    if (which >= kPnormFwd && which <= kNormalizeBwd) flavour = thn::kP2;
+    if (which >= kPnormFwd && which <= kNormalizeBwd) {
+        flavour = thn::kP2 | ((which == kPnormFwd && is_layernorm != 0) ? 4 : 0);      // 4: the forward also normalises
+    }
     if (which == kFusedFwd || which == kFusedBwd) {
         if (is_layernorm < 0 || !fusable(is_layernorm >> 1)) return THN_E_SHAPE;
         flavour = is_layernorm;                     // bit 0 = LayerNorm, bits 1.. = activation
