@@ -373,7 +373,8 @@ def test_every_compiled_launch_shape(dtype):
 
 def test_launch_rules_of_16_bit_rows_off_the_128_bit_path():
     """normalize: the forward over 769 to 1024 vectors runs 2 x 512 in 512 threads (the p-norm by itself keeps 4 x 256),
-    the backward takes its forward's 3-vector shape for rows of 129 to 191 and 257 to 383 vectors (on the path too),
+    the backward takes its forward's 3-vector shape for rows of 129 to 191 and 257 to 383 vectors (on the path up to 144
+    and 288),
     4 x 128 for 385 to 512 vectors, and one workgroup per compute unit in 512 threads.  Each against the oracle."""
     cus = torch.cuda.get_device_properties(0).multi_processor_count
     bf16, f16, f32 = torch.bfloat16, torch.float16, torch.float32
@@ -381,7 +382,8 @@ def test_launch_rules_of_16_bit_rows_off_the_128_bit_path():
     assert query_launch(4, False, 8192, 8191, bf16)[:3] == (4, 256, 256)
     assert query_launch(4, True, 8192, 8192, bf16)[:3] == (4, 256, 256)
     for n, want in ((1025, (3, 64, 256)), (1152, (3, 64, 256)), (1281, (3, 64, 256)), (2050, (3, 128, 256)),
-                    (2304, (3, 128, 256)), (3072, (2, 256, 256)), (1536, (2, 128, 256)), (3999, (4, 128, 256))):
+                    (2304, (3, 128, 256)), (1280, (2, 128, 256)), (2560, (2, 256, 256)), (3072, (2, 256, 256)),
+                    (1536, (2, 128, 256)), (3999, (4, 128, 256))):
         assert query_launch(6, False, 1 << 15, n, bf16)[:3] == want, n
         assert query_launch(6, False, 1 << 15, n, f16)[:3] == want, n
     assert query_launch(6, False, 1 << 15, 516, f32)[:3] == (2, 128, 256)

@@ -601,15 +601,18 @@ int plan_launch(int which, int flavour, bool aligned, int64_t M, int64_t N, int 
             wide_ragged_forward = true;
         }
     }
-    // The normalize backward over 16-bit rows of 129 to 191 and 257 to 383 vectors: 3 x 64 / 3 x 128 vectors, the shape
+    // The normalize backward over 16-bit rows of 129 to 191 and 257 to 383 vectors (129 to 144 and 257 to 288 on the
+    // 128-bit path): 3 x 64 / 3 x 128 vectors, the shape
     // (and the rows per workgroup) of its forward, instead of 2 x 128 / 2 x 256 -- by itself the kernel is as fast either
     // way on the 128-bit path, but a row then stays on one XCD through forward and backward, and off the path the
     // fuller shape is faster by itself as well.  bfloat16, forward + backward of 2^26 elements: N = 1032 117.3 -> 114.1
     // us, 1152 107.6 -> 103.6, 1280 104.2 -> 103.8, 2304 106.5 -> 103.1, 2560 104.1 -> 103.9; off the path N = 1025
     // 135.9 -> 123.5, 1281 120.1 -> 116.0, 2050 122.9 -> 117.2, 2900 112.7 -> 110.7 (float32 rows lose 1 % that way, and
-    // rows that fill the 3-vector shape exactly lose as much: N = 3072 102.1 -> 102.9).
+    // rows that fill the 3-vector shape exactly lose as much: N = 3072 102.1 -> 102.9).  On the path only up to 9/8 of
+    // the 2-vector shape's threads (N = 1152, 2304): rows of 5/4 (1280, 2560) gain 0.3 % with a backward that follows
+    // its forward and lose 1.8 % with one that does not.
     if (which == kNormalizeBwd && bytes == 2 && N >= vec_elems && s.k == 2 && s.block == 256 &&
-        (s.tpr == 128 || s.tpr == 256) && 2 * n_vecs < 3 * s.tpr) {
+        (s.tpr == 128 || s.tpr == 256) && (aligned ? 8 * n_vecs <= 9 * s.tpr : 2 * n_vecs < 3 * s.tpr)) {
         const Shape three{3, s.tpr / 2, 256};
         if (shape_compiled(which, aligned, ln16, three)) s = three;
     }
