@@ -319,7 +319,8 @@ constexpr int kTprList[] = {8, 16, 32, 64, 128, 256, 512, 1024};
 //             wave: the float64 column sums need the instruction-level parallelism) and for rows that 1024
 //             threads cannot cover otherwise; 512-thread workgroups once a row spans two waves or more, which
 //             also halves the number of partial rows;
-//   softmax / normalize / epilogue backward (two or three input streams): kmax 2 up to 32 KiB rows.
+//   normalize / epilogue backward (two or three input streams): kmax 2 up to 32 KiB rows; the softmax backward the
+//             forward's shape up to 8 KiB rows and kmax 2 from there to 32 KiB.
 // A second finding runs through the norm rules of plan_launch(): a compute unit wants eight waves of a row kernel,
 // not four.  One 256-thread workgroup per compute unit (one wave per SIMD) leaves a row's arithmetic and reduction
 // rounds uncovered -- the 16-bit LayerNorm forward then takes 1.3 us per row at any width -- so the backward of
@@ -364,9 +365,10 @@ Shape heuristic_shape(int which, bool aligned, bool ln16, int n_vecs) {
     }
     if (which == kNormBwd && n_vecs > 8 && n_vecs <= 16) s.tpr = 16;      // 256-byte rows: one vector per thread
     s.k = ceil_div(n_vecs, s.tpr);
-    // The softmax backward prefers 2 vectors per thread, but a row of 3 * 2^k vectors (or a little less) would
-    // leave a quarter to a half of the slots without work: then 3 vectors on half the threads (bf16 N = 1280 /
-    // 2560 / 3072: 5.0 / 5.0 / 5.5 -> 6.0 / 6.4 / 6.3 TB/s; the normalize backward lost 5 % with the same change).
+    // The softmax backward over rows of more than 8 KiB prefers 2 vectors per thread, but a row of 3 * 2^k vectors (or
+    // a little less) would leave a quarter to a half of the slots without work: then 3 vectors on half the threads
+    // (measured when narrower rows had 2 vectors as well: bf16 N = 1280 / 2560 / 3072: 5.0 / 5.0 / 5.5 -> 6.0 / 6.4 /
+    // 6.3 TB/s).
     if (which == kSoftmaxBwd && s.k == 2 && s.tpr >= 128) {
         const int half = s.tpr / 2;
         if (3 * half >= n_vecs) {          // at most three quarters of the 2-vector slots would have work
