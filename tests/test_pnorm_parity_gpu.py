@@ -389,6 +389,22 @@ def test_launch_rules_of_16_bit_rows_off_the_128_bit_path():
     assert query_launch(6, False, 1 << 15, 516, f32)[:3] == (2, 128, 256)
     for n in (4098, 6001, 8191):
         assert query_launch(6, False, 1 << 15, n, bf16)[2:4] == (512, cus), n
+    # rows of 33 to 48 and 65 to 96 vectors: the forward 3 x 16 / 3 x 32 in every storage type, the 16-bit normalize
+    # backward up to 40 and 80 vectors
+    for which_fwd in (False, True):
+        assert query_launch(4, which_fwd, 1 << 15, 264, bf16)[:3] == (3, 16, 256)
+        assert query_launch(4, which_fwd, 1 << 15, 576, f16)[:3] == (3, 32, 256)
+        assert query_launch(4, which_fwd, 1 << 15, 132, f32)[:3] == (3, 16, 256)
+        assert query_launch(4, which_fwd, 1 << 15, 301, f32)[:3] == (3, 32, 256)
+    assert query_launch(6, False, 1 << 15, 264, bf16)[:3] == (3, 16, 256) and query_launch(6, False, 1 << 15, 320, f16)[:3] == (3, 16, 256)
+    assert query_launch(6, False, 1 << 15, 384, bf16)[:3] == (2, 32, 256) and query_launch(6, False, 1 << 15, 132, f32)[:3] == (2, 32, 256)
+    assert query_launch(6, False, 1 << 15, 577, bf16)[:3] == (3, 32, 256) and query_launch(6, False, 1 << 15, 768, bf16)[:3] == (2, 64, 256)
+    for n, dt in ((264, bf16), (301, f16), (577, bf16), (640, f16), (132, f32), (301, f32)):
+        announce(f"three-vector shapes K={n} {dt}")
+        x, gn, gy = make((3, 37, n), dt, seed=n)
+        for p in (1, 2, 3):
+            compare_norm(x, gn, p, 1e-6, f"norm K={n} p={p}")
+            compare_normalize(x, gy, p, 1e-6, f"normalize K={n} p={p}")
     for n, dt in ((8191, bf16), (7001, f16), (1025, bf16), (1152, f16), (2050, bf16), (2304, bf16), (3999, f16)):
         announce(f"launch rules K={n} {dt}")
         x, gn, gy = make((2, 11, n), dt, seed=n)

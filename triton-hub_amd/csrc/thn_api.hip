@@ -565,6 +565,21 @@ int plan_launch(int which, int flavour, bool aligned, int64_t M, int64_t N, int 
             narrow_forward_pair = which == kSoftmaxFwd;
         }
     }
+    // The p-norm / normalize family at the same widths: the forward 3 x 16 / 3 x 32 in every storage type (normalize,
+    // 2^26 elements, forward: bfloat16 N = 264 59.2 -> 52.9 us, 272 56.5 -> 52.3, 384 49.2 -> 47.0, 520 58.2 -> 53.6;
+    // float32 N = 132 115.0 -> 105.6, 160 96.5 -> 92.4, 260 114.7 -> 107.5, 384 95.8 -> 92.9); the 16-bit normalize
+    // backward for rows of 33 to 40 and 65 to 80 vectors, where 2 x 32 / 2 x 64 are five eighths full at most (forward
+    // + backward with both: N = 264 132.3 -> 120.2 us, 320 107.6 -> 103.5, 520 126.1 -> 116.7, 576 110.0 -> 103.3, 640
+    // 107.1 -> 103.4; fuller rows and float32 rows lose 3-10 % in the backward that way).
+    if (which == kPnormFwd && N >= vec_elems && (fills_three_16 || fills_three_32)) {
+        const Shape three{3, fills_three_16 ? 16 : 32, 256};
+        if (shape_compiled(which, aligned, ln16, three)) s = three;
+    }
+    if (which == kNormalizeBwd && bytes == 2 && N >= vec_elems &&
+        ((n_vecs > 32 && n_vecs <= 40) || (n_vecs > 64 && n_vecs <= 80))) {
+        const Shape three{3, n_vecs <= 40 ? 16 : 32, 256};
+        if (shape_compiled(which, aligned, ln16, three)) s = three;
+    }
     if (which == kNormBwd && ln16 && (fills_three_16 || fills_three_32 || (n_vecs > 128 && n_vecs <= 160))) {
         const Shape three{3, fills_three_16 ? 16 : (fills_three_32 ? 32 : 64), 512};
         if (shape_compiled(which, aligned, ln16, three)) {

@@ -8,10 +8,11 @@
 namespace thn {
 
 // X(K, TPR, BLOCK): the shapes the launch heuristic can reach (fewest threads per row with at most 4, or at
-// most 2, vectors each).
+// most 2, vectors each; 3 x 16 and 3 x 32 for rows of 33 to 48 and 65 to 96 vectors, as in the norm and softmax
+// families).
 #define THN_ROW_SHAPES(X)                                                            \
     X(1, 8, 256) X(2, 8, 256) X(4, 8, 256)                                           \
-    X(2, 16, 256) X(4, 16, 256) X(2, 32, 256) X(4, 32, 256)                          \
+    X(2, 16, 256) X(3, 16, 256) X(4, 16, 256) X(2, 32, 256) X(3, 32, 256) X(4, 32, 256) \
     X(2, 64, 256) X(3, 64, 256) X(4, 64, 256)                                        \
     X(2, 128, 256) X(3, 128, 256) X(4, 128, 256)                                     \
     X(2, 256, 256) X(3, 256, 256) X(4, 256, 256)                                     \
