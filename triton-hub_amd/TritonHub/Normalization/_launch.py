@@ -261,7 +261,9 @@ def norm_bwd(x: torch.Tensor, dout: torch.Tensor, weight, bias, mean, rstd, laye
 
 
 def query_launch(which: int, layernorm: bool, m: int, n: int, dtype: torch.dtype):
-    """(vecs_per_thread, threads_per_row, block_threads, grid_blocks, vector_path) the library would use."""
+    """(vecs_per_thread, threads_per_row, block_threads, grid_blocks, vector_path) the library would use.
+    `layernorm` is the flavour within the family `which` names: LayerNorm against RMSNorm (0, 1), log-softmax against
+    softmax (2, 3), normalize against the p-norm by itself (4); the activation code too for the epilogue families."""
     shape = (ctypes.c_int32 * 5)()
     _native.check(_native.lib().thn_norm_query_launch(which, int(layernorm), m, n, _native.dtype_code(dtype), shape))
     return tuple(shape)
