@@ -333,6 +333,10 @@ def compiled_forward_shapes():
     text = open(os.path.join(ROOT, "triton-hub_amd", "csrc", "thn_dispatch.h")).read()
     body = re.search(r"#define THN_FWD_SHAPES\(X\)(.*?)\n\n", text, re.S).group(1)
     body += re.search(r"#define THN_FWD_SHAPES_THREE\(X\)(.*?)\n\n", text, re.S).group(1)     # 3 x 16, 3 x 32
+    text = open(os.path.join(ROOT, "triton-hub_amd", "csrc", "thn_softmax_dispatch.h")).read()
+    five = re.search(r"#define THN_SM_SHAPES_FIVE\(X\)(.*?)\n\n", text, re.S).group(1)          # 5 x 32 ... 5 x 256
+    assert len(re.findall(r"X\(5, ", five)) == 4
+    body += five
     return [(int(k), int(t), int(b)) for k, t, b in re.findall(r"X\((\d+), (\d+), (\d+)\)", body)]
 
 
@@ -390,4 +394,27 @@ def test_launch_rules_of_rows_off_the_128_bit_path_and_of_the_backward():
         for n, dt in ((8191, bf16), (7001, torch.float16), (1792, bf16), (4095, bf16), (896, f32)):
             announce(f"launch rules {kind} N={n} {dt}")
             x, dy = make((21, n), dt, seed=n, scale=3.0)
+            run_and_compare(kind, x, dy, f"{kind} N={n} {dt}")
+
+
+def test_five_vector_shapes_for_rows_just_above_a_power_of_two_of_vectors():
+    """Rows of 4 t + 1 to 5 t vectors (t = 32 ... 256) take 5 x t vectors per row in the forward; the backward follows
+    where measured to pay.  The launches the library picks, each against the oracle."""
+    from TritonHub.Normalization._launch import query_launch
+    bf16, f16, f32 = torch.bfloat16, torch.float16, torch.float32
+    want = {(1032, bf16): ((5, 32, 256), (5, 32, 256)), (1152, f16): ((5, 32, 256), (5, 32, 256)),
+            (1280, bf16): ((5, 32, 256), (3, 64, 256)), (2056, bf16): ((5, 64, 256), (5, 64, 256)),
+            (4104, f16): ((5, 128, 256), (5, 128, 256)), (5120, bf16): ((5, 128, 256), (3, 256, 256)),
+            (8200, bf16): ((5, 256, 256), (5, 256, 256)), (10240, bf16): ((5, 256, 256), (3, 512, 512)),
+            (516, f32): ((5, 32, 256), (5, 32, 256)), (2052, f32): ((5, 128, 256), (3, 256, 256)),
+            (1025, bf16): ((5, 32, 256), (3, 64, 256)), (5001, bf16): ((5, 128, 256), (5, 128, 256)),
+            (1024, bf16): ((4, 32, 256), (4, 32, 256)), (1288, bf16): ((3, 64, 256), (3, 64, 256))}
+    for (n, dt), (f, b) in want.items():
+        assert query_launch(2, False, 1 << 14, n, dt)[:3] == f, (n, dt)
+        assert query_launch(3, False, 1 << 14, n, dt)[:3] == b, (n, dt)
+    for kind in KINDS:
+        for n, dt in ((1032, bf16), (1280, f16), (2056, bf16), (4104, f16), (8200, bf16), (516, f32), (2052, f32),
+                      (1025, bf16), (5001, f16), (4098, bf16)):
+            announce(f"five-vector shapes {kind} N={n} {dt}")
+            x, dy = make((19, n), dt, seed=n, scale=3.0)
             run_and_compare(kind, x, dy, f"{kind} N={n} {dt}")

@@ -111,6 +111,9 @@ bool shape_compiled(int which, bool aligned, bool ln16, Shape s) {
             THN_FWD_SHAPES_AS_BACKWARD(THN_MATCH)
         }
         THN_FWD_SHAPES_THREE(THN_MATCH)
+        if (which == kSoftmaxFwd || which == kSoftmaxBwd) {
+            THN_SM_SHAPES_FIVE(THN_MATCH)
+        }
     }
 #undef THN_MATCH
     return false;
@@ -563,6 +566,26 @@ int plan_launch(int which, int flavour, bool aligned, int64_t M, int64_t N, int 
         if ((which == kSoftmaxFwd || fills_three_16) && shape_compiled(which, aligned, ln16, three)) {
             s = three;
             narrow_forward_pair = which == kSoftmaxFwd;
+        }
+    }
+    // The softmax family over rows of 4 * t + 1 to 5 * t vectors, t = 32 ... 256 (THN_SM_SHAPES_FIVE): 5 x t vectors, one
+    // workgroup per compute unit on the 128-bit path, instead of 3 x 2t with a third to a sixth of the slots idle.
+    // Forward, 2^26 elements: bfloat16 N = 1032 52.7 -> 48.3 us, 1152 50.6 -> 47.3, 2056 59.5 -> 49.0, 2304 50.9 -> 47.5,
+    // 4104 62.5 -> 48.2, 4608 51.4 -> 48.2, 5120 50.9 -> 48.1; float32 N = 516 99.0 -> 94.0, 2052 115.0 -> 96.3; off the
+    // path N = 2050 56.9 -> 53.4, 4098 58.2 -> 51.7, 5001 60.0 -> 53.9.  The backward follows (the same rows per
+    // workgroup: forward + backward N = 1032 113.9 -> 106.1 us, 2056 110.8 -> 105.2, 8200 108.6 -> 103.9, 9216 103.6 ->
+    // 101.3, float32 516 220.3 -> 203.5, 1025 214.4 -> 201.5, off the path 5001 127.3 -> 111.1) except where it was
+    // measured to lose by itself more than the shared rows gain: rows of more than 4.5 * t vectors on the path (N =
+    // 1280, 2560, 5120: 0.2-0.7 %), float32 rows from t = 128 (N = 2052 207.7 -> 217.8 us) and rows just above 4 * t
+    // vectors off the path (N = 1025 116.6 -> 118.1).
+    if ((which == kSoftmaxFwd || which == kSoftmaxBwd) && N >= vec_elems && n_vecs > 128 && n_vecs <= 1280) {
+        int t = 32;
+        while (5 * t < n_vecs) t *= 2;
+        if (n_vecs > 4 * t) {
+            const bool bwd_keeps = (aligned && 2 * n_vecs > 9 * t) || (bytes >= 4 && t >= 128) ||
+                                   (!aligned && 8 * n_vecs <= 33 * t);
+            const Shape five{5, t, 256};
+            if ((which == kSoftmaxFwd || !bwd_keeps) && shape_compiled(which, aligned, ln16, five)) s = five;
         }
     }
     // The p-norm / normalize family at the same widths: the forward 3 x 16 / 3 x 32 in every storage type (normalize,

@@ -19,6 +19,11 @@ THN_DECLARE_SOFTMAX_LAUNCHERS(f16)
 THN_DECLARE_SOFTMAX_LAUNCHERS(bf16)
 THN_DECLARE_SOFTMAX_LAUNCHERS(f64)
 
+// Rows of 4 * TPR + 1 to 5 * TPR vectors (a width just above a power of two of vectors, and 5 * 2^k: 1032 ... 1280,
+// 2056 ... 2560, 4104 ... 5120, 8200 ... 10240 columns in 16-bit storage): 5 vectors per thread fill 4/5 or more of the
+// shape where 3 vectors on twice the threads fill 2/3 to 5/6.
+#define THN_SM_SHAPES_FIVE(X) X(5, 32, 256) X(5, 64, 256) X(5, 128, 256) X(5, 256, 256)
+
 #define THN_SM_CASE(KERNEL, ARGS_T, AL, K_, TPR_, BLOCK_)                                                      \
     if (s.k == K_ && s.tpr == TPR_ && s.block == BLOCK_) {                                                     \
         return is_log ? run_kernel<ARGS_T>(KERNEL<T, true, K_, TPR_, BLOCK_, AL>, a, grid, BLOCK_, st, occupancy) \
@@ -44,9 +49,11 @@ THN_DECLARE_SOFTMAX_LAUNCHERS(f64)
         if (aligned) {                                                                                          \
             THN_FWD_SHAPES(THN_SMF_AL)                                                                          \
             THN_FWD_SHAPES_THREE(THN_SMF_AL)                                                                    \
+            THN_SM_SHAPES_FIVE(THN_SMF_AL)                                                                      \
         } else if (a.n_cols >= TYPE::VEC) { \
             THN_FWD_SHAPES(THN_SMF_SC) \
             THN_FWD_SHAPES_THREE(THN_SMF_SC) \
+            THN_SM_SHAPES_FIVE(THN_SMF_SC) \
         } else { \
             using T = ElemIo<TYPE>; \
             THN_SMF_SC(4, 8, 256) \
@@ -59,9 +66,11 @@ THN_DECLARE_SOFTMAX_LAUNCHERS(f64)
         if (aligned) {                                                                                          \
             THN_FWD_SHAPES(THN_SMB_AL)                                                                          \
             THN_FWD_SHAPES_THREE(THN_SMB_AL)                                                                    \
+            THN_SM_SHAPES_FIVE(THN_SMB_AL)                                                                      \
         } else if (a.n_cols >= TYPE::VEC) { \
             THN_FWD_SHAPES(THN_SMB_SC) \
             THN_FWD_SHAPES_THREE(THN_SMB_SC) \
+            THN_SM_SHAPES_FIVE(THN_SMB_SC) \
         } else { \
             using T = ElemIo<TYPE>; \
             THN_SMB_SC(4, 8, 256) \
