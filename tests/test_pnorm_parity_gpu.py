@@ -336,7 +336,9 @@ def test_c_abi_direct_calls_and_errors():
 def row_shapes():
     text = open(os.path.join(ROOT, "triton-hub_amd", "csrc", "thn_pnorm_dispatch.h")).read()
     body = re.search(r"#define THN_ROW_SHAPES\(X\)(.*?)\n\n", text, re.S).group(1)
-    return [(int(k), int(t), int(b)) for k, t, b in re.findall(r"X\((\d+), (\d+), (\d+)\)", body)]
+    five = re.search(r"#define THN_PN_SHAPES_FIVE\(X\)(.*?)\n\n", text, re.S).group(1)    # forward, normalize backward
+    assert len(re.findall(r"X\(5, ", five)) == 4
+    return [(int(k), int(t), int(b)) for k, t, b in re.findall(r"X\((\d+), (\d+), (\d+)\)", body + five)]
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
@@ -361,6 +363,9 @@ def test_every_compiled_launch_shape(dtype):
                     for which in (4, 5, 6):
                         assert lib.thn_norm_set_launch_override(which, k, tpr, block, 0) == 0
                         q = query_launch(which, False, m, n, dtype)
+                        if k == 5 and which == 5:       # the norm backward has no 5-vector instances: keeps its own shape
+                            assert q[0] != 5
+                            continue
                         assert q[:3] == (k, tpr, block) and q[4] == (1 if on_path else 0), q
                     x, gn, gy = make((1, m, n), dtype, seed=k * 1000 + tpr)
                     for p in (1, 2, 3):
@@ -381,13 +386,14 @@ def test_launch_rules_of_16_bit_rows_off_the_128_bit_path():
     assert query_launch(4, True, 8192, 8191, bf16)[:4] == (2, 512, 512, cus)
     assert query_launch(4, False, 8192, 8191, bf16)[:3] == (4, 256, 256)
     assert query_launch(4, True, 8192, 8192, bf16)[:3] == (4, 256, 256)
-    for n, want in ((1025, (3, 64, 256)), (1152, (3, 64, 256)), (1281, (3, 64, 256)), (2050, (3, 128, 256)),
-                    (2304, (3, 128, 256)), (1280, (2, 128, 256)), (2560, (2, 256, 256)), (3072, (2, 256, 256)),
+    # (rows of 4 t + 1 to 5 t vectors off the path take 5 x t, below)
+    for n, want in ((1152, (3, 64, 256)), (1288, (2, 128, 256)), (1500, (3, 64, 256)), (2304, (3, 128, 256)),
+                    (2900, (3, 128, 256)), (1280, (2, 128, 256)), (2560, (2, 256, 256)), (3072, (2, 256, 256)),
                     (1536, (2, 128, 256)), (3999, (4, 128, 256))):
         assert query_launch(6, False, 1 << 15, n, bf16)[:3] == want, n
         assert query_launch(6, False, 1 << 15, n, f16)[:3] == want, n
     assert query_launch(6, False, 1 << 15, 516, f32)[:3] == (2, 128, 256)
-    for n in (4098, 6001, 8191):
+    for n in (5400, 6001, 8191):
         assert query_launch(6, False, 1 << 15, n, bf16)[2:4] == (512, cus), n
     # rows of 33 to 48 and 65 to 96 vectors: the forward 3 x 16 / 3 x 32 in every storage type, the 16-bit normalize
     # backward up to 40 and 80 vectors
@@ -405,7 +411,20 @@ def test_launch_rules_of_16_bit_rows_off_the_128_bit_path():
         for p in (1, 2, 3):
             compare_norm(x, gn, p, 1e-6, f"norm K={n} p={p}")
             compare_normalize(x, gy, p, 1e-6, f"normalize K={n} p={p}")
-    for n, dt in ((8191, bf16), (7001, f16), (1025, bf16), (1152, f16), (2050, bf16), (2304, bf16), (3999, f16)):
+    # rows of 4 t + 1 to 5 t vectors: the normalize forward 5 x t with one workgroup per compute unit (t up to 128), the
+    # 16-bit backward 5 x t off the path and just above 4 t vectors on it
+    for n, dt, f, b in ((1032, bf16, (5, 32, 256), (3, 64, 256)), (2056, bf16, (5, 64, 256), (5, 64, 256)),
+                        (4104, f16, (5, 128, 256), (5, 128, 256)), (5120, bf16, (5, 128, 256), (2, 512, 512)),
+                        (8200, bf16, (5, 256, 256), (5, 256, 256)), (10240, bf16, (3, 512, 512), (2, 1024, 1024)),
+                        (516, f32, (5, 32, 256), (2, 128, 256)), (2052, f32, (5, 128, 256), (2, 512, 512)),
+                        (1025, bf16, (5, 32, 256), (5, 32, 256)), (2050, f16, (5, 64, 256), (5, 64, 256)),
+                        (5001, bf16, (5, 128, 256), (5, 128, 256))):
+        q = query_launch(4, True, 1 << 15, n, dt)
+        assert q[:3] == f and (q[3] <= cus or f[0] != 5), (n, dt, q)
+        assert query_launch(6, False, 1 << 15, n, dt)[:3] == b, (n, dt)
+        assert query_launch(4, False, 1 << 15, n, dt)[0] != 5, (n, dt)         # the p-norm by itself keeps its shapes
+    for n, dt in ((8191, bf16), (7001, f16), (1025, bf16), (1152, f16), (2050, bf16), (2304, bf16), (3999, f16),
+                  (1032, bf16), (2056, f16), (4104, bf16), (8200, f16), (516, f32), (2052, f32), (5001, bf16)):
         announce(f"launch rules K={n} {dt}")
         x, gn, gy = make((2, 11, n), dt, seed=n)
         for p in (1, 2, 3):

@@ -104,6 +104,9 @@ bool shape_compiled(int which, bool aligned, bool ln16, Shape s) {
         }
     } else if (which >= kPnormFwd) {
         THN_ROW_SHAPES(THN_MATCH)
+        if (which != kPnormBwd) {
+            THN_PN_SHAPES_FIVE(THN_MATCH)
+        }
     } else {
         THN_FWD_SHAPES(THN_MATCH)
         if (which == kNormFwd) {
@@ -588,6 +591,25 @@ int plan_launch(int which, int flavour, bool aligned, int64_t M, int64_t N, int 
             if ((which == kSoftmaxFwd || !bwd_keeps) && shape_compiled(which, aligned, ln16, five)) s = five;
         }
     }
+    // normalize over the same rows (THN_PN_SHAPES_FIVE): the forward 5 x t vectors, t = 32 ... 128, ONE workgroup per
+    // compute unit (2^26 elements, forward: bfloat16 N = 1032 51.8 -> 49.4 us, 2056 57.3 -> 49.6, 4104 61.1 -> 48.2, 5120
+    // 48.6 -> 47.0; float32 N = 516 101.4 -> 93.7, 2052 114.8 -> 92.8; off the path N = 4098 56.8 -> 49.3, 5001 59.9 ->
+    // 52.6); the 16-bit backward 5 x t as well off the path and, from t = 64, for rows just above 4 * t vectors on it
+    // (forward + backward: N = 2056 117.5 -> 110.4 us, 4104 123.9 -> 108.8, 8200 106.7 -> 104.6; off the path N = 1025
+    // 124.5 -> 119.7, 4098 118.6 -> 109.8, 5001 133.8 -> 113.8; fuller rows on the path and float32 rows lose 1-5 % in the
+    // backward that way).  The p-norm by itself keeps its shapes.
+    if ((which == kNormalizeBwd || (which == kPnormFwd && (flavour & 4) != 0)) && N >= vec_elems && n_vecs > 128 &&
+        n_vecs <= 1280) {
+        int t = 32;
+        while (5 * t < n_vecs) t *= 2;
+        if (n_vecs > 4 * t) {
+            const bool just_above = 8 * n_vecs <= 33 * t;
+            const bool bwd_takes = bytes == 2 && (!aligned || (just_above && t >= 64));
+            const bool fwd_takes = t <= 128 || (bwd_takes && aligned);
+            const Shape five{5, t, 256};
+            if ((which == kPnormFwd ? fwd_takes : bwd_takes) && shape_compiled(which, aligned, ln16, five)) s = five;
+        }
+    }
     // The p-norm / normalize family at the same widths: the forward 3 x 16 / 3 x 32 in every storage type (normalize,
     // 2^26 elements, forward: bfloat16 N = 264 59.2 -> 52.9 us, 272 56.5 -> 52.3, 384 49.2 -> 47.0, 520 58.2 -> 53.6;
     // float32 N = 132 115.0 -> 105.6, 160 96.5 -> 92.4, 260 114.7 -> 107.5, 384 95.8 -> 92.9); the 16-bit normalize
@@ -761,6 +783,7 @@ int plan_launch(int which, int flavour, bool aligned, int64_t M, int64_t N, int 
             cap = 2;
         }
         if ((narrow_forward_pair || narrow_backward_pair) && cap < 2) cap = 2;
+        if (which == kPnormFwd && s.k == 5) cap = 1;       // 1280 vectors per workgroup step: see THN_PN_SHAPES_FIVE above
     }
     if (cap < bpc) bpc = cap;
     const int rows_per_block = s.block / s.tpr;

@@ -19,6 +19,10 @@ namespace thn {
     X(2, 512, 512) X(3, 512, 512) X(4, 512, 512)                                     \
     X(2, 1024, 1024) X(3, 1024, 1024) X(4, 1024, 1024)
 
+// Forward and normalize backward only: 5 vectors per thread for rows of 4 * TPR + 1 to 5 * TPR vectors, as in the
+// softmax family (THN_SM_SHAPES_FIVE).
+#define THN_PN_SHAPES_FIVE(X) X(5, 32, 256) X(5, 64, 256) X(5, 128, 256) X(5, 256, 256)
+
 // mode: kP1 / kP2 / kPInt.  task of the looping kernels: 0 norm forward, 1 normalize forward.
 #define THN_DECLARE_PNORM_LAUNCHERS(NAME)                                                                       \
     int launch_pnorm_fwd_##NAME(int mode, bool normalize, bool aligned, Shape s, const PnormFwdArgs& a,         \
@@ -66,8 +70,10 @@ THN_DECLARE_PNORM_LAUNCHERS(f64)
         using T = TYPE;                                                                                         \
         if (aligned) {                                                                                          \
             THN_ROW_SHAPES(THN_PNF_AL)                                                                          \
+            THN_PN_SHAPES_FIVE(THN_PNF_AL)                                                                      \
         } else if (a.n_cols >= TYPE::VEC) { \
             THN_ROW_SHAPES(THN_PNF_SC) \
+            THN_PN_SHAPES_FIVE(THN_PNF_SC) \
         } else { \
             using T = ElemIo<TYPE>; \
             THN_PNF_SC(4, 8, 256) \
@@ -98,8 +104,10 @@ THN_DECLARE_PNORM_LAUNCHERS(f64)
         using T = TYPE;                                                                                         \
         if (aligned) {                                                                                          \
             THN_ROW_SHAPES(THN_NZB_AL)                                                                          \
+            THN_PN_SHAPES_FIVE(THN_NZB_AL)                                                                      \
         } else if (a.n_cols >= TYPE::VEC) { \
             THN_ROW_SHAPES(THN_NZB_SC) \
+            THN_PN_SHAPES_FIVE(THN_NZB_SC) \
         } else { \
             using T = ElemIo<TYPE>; \
             THN_NZB_SC(4, 8, 256) \
